@@ -1,0 +1,915 @@
+"""
+Typed DAG -> HIP C++ for gfx950.
+
+The generated text is appended to ``neon_device.h`` and compiled with hiprtc.
+It replaces the reference's string templates (cuda_templates.py:45-135 filled
+in by float_ew.py:268-617) but is organised around how CDNA4 wants to be fed
+rather than around one-thread-block-per-line:
+
+  * every global access is one ``nh_raw<T,V>`` / ``nh_out<T,V>`` tile per lane:
+    V consecutive elements, 16 bytes wherever layout and alignment allow;
+  * lanes always run along the contiguous (column) axis, for axis-0 reductions
+    too, where the reference walked down a strided column per thread
+    (float_ew.py:709-711);
+  * a line that has to be swept more than once (softmax, variance,
+    normalisation) is loaded once and kept in registers in storage format;
+  * reductions are wave64 DPP all-reduces; LDS only joins waves; workgroups
+    that share a long column strip combine through a ticket, never by waiting.
+
+Kernel families
+  ``ew``       no reduction; one or several assign statements per launch
+  ``row``      reductions along axis 1; a team of LX lanes owns a row
+  ``col``      reductions along axis 0; a workgroup owns a strip of columns
+               and all rows, which stay in registers
+  ``colsplit`` one level of axis-0 reductions over many rows; (strip x row
+               chunk) workgroups, partials folded by the last one to finish
+
+Arithmetic is fp32 whatever the storage type.  Parameters, in order: per
+tensor slot ``(pointer, row stride, column stride)`` in elements, one float per
+constant slot, ``R``, ``C``, then family-specific extras.
+"""
+import hashlib
+
+from neon_amd.backends.hip.optree_ir import DTYPE_CODE, used_nodes
+
+CTYPE = {"f4": "float", "f2": "nh_f16", "i4": "nh_i32", "u4": "nh_u32",
+         "i2": "nh_i16", "u2": "nh_u16", "i1": "nh_i8", "u1": "nh_u8"}
+
+_BIN = {"add": "({0} + {1})", "sub": "({0} - {1})", "mul": "({0} * {1})",
+        "div": "({0} / {1})",
+        "eq": "(({0} == {1}) ? 1.0f : 0.0f)", "ne": "(({0} != {1}) ? 1.0f : 0.0f)",
+        "lt": "(({0} < {1}) ? 1.0f : 0.0f)", "le": "(({0} <= {1}) ? 1.0f : 0.0f)",
+        "gt": "(({0} > {1}) ? 1.0f : 0.0f)", "ge": "(({0} >= {1}) ? 1.0f : 0.0f)",
+        "pow": "powf({0}, {1})", "minimum": "nh_min({0}, {1})",
+        "maximum": "nh_max({0}, {1})"}
+_UN = {"neg": "(-{0})", "abs": "__builtin_fabsf({0})", "sgn": "nh_sgn({0})",
+       "sqrt": "sqrtf({0})", "sqr": "nh_sqr({0})", "exp": "expf({0})",
+       "log": "logf({0})", "exp2": "exp2f({0})", "log2": "log2f({0})",
+       "sig": "nh_sig({0})", "sig2": "nh_sig2({0})", "tanh": "tanhf({0})",
+       "tanh2": "nh_tanh2({0})", "safelog": "nh_safelog({0})",
+       "rint": "rintf({0})", "finite": "nh_finite({0})", "ident": "({0})"}
+_RED_OP = {"sum": "nh_op_sum", "max": "nh_op_max", "min": "nh_op_min",
+           "argmax": "nh_op_argmax", "argmin": "nh_op_argmin"}
+
+
+class Spec(object):
+    """Everything the launcher needs for one generated kernel."""
+
+    def __init__(self, family, name, source, fmt, block, lds_bytes, params):
+        self.family = family
+        self.name = name
+        self.source = source
+        self.fmt = fmt                # struct format of the packed arguments
+        self.block = block            # threads per workgroup
+        self.lds_bytes = lds_bytes    # static LDS is declared in the source; kept for reports
+        self.params = params          # tiling parameters (dict) used to size the grid
+
+
+class _Lines(object):
+    def __init__(self):
+        self.out = []
+        self.ind = 0
+
+    def __call__(self, text=""):
+        self.out.append(("    " * self.ind + text) if text else "")
+
+    def open(self, text):
+        self(text + " {")
+        self.ind += 1
+
+    def close(self, tail=""):
+        self.ind -= 1
+        self("}" + tail)
+
+    def text(self):
+        return "\n".join(self.out) + "\n"
+
+
+class _Gen(object):
+    """State shared by the family emitters for one program."""
+
+    def __init__(self, prog, V):
+        self.prog = prog
+        self.V = V
+        self.R, self.C = prog.domain
+        self.axis = prog.axis
+        self.L = _Lines()
+
+    # -- parameters -----------------------------------------------------------------
+    def slot_ctype(self, slot):
+        return CTYPE[DTYPE_CODE[slot.dtype]]
+
+    def col_unit(self, slot):
+        """True when the slot's column stride is the literal 1."""
+        return slot.shape[1] > 1 and slot.strides[1] == 1
+
+    def param_list(self, extras):
+        ps, fmt = [], ""
+        no_alias = not self.prog.overlapping_slots()
+        for t in self.prog.tensors:
+            qual = "" if t.written else "const "
+            restrict = " __restrict__" if no_alias else ""
+            ps.append("%s%s*%s a%d" % (qual, self.slot_ctype(t), restrict, t.index))
+            ps.append("long long sr%d" % t.index)
+            ps.append("long long sc%d" % t.index)
+            fmt += "Pqq"
+        for i in range(len(self.prog.consts)):
+            ps.append("float k%d" % i)
+            fmt += "f"
+        ps += ["int R", "int C"]
+        fmt += "ii"
+        for decl, f in extras:
+            ps.append(decl)
+            fmt += f
+        return ", ".join(ps), "@" + fmt
+
+    # -- addresses ------------------------------------------------------------------
+    def addr(self, slot, r, c):
+        """Element address of (r, c) in a slot, honouring broadcast dims."""
+        parts = ["a%d" % slot.index]
+        if slot.shape[0] > 1:
+            parts.append("(long long)(%s) * sr%d" % (r, slot.index))
+        if slot.shape[1] > 1:
+            if self.col_unit(slot):
+                parts.append("(long long)(%s)" % c)
+            else:
+                parts.append("(long long)(%s) * sc%d" % (c, slot.index))
+        return " + ".join(parts)
+
+    # -- loads -------------------------------------------------------------------------
+    def leaf_nodes(self, nodes):
+        return [n for n in nodes if n.kind in ("T", "H")]
+
+    def tile_name(self, n, sfx):
+        return ("x%d%s" % (n.slot, sfx)) if n.kind == "T" else ("h%d_%d%s" % (n.slot, n.axis, sfx))
+
+    def tile_width(self, n, V):
+        if n.kind == "T":
+            return V if self.prog.tensors[n.slot].shape[1] > 1 else 1
+        return V if n.axis == 0 else 1
+
+    def tile_type(self, n, V):
+        slot = self.prog.tensors[n.slot]
+        return "nh_raw<%s, %d>" % (self.slot_ctype(slot), self.tile_width(n, V))
+
+    def tile_addr(self, n, r, c):
+        slot = self.prog.tensors[n.slot]
+        if n.kind == "T":
+            return self.addr(slot, r, c)
+        # one-hot index vector: flat, contiguous; indexed by the position along
+        # the axis that is *not* hot
+        return "a%d + (long long)(%s)" % (slot.index, c if n.axis == 0 else r)
+
+    def emit_load(self, n, r, c, V, sfx, declare=True, target=None):
+        name = target or self.tile_name(n, sfx)
+        if declare:
+            self.L("%s %s;" % (self.tile_type(n, V), name))
+        self.L("%s.load(%s);" % (name, self.tile_addr(n, r, c)))
+
+    # -- expressions -----------------------------------------------------------------
+    def leaf_value(self, n, tile, r, c, V):
+        w = self.tile_width(n, V)
+        j = "j" if w > 1 else "0"
+        if n.kind == "T":
+            return "%s.get(%s)" % (tile, j)
+        if n.axis == 0:
+            return "((%s.geti(%s) == (int)(%s)) ? 1.0f : 0.0f)" % (tile, j, r)
+        return "((%s.geti(0) == (int)((%s) + j)) ? 1.0f : 0.0f)" % (tile, c)
+
+    def emit_exprs(self, nodes, ref, skip):
+        """Emit ``const float t<id> = ...;`` for E nodes of ``nodes`` not in
+        ``skip``; ``ref(node)`` names the value of any operand."""
+        for n in nodes:
+            if n.kind != "E" or n.nid in skip:
+                continue
+            a = [ref(x) for x in n.args]
+            if n.op.startswith("quant:"):
+                e = "nh_quant<%s>(%s)" % (CTYPE[n.op.split(":")[1]], a[0])
+            elif n.op == "zero_index":
+                e = "0.0f"
+            elif len(a) == 1:
+                e = _UN[n.op].format(*a)
+            else:
+                e = _BIN[n.op].format(*a)
+            self.L("const float t%d = %s;" % (n.nid, e))
+
+
+def _needed(targets, available):
+    """Nodes to evaluate for ``targets`` given already-available reductions."""
+    seen = {}
+    todo = list(targets)
+    while todo:
+        n = todo.pop()
+        if n.nid in seen or n.nid in available:
+            continue
+        seen[n.nid] = n
+        todo.extend(n.args)
+    return [seen[k] for k in sorted(seen)]
+
+
+def _kernel_name(family, source_body):
+    return "nk_%s_%s" % (family, hashlib.sha1(source_body.encode()).hexdigest()[:16])
+
+
+def _finish(family, g, head, fmt, block, lds, params):
+    body = g.L.text()
+    name = _kernel_name(family, head + body + repr(sorted(params.items())))
+    src = head.replace("@NAME@", name) + body
+    return Spec(family, name, src, fmt, block, lds, params)
+
+
+# =====================================================================================
+# family: ew
+# =====================================================================================
+def gen_ew(prog, V, LX, LY, UC, UR, tail):
+    """Elementwise kernel.  Workgroup = LX column-lanes x LY row-lanes; a lane
+    handles UC column tiles x UR rows per step, all loads issued before the
+    first store.  ``tail``: emit a scalar path for a last partial tile
+    (only needed when C % V != 0, which the planner allows for single-row
+    domains)."""
+    g = _Gen(prog, V)
+    L = g.L
+    T = LX * LY
+    params, fmt = g.param_list([("int row_tiles", "i")])
+    head = ('extern "C" __global__ __launch_bounds__(%d) void @NAME@(%s)\n' % (T, params))
+    roots = [st.root for st in prog.statements]
+    nodes = _needed(roots, {})
+    leaves = g.leaf_nodes(nodes)
+
+    def ref_for(sfx, r, c, Vv):
+        def ref(n):
+            if n.kind == "C":
+                return "k%d" % n.slot
+            if n.kind in ("T", "H"):
+                return g.leaf_value(n, g.tile_name(n, sfx), r, c, Vv)
+            return "t%d" % n.nid
+        return ref
+
+    def body(sfx, r, c, Vv, loads_only=False, compute_only=False):
+        if not compute_only:
+            for n in leaves:
+                g.emit_load(n, r, c, Vv, sfx, declare=False)
+        if loads_only:
+            return
+        for st in prog.statements:
+            w = Vv if st.out.shape[1] > 1 else 1
+            L("nh_out<%s, %d> o%d%s; o%d%s.clear();" % (g.slot_ctype(st.out), w, st.out.index, sfx,
+                                                       st.out.index, sfx))
+        if Vv > 1:
+            L("#pragma unroll")
+        L.open("for (int j = 0; j < %d; ++j)" % Vv)
+        g.emit_exprs(nodes, ref_for(sfx, r, c, Vv), {})
+        for st in prog.statements:
+            w = Vv if st.out.shape[1] > 1 else 1
+            jj = "j" if w > 1 else "0"
+            val = ref_for(sfx, r, c, Vv)(st.root)
+            if w == 1 and Vv > 1:
+                L("if (j == 0) o%d%s.set(0, %s);" % (st.out.index, sfx, val))
+            else:
+                L("o%d%s.set(%s, %s);" % (st.out.index, sfx, jj, val))
+        L.close()
+        for st in prog.statements:
+            L("o%d%s.store(%s);" % (st.out.index, sfx, g.addr(st.out, r, c)))
+
+    L.open("")
+    L("const int tx = threadIdx.x %% %d, ty = threadIdx.x / %d;" % (LX, LX))
+    L.open("for (int rt = blockIdx.y; rt < row_tiles; rt += gridDim.y)")
+    units = [(uc, ur) for uc in range(UC) for ur in range(UR)]
+    for (uc, ur) in units:
+        s = "_%d_%d" % (uc, ur)
+        L("const long long c%s = ((long long)(blockIdx.x * %d + %d) * %d + tx) * %d;" % (s, UC, uc, LX, V))
+        L("const long long r%s = ((long long)rt * %d + %d) * %d + ty;" % (s, UR, ur, LY))
+        L("const bool ok%s = (r%s < R) && (c%s + %d <= C);" % (s, s, s, V))
+        for n in leaves:
+            L("%s %s; %s.zero();" % (g.tile_type(n, V), g.tile_name(n, s), g.tile_name(n, s)))
+    for (uc, ur) in units:
+        s = "_%d_%d" % (uc, ur)
+        L.open("if (ok%s)" % s)
+        body(s, "r" + s, "c" + s, V, loads_only=True)
+        L.close()
+    for (uc, ur) in units:
+        s = "_%d_%d" % (uc, ur)
+        L.open("if (ok%s)" % s)
+        body(s, "r" + s, "c" + s, V, compute_only=True)
+        L.close()
+        if tail and V > 1:
+            L.open("else if (r%s < R && c%s < C)" % (s, s))
+            L.open("for (long long e = c%s; e < C; ++e)" % s)
+            for n in leaves:
+                L("%s %s;" % (g.tile_type(n, 1), g.tile_name(n, "_e")))
+            body("_e", "r" + s, "e", 1)
+            L.close()
+            L.close()
+    L.close()
+    L.close()
+    return _finish("ew", g, head, fmt, T, 0,
+                   dict(V=V, LX=LX, LY=LY, UC=UC, UR=UR, tail=bool(tail)))
+
+
+# =====================================================================================
+# shared pieces of the reduction families
+# =====================================================================================
+def _levels(prog):
+    """reductions grouped by the sweep that produces them: sweep s yields the
+    reductions of level s+1."""
+    per = {}
+    for n in prog.nodes:
+        if n.kind == "R":
+            per.setdefault(n.level - 1, []).append(n)
+    return per
+
+
+def _live_reductions(prog):
+    roots = [st.root for st in prog.statements]
+    return [n for n in used_nodes(roots) if n.kind == "R"]
+
+
+class _RedGen(_Gen):
+    """Common machinery of row / col / colsplit."""
+
+    def __init__(self, prog, V):
+        super(_RedGen, self).__init__(prog, V)
+        self.col_axis = (prog.axis == 0)   # reductions leave one value per column
+
+    # value of a finished reduction at element j of the lane's tile
+    def red_ref(self, n):
+        if self.col_axis:
+            return ("(float)ri%d[j]" % n.nid) if n.is_index else ("rv%d[j]" % n.nid)
+        return ("(float)ri%d" % n.nid) if n.is_index else ("rv%d" % n.nid)
+
+    def make_ref(self, sfx, r, c, Vv, tiles=None):
+        def ref(n):
+            if n.kind == "C":
+                return "k%d" % n.slot
+            if n.kind in ("T", "H"):
+                tile = tiles[n.nid] if tiles and n.nid in tiles else self.tile_name(n, sfx)
+                return self.leaf_value(n, tile, r, c, Vv)
+            if n.kind == "R":
+                return self.red_ref(n)
+            return "t%d" % n.nid
+        return ref
+
+    def declare_acc(self, n):
+        L = self.L
+        op = _RED_OP[n.op]
+        if self.col_axis:
+            if n.is_index:
+                L("nh_pair acc%d[%d];" % (n.nid, self.V))
+            else:
+                L("float acc%d[%d];" % (n.nid, self.V))
+            L("#pragma unroll")
+            L("for (int j = 0; j < %d; ++j) acc%d[j] = %s::init();" % (self.V, n.nid, op))
+        else:
+            L("%s acc%d = %s::init();" % ("nh_pair" if n.is_index else "float", n.nid, op))
+
+    def accumulate(self, n, val, index):
+        """fold one element into the lane's accumulator (inside the j loop)"""
+        op = _RED_OP[n.op]
+        acc = ("acc%d[j]" % n.nid) if self.col_axis else ("acc%d" % n.nid)
+        if n.is_index:
+            self.L("%s::step(%s, %s, (int)(%s));" % (op, acc, val, index))
+        else:
+            self.L("%s = %s::f(%s, %s);" % (acc, op, acc, val))
+
+
+# =====================================================================================
+# family: row  (axis 1)
+# =====================================================================================
+def gen_row(prog, V, LX, LY, NCH):
+    """Axis-1 reductions.  A team of LX lanes (a power of two up to 64, or the
+    whole workgroup) owns one row; the workgroup holds LY rows.  A lane visits
+    column tiles tx, tx+LX, ...; with ``NCH`` > 0 that loop has a fixed trip
+    count and the tiles loaded in the first sweep stay in registers for the
+    later ones; with ``NCH`` == 0 every sweep streams the row again."""
+    g = _RedGen(prog, V)
+    L = g.L
+    T = LX * LY
+    assert LX <= 64 or LY == 1
+    resident = NCH > 0
+    params, fmt = g.param_list([])
+    head = ('extern "C" __global__ __launch_bounds__(%d) void @NAME@(%s)\n' % (T, params))
+    per_level = _levels(prog)
+    nsweeps = prog.nlevels
+    full_out = [st for st in prog.statements if st.out.shape[1] > 1 or g.C == 1]
+    line_out = [st for st in prog.statements if st not in full_out]
+    done = {}      # nid -> node of reductions already finished
+    cached = {}    # leaf nid -> resident tile array name
+
+    L.open("")
+    if LX > 64:
+        L("__shared__ float s_f[%d];" % (T // 64))
+        L("__shared__ nh_pair s_p[%d];" % (T // 64))
+    L("const int tx = threadIdx.x %% %d, ty = threadIdx.x / %d;" % (LX, LX))
+    L("const long long r = (long long)blockIdx.x * %d + ty;" % LY)
+    L("const bool row_ok = r < R;")
+    L("const long long rr = row_ok ? r : 0;")   # address clamp for idle teams
+    if not resident:
+        L("const int nch = (C + %d - 1) / %d;" % (LX * V, LX * V))
+
+    def chunk_loop_open():
+        if resident:
+            L("#pragma unroll")
+            L.open("for (int k = 0; k < %d; ++k)" % NCH)
+        else:
+            L("#pragma unroll 2")
+            L.open("for (int k = 0; k < nch; ++k)")
+        L("const long long c = ((long long)k * %d + tx) * %d;" % (LX, V))
+        L("const bool ok = row_ok && (c < C);")
+
+    line_tiles = {}   # leaf nid -> tile that does not change along the row
+
+    def varies_in_loop(n):
+        return g.tile_width(n, 2) == 2      # tile spans columns
+
+    def load_leaves(leaves, first_use):
+        """make tiles for ``leaves`` available inside the chunk loop"""
+        tiles = {}
+        for n in leaves:
+            if not varies_in_loop(n):
+                tiles[n.nid] = line_tiles[n.nid]
+                continue
+            if resident and n.nid in cached:
+                tiles[n.nid] = "%s[k]" % cached[n.nid]
+                continue
+            if resident:
+                name = "keep%d" % n.nid
+                cached[n.nid] = name
+                tiles[n.nid] = "%s[k]" % name
+                L("if (ok) %s[k].load(%s); else %s[k].zero();" % (name, g.tile_addr(n, "rr", "c"), name))
+            else:
+                name = g.tile_name(n, "_s")
+                tiles[n.nid] = name
+                L("%s %s; %s.zero();" % (g.tile_type(n, V), name, name))
+                L("if (ok) %s.load(%s);" % (name, g.tile_addr(n, "rr", "c")))
+        return tiles
+
+    def declare_tiles(leaves):
+        """function-scope declarations needed before a sweep's loop"""
+        for n in leaves:
+            if not varies_in_loop(n):
+                if n.nid not in line_tiles:
+                    name = "line%d" % n.nid
+                    line_tiles[n.nid] = name
+                    L("%s %s;" % (g.tile_type(n, V), name))
+                    L("%s.load(%s);" % (name, g.tile_addr(n, "rr", "0")))
+            elif resident and n.nid not in cached:
+                L("%s keep%d[%d];" % (g.tile_type(n, V), n.nid, NCH))
+        if resident:
+            for nid, name in cached.items():
+                L("#pragma unroll")
+                L("for (int k = 0; k < %d; ++k) %s[k].keep();" % (NCH, name))
+
+    # operands that do not change along the row are fetched once, up front, so
+    # their latency overlaps the first sweep
+    declare_tiles([n for n in g.leaf_nodes(used_nodes([st.root for st in prog.statements]))
+                   if not varies_in_loop(n)])
+
+    for s in range(nsweeps):
+        reds = [n for n in per_level.get(s, [])]
+        if not reds:
+            continue
+        args = [n.args[0] for n in reds]
+        nodes = _needed(args, done)
+        leaves = g.leaf_nodes(nodes)
+        declare_tiles(leaves)
+        for n in reds:
+            g.declare_acc(n)
+        chunk_loop_open()
+        tiles = load_leaves(leaves, True)
+        L.open("if (ok)")
+        if V > 1:
+            L("#pragma unroll")
+        L.open("for (int j = 0; j < %d; ++j)" % V)
+        ref = g.make_ref("_s", "rr", "c", V, tiles)
+        g.emit_exprs(nodes, ref, done)
+        for n in reds:
+            g.accumulate(n, ref(n.args[0]), "c + j")
+        L.close()
+        L.close()
+        L.close()
+        for n in reds:
+            op = _RED_OP[n.op]
+            ty_ = "nh_pair" if n.is_index else "float"
+            if LX <= 64:
+                L("const %s red%d = nh_wave_allreduce<%s, %d, %s>(acc%d);" % (ty_, n.nid, op, LX, ty_, n.nid))
+            else:
+                L("const %s red%d = nh_block_allreduce<%s, %d, %s>(acc%d, %s);"
+                  % (ty_, n.nid, op, T // 64, ty_, n.nid, "s_p" if n.is_index else "s_f"))
+            if n.is_index:
+                L("const int ri%d = red%d.i;" % (n.nid, n.nid))
+            else:
+                L("const float rv%d = red%d;" % (n.nid, n.nid))
+            done[n.nid] = n
+
+    # outputs that have one value per row
+    if line_out:
+        roots = [st.root for st in line_out]
+        nodes = _needed(roots, done)
+        leaves = g.leaf_nodes(nodes)
+        L.open("if (row_ok && tx == 0)")
+        for n in leaves:
+            g.emit_load(n, "r", "0", 1, "_l")
+        L.open("")
+        L("const int j = 0; (void)j;")
+        ref = g.make_ref("_l", "r", "0", 1)
+        g.emit_exprs(nodes, ref, done)
+        for st in line_out:
+            L("nh_out<%s, 1> o%d; o%d.clear();" % (g.slot_ctype(st.out), st.out.index, st.out.index))
+            if st.root.kind == "R" and st.root.is_index:
+                L("o%d.seti(0, ri%d);" % (st.out.index, st.root.nid))
+            else:
+                L("o%d.set(0, %s);" % (st.out.index, ref(st.root)))
+            L("o%d.store(%s);" % (st.out.index, g.addr(st.out, "r", "0")))
+        L.close()
+        L.close()
+
+    # outputs with the full shape: one more sweep
+    if full_out:
+        roots = [st.root for st in full_out]
+        nodes = _needed(roots, done)
+        leaves = g.leaf_nodes(nodes)
+        declare_tiles(leaves)
+        chunk_loop_open()
+        tiles = load_leaves(leaves, False)
+        L.open("if (ok)")
+        for st in full_out:
+            L("nh_out<%s, %d> o%d; o%d.clear();" % (g.slot_ctype(st.out), V, st.out.index, st.out.index))
+        if V > 1:
+            L("#pragma unroll")
+        L.open("for (int j = 0; j < %d; ++j)" % V)
+        ref = g.make_ref("_s", "rr", "c", V, tiles)
+        g.emit_exprs(nodes, ref, done)
+        for st in full_out:
+            if st.root.kind == "R" and st.root.is_index:
+                L("o%d.seti(j, ri%d);" % (st.out.index, st.root.nid))
+            else:
+                L("o%d.set(j, %s);" % (st.out.index, ref(st.root)))
+        L.close()
+        for st in full_out:
+            L("o%d.store(%s);" % (st.out.index, g.addr(st.out, "r", "c")))
+        L.close()
+        L.close()
+    L.close()
+    return _finish("row", g, head, fmt, T, 0, dict(V=V, LX=LX, LY=LY, NCH=NCH))
+
+
+# =====================================================================================
+# families: col / colsplit  (axis 0)
+# =====================================================================================
+def _emit_col_fold(g, L, n, LX, LY, T, V, src, dst_decl=True):
+    """Join the row-lanes of every column of the workgroup.  ``src`` is the
+    per-lane accumulator array; afterwards every lane holds the result in
+    rv<id>[] / ri<id>[].  Lanes of one wave that share a column tile are
+    folded with lane-xor exchanges first; LDS then joins the wave groups in
+    row order."""
+    op = _RED_OP[n.op]
+    ty_ = "nh_pair" if n.is_index else "float"
+    if LX < 64:
+        stride = LX
+        while stride < 64:
+            L("#pragma unroll")
+            L("for (int j = 0; j < %d; ++j) %s[j] = %s::f(%s[j], nh_lane_xor<%d>(%s[j]));"
+              % (V, src, op, src, stride, src))
+            stride *= 2
+        WY = T // 64
+        wy = "(threadIdx.x >> 6)"
+        writer = "((threadIdx.x & 63) < %d)" % LX
+    else:
+        WY = LY
+        wy = "ty"
+        writer = "true"
+    if dst_decl:
+        if n.is_index:
+            L("int ri%d[%d];" % (n.nid, V))
+        else:
+            L("float rv%d[%d];" % (n.nid, V))
+    buf = "s_p" if n.is_index else "s_f"
+    if WY == 1:
+        L("#pragma unroll")
+        if n.is_index:
+            L("for (int j = 0; j < %d; ++j) ri%d[j] = %s[j].i;" % (V, n.nid, src))
+        else:
+            L("for (int j = 0; j < %d; ++j) rv%d[j] = %s[j];" % (V, n.nid, src))
+        return
+    L.open("if (%s)" % writer)
+    L("#pragma unroll")
+    L("for (int j = 0; j < %d; ++j) %s[%s][tx * %d + j] = %s[j];" % (V, buf, wy, V, src))
+    L.close()
+    L("__syncthreads();")
+    L("#pragma unroll")
+    L.open("for (int j = 0; j < %d; ++j)" % V)
+    L("%s f = %s[0][tx * %d + j];" % (ty_, buf, V))
+    L("for (int y = 1; y < %d; ++y) f = %s::f(f, %s[y][tx * %d + j]);" % (WY, op, buf, V))
+    if n.is_index:
+        L("ri%d[j] = f.i; %s[j] = f;" % (n.nid, src))
+    else:
+        L("rv%d[j] = f; %s[j] = f;" % (n.nid, src))
+    L.close()
+    L("__syncthreads();")
+
+
+def _col_lds(L, LX, LY, T, V, any_index):
+    WY = (T // 64) if LX < 64 else LY
+    L("__shared__ float s_f[%d][%d];" % (WY, LX * V + 1))
+    if any_index:
+        L("__shared__ nh_pair s_p[%d][%d];" % (WY, LX * V + 1))
+    return WY * (LX * V + 1) * (4 + (8 if any_index else 0))
+
+
+def gen_col(prog, V, LX, LY, NR):
+    """Axis-0 reductions with all rows of a column strip inside one workgroup
+    (LX column-lanes x LY row-lanes, NR rows per lane, kept in registers)."""
+    g = _RedGen(prog, V)
+    L = g.L
+    T = LX * LY
+    params, fmt = g.param_list([])
+    head = ('extern "C" __global__ __launch_bounds__(%d) void @NAME@(%s)\n' % (T, params))
+    per_level = _levels(prog)
+    nsweeps = prog.nlevels
+    full_out = [st for st in prog.statements if st.out.shape[0] > 1 or g.R == 1]
+    line_out = [st for st in prog.statements if st not in full_out]
+    any_index = any(n.is_index for n in prog.nodes if n.kind == "R")
+    done, cached = {}, {}
+
+    L.open("")
+    lds = _col_lds(L, LX, LY, T, V, any_index)
+    L("const int tx = threadIdx.x %% %d, ty = threadIdx.x / %d;" % (LX, LX))
+    L("const long long c = ((long long)blockIdx.x * %d + tx) * %d;" % (LX, V))
+    L("const bool col_ok = c < C;")
+    L("const long long cc = col_ok ? c : 0;")
+
+    def row_loop_open():
+        L("#pragma unroll")
+        L.open("for (int i = 0; i < %d; ++i)" % NR)
+        L("const long long r = (long long)i * %d + ty;" % LY)
+        L("const bool ok = col_ok && (r < R);")
+
+    def keep_all():
+        for nid, name in cached.items():
+            L("#pragma unroll")
+            L("for (int i = 0; i < %d; ++i) %s[i].keep();" % (NR, name))
+
+    line_tiles = {}   # leaf nid -> tile that does not change down the column
+
+    def varies_in_loop(n):
+        if n.kind == "T":
+            return prog.tensors[n.slot].shape[0] > 1
+        return n.axis == 1           # one-hot along axis 1 reads idx[r]
+
+    def load_leaves(leaves):
+        tiles = {}
+        for n in leaves:
+            if not varies_in_loop(n):
+                tiles[n.nid] = line_tiles[n.nid]
+                continue
+            if n.nid not in cached:
+                cached[n.nid] = "keep%d" % n.nid
+                L("if (ok) keep%d[i].load(%s); else keep%d[i].zero();" % (n.nid, g.tile_addr(n, "r", "cc"), n.nid))
+            tiles[n.nid] = "keep%d[i]" % n.nid
+        return tiles
+
+    def declare_tiles(leaves):
+        keep_all()
+        for n in leaves:
+            if not varies_in_loop(n):
+                if n.nid not in line_tiles:
+                    name = "line%d" % n.nid
+                    line_tiles[n.nid] = name
+                    L("%s %s;" % (g.tile_type(n, V), name))
+                    L("%s.load(%s);" % (name, g.tile_addr(n, "0", "cc")))
+            elif n.nid not in cached:
+                L("%s keep%d[%d];" % (g.tile_type(n, V), n.nid, NR))
+
+    declare_tiles([n for n in g.leaf_nodes(used_nodes([st.root for st in prog.statements]))
+                   if not varies_in_loop(n)])
+
+    for s in range(nsweeps):
+        reds = per_level.get(s, [])
+        if not reds:
+            continue
+        args = [n.args[0] for n in reds]
+        nodes = _needed(args, done)
+        leaves = g.leaf_nodes(nodes)
+        declare_tiles(leaves)
+        for n in reds:
+            g.declare_acc(n)
+        row_loop_open()
+        tiles = load_leaves(leaves)
+        L.open("if (ok)")
+        if V > 1:
+            L("#pragma unroll")
+        L.open("for (int j = 0; j < %d; ++j)" % V)
+        ref = g.make_ref("_s", "r", "cc", V, tiles)
+        g.emit_exprs(nodes, ref, done)
+        for n in reds:
+            g.accumulate(n, ref(n.args[0]), "r")
+        L.close()
+        L.close()
+        L.close()
+        for n in reds:
+            _emit_col_fold(g, L, n, LX, LY, T, V, "acc%d" % n.nid)
+            done[n.nid] = n
+
+    if line_out:
+        roots = [st.root for st in line_out]
+        nodes = _needed(roots, done)
+        leaves = g.leaf_nodes(nodes)
+        L.open("if (col_ok && ty == 0)")
+        for n in leaves:
+            g.emit_load(n, "0", "c", V, "_l")
+        for st in line_out:
+            L("nh_out<%s, %d> o%d; o%d.clear();" % (g.slot_ctype(st.out), V, st.out.index, st.out.index))
+        if V > 1:
+            L("#pragma unroll")
+        L.open("for (int j = 0; j < %d; ++j)" % V)
+        ref = g.make_ref("_l", "0", "c", V)
+        g.emit_exprs(nodes, ref, done)
+        for st in line_out:
+            if st.root.kind == "R" and st.root.is_index:
+                L("o%d.seti(j, ri%d[j]);" % (st.out.index, st.root.nid))
+            else:
+                L("o%d.set(j, %s);" % (st.out.index, ref(st.root)))
+        L.close()
+        for st in line_out:
+            L("o%d.store(%s);" % (st.out.index, g.addr(st.out, "0", "c")))
+        L.close()
+
+    if full_out:
+        roots = [st.root for st in full_out]
+        nodes = _needed(roots, done)
+        leaves = g.leaf_nodes(nodes)
+        declare_tiles(leaves)
+        row_loop_open()
+        tiles = load_leaves(leaves)
+        L.open("if (ok)")
+        for st in full_out:
+            L("nh_out<%s, %d> o%d; o%d.clear();" % (g.slot_ctype(st.out), V, st.out.index, st.out.index))
+        if V > 1:
+            L("#pragma unroll")
+        L.open("for (int j = 0; j < %d; ++j)" % V)
+        ref = g.make_ref("_s", "r", "cc", V, tiles)
+        g.emit_exprs(nodes, ref, done)
+        for st in full_out:
+            if st.root.kind == "R" and st.root.is_index:
+                L("o%d.seti(j, ri%d[j]);" % (st.out.index, st.root.nid))
+            else:
+                L("o%d.set(j, %s);" % (st.out.index, ref(st.root)))
+        L.close()
+        for st in full_out:
+            L("o%d.store(%s);" % (st.out.index, g.addr(st.out, "r", "c")))
+        L.close()
+        L.close()
+    L.close()
+    return _finish("col", g, head, fmt, T, lds, dict(V=V, LX=LX, LY=LY, NR=NR))
+
+
+def gen_colsplit(prog, V, LX, LY):
+    """One level of axis-0 reductions over a tall matrix.  grid = (column
+    strips, row chunks).  Each workgroup reduces its chunk, leaves one partial
+    per column in the workspace and takes a ticket; the workgroup that draws
+    the last ticket of its strip folds the partials in chunk order, evaluates
+    the statements (one value per column) and stores them.  Tickets live in
+    the workspace, start at zero and are reset by their last user.
+
+    Extra parameters: ``rows_per_chunk``, workspace pointer (partials first,
+    tickets after ``ticket_offset`` bytes)."""
+    assert prog.nlevels == 1
+    g = _RedGen(prog, V)
+    L = g.L
+    T = LX * LY
+    params, fmt = g.param_list([("int rows_per_chunk", "i"), ("char* ws", "P"),
+                                ("long long ticket_offset", "q")])
+    head = ('extern "C" __global__ __launch_bounds__(%d) void @NAME@(%s)\n' % (T, params))
+    reds = _live_reductions(prog)
+    any_index = any(n.is_index for n in reds)
+    for st in prog.statements:
+        assert st.out.shape[0] == 1
+    done = {}
+
+    L.open("")
+    lds = _col_lds(L, LX, LY, T, V, any_index)
+    L("__shared__ int s_last;")
+    L("const int tx = threadIdx.x %% %d, ty = threadIdx.x / %d;" % (LX, LX))
+    L("const long long c = ((long long)blockIdx.x * %d + tx) * %d;" % (LX, V))
+    L("const bool col_ok = c < C;")
+    L("const long long cc = col_ok ? c : 0;")
+    L("const long long r0 = (long long)blockIdx.y * rows_per_chunk;")
+    L("const long long r1 = (r0 + rows_per_chunk < R) ? (r0 + rows_per_chunk) : (long long)R;")
+    L("const int nchunks = gridDim.y;")
+    args = [n.args[0] for n in reds]
+    nodes = _needed(args, {})
+    leaves = g.leaf_nodes(nodes)
+    for n in reds:
+        g.declare_acc(n)
+    U = 4
+    # main loop: U independent rows in flight per lane
+    L.open("if (col_ok)")
+    L("long long r = r0 + ty;")
+    L.open("for (; r + %d < r1; r += %d)" % ((U - 1) * LY, U * LY))
+    for u in range(U):
+        for n in leaves:
+            g.emit_load(n, "r + %d" % (u * LY), "c", V, "_%d" % u)
+    for u in range(U):
+        if V > 1:
+            L("#pragma unroll")
+        L.open("for (int j = 0; j < %d; ++j)" % V)
+        ref = g.make_ref("_%d" % u, "r + %d" % (u * LY), "c", V)
+        g.emit_exprs(nodes, ref, {})
+        for n in reds:
+            g.accumulate(n, ref(n.args[0]), "r + %d" % (u * LY))
+        L.close()
+    L.close()
+    L.open("for (; r < r1; r += %d)" % LY)
+    for n in leaves:
+        g.emit_load(n, "r", "c", V, "_t")
+    if V > 1:
+        L("#pragma unroll")
+    L.open("for (int j = 0; j < %d; ++j)" % V)
+    ref = g.make_ref("_t", "r", "c", V)
+    g.emit_exprs(nodes, ref, {})
+    for n in reds:
+        g.accumulate(n, ref(n.args[0]), "r")
+    L.close()
+    L.close()
+    L.close()
+    for n in reds:
+        _emit_col_fold(g, L, n, LX, LY, T, V, "acc%d" % n.nid)
+
+    # partial buffers: reduction k occupies [k*nchunks*C, (k+1)*nchunks*C) entries
+    # of 8 bytes (value, index)
+    L.open("if (nchunks > 1)")
+    for k, n in enumerate(reds):
+        L("nh_pair* part%d = reinterpret_cast<nh_pair*>(ws) + (long long)%d * nchunks * C;" % (n.nid, k))
+    L("unsigned int* tickets = reinterpret_cast<unsigned int*>(ws + ticket_offset);")
+    L.open("if (col_ok && ty == 0)")
+    L("#pragma unroll")
+    L.open("for (int j = 0; j < %d; ++j)" % V)
+    for n in reds:
+        L("nh_pair p%d; p%d.v = %s; p%d.i = %s;" % (n.nid, n.nid,
+                                                     ("acc%d[j].v" % n.nid) if n.is_index else ("rv%d[j]" % n.nid),
+                                                     n.nid,
+                                                     ("acc%d[j].i" % n.nid) if n.is_index else "0"))
+        L("part%d[(long long)blockIdx.y * C + c + j] = p%d;" % (n.nid, n.nid))
+    L.close()
+    L.close()
+    L("__threadfence();")
+    L("__syncthreads();")
+    L.open("if (threadIdx.x == 0)")
+    L("const unsigned int t = atomicAdd(&tickets[blockIdx.x], 1u);")
+    L("s_last = (t == (unsigned int)(nchunks - 1));")
+    L.close()
+    L("__syncthreads();")
+    L("if (!s_last) return;")
+    L("__threadfence();")
+    for n in reds:
+        op = _RED_OP[n.op]
+        L("#pragma unroll")
+        if n.is_index:
+            L("for (int j = 0; j < %d; ++j) acc%d[j] = %s::init();" % (V, n.nid, op))
+        else:
+            L("for (int j = 0; j < %d; ++j) acc%d[j] = %s::init();" % (V, n.nid, op))
+    L.open("if (col_ok)")
+    L.open("for (int q = ty; q < nchunks; q += %d)" % LY)
+    L("#pragma unroll")
+    L.open("for (int j = 0; j < %d; ++j)" % V)
+    for n in reds:
+        op = _RED_OP[n.op]
+        L("const nh_pair p%d = part%d[(long long)q * C + c + j];" % (n.nid, n.nid))
+        if n.is_index:
+            L("acc%d[j] = %s::f(acc%d[j], p%d);" % (n.nid, op, n.nid, n.nid))
+        else:
+            L("acc%d[j] = %s::f(acc%d[j], p%d.v);" % (n.nid, op, n.nid, n.nid))
+    L.close()
+    L.close()
+    L.close()
+    for n in reds:
+        _emit_col_fold(g, L, n, LX, LY, T, V, "acc%d" % n.nid, dst_decl=False)
+    L("if (threadIdx.x == 0) tickets[blockIdx.x] = 0u;")
+    L.close()
+    for n in reds:
+        done[n.nid] = n
+
+    roots = [st.root for st in prog.statements]
+    nodes = _needed(roots, done)
+    leaves = g.leaf_nodes(nodes)
+    L.open("if (col_ok && ty == 0)")
+    for n in leaves:
+        g.emit_load(n, "0", "c", V, "_l")
+    for st in prog.statements:
+        L("nh_out<%s, %d> o%d; o%d.clear();" % (g.slot_ctype(st.out), V, st.out.index, st.out.index))
+    if V > 1:
+        L("#pragma unroll")
+    L.open("for (int j = 0; j < %d; ++j)" % V)
+    ref = g.make_ref("_l", "0", "c", V)
+    g.emit_exprs(nodes, ref, done)
+    for st in prog.statements:
+        if st.root.kind == "R" and st.root.is_index:
+            L("o%d.seti(j, ri%d[j]);" % (st.out.index, st.root.nid))
+        else:
+            L("o%d.set(j, %s);" % (st.out.index, ref(st.root)))
+    L.close()
+    for st in prog.statements:
+        L("o%d.store(%s);" % (st.out.index, g.addr(st.out, "0", "c")))
+    L.close()
+    L.close()
+    return _finish("colsplit", g, head, fmt, T, lds, dict(V=V, LX=LX, LY=LY, NRED=len(reds)))

@@ -1,0 +1,443 @@
+"""
+Op-tree -> typed DAG.
+
+Takes the postfix stacks of one or more ``assign`` trees (a *program*; several
+statements are fused when the backend was asked to, one otherwise) and builds a
+DAG in which
+
+  * every distinct tensor (same object, or same memory + geometry) and every
+    distinct constant gets one kernel-argument *slot*;
+  * identical sub-expressions are one node (structural hashing over the whole
+    tree -- the reference only merges duplicates at reduction boundaries,
+    float_ew.py:147-190, so softmax's repeated ``exp(x - max)`` was evaluated
+    twice per element there);
+  * sub-trees made of numbers only (Adam's ``lr*sqrt(1-b2**t)/(1-b1**t)``) are
+    folded on the host in double precision -- what the CPU backend's numpy
+    calls do with Python floats -- and become a single constant slot;
+  * each node knows along which axes it varies (``vr``, ``vc``) and its
+    reduction *level*: how many nested reductions must have completed before
+    it can be evaluated.
+
+The same walk yields the cache key: two programs with equal keys generate
+byte-identical kernels and bind arguments in the same order.
+
+Host-side checks raise before anything is generated, with the exception types
+of the reference launcher (float_ew.py:682-690, 724-726, 821-825, 900-906):
+reduction axis outside {0,1} or two different axes -> ValueError; operand
+shapes that do not broadcast -> TypeError; unknown op or operand -> TypeError.
+"""
+import math
+
+import numpy as np
+
+from neon_amd.backends.backend import OpCollection, Tensor
+
+UNARY = {"neg", "abs", "sgn", "sqrt", "sqr", "exp", "log", "exp2", "log2", "sig",
+         "sig2", "tanh", "tanh2", "safelog", "rint", "finite"}
+BINARY = {"add", "sub", "mul", "div", "eq", "ne", "lt", "le", "gt", "ge", "pow",
+          "minimum", "maximum"}
+REDUCE = {"sum", "max", "min", "argmax", "argmin"}
+
+# storage dtype -> short code used in keys and kernel names
+DTYPE_CODE = {np.dtype(np.float32): "f4", np.dtype(np.float16): "f2",
+              np.dtype(np.int32): "i4", np.dtype(np.uint32): "u4",
+              np.dtype(np.int16): "i2", np.dtype(np.uint16): "u2",
+              np.dtype(np.int8): "i1", np.dtype(np.uint8): "u1"}
+
+
+def _fold_unary(op, x):
+    """Host evaluation of a unary op on a number, numpy semantics in double."""
+    x = float(x)
+    with np.errstate(all="ignore"):
+        if op == "neg":
+            return -x
+        if op == "abs":
+            return abs(x)
+        if op == "sgn":
+            return float(np.sign(x))
+        if op == "sqrt":
+            return float(np.sqrt(x))
+        if op == "sqr":
+            return x * x
+        if op == "exp":
+            return float(np.exp(x))
+        if op == "log":
+            return float(np.log(x))
+        if op == "safelog":
+            return float(np.log(np.maximum(x, np.exp(-50.))))
+        if op == "exp2":
+            return float(np.exp2(x))
+        if op == "log2":
+            return float(np.log2(x))
+        if op == "sig":
+            return float(1. / (1. + np.exp(-x)))
+        if op == "sig2":
+            return float(1. / (1. + np.exp2(-x)))
+        if op == "tanh":
+            return float(np.tanh(x))
+        if op == "tanh2":
+            return float((np.exp2(2. * x) - 1.) / (np.exp2(2. * x) + 1.))
+        if op == "rint":
+            return float(np.rint(x))
+        if op == "finite":
+            return float(np.isfinite(x))
+    raise TypeError("unknown unary op %s" % op)
+
+
+def _fold_binary(op, a, b):
+    a, b = float(a), float(b)
+    with np.errstate(all="ignore"):
+        if op == "add":
+            return a + b
+        if op == "sub":
+            return a - b
+        if op == "mul":
+            return a * b
+        if op == "div":
+            return float(np.float64(a) / np.float64(b))
+        if op == "pow":
+            return float(np.power(np.float64(a), np.float64(b)))
+        if op == "minimum":
+            return float(np.minimum(a, b))
+        if op == "maximum":
+            return float(np.maximum(a, b))
+        if op == "eq":
+            return float(a == b)
+        if op == "ne":
+            return float(a != b)
+        if op == "lt":
+            return float(a < b)
+        if op == "le":
+            return float(a <= b)
+        if op == "gt":
+            return float(a > b)
+        if op == "ge":
+            return float(a >= b)
+    raise TypeError("unknown binary op %s" % op)
+
+
+class MixedAxes(ValueError):
+    """Reductions along both axes in one tree: needs more than one kernel."""
+
+
+class Node(object):
+    """DAG node.  kind: 'T' tensor leaf, 'C' constant slot, 'E' elementwise op,
+    'R' reduction, 'H' one-hot of an index tensor."""
+    __slots__ = ("kind", "op", "args", "slot", "axis", "vr", "vc", "level",
+                 "nid", "is_index", "shape")
+
+    def __init__(self, kind, op=None, args=(), slot=None, axis=None):
+        self.kind = kind
+        self.op = op
+        self.args = tuple(args)
+        self.slot = slot
+        self.axis = axis
+        self.vr = self.vc = False
+        self.level = 0
+        self.nid = -1
+        self.is_index = False
+        self.shape = (1, 1)
+
+    def __repr__(self):
+        return "N%d<%s %s %s>" % (self.nid, self.kind, self.op or "", self.slot if self.slot is not None else "")
+
+
+class TensorSlot(object):
+    """One kernel pointer argument: a distinct (memory, geometry, dtype)."""
+    __slots__ = ("index", "tensor", "dtype", "shape", "strides", "ptr", "written",
+                 "read", "geom")
+
+    def __init__(self, index, tensor, shape, strides):
+        self.index = index
+        self.tensor = tensor
+        self.dtype = np.dtype(tensor.dtype)
+        self.shape = shape
+        self.strides = strides
+        self.ptr = tensor.ptr
+        self.written = False
+        self.read = False
+        self.geom = (tensor.ptr, shape, strides, self.dtype)
+
+
+class Statement(object):
+    __slots__ = ("out", "root")
+
+    def __init__(self, out, root):
+        self.out = out      # TensorSlot
+        self.root = root    # Node
+
+
+def view_2d(tensor):
+    """(shape, element strides) of a tensor as the 2-d object the kernels see.
+    Tensors with more than two dims are accepted only when contiguous and are
+    flattened to (dim0, rest)."""
+    shape, strides = tuple(tensor.shape), tuple(tensor.strides)
+    if len(shape) == 2:
+        return shape, strides
+    if len(shape) == 1:
+        return (shape[0], 1), (strides[0], 1)
+    if not tensor.is_contiguous:
+        raise ValueError("op-trees on non-contiguous tensors with more than 2 "
+                         "dimensions are not supported")
+    rest = 1
+    for d in shape[1:]:
+        rest *= d
+    return (shape[0], rest), (rest, 1)
+
+
+class Program(object):
+    """DAG of one fused group of assign statements."""
+
+    def __init__(self):
+        self.tensors = []          # TensorSlot list, in first-use order
+        self.consts = []           # python floats, in first-use order
+        self.statements = []
+        self.nodes = []            # topological order
+        self._tensor_by_geom = {}
+        self._tensor_by_id = {}
+        self._cse = {}
+        self._const_slot = {}
+        self._current = {}         # tensor slot index -> node holding its newest value
+        self.key_parts = []
+        self.axis = None           # the one reduction axis, if any
+        self.domain = None
+        self.nlevels = 0
+
+    # -- slots -----------------------------------------------------------------
+    def tensor_slot(self, t):
+        slot = self._tensor_by_id.get(id(t))
+        if slot is not None:
+            return slot
+        if getattr(t, "take_array", None):
+            raise NotImplementedError("fancy-indexed views inside op-trees")
+        shape, strides = view_2d(t)
+        geom = (t.ptr, shape, strides, np.dtype(t.dtype))
+        slot = self._tensor_by_geom.get(geom)
+        if slot is None:
+            if np.dtype(t.dtype) not in DTYPE_CODE:
+                raise TypeError("unsupported tensor dtype %s" % t.dtype)
+            slot = TensorSlot(len(self.tensors), t, shape, strides)
+            self.tensors.append(slot)
+            self._tensor_by_geom[geom] = slot
+        self._tensor_by_id[id(t)] = slot
+        return slot
+
+    def const_node(self, value):
+        value = float(value)
+        # every occurrence of an equal number shares a slot; the *value* is a
+        # run-time argument, so the key records only the slot pattern
+        slot = self._const_slot.get(value)
+        if slot is None:
+            slot = len(self.consts)
+            self.consts.append(value)
+            self._const_slot[value] = slot
+        self.key_parts.append(("C", slot))
+        return self._intern(("C", slot), lambda: Node("C", slot=slot))
+
+    def _intern(self, key, make):
+        n = self._cse.get(key)
+        if n is None:
+            n = make()
+            n.nid = len(self.nodes)
+            self.nodes.append(n)
+            self._cse[key] = n
+        return n
+
+    # -- building ------------------------------------------------------------------
+    def add_statement(self, optree):
+        """Append ``assign(out, expr)`` given as an OpTreeNode."""
+        assert optree[0]["op"] == "assign"
+        out_t, value = optree[1], optree[2]
+        if not isinstance(out_t, Tensor):
+            raise TypeError("assignment target must be a tensor")
+        out_slot = self.tensor_slot(out_t)
+        stack = []
+        postfix = []
+        if isinstance(value, (int, float)):
+            postfix = [value]
+        elif isinstance(value, Tensor):
+            postfix = [value]
+        else:
+            value.traverse(postfix)
+        for p in postfix:
+            if isinstance(p, dict):
+                self._apply(p, stack)
+            elif isinstance(p, Tensor):
+                stack.append(self._read_tensor(p))
+            elif isinstance(p, (int, float)):
+                stack.append(float(p))          # folded lazily
+            else:
+                raise TypeError("args must be instance of Tensor, int, float, or dict (for operators)")
+        if len(stack) != 1:
+            raise TypeError("malformed op-tree")
+        root = stack[0]
+        if not isinstance(root, Node):
+            root = self.const_node(root)
+        out_slot.written = True
+        st = Statement(out_slot, root)
+        self.statements.append(st)
+        self.key_parts.append(("=", out_slot.index))
+        self._current[out_slot.index] = root
+        return st
+
+    def _read_tensor(self, t):
+        slot = self.tensor_slot(t)
+        self.key_parts.append(("T", slot.index))
+        cur = self._current.get(slot.index)
+        if cur is not None:
+            # value written by an earlier statement of this program: forward it,
+            # rounded the way the store rounds it
+            if slot.dtype == np.dtype(np.float32):
+                return cur
+            return self._intern(("Q", cur.nid, DTYPE_CODE[slot.dtype]),
+                                lambda: Node("E", op="quant:" + DTYPE_CODE[slot.dtype], args=(cur,)))
+        slot.read = True
+        return self._intern(("T", slot.index), lambda: Node("T", slot=slot.index))
+
+    def _as_node(self, x):
+        return x if isinstance(x, Node) else self.const_node(x)
+
+    def _apply(self, d, stack):
+        op = d["op"]
+        if op in UNARY:
+            x = stack.pop()
+            if not isinstance(x, Node):
+                self.key_parts.append(("fold1", op))
+                stack.append(_fold_unary(op, x))
+                return
+            self.key_parts.append(op)
+            stack.append(self._intern(("E", op, x.nid), lambda: Node("E", op=op, args=(x,))))
+        elif op in BINARY:
+            b = stack.pop()
+            a = stack.pop()
+            if not isinstance(a, Node) and not isinstance(b, Node):
+                self.key_parts.append(("fold2", op))
+                stack.append(_fold_binary(op, a, b))
+                return
+            self.key_parts.append(op)
+            a, b = self._as_node(a), self._as_node(b)
+            stack.append(self._intern(("E", op, a.nid, b.nid), lambda: Node("E", op=op, args=(a, b))))
+        elif op in REDUCE:
+            x = stack.pop()
+            axis = d.get("axis", None)
+            if axis not in (0, 1):
+                raise ValueError("Only reduction along an axis currently supported")
+            self.key_parts.append((op, axis))
+            x = self._as_node(x)
+            n = self._intern(("R", op, axis, x.nid), lambda: Node("R", op=op, args=(x,), axis=axis))
+            n.is_index = op in ("argmax", "argmin")
+            stack.append(n)
+        elif op == "onehot":
+            idx = d["idx"]
+            slot = self.tensor_slot(idx)
+            slot.read = True
+            axis = d["axis"]
+            self.key_parts.append(("onehot", slot.index, axis))
+            stack.append(self._intern(("H", slot.index, axis),
+                                      lambda: Node("H", op="onehot", slot=slot.index, axis=axis)))
+        elif op in ("dot", "transpose", "rand", "binarize", "shift", "assign"):
+            raise NotImplementedError("op '%s' cannot be part of a fused op-tree kernel" % op)
+        else:
+            raise TypeError("%s is not a valid operation" % op)
+
+    # -- analysis --------------------------------------------------------------------
+    def finalize(self):
+        """Infer the iteration domain, per-node variance and reduction levels;
+        verify broadcast compatibility."""
+        index_only = set(n.slot for n in self.nodes if n.kind == "H")
+        index_only -= set(n.slot for n in self.nodes if n.kind == "T")
+        index_only -= set(st.out.index for st in self.statements)
+        shaped = [t for t in self.tensors if t.index not in index_only]
+        R = C = 1
+        for t in shaped:
+            R, C = max(R, t.shape[0]), max(C, t.shape[1])
+        axes = set(n.axis for n in self.nodes if n.kind == "R")
+        if len(axes) > 1:
+            raise MixedAxes("Reduction along only one axis is supported per kernel")
+        self.axis = axes.pop() if axes else None
+        self.domain = (R, C)
+        for t in shaped:
+            if t.shape[0] not in (1, R) or t.shape[1] not in (1, C):
+                raise TypeError("Input shape:%s not compatible with %s" % (t.shape, (R, C)))
+        for n in self.nodes:
+            if n.kind == "T":
+                shp = self.tensors[n.slot].shape
+                n.vr, n.vc, n.level = shp[0] > 1, shp[1] > 1, 0
+            elif n.kind == "C":
+                n.vr = n.vc = False
+                n.level = 0
+            elif n.kind == "H":
+                # one-hot of a vector of indices: full variance wherever the
+                # index vector and the hot axis have extent
+                n.vr, n.vc, n.level = R > 1, C > 1, 0
+            elif n.kind == "E":
+                n.vr = any(a.vr for a in n.args)
+                n.vc = any(a.vc for a in n.args)
+                n.level = max(a.level for a in n.args)
+            elif n.kind == "R":
+                a = n.args[0]
+                varies = a.vr if n.axis == 0 else a.vc
+                if not varies:
+                    # extent 1 along the reduced axis: the reduction is the
+                    # identity (index reductions give 0), as numpy has it
+                    n.kind = "E"
+                    n.op = "zero_index" if n.is_index else "ident"
+                    n.is_index = False
+                    n.vr, n.vc, n.level = a.vr, a.vc, a.level
+                else:
+                    n.vr = a.vr and n.axis != 0
+                    n.vc = a.vc and n.axis != 1
+                    n.level = a.level + 1
+            n.shape = (R if n.vr else 1, C if n.vc else 1)
+        if not any(n.kind == "R" for n in self.nodes):
+            self.axis = None
+        self.nlevels = max([n.level for n in self.nodes] + [0])
+        for st in self.statements:
+            rs, os_ = st.root.shape, st.out.shape
+            if (rs[0] not in (1, os_[0])) or (rs[1] not in (1, os_[1])):
+                raise TypeError("Input shape:%s not compatible with %s" % (rs, os_))
+        return self
+
+    def key(self):
+        """Hashable identity of the program's structure and operand geometry."""
+        geo = tuple((DTYPE_CODE[t.dtype], t.shape, t.strides, t.ptr % 16 == 0, t.written)
+                    for t in self.tensors)
+        return (tuple(self.key_parts), geo, self._alias_signature())
+
+    def _alias_signature(self):
+        """Which slots overlap in memory (matters for what may be declared
+        non-aliasing in the generated kernel)."""
+        spans = []
+        for t in self.tensors:
+            isz = t.dtype.itemsize
+            extent = 1 + sum((s - 1) * abs(st) for s, st in zip(t.shape, t.strides) if s > 0)
+            spans.append((t.ptr, t.ptr + extent * isz))
+        sig = []
+        for i in range(len(spans)):
+            for j in range(i + 1, len(spans)):
+                if spans[i][0] < spans[j][1] and spans[j][0] < spans[i][1]:
+                    sig.append((i, j))
+        return tuple(sig)
+
+    def overlapping_slots(self):
+        return self._alias_signature()
+
+
+def build_program(optrees):
+    prog = Program()
+    for tree in optrees:
+        prog.add_statement(tree)
+    return prog.finalize()
+
+
+def used_nodes(roots):
+    """Nodes reachable from ``roots`` in topological (id) order."""
+    seen = {}
+    todo = list(roots)
+    while todo:
+        n = todo.pop()
+        if n.nid in seen:
+            continue
+        seen[n.nid] = n
+        todo.extend(n.args)
+    return [seen[k] for k in sorted(seen)]

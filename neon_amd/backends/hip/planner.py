@@ -1,0 +1,380 @@
+"""
+Shape-class selection, kernel cache and launch plans.
+
+``make_plan(prog, rt, cache)`` looks at a finalized program (optree_ir) and
+picks a kernel family and its tiling from the actual geometry, generates the
+source, compiles it (or finds it in the cache) and returns a ``Plan`` whose
+``launch`` packs arguments and enqueues.  The reference did the equivalent in
+``call_compound_kernel`` (float_ew.py:644-940) with three hard-wired block
+sizes tuned for a 24-SM part; here the choice is driven by what fills 256
+compute units and keeps every access a 16-byte vector.
+
+``NeedsSplit`` tells the backend that the tree must be broken into several
+programs through temporaries (the job of ``_split_to_stacks`` in the
+reference, nervanagpu.py:1099-1237).
+"""
+import hashlib
+import os
+import tempfile
+
+import numpy as np
+
+from neon_amd.backends.hip import codegen
+from neon_amd.backends.hip import runtime as hiprt
+from neon_amd.backends.hip.optree_ir import used_nodes
+
+
+class NeedsSplit(Exception):
+    """The program cannot run as one kernel; evaluate reductions separately."""
+
+
+def _pow2ceil(x):
+    p = 1
+    while p < x:
+        p *= 2
+    return p
+
+
+def _pow2floor(x):
+    p = 1
+    while p * 2 <= x:
+        p *= 2
+    return p
+
+
+def _ceil_div(a, b):
+    return -(-a // b)
+
+
+# ---------------------------------------------------------------------------------------
+# kernel cache: in-process dict in front of an on-disk store of code objects
+# (the role of neon/backends/util/source_module.py:16-22 for the reference)
+# ---------------------------------------------------------------------------------------
+class KernelCache(object):
+    def __init__(self, arch, cache_dir=None):
+        self.arch = arch
+        with open(hiprt.DEVICE_HEADER) as f:
+            self.header = f.read()
+        if cache_dir is None:
+            cache_dir = os.environ.get("NEON_HIP_CACHE_DIR")
+        if cache_dir is None and os.environ.get("NEON_CACHE_DIR"):
+            cache_dir = os.path.join(os.environ["NEON_CACHE_DIR"], "hip")
+        if cache_dir is None:
+            # next to the prebuilt library, so kernels compiled at build time are
+            # found at run time; a read-only install falls back to the home dir
+            local = os.path.join(os.path.dirname(hiprt.LIB_PATH), "kcache")
+            try:
+                os.makedirs(local, exist_ok=True)
+                cache_dir = local if os.access(local, os.W_OK) else None
+            except OSError:
+                cache_dir = None
+        if cache_dir is None:
+            cache_dir = os.path.join(os.path.expanduser("~"), ".cache", "neon_amd", "hip")
+        self.cache_dir = cache_dir
+        self.loaded = {}      # kernel name -> runtime.Kernel
+        self.stats = {"hit_mem": 0, "hit_disk": 0, "compiled": 0}
+        self.dump_dir = os.environ.get("NEON_HIP_DUMP")
+
+    def _digest(self, source):
+        h = hashlib.sha256()
+        h.update(self.arch.encode())
+        h.update(" ".join(hiprt.RTC_OPTIONS).encode())
+        h.update(self.header.encode())
+        h.update(source.encode())
+        return h.hexdigest()
+
+    def code_object(self, spec):
+        """code-object bytes for a Spec, compiling on a miss"""
+        full = self.header + "\n" + spec.source
+        path = os.path.join(self.cache_dir, self._digest(spec.source) + ".hsaco")
+        if self.dump_dir:
+            os.makedirs(self.dump_dir, exist_ok=True)
+            with open(os.path.join(self.dump_dir, spec.name + ".hip"), "w") as f:
+                f.write(spec.source)
+        try:
+            with open(path, "rb") as f:
+                self.stats["hit_disk"] += 1
+                return f.read()
+        except (IOError, OSError):
+            pass
+        code, _log = hiprt.rtc_compile(full, spec.name + ".hip", self.arch)
+        self.stats["compiled"] += 1
+        try:
+            os.makedirs(self.cache_dir, exist_ok=True)
+            fd, tmp = tempfile.mkstemp(dir=self.cache_dir)
+            with os.fdopen(fd, "wb") as f:
+                f.write(code)
+            os.replace(tmp, path)
+        except (IOError, OSError):
+            pass       # a read-only cache directory only costs recompiles
+        return code
+
+    def kernel(self, rt, spec):
+        k = self.loaded.get(spec.name)
+        if k is not None:
+            self.stats["hit_mem"] += 1
+            return k
+        code = self.code_object(spec)
+        k = rt.load_kernel(code, spec.name, spec.fmt)
+        self.loaded[spec.name] = k
+        return k
+
+
+# ---------------------------------------------------------------------------------------
+# vector width
+# ---------------------------------------------------------------------------------------
+def _vector_width(prog, single_row_tail_ok):
+    """Largest V (elements per lane access) such that every column-varying
+    operand can be touched with aligned vector instructions."""
+    R, C = prog.domain
+    cols = [t for t in prog.tensors if t.shape[1] > 1]
+    used = used_nodes([st.root for st in prog.statements])
+    hot0 = [prog.tensors[n.slot] for n in used if n.kind == "H" and n.axis == 0]
+    if not cols and not hot0:
+        return 1
+    if any(t.strides[1] != 1 for t in cols):
+        return 1
+    isz_min = min([t.dtype.itemsize for t in cols] + [4 for _ in hot0])
+    V = min(8, 16 // isz_min)
+    while V > 1:
+        ok = (C % V == 0) or (single_row_tail_ok and R == 1)
+        for t in cols:
+            align = min(16, V * t.dtype.itemsize)
+            if t.ptr % align:
+                ok = False
+            if t.shape[0] > 1 and (t.strides[0] * t.dtype.itemsize) % align:
+                ok = False
+        for t in hot0:
+            if t.ptr % min(16, V * 4):
+                ok = False
+        if ok:
+            break
+        V //= 2
+    return V
+
+
+def _check_onehot(prog):
+    R, C = prog.domain
+    for n in used_nodes([st.root for st in prog.statements]):
+        if n.kind == "H":
+            t = prog.tensors[n.slot]
+            want = C if n.axis == 0 else R
+            size = t.shape[0] * t.shape[1]
+            contiguous = t.strides == (t.shape[1], 1) or 1 in t.shape and (
+                t.strides[0 if t.shape[1] == 1 else 1] == 1)
+            if size != want or not contiguous:
+                raise TypeError("onehot index vector of size %d does not match extent %d" % (size, want))
+
+
+def _try_flatten(prog):
+    """A reduction-free program whose tensors all have the domain's shape and
+    are contiguous (or are 1x1) is a 1-d problem: view it as one long row."""
+    R, C = prog.domain
+    if R == 1:
+        return
+    for t in prog.tensors:
+        if t.shape == (1, 1):
+            continue
+        if t.shape != (R, C) or t.strides != (C, 1):
+            return
+    for n in prog.nodes:
+        if n.kind == "H":
+            return
+    N = R * C
+    for t in prog.tensors:
+        if t.shape != (1, 1):
+            t.shape, t.strides = (1, N), (N, 1)
+    prog.domain = (1, N)
+
+
+# ---------------------------------------------------------------------------------------
+# plans
+# ---------------------------------------------------------------------------------------
+class Plan(object):
+    """A compiled kernel + grid; ``launch(prog)`` binds the argument values of
+    any program with the same key."""
+
+    def __init__(self, rt, kernel, spec, grid, extras_fn=None, workspace=None):
+        self.rt = rt
+        self.kernel = kernel
+        self.spec = spec
+        self.grid = grid
+        self.block = (spec.block, 1, 1)
+        self.extras_fn = extras_fn
+        self.workspace = workspace     # device allocation owned by the plan
+        self.domain = None             # set by make_plan: the (R, C) the kernel iterates
+
+    def launch(self, prog):
+        vals = []
+        for t in prog.tensors:
+            vals.append(t.ptr)
+            vals.append(t.strides[0])
+            vals.append(t.strides[1])
+        nconst0 = len(vals)
+        vals.extend(prog.consts)
+        vals.append(self.domain[0])
+        vals.append(self.domain[1])
+        if self.extras_fn is not None:
+            vals.extend(self.extras_fn())
+        try:
+            self.rt.launch(self.kernel, self.grid, self.block, 0, *vals)
+        except OverflowError:
+            # a constant beyond the fp32 range becomes +-inf, as a numpy cast would
+            for i in range(nconst0, nconst0 + len(prog.consts)):
+                with np.errstate(over="ignore"):
+                    vals[i] = float(np.float32(vals[i]))
+            self.rt.launch(self.kernel, self.grid, self.block, 0, *vals)
+
+    def release(self):
+        if self.workspace:
+            self.rt.free(self.workspace)
+            self.workspace = None
+
+
+def _words_per_tile(prog, V, axis):
+    """registers one resident tile position costs, summed over the tensor
+    leaves that vary along the reduced axis (the others are loaded once)"""
+    total = 0
+    for t in prog.tensors:
+        if not t.read or t.shape[axis] == 1:
+            continue
+        w = V if t.shape[1] > 1 else 1
+        total += max(1, (w * t.dtype.itemsize + 3) // 4)
+    return max(total, 1)
+
+
+class Choice(object):
+    """Outcome of shape-class selection: generated kernel, grid and what the
+    extra kernel parameters are.  Needs no device."""
+
+    def __init__(self, spec, grid, extras=(), workspace=None):
+        self.spec = spec
+        self.grid = grid
+        self.extras = tuple(extras)          # literal values appended after R, C
+        self.workspace = workspace           # None or (bytes, ticket_offset, n_tickets)
+
+
+def choose(prog, cu_count=256):
+    """Pick family + tiling for a finalized program and generate its source."""
+    R, C = prog.domain
+    if R > 0x7FFFFFFF or C > 0x7FFFFFFF:
+        raise ValueError("tensor dimension too large")
+    _check_onehot(prog)
+    if prog.axis is None:
+        return _plan_ew(prog, cu_count)
+    if prog.axis == 1:
+        return _plan_row(prog, cu_count)
+    return _plan_col(prog, cu_count)
+
+
+def make_plan(prog, rt, cache, cu_count):
+    ch = choose(prog, cu_count)
+    kernel = cache.kernel(rt, ch.spec)
+    extras = ch.extras
+    ws = None
+    if ch.workspace is not None:
+        ws_bytes, ticket_off, n_tickets = ch.workspace
+        ws = rt.malloc(ws_bytes)
+        rt.memset(ws + ticket_off, 0, n_tickets, 4)   # tickets start at zero and reset themselves
+        extras = extras + (ws, ticket_off)
+    plan = Plan(rt, kernel, ch.spec, ch.grid, extras_fn=(lambda e=extras: e) if extras else None,
+                workspace=ws)
+    plan.domain = tuple(prog.domain)
+    return plan
+
+
+def _plan_ew(prog, cu_count):
+    _try_flatten(prog)
+    R, C = prog.domain
+    V = _vector_width(prog, single_row_tail_ok=True)
+    nvec = _ceil_div(C, V)
+    if R == 1:
+        LX, LY, UR = 256, 1, 1
+        UC = max(1, min(4, nvec // (256 * 4 * cu_count)))
+    else:
+        LX = min(256, _pow2ceil(nvec))
+        LY = 256 // LX
+        UC = 1
+        UR = max(1, min(4, R // (LY * 8)))
+    tail = (C % V) != 0
+    spec = codegen.gen_ew(prog, V, LX, LY, UC, UR, tail)
+    gx = _ceil_div(nvec, LX * UC)
+    row_tiles = _ceil_div(R, LY * UR)
+    gy = min(row_tiles, 65535)
+    if gx > 0x7FFFFFFF:
+        raise ValueError("tensor too large for one launch")
+    return Choice(spec, (gx, gy, 1), extras=(row_tiles,))
+
+
+def _plan_row(prog, cu_count):
+    R, C = prog.domain
+    V = _vector_width(prog, single_row_tail_ok=False)
+    nvec = _ceil_div(C, V)
+    words = _words_per_tile(prog, V, 1)
+    options = []
+    if nvec <= 64 * 8:
+        options.append((max(1, min(64, _pow2ceil(_ceil_div(nvec, 4)))), 256))
+    options += [(256, 256), (512, 512), (1024, 1024)]
+    LX, T, NCH = 1024, 1024, 0          # fallback: stream the row on every sweep
+    for lx, t in options:
+        nch = _ceil_div(nvec, lx)
+        budget = 64 if t == 1024 else 128
+        if nch <= 16 and nch * words <= budget:
+            LX, T, NCH = lx, t, nch
+            break
+    LY = T // LX
+    spec = codegen.gen_row(prog, V, LX, LY, NCH)
+    gx = _ceil_div(R, LY)
+    return Choice(spec, (gx, 1, 1))
+
+
+def _plan_col(prog, cu_count):
+    R, C = prog.domain
+    V = _vector_width(prog, single_row_tail_ok=False)
+    nvec = _ceil_div(C, V)
+    isz = max([t.dtype.itemsize for t in prog.tensors if t.shape[1] > 1] + [1])
+    words = _words_per_tile(prog, V, 0)
+    line_only = all(st.out.shape[0] == 1 and R > 1 for st in prog.statements)
+
+    # (a) whole column strip inside one workgroup, rows resident in registers
+    lx_min = max(1, min(64, 64 // (V * isz)))
+    LX = max(lx_min, min(64, _pow2floor(max(1, nvec // 32))))
+    LX = min(LX, _pow2ceil(nvec))
+    fit = None
+    strips = _ceil_div(nvec, LX)
+    # few strips: spend more lanes on each so the rows-per-lane count drops
+    for T in ((256, 512, 1024) if strips >= cu_count else (1024, 512, 256)):
+        LY = T // LX
+        NR = _ceil_div(R, LY)
+        budget = 64 if T == 1024 else 128
+        if NR <= 16 and NR * words <= budget:
+            fit = (T, LY, NR)
+            break
+    single_level = prog.nlevels == 1
+    big = R * C >= (1 << 18)
+    if fit and not (single_level and line_only and big and R >= 512):
+        T, LY, NR = fit
+        spec = codegen.gen_col(prog, V, LX, LY, NR)
+        return Choice(spec, (_ceil_div(nvec, LX), 1, 1))
+
+    # (b) one level, one value per column, many rows: split rows over workgroups
+    if single_level and line_only:
+        LX = max(lx_min, min(16, _pow2ceil(nvec)))
+        LY = 256 // LX
+        strips = _ceil_div(nvec, LX)
+        target = 4 * cu_count
+        chunks = max(1, min(128, target // strips))
+        rpc = max(4 * LY, _ceil_div(R, chunks))
+        rpc = _ceil_div(rpc, LY) * LY
+        chunks = _ceil_div(R, rpc)
+        if chunks > 65535:
+            raise ValueError("tensor too large for one launch")
+        spec = codegen.gen_colsplit(prog, V, LX, LY)
+        nred = spec.params["NRED"]
+        part_bytes = nred * chunks * C * 8
+        ticket_off = _ceil_div(part_bytes, 256) * 256
+        ws_bytes = ticket_off + strips * 4
+        return Choice(spec, (strips, chunks, 1), extras=(rpc,),
+                      workspace=(ws_bytes, ticket_off, strips))
+
+    raise NeedsSplit()

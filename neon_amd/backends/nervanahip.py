@@ -1,0 +1,666 @@
+"""
+``hip`` backend: ``HIPTensor`` and ``NervanaHIP`` (``gen_backend('hip')``, ``-b hip``).
+
+The op-tree path of the reference's accelerator backend (``GPUTensor`` and
+``NervanaGPU.execute``, neon/backends/nervanagpu.py:48-659, 1099-1283) rebuilt
+for one MI355X: tensors are device allocations reached through the C ABI of
+libneonhip.so, ``execute`` turns an assign tree into a typed DAG, picks a
+kernel family from the operand geometry, generates HIP C++, compiles it with
+hiprtc (cached in memory and on disk) and launches it.  There is no CPU
+fallback: without the library or a device, constructing the backend raises.
+
+Result semantics follow the reference's CPU backend (nervanacpu.py:480-522)
+wherever its two backends differ.
+"""
+import logging
+import struct
+
+import numpy as np
+
+from neon_amd.backends.backend import Backend, OpTreeNode, Tensor
+from neon_amd.backends.hip import runtime as hiprt
+from neon_amd.backends.hip.optree_ir import MixedAxes, Program, REDUCE
+from neon_amd.backends.hip.planner import KernelCache, NeedsSplit, make_plan
+
+logger = logging.getLogger(__name__)
+
+_none_slice = slice(None, None, None)
+_DTYPES = (np.float16, np.float32, np.uint8, np.int8, np.uint16, np.int16,
+           np.uint32, np.int32)
+
+
+def _contiguous_strides(shape):
+    """C-order element strides (reference nervanagpu.py:3234-3241)."""
+    strides, acc = [], 1
+    for d in reversed(shape):
+        strides.append(acc)
+        acc *= d
+    return tuple(reversed(strides))
+
+
+def _reshape_strides(strides, shape, new_shape):
+    """Strides of a reshaped view; only a contiguous trailing block may change
+    shape (reference nervanagpu.py:3243-3263)."""
+    matched = 0
+    for o, n in zip(shape, new_shape):
+        if o != n:
+            break
+        matched += 1
+    shape = tuple(shape) + (1,) * (len(new_shape) - len(shape))
+    strides = tuple(strides) + (1,) * (len(new_shape) - len(strides))
+    if matched == len(new_shape):
+        return tuple(strides[:matched])
+    tail_new = int(np.prod(new_shape[matched:]))
+    tail_old = int(strides[matched]) * int(shape[matched])
+    if tail_old != tail_new:
+        raise ValueError("Reshaping of non-contiguous dimensions unsupported.")
+    return tuple(strides[:matched]) + _contiguous_strides(new_shape[matched:])
+
+
+class HIPTensor(Tensor):
+    """Device tensor: a pointer into an allocation plus shape and element
+    strides; indexing produces views (reference GPUTensor,
+    nervanagpu.py:48-659)."""
+
+    def __init__(self, backend, shape=None, dtype=np.float32, name=None,
+                 persist_values=True, base=None, gpudata=None, strides=None,
+                 take_array=None, is_trans=False, rounding=0):
+        super(HIPTensor, self).__init__(backend, shape, dtype, name, persist_values)
+        dtype = np.dtype(dtype)
+        assert dtype.type in _DTYPES, "unsupported dtype %s" % dtype
+        if not isinstance(shape, (tuple, list)):
+            assert isinstance(shape, (int, np.integer))
+            shape = (int(shape),)
+        if len(shape) < self._min_dims:
+            shape = tuple(shape) + (1,) * (self._min_dims - len(shape))
+        dims, size = [], 1
+        for d in shape:
+            if int(d) != d:
+                raise TypeError("shape dims must be integer values [%s]" % str(d))
+            dims.append(int(d))
+            size *= int(d)
+        self.shape = tuple(dims)
+        self.size = size
+        self.dtype = dtype
+        self.nbytes = dtype.itemsize * size
+        self.strides = _contiguous_strides(self.shape) if strides is None else tuple(int(s) for s in strides)
+        self.base = base
+        self.take_array = take_array
+        self.is_trans = is_trans
+        self.rounding = rounding
+        self.kahan_count = 0
+        self.kahan_reset = 0
+        self._owns = False
+        if gpudata is None:
+            assert base is None
+            self.gpudata = backend._mem_alloc(self.nbytes) if size else 0
+            self._owns = bool(size)
+        else:
+            self.gpudata = int(gpudata)
+        self.is_contiguous = (not take_array and
+                              self.strides == _contiguous_strides(self.shape))
+
+    def __del__(self):
+        if getattr(self, "_owns", False) and self.gpudata:
+            be = self.backend
+            if be is not None and getattr(be, "rt", None) is not None:
+                try:
+                    be._mem_free(self.gpudata)
+                except Exception:       # interpreter shutdown
+                    pass
+            self.gpudata = 0
+
+    @property
+    def ptr(self):
+        return self.gpudata
+
+    def __int__(self):
+        return int(self.gpudata)
+
+    def __str__(self):
+        return ("HIPTensor(base 0x%x) name:%s shape:%s dtype:%s strides:%s "
+                "is_trans:%s is_contiguous:%s" % (self.gpudata, self.name, self.shape, self.dtype,
+                                                  self.strides, self.is_trans, self.is_contiguous))
+
+    __repr__ = __str__
+
+    def __len__(self):
+        return self.shape[0] if len(self.shape) else 0
+
+    def __setitem__(self, index, value):
+        self.__getitem__(index)._assign(value)
+
+    def __getitem__(self, index):
+        """Basic slicing -> view.  An int index keeps its axis (size 1) while
+        the tensor has fewer than 3 dims; a tensor / array / list index along
+        one axis is a gather view (reference nervanagpu.py:193-323)."""
+        if not isinstance(index, tuple):
+            if isinstance(index, slice) and index == _none_slice:
+                return self
+            index = (index,)
+        new_shape, new_strides, offset = [], [], 0
+        take = None
+        seen_ellipsis = False
+        ia = aa = 0
+        while ia < len(index):
+            entry = index[ia]
+            if aa > len(self.shape):
+                raise IndexError("too many axes in index")
+            if isinstance(entry, slice):
+                start, stop, step = entry.indices(self.shape[aa])
+                new_shape.append(max(0, -((start - stop) // step)))
+                new_strides.append(step * self.strides[aa])
+                offset += self.strides[aa] * start * self.dtype.itemsize
+                ia += 1
+                aa += 1
+            elif isinstance(entry, (HIPTensor, np.ndarray, list, tuple)):
+                if isinstance(entry, (list, tuple)):
+                    entry = np.array(entry, dtype=np.int32)
+                if isinstance(entry, np.ndarray):
+                    entry = self.__class__(self.backend, entry.shape, dtype=np.int32).set(entry)
+                size = max(entry.shape)
+                if size != entry.size:
+                    raise IndexError("Fancy indexing only currently supported dim > 1 in a single dimension.")
+                if take is not None:
+                    raise IndexError("Fancy indexing only currently supported one axis at a time.")
+                if entry.dtype.type is not np.int32:
+                    raise IndexError("Fancy indexing only currently supported with int32 types.")
+                take = (entry, aa)
+                new_shape.append(size)
+                new_strides.append(self.strides[aa])
+                ia += 1
+                aa += 1
+            elif isinstance(entry, (int, np.integer)):
+                dim = self.shape[aa]
+                entry = int(entry)
+                if entry < 0:
+                    entry += dim
+                if not 0 <= entry < dim:
+                    raise IndexError("subindex in axis %d out of range" % ia)
+                offset += self.strides[aa] * entry * self.dtype.itemsize
+                if len(self.shape) < 3:
+                    new_shape.append(1)
+                    new_strides.append(self.strides[aa])
+                ia += 1
+                aa += 1
+            elif entry is Ellipsis:
+                ia += 1
+                target = len(self.shape) - (len(index) - ia)
+                if target < aa:
+                    raise IndexError("invalid use of ellipsis in index")
+                while aa < target:
+                    new_shape.append(self.shape[aa])
+                    new_strides.append(self.strides[aa])
+                    aa += 1
+                if seen_ellipsis:
+                    raise IndexError("more than one ellipsis not allowed in index")
+                seen_ellipsis = True
+            else:
+                raise IndexError("invalid subindex in axis %d" % ia)
+        while aa < len(self.shape):
+            new_shape.append(self.shape[aa])
+            new_strides.append(self.strides[aa])
+            aa += 1
+        return self.__class__(backend=self.backend, shape=tuple(new_shape), dtype=self.dtype,
+                              base=self, gpudata=self.gpudata + offset, strides=new_strides,
+                              take_array=take, name=self.name, rounding=self.rounding)
+
+    def _assign(self, value):
+        """Constant fill and same-layout copy use the device's fill / copy
+        engines; everything else is an op-tree kernel
+        (reference nervanagpu.py:334-383)."""
+        be = self.backend
+        if isinstance(value, (int, float)):
+            if self.is_contiguous and not be._fusing:
+                if self.size:
+                    bits = np.array([value]).astype(self.dtype).view(
+                        {1: np.uint8, 2: np.uint16, 4: np.uint32}[self.dtype.itemsize])[0]
+                    be.rt.memset(self.gpudata, int(bits), self.size, self.dtype.itemsize)
+            else:
+                OpTreeNode.build("assign", self, value)
+        elif isinstance(value, HIPTensor):
+            if (self.is_contiguous and value.is_contiguous and self.dtype == value.dtype and
+                    self.shape == value.shape and not be._fusing):
+                if self.nbytes:
+                    be.rt.memcpy_d2d(self.gpudata, value.gpudata, self.nbytes)
+            else:
+                OpTreeNode.build("assign", self, value)
+        elif isinstance(value, OpTreeNode):
+            OpTreeNode.build("assign", self, value)
+        elif isinstance(value, np.ndarray):
+            self.set(value)
+        else:
+            raise TypeError("Invalid type for assignment: %s" % type(value))
+        return self
+
+    def set(self, ary):
+        """Host array -> device (reference nervanagpu.py:385-416)."""
+        ary = np.asarray(ary)
+        if ary.size != self.size:
+            raise TypeError("ary.size {} != self.size {}".format(ary.size, self.size))
+        assert self.is_contiguous, "Array in set() must be contiguous"
+        if ary.dtype != self.dtype:
+            ary = ary.astype(self.dtype)
+        ary = np.ascontiguousarray(ary)
+        self.backend._flush()
+        if self.nbytes:
+            self.backend.rt.memcpy_h2d(self.gpudata, ary)
+        return self
+
+    def get(self, stream=None):
+        """Device -> fresh host array; a non-contiguous view is first packed
+        into a temporary on the device (reference nervanagpu.py:418-435)."""
+        be = self.backend
+        be._flush()
+        out = np.empty(self.shape, self.dtype)
+        if not self.size:
+            return out
+        if self.is_contiguous:
+            be.rt.memcpy_d2h(out, self.gpudata)
+        else:
+            tmp = be.empty(self.shape, self.dtype)
+            tmp.copy(self)
+            be._flush()
+            be.rt.memcpy_d2h(out, tmp.gpudata)
+        return out
+
+    def raw(self):
+        return self.gpudata
+
+    def asnumpyarray(self):
+        return self.get()
+
+    def take(self, indices, axis, out=None):
+        if axis == 1:
+            view = self.__getitem__((_none_slice, indices))
+        else:
+            view = self.__getitem__((indices, _none_slice))
+        if out:
+            return out._assign(view)
+        return view
+
+    def fill(self, value):
+        return self._assign(value)
+
+    def copy(self, a):
+        return self._assign(a)
+
+    def copy_from(self, a):
+        return self.set(a)
+
+    def reshape(self, *shape):
+        """View with a new shape; ``-1`` infers one extent
+        (reference nervanagpu.py:514-550)."""
+        if isinstance(shape[0], (tuple, list)):
+            shape = tuple(shape[0])
+        if len(shape) < self._min_dims:
+            shape = tuple(shape) + (1,)
+        if -1 in shape:
+            missing = -self.size // int(np.prod(shape))
+            shape = tuple(missing if x == -1 else x for x in shape)
+        shape = tuple(int(x) for x in shape)
+        if shape == self.shape:
+            return self
+        if int(np.prod(shape)) != self.size:
+            raise ValueError("total size of new array must be unchanged")
+        if self.take_array:
+            raise TypeError("reshaping of non-contiguous arrays is not yet supported")
+        strides = _reshape_strides(self.strides, self.shape, shape)
+        return self.__class__(backend=self.backend, shape=shape, dtype=self.dtype, base=self,
+                              gpudata=self.gpudata, strides=strides, name=self.name,
+                              rounding=self.rounding)
+
+    @property
+    def T(self):
+        """Transposed view: swapped strides, no data movement
+        (reference nervanagpu.py:552-578)."""
+        if len(self.shape) <= 2:
+            shape, strides = self.shape[::-1], self.strides[::-1]
+        else:
+            shape = list(self.shape[::-1])
+            strides = list(self.strides[::-1])
+            shape = tuple(shape[-1:] + shape[:-1])
+            strides = tuple(strides[-1:] + strides[:-1])
+        return self.__class__(backend=self.backend, shape=shape, dtype=self.dtype, base=self,
+                              gpudata=self.gpudata, strides=strides, is_trans=not self.is_trans,
+                              name=self.name, rounding=self.rounding)
+
+    def transpose(self, out=None):
+        if out:
+            return OpTreeNode.build("assign", out, self.T)
+        return self.T
+
+    def share(self, shape, dtype=None, name=None):
+        """New tensor over the first ``prod(shape)`` elements of this one's
+        memory (reference nervanagpu.py:589-618)."""
+        size = int(np.prod(shape))
+        if size > self.size:
+            raise ValueError("total size of new array must <= size of parent")
+        if not self.is_contiguous:
+            raise TypeError("sharing of non-contigous arrays is not yet supported")
+        dtype = self.dtype if dtype is None else np.dtype(dtype)
+        base = self if self.base is None else self.base
+        return self.__class__(backend=self.backend, shape=shape, dtype=dtype, base=base,
+                              gpudata=self.gpudata, strides=_contiguous_strides(tuple(shape)),
+                              name=name, rounding=self.rounding)
+
+
+class _FuseScope(object):
+    def __init__(self, be):
+        self.be = be
+
+    def __enter__(self):
+        self.be._fuse_depth += 1
+        self.be._fusing = True
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        self.be._fuse_depth -= 1
+        if self.be._fuse_depth == 0:
+            self.be._fusing = False
+            if exc_type is None:
+                self.be._flush()
+            else:
+                self.be._pending = []
+        return False
+
+
+class NervanaHIP(Backend):
+    """MI355X backend for the op-tree path.
+
+    Arguments mirror ``gen_backend``'s keyword set (reference
+    neon/backends/__init__.py:107-114).  ``stochastic_round`` is accepted and
+    must be falsy: rounding is to nearest even.
+    """
+    backend_name = "hip"
+
+    def __init__(self, rng_seed=None, default_dtype=np.float32, stochastic_round=False,
+                 deterministic=None, device_id=0, bench=False, scratch_size=0,
+                 hist_bins=64, hist_offset=-48, compat_mode=None, num_devices=None,
+                 cache_dir=None):
+        if default_dtype not in (np.float16, np.float32):
+            raise ValueError("Default data type for the hip backend must be float16 or 32")
+        if stochastic_round:
+            raise NotImplementedError("stochastic rounding is not implemented by the hip backend")
+        self.rt = None
+        self.rt = hiprt.Runtime(device_id or 0)       # raises if library or device is missing
+        if not self.rt.arch.startswith("gfx950"):
+            logger.warning("hip backend is written for gfx950; found %s", self.rt.arch)
+        super(NervanaHIP, self).__init__(rng_seed, default_dtype, compat_mode=compat_mode)
+        self.tensor_cls = HIPTensor
+        self.device_type = 1
+        self.device_id = device_id or 0
+        self.round_mode = None
+        self.bench = bench
+        self.stream = None
+        self.use_pinned_mem = False
+        self.hist_bins, self.hist_offset = hist_bins, hist_offset
+        self.cu_count = int(self.rt.props.compute_units)
+        self.kernels = KernelCache(self.rt.arch.split(":")[0], cache_dir)
+        self.plans = {}
+        self.plan_stats = {"hit": 0, "miss": 0, "split": 0, "launches": 0}
+        self._pending = []
+        self._fusing = False
+        self._fuse_depth = 0
+        self._temp_pool = {}
+        self._live_allocs = 0
+
+    # -- memory ---------------------------------------------------------------------
+    def _mem_alloc(self, nbytes):
+        self._live_allocs += 1
+        return self.rt.malloc(nbytes)
+
+    def _mem_free(self, ptr):
+        self._live_allocs -= 1
+        self.rt.free(ptr)
+
+    def cleanup_backend(self):
+        rt = getattr(self, "rt", None)
+        if rt is None:
+            return
+        try:
+            self._pending = []
+            rt.synchronize()
+            for plan in self.plans.values():
+                for p in (plan if isinstance(plan, list) else [plan]):
+                    p.release()
+            self.plans = {}
+            self._temp_pool = {}
+        except Exception:
+            pass
+
+    def synchronize(self):
+        self._flush()
+        self.rt.synchronize()
+
+    # -- allocation API (reference nervanagpu.py:1285-1439) --------------------------
+    def empty(self, shape, dtype=None, name=None, persist_values=True,
+              parallel=False, distributed=False, allocator=None):
+        dtype = self.default_dtype if dtype is None else dtype
+        return HIPTensor(self, shape, dtype=dtype, name=name, persist_values=persist_values)
+
+    def array(self, ary, dtype=None, name=None, persist_values=True,
+              parallel=False, distributed=False, allocator=None):
+        dtype = self.default_dtype if dtype is None else dtype
+        ary = np.asarray(ary)
+        if ary.ndim < self._min_dims:
+            ary = ary.reshape(ary.size, 1)
+        if ary.dtype != np.dtype(dtype):
+            ary = ary.astype(dtype)
+        return HIPTensor(self, ary.shape, dtype=dtype, name=name,
+                         persist_values=persist_values).set(ary)
+
+    def zeros(self, shape, dtype=None, name=None, persist_values=True,
+              parallel=False, distributed=False, allocator=None):
+        return self.empty(shape, dtype, name, persist_values)._assign(0)
+
+    def ones(self, shape, dtype=None, name=None, persist_values=True,
+             parallel=False, distributed=False, allocator=None):
+        return self.empty(shape, dtype, name, persist_values)._assign(1)
+
+    def empty_like(self, other_ary, name=None, persist_values=True):
+        return HIPTensor(self, other_ary.shape, dtype=other_ary.dtype, name=name,
+                         persist_values=persist_values)
+
+    def zeros_like(self, other_ary, name=None, persist_values=True):
+        return self.empty_like(other_ary, name, persist_values)._assign(0)
+
+    # -- timing marks (reference nervanagpu.py:3138-3177) -----------------------------
+    def init_mark(self):
+        return self.rt.event()
+
+    def record_mark(self, marker):
+        self._flush()
+        self.rt.event_record(marker)
+
+    def synchronize_mark(self, marker):
+        self.rt.event_sync(marker)
+
+    def get_time(self, start, end):
+        return self.rt.event_elapsed_ms(start, end)
+
+    # -- statement fusion ----------------------------------------------------------------
+    def fused(self):
+        """Context manager: elementwise assigns issued inside are queued and run
+        as ONE multi-output kernel when the block ends (or as soon as a
+        statement arrives that cannot join the group).  Later statements see
+        the values written by earlier ones, as if run one by one.  This is
+        what turns Adam's three assigns (reference optimizer.py:925-930) into a
+        single pass over the four tensors."""
+        return _FuseScope(self)
+
+    def begin(self, block, identifier):
+        """``Block.update`` opens a fusion group (the reference documents
+        begin/end as optimisation hints, backend.py:671-709)."""
+        from neon_amd.backends.backend import Block
+        if block == Block.update:
+            self._fuse_depth += 1
+            self._fusing = True
+
+    def end(self, block, identifier):
+        from neon_amd.backends.backend import Block
+        if block == Block.update and self._fuse_depth > 0:
+            self._fuse_depth -= 1
+            if self._fuse_depth == 0:
+                self._fusing = False
+                self._flush()
+
+    def _flush(self):
+        if self._pending:
+            trees, self._pending = self._pending, []
+            self._run(trees)
+
+    @staticmethod
+    def _is_elementwise(tree):
+        for p in tree.traverse(list()):
+            if isinstance(p, dict) and (p["op"] in REDUCE or p["op"] in ("dot", "transpose", "onehot")):
+                return False
+        return True
+
+    def _can_join(self, tree):
+        """A statement joins the pending group when it is purely elementwise,
+        every tensor in it has the group's shape and is contiguous (or is
+        1x1), so each lane only ever touches its own elements."""
+        if not self._is_elementwise(tree):
+            return False
+        shape = tree[1].shape
+        for p in [tree[1]] + [q for q in tree.traverse(list()) if isinstance(q, Tensor)]:
+            if p.size == 1 and p.is_contiguous:
+                if any(p.ptr == q[1].ptr for q in self._pending + [tree]):
+                    return False        # a scalar that is also written: order matters
+                continue
+            if p.shape != shape or not p.is_contiguous:
+                return False
+        if self._pending and self._pending[0][1].shape != shape:
+            return False
+        return True
+
+    # -- execution -----------------------------------------------------------------------
+    def execute(self, optree):
+        """Run ``assign(out, expr)`` (reference nervanagpu.py:1255-1283)."""
+        assert optree[0]["op"] == "assign"
+        if self._fusing:
+            if self._can_join(optree):
+                self._pending.append(optree)
+                return optree[1]
+            self._flush()
+        self._run([optree])
+        return optree[1]
+
+    def _run(self, trees):
+        try:
+            prog = Program()
+            for t in trees:
+                prog.add_statement(t)
+            prog.finalize()
+            key = prog.key()
+            plan = self.plans.get(key)
+            if plan is None:
+                self.plan_stats["miss"] += 1
+                plan = make_plan(prog, self.rt, self.kernels, self.cu_count)
+                self.plans[key] = plan
+            else:
+                self.plan_stats["hit"] += 1
+            plan.launch(prog)
+            self.plan_stats["launches"] += 1
+        except (NeedsSplit, MixedAxes, NotImplementedError) as e:
+            if len(trees) != 1:
+                for t in trees:
+                    self._run([t])
+                return
+            if isinstance(e, NotImplementedError) and not _splittable(trees[0]):
+                raise
+            self.plan_stats["split"] += 1
+            self._run_split(trees[0])
+
+    def _run_split(self, tree):
+        """Evaluate a tree that does not fit one kernel stage by stage through
+        temporaries: every reduction (innermost first) and every transposed
+        sub-expression is materialised, then the remaining elementwise tree is
+        assigned (the role of _split_to_stacks, reference
+        nervanagpu.py:1099-1237)."""
+        out, expr = tree[1], tree[2]
+        temps = []
+        memo = {}
+
+        def lower(node, top=False):
+            if not isinstance(node, OpTreeNode):
+                return node
+            op = node[0]["op"]
+            if op == "dot":
+                raise NotImplementedError("dot inside an op-tree is outside the hip backend's scope")
+            left = lower(node[1])
+            right = lower(node[2])
+            if op == "transpose":
+                if isinstance(left, HIPTensor):
+                    return left.T
+                tmp = self._temp(left.shape, np.float32, temps)
+                self._run([OpTreeNode({"op": "assign"}, tmp, left)])
+                return tmp.T
+            rebuilt = OpTreeNode(node[0], left, right)
+            if op in REDUCE:
+                if top:
+                    return rebuilt
+                k = rebuilt.key()
+                if k in memo:
+                    return memo[k]
+                tmp = self._temp(node[0]["shape"], np.float32, temps)
+                self._run([OpTreeNode({"op": "assign"}, tmp, rebuilt)])
+                memo[k] = tmp
+                return tmp
+            return rebuilt
+
+        try:
+            lowered = lower(expr, top=True)
+            self._run_leaf(OpTreeNode({"op": "assign"}, out, lowered))
+        finally:
+            for t in temps:
+                self._temp_release(t)
+
+    def _run_leaf(self, tree):
+        prog = Program()
+        prog.add_statement(tree)
+        prog.finalize()
+        key = prog.key()
+        plan = self.plans.get(key)
+        if plan is None:
+            self.plan_stats["miss"] += 1
+            try:
+                plan = make_plan(prog, self.rt, self.kernels, self.cu_count)
+            except NeedsSplit:
+                raise ValueError("op-tree cannot be mapped to the available kernel families")
+            self.plans[key] = plan
+        else:
+            self.plan_stats["hit"] += 1
+        plan.launch(prog)
+        self.plan_stats["launches"] += 1
+
+    def _temp(self, shape, dtype, temps):
+        key = (tuple(shape), np.dtype(dtype))
+        pool = self._temp_pool.setdefault(key, [])
+        t = pool.pop() if pool else HIPTensor(self, shape, dtype=dtype)
+        temps.append(t)
+        return t
+
+    def _temp_release(self, t):
+        # kernels run in stream order, so the buffer may be handed out again as
+        # soon as its last consumer has been enqueued
+        self._temp_pool.setdefault((t.shape, t.dtype), []).append(t)
+
+    # -- layer-level helpers that are plain op-trees ----------------------------------------
+    def consume(self, buf_index, hostlist, devlist):
+        assert 0 <= buf_index < 2, "Can only double buffer"
+        self._flush()
+        if devlist[buf_index] is None:
+            devlist[buf_index] = self.empty_like(hostlist[buf_index])
+        devlist[buf_index].set(hostlist[buf_index])
+
+    def set_hist_buffers(self, hist_bins, hist_offset):
+        self.hist_bins, self.hist_offset = hist_bins, hist_offset
+
+
+def _splittable(tree):
+    for p in tree.traverse(list()):
+        if isinstance(p, dict) and p["op"] == "transpose":
+            return True
+    return False

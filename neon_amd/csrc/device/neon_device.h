@@ -1,0 +1,298 @@
+// neon_device.h -- device-side building blocks for gfx950 (CDNA4, wave64).
+//
+// Shared by the prebuilt kernels (compiled with hipcc) and by every kernel the
+// op-tree code generator emits (this text is prepended to the generated source
+// and compiled with hiprtc).  Nothing here includes a system header so the
+// same text works in both places.
+//
+// Contents
+//   * storage types and conversions: fp32 compute, fp16 / bf16 / integer storage
+//   * 16-byte vector loads and stores
+//   * per-op scalar semantics matching the numpy CPU backend of the reference
+//     (neon/backends/nervanacpu.py:480-522)
+//   * wave64 cross-lane reductions built on DPP, and the LDS step that
+//     combines the waves of a workgroup
+#ifndef NEON_DEVICE_H
+#define NEON_DEVICE_H
+
+#define NEON_WAVE 64
+#define NEON_DEV __device__ __forceinline__
+
+typedef _Float16 nh_f16;
+typedef __bf16 nh_bf16;
+typedef signed char nh_i8;
+typedef unsigned char nh_u8;
+typedef short nh_i16;
+typedef unsigned short nh_u16;
+typedef int nh_i32;
+typedef unsigned int nh_u32;
+
+#define NH_INF __builtin_inff()
+#define NH_FLT_MAX 3.402823466e+38f
+
+// ---------------------------------------------------------------------------
+// storage <-> fp32
+// Loads widen exactly.  Stores follow numpy's unsafe cast, which is what the
+// CPU backend's `left[:] = right` does (nervanacpu.py:476-477): floating
+// targets round to nearest even, integer targets truncate toward zero.
+// ---------------------------------------------------------------------------
+template <typename T> NEON_DEV float nh_load_cvt(T x) { return (float)x; }
+
+template <typename T> struct nh_store_cvt;
+template <> struct nh_store_cvt<float>   { static NEON_DEV float   f(float x) { return x; } };
+template <> struct nh_store_cvt<nh_f16>  { static NEON_DEV nh_f16  f(float x) { return (nh_f16)x; } };
+template <> struct nh_store_cvt<nh_bf16> { static NEON_DEV nh_bf16 f(float x) { return (nh_bf16)x; } };
+template <> struct nh_store_cvt<nh_i32>  { static NEON_DEV nh_i32  f(float x) { return (nh_i32)x; } };
+template <> struct nh_store_cvt<nh_u32>  { static NEON_DEV nh_u32  f(float x) { return (nh_u32)(long long)x; } };
+template <> struct nh_store_cvt<nh_i16>  { static NEON_DEV nh_i16  f(float x) { return (nh_i16)(nh_i32)x; } };
+template <> struct nh_store_cvt<nh_u16>  { static NEON_DEV nh_u16  f(float x) { return (nh_u16)(nh_i32)x; } };
+template <> struct nh_store_cvt<nh_i8>   { static NEON_DEV nh_i8   f(float x) { return (nh_i8)(nh_i32)x; } };
+template <> struct nh_store_cvt<nh_u8>   { static NEON_DEV nh_u8   f(float x) { return (nh_u8)(nh_i32)x; } };
+
+// An index produced by argmax/argmin goes to an integer target unchanged and
+// to a floating target as its value.
+template <typename T> NEON_DEV T nh_store_index(int i) { return (T)i; }
+
+// ---------------------------------------------------------------------------
+// vector access: V consecutive elements, at most 16 bytes per instruction
+// ---------------------------------------------------------------------------
+template <typename T, int V> struct __attribute__((aligned(sizeof(T) * V > 16 ? 16 : sizeof(T) * V))) nh_vec {
+    T v[V];
+};
+
+template <typename T, int V> NEON_DEV void nh_load_vec(const T* __restrict__ p, T (&raw)[V]) {
+    const nh_vec<T, V> t = *reinterpret_cast<const nh_vec<T, V>*>(p);
+#pragma unroll
+    for (int j = 0; j < V; ++j) raw[j] = t.v[j];
+}
+
+template <typename T, int V> NEON_DEV void nh_store_vec(T* p, const T (&raw)[V]) {
+    nh_vec<T, V> t;
+#pragma unroll
+    for (int j = 0; j < V; ++j) t.v[j] = raw[j];
+    *reinterpret_cast<nh_vec<T, V>*>(p) = t;
+}
+
+// Packed 16-bit storage kept in 32-bit registers (two elements per register).
+typedef nh_f16 nh_f16x2 __attribute__((ext_vector_type(2)));
+NEON_DEV float nh_f16_lo(nh_u32 w) { return (float)__builtin_bit_cast(nh_f16x2, w).x; }
+NEON_DEV float nh_f16_hi(nh_u32 w) { return (float)__builtin_bit_cast(nh_f16x2, w).y; }
+NEON_DEV nh_u32 nh_f16_pack(float lo, float hi) {
+    nh_f16x2 h; h.x = (nh_f16)lo; h.y = (nh_f16)hi;
+    return __builtin_bit_cast(nh_u32, h);
+}
+NEON_DEV float nh_bf16_lo(nh_u32 w) { return __builtin_bit_cast(float, w << 16); }
+NEON_DEV float nh_bf16_hi(nh_u32 w) { return __builtin_bit_cast(float, w & 0xFFFF0000u); }
+// Compiler barrier on register-resident data: the values are unchanged but
+// treated as new, so work derived from them before the call (e.g. widened
+// copies) is not kept alive across it.
+template <int N> NEON_DEV void nh_keep_packed(nh_u32 (&w)[N]) {
+#pragma unroll
+    for (int j = 0; j < N; ++j) asm volatile("" : "+v"(w[j]));
+}
+
+// ---------------------------------------------------------------------------
+// Register tiles.  nh_raw<T,V> holds V consecutive elements of storage type T
+// exactly as they sit in memory (32-bit words, 16-bit types two per word), so
+// a tile that stays resident across several sweeps costs V*sizeof(T)/4
+// registers; get(j) widens one element to fp32 on use.  nh_out<T,V> is the
+// store-side mirror: set(j, x) narrows, store() writes the words.
+// When V*sizeof(T) is not a multiple of 4 (V == 1 with a narrow type) the
+// single element lives in word 0.
+// ---------------------------------------------------------------------------
+template <typename T> struct nh_is_float { static constexpr bool value = false; };
+template <> struct nh_is_float<float> { static constexpr bool value = true; };
+template <> struct nh_is_float<nh_f16> { static constexpr bool value = true; };
+template <> struct nh_is_float<nh_bf16> { static constexpr bool value = true; };
+
+template <typename T> NEON_DEV nh_u32 nh_bits_of(T x) {
+    if constexpr (sizeof(T) == 4) return __builtin_bit_cast(nh_u32, x);
+    else if constexpr (sizeof(T) == 2) return (nh_u32)__builtin_bit_cast(nh_u16, x);
+    else return (nh_u32)__builtin_bit_cast(nh_u8, x);
+}
+template <typename T> NEON_DEV T nh_from_bits(nh_u32 b) {
+    if constexpr (sizeof(T) == 4) return __builtin_bit_cast(T, b);
+    else if constexpr (sizeof(T) == 2) return __builtin_bit_cast(T, (nh_u16)b);
+    else return __builtin_bit_cast(T, (nh_u8)b);
+}
+
+template <typename T, int V> struct nh_raw {
+    static constexpr int BYTES = (int)sizeof(T) * V;
+    static constexpr bool PACKED = (BYTES % 4) == 0;
+    static constexpr int NW = PACKED ? BYTES / 4 : 1;
+    static constexpr int PER = 4 / (int)sizeof(T);  // elements per word
+    nh_u32 w[NW];
+
+    NEON_DEV void load(const T* p) {
+        if constexpr (PACKED) nh_load_vec<nh_u32, NW>(reinterpret_cast<const nh_u32*>(p), w);
+        else w[0] = nh_bits_of<T>(*p);
+    }
+    NEON_DEV void zero() {
+#pragma unroll
+        for (int i = 0; i < NW; ++i) w[i] = 0u;
+    }
+    NEON_DEV float get(int j) const {
+        const nh_u32 word = w[PACKED ? j / PER : 0];
+        const int sub = PACKED ? j % PER : 0;
+        const nh_u32 bits = (sizeof(T) == 4) ? word : (word >> (8 * (int)sizeof(T) * sub));
+        return (float)nh_from_bits<T>(bits);
+    }
+    NEON_DEV int geti(int j) const {  // integer view, for index tensors
+        const nh_u32 word = w[PACKED ? j / PER : 0];
+        const int sub = PACKED ? j % PER : 0;
+        const nh_u32 bits = (sizeof(T) == 4) ? word : (word >> (8 * (int)sizeof(T) * sub));
+        return (int)nh_from_bits<T>(bits);
+    }
+    NEON_DEV void keep() {
+#pragma unroll
+        for (int i = 0; i < NW; ++i) asm volatile("" : "+v"(w[i]));
+    }
+};
+
+template <typename T, int V> struct nh_out {
+    static constexpr int BYTES = (int)sizeof(T) * V;
+    static constexpr bool PACKED = (BYTES % 4) == 0;
+    static constexpr int NW = PACKED ? BYTES / 4 : 1;
+    static constexpr int PER = 4 / (int)sizeof(T);
+    nh_u32 w[NW];
+
+    NEON_DEV void clear() {
+#pragma unroll
+        for (int i = 0; i < NW; ++i) w[i] = 0u;
+    }
+    NEON_DEV void put_bits(int j, nh_u32 bits) {
+        if constexpr (sizeof(T) == 4) w[PACKED ? j : 0] = bits;
+        else w[PACKED ? j / PER : 0] |= bits << (8 * (int)sizeof(T) * (PACKED ? j % PER : 0));
+    }
+    NEON_DEV void set(int j, float x) { put_bits(j, nh_bits_of<T>(nh_store_cvt<T>::f(x))); }
+    NEON_DEV void seti(int j, int i) { put_bits(j, nh_bits_of<T>(nh_store_index<T>(i))); }
+    NEON_DEV void store(T* p) const {
+        if constexpr (PACKED) nh_store_vec<nh_u32, NW>(reinterpret_cast<nh_u32*>(p), w);
+        else *p = nh_from_bits<T>(w[0]);
+    }
+};
+
+// value after a round trip through storage type T (what a later read of a
+// just-written tensor would see)
+template <typename T> NEON_DEV float nh_quant(float x) { return (float)nh_store_cvt<T>::f(x); }
+
+// ---------------------------------------------------------------------------
+// scalar op semantics (CPU-backend flavour where the two backends of the
+// reference differ: safelog clamps its argument, sign(nan) is nan,
+// minimum/maximum and max/min reductions propagate nan like numpy)
+// ---------------------------------------------------------------------------
+NEON_DEV float nh_max(float a, float b) { return (a != a) ? a : ((b != b) ? b : __builtin_fmaxf(a, b)); }
+NEON_DEV float nh_min(float a, float b) { return (a != a) ? a : ((b != b) ? b : __builtin_fminf(a, b)); }
+NEON_DEV float nh_sgn(float x) { return (x != x) ? x : (float)((x > 0.0f) - (x < 0.0f)); }
+NEON_DEV float nh_sqr(float x) { return x * x; }
+NEON_DEV float nh_safelog(float x) { return logf(nh_max(x, 1.9287498479639178e-22f)); }  // exp(-50)
+NEON_DEV float nh_sig(float x) { return 1.0f / (1.0f + expf(-x)); }
+NEON_DEV float nh_sig2(float x) { return 1.0f / (1.0f + exp2f(-x)); }
+NEON_DEV float nh_tanh2(float x) { const float e = exp2f(2.0f * x); return (e - 1.0f) / (e + 1.0f); }
+NEON_DEV float nh_finite(float x) { return (__builtin_fabsf(x) <= NH_FLT_MAX) ? 1.0f : 0.0f; }
+
+// ---------------------------------------------------------------------------
+// DPP lane permutations.  Every lane of the wave must be active at the call.
+// ---------------------------------------------------------------------------
+#define NH_DPP_XOR1 0xB1        // quad_perm:[1,0,3,2]
+#define NH_DPP_XOR2 0x4E        // quad_perm:[2,3,0,1]
+#define NH_DPP_HALF_MIRROR 0x141  // lane i <-> 7-i inside each group of 8
+#define NH_DPP_MIRROR 0x140     // lane i <-> 15-i inside each row of 16
+#define NH_SWIZZLE_XOR16 0x401F // ds_swizzle bit mode: and 0x1f, or 0, xor 0x10
+
+template <int CTRL> NEON_DEV float nh_dpp(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+template <int CTRL> NEON_DEV int nh_dpp(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false);
+}
+NEON_DEV float nh_swz16(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), NH_SWIZZLE_XOR16));
+}
+NEON_DEV int nh_swz16(int v) { return __builtin_amdgcn_ds_swizzle(v, NH_SWIZZLE_XOR16); }
+template <int LANE> NEON_DEV float nh_readlane(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), LANE));
+}
+template <int LANE> NEON_DEV int nh_readlane(int v) { return __builtin_amdgcn_readlane(v, LANE); }
+
+// ---------------------------------------------------------------------------
+// reduction operators.  A value-reduction carries one float; an arg-reduction
+// carries (value, index) and breaks ties toward the lower index, which is what
+// np.argmax / np.argmin return (first occurrence).
+// ---------------------------------------------------------------------------
+struct nh_op_sum { static NEON_DEV float init() { return 0.0f; }      static NEON_DEV float f(float a, float b) { return a + b; } };
+struct nh_op_max { static NEON_DEV float init() { return -NH_INF; }   static NEON_DEV float f(float a, float b) { return nh_max(a, b); } };
+struct nh_op_min { static NEON_DEV float init() { return NH_INF; }    static NEON_DEV float f(float a, float b) { return nh_min(a, b); } };
+
+struct nh_pair { float v; int i; };
+struct nh_op_argmax {
+    static NEON_DEV nh_pair init() { nh_pair p; p.v = -NH_INF; p.i = 0; return p; }
+    static NEON_DEV nh_pair f(nh_pair a, nh_pair b) {
+        const bool take_b = (b.v > a.v) || (b.v == a.v && b.i < a.i);
+        nh_pair r; r.v = take_b ? b.v : a.v; r.i = take_b ? b.i : a.i; return r;
+    }
+    // sequential update with strictly increasing indices keeps the first hit
+    static NEON_DEV void step(nh_pair& a, float v, int i) { if (v > a.v) { a.v = v; a.i = i; } }
+};
+struct nh_op_argmin {
+    static NEON_DEV nh_pair init() { nh_pair p; p.v = NH_INF; p.i = 0; return p; }
+    static NEON_DEV nh_pair f(nh_pair a, nh_pair b) {
+        const bool take_b = (b.v < a.v) || (b.v == a.v && b.i < a.i);
+        nh_pair r; r.v = take_b ? b.v : a.v; r.i = take_b ? b.i : a.i; return r;
+    }
+    static NEON_DEV void step(nh_pair& a, float v, int i) { if (v < a.v) { a.v = v; a.i = i; } }
+};
+
+template <int CTRL> NEON_DEV nh_pair nh_dpp(nh_pair p) { nh_pair r; r.v = nh_dpp<CTRL>(p.v); r.i = nh_dpp<CTRL>(p.i); return r; }
+NEON_DEV nh_pair nh_swz16(nh_pair p) { nh_pair r; r.v = nh_swz16(p.v); r.i = nh_swz16(p.i); return r; }
+template <int LANE> NEON_DEV nh_pair nh_readlane(nh_pair p) { nh_pair r; r.v = nh_readlane<LANE>(p.v); r.i = nh_readlane<LANE>(p.i); return r; }
+
+// Exchange with the lane whose index differs in bit log2(S).  Strides below 32
+// use ds_swizzle in bit mode (crossbar only, no LDS memory); 32 crosses the two
+// halves of the wave with ds_bpermute.
+template <int S> NEON_DEV int nh_lane_xor(int v) {
+    if constexpr (S < 32) return __builtin_amdgcn_ds_swizzle(v, 0x1F | (S << 10));
+    else return __builtin_amdgcn_ds_bpermute((int)((__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)) ^ 32u) << 2), v);
+}
+template <int S> NEON_DEV float nh_lane_xor(float v) {
+    return __builtin_bit_cast(float, nh_lane_xor<S>(__builtin_bit_cast(int, v)));
+}
+template <int S> NEON_DEV nh_pair nh_lane_xor(nh_pair p) {
+    nh_pair r; r.v = nh_lane_xor<S>(p.v); r.i = nh_lane_xor<S>(p.i); return r;
+}
+
+// All-reduce over aligned groups of WIDTH lanes (WIDTH in 1,2,4,...,64): every
+// lane of a group ends with the group's result.  Steps 1-2 are quad
+// permutes; steps 4 and 8 use the mirror patterns, valid because the previous
+// steps made each group of 4 / 8 lanes uniform; 16 uses ds_swizzle (no LDS
+// memory is touched); 64 finishes through four scalar lane reads.
+template <class OP, int WIDTH, typename T> NEON_DEV T nh_wave_allreduce(T v) {
+    if (WIDTH >= 2) v = OP::f(v, nh_dpp<NH_DPP_XOR1>(v));
+    if (WIDTH >= 4) v = OP::f(v, nh_dpp<NH_DPP_XOR2>(v));
+    if (WIDTH >= 8) v = OP::f(v, nh_dpp<NH_DPP_HALF_MIRROR>(v));
+    if (WIDTH >= 16) v = OP::f(v, nh_dpp<NH_DPP_MIRROR>(v));
+    if (WIDTH == 32) v = OP::f(v, nh_swz16(v));
+    if (WIDTH == 64) {
+        const T a = nh_readlane<0>(v), b = nh_readlane<16>(v), c = nh_readlane<32>(v), d = nh_readlane<48>(v);
+        v = OP::f(OP::f(a, b), OP::f(c, d));
+    }
+    return v;
+}
+
+// Workgroup all-reduce: DPP inside each wave, then one LDS slot per wave.
+// `slots` must hold NWAVES entries of T; the two barriers make the buffer
+// reusable by the next call.  All threads of the workgroup must call it.
+template <class OP, int NWAVES, typename T> NEON_DEV T nh_block_allreduce(T v, T* slots) {
+    v = nh_wave_allreduce<OP, 64>(v);
+    if (NWAVES == 1) return v;
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) slots[wave] = v;
+    __syncthreads();
+    T r = slots[0];
+#pragma unroll
+    for (int w = 1; w < NWAVES; ++w) r = OP::f(r, slots[w]);
+    __syncthreads();
+    return r;
+}
+
+#endif  // NEON_DEVICE_H

@@ -1,0 +1,460 @@
+// Prebuilt hand-written gfx950 kernels behind the direct entry points of
+// include/neonhip.h.  All of them are HBM-bound streaming kernels: every
+// global access is a 16-byte vector per lane, arithmetic is fp32, and nothing
+// is read twice.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "neonhip.h"
+#include "device/neon_device.h"
+
+bool nh_internal_ready();
+int nh_internal_fail(int code, const char* msg);
+int nh_internal_cu_count();
+
+namespace {
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int launch_status(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return nh_internal_fail((int)e, what);
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Streaming elementwise kernels: 256 threads, each owning EW_U vectors of V
+// floats spaced a workgroup apart (so every wave touches 1 KiB contiguous per
+// instruction).  All loads of a tile are issued before the first use.
+// ---------------------------------------------------------------------------
+constexpr int EW_T = 256;
+constexpr int EW_U = 4;
+
+template <int V, class F>
+__global__ __launch_bounds__(EW_T) void ew_stream_kernel(F f, size_t n) {
+    const size_t tile = (size_t)blockIdx.x * (EW_T * EW_U * V);
+    const int tid = threadIdx.x;
+    if (tile + (size_t)EW_T * EW_U * V <= n) {
+        typename F::template regs<V> r[EW_U];
+#pragma unroll
+        for (int u = 0; u < EW_U; ++u) f.template load<V>(r[u], tile + (size_t)(u * EW_T + tid) * V);
+#pragma unroll
+        for (int u = 0; u < EW_U; ++u) {
+            f.template compute<V>(r[u]);
+            f.template store<V>(r[u], tile + (size_t)(u * EW_T + tid) * V);
+        }
+    } else {
+        for (size_t i = tile + tid; i < n; i += EW_T) {
+            typename F::template regs<1> r;
+            f.template load<1>(r, i);
+            f.template compute<1>(r);
+            f.template store<1>(r, i);
+        }
+    }
+}
+
+struct AxpbyF {
+    float* out; const float* x; const float* y; float a, b;
+    template <int V> struct regs { float x[V], y[V]; };
+    template <int V> __device__ void load(regs<V>& r, size_t i) const { nh_load_vec<float, V>(x + i, r.x); nh_load_vec<float, V>(y + i, r.y); }
+    template <int V> __device__ void compute(regs<V>& r) const {
+#pragma unroll
+        for (int j = 0; j < V; ++j) r.x[j] = a * r.x[j] + b * r.y[j];
+    }
+    template <int V> __device__ void store(const regs<V>& r, size_t i) const { nh_store_vec<float, V>(out + i, r.x); }
+};
+
+struct SigmoidF {
+    float* out; const float* x;
+    template <int V> struct regs { float x[V]; };
+    template <int V> __device__ void load(regs<V>& r, size_t i) const { nh_load_vec<float, V>(x + i, r.x); }
+    template <int V> __device__ void compute(regs<V>& r) const {
+#pragma unroll
+        for (int j = 0; j < V; ++j) r.x[j] = nh_sig(r.x[j]);
+    }
+    template <int V> __device__ void store(const regs<V>& r, size_t i) const { nh_store_vec<float, V>(out + i, r.x); }
+};
+
+// The three assigns of the reference's Adam.optimize
+// (neon/optimizers/optimizer.py:925-930) fused: 4 tensors read, 3 written.
+// Operation order follows the Python expressions so that, with contraction
+// off, the result is the one numpy computes in fp32.
+struct AdamF {
+    float* p; float* m; float* v; const float* g;
+    float lr, b1, omb1, b2, omb2, eps;
+    template <int V> struct regs { float p[V], m[V], v[V], g[V]; };
+    template <int V> __device__ void load(regs<V>& r, size_t i) const {
+        nh_load_vec<float, V>(g + i, r.g); nh_load_vec<float, V>(m + i, r.m);
+        nh_load_vec<float, V>(v + i, r.v); nh_load_vec<float, V>(p + i, r.p);
+    }
+    template <int V> __device__ void compute(regs<V>& r) const {
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            const float gj = r.g[j];
+            const float mj = r.m[j] * b1 + omb1 * gj;
+            const float vj = r.v[j] * b2 + (omb2 * gj) * gj;
+            r.m[j] = mj;
+            r.v[j] = vj;
+            r.p[j] = r.p[j] - (lr * mj) / (sqrtf(vj) + eps);
+        }
+    }
+    template <int V> __device__ void store(const regs<V>& r, size_t i) const {
+        nh_store_vec<float, V>(m + i, r.m); nh_store_vec<float, V>(v + i, r.v); nh_store_vec<float, V>(p + i, r.p);
+    }
+};
+
+template <class F> int launch_ew(const F& f, size_t n, bool vec_ok, void* stream, const char* what) {
+    if (!nh_internal_ready()) return nh_internal_fail(NH_ENOTINIT, "nh_init has not been called");
+    if (n == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (vec_ok) {
+        const size_t per_block = (size_t)EW_T * EW_U * 4;
+        const size_t blocks = (n + per_block - 1) / per_block;
+        if (blocks > 0x7FFFFFFFull) return nh_internal_fail(NH_EINVAL, "tensor too large for one launch");
+        hipLaunchKernelGGL((ew_stream_kernel<4, F>), dim3((unsigned)blocks), dim3(EW_T), 0, s, f, n);
+    } else {
+        const size_t per_block = (size_t)EW_T * EW_U;
+        const size_t blocks = (n + per_block - 1) / per_block;
+        if (blocks > 0x7FFFFFFFull) return nh_internal_fail(NH_EINVAL, "tensor too large for one launch");
+        hipLaunchKernelGGL((ew_stream_kernel<1, F>), dim3((unsigned)blocks), dim3(EW_T), 0, s, f, n);
+    }
+    return launch_status(what);
+}
+
+// ---------------------------------------------------------------------------
+// Row normalisation, fp16 storage / fp32 statistics.  One workgroup of 1024
+// threads owns one row and keeps it in registers as raw fp16 vectors (NCH
+// chunks of 8 halves per thread), so the row is read from HBM exactly once:
+// sweep 1 sums, sweep 2 sums squared deviations, sweep 3 normalises and
+// stores.  Cross-lane sums use DPP; LDS only joins the 16 waves.
+// ---------------------------------------------------------------------------
+constexpr int RN_T = 1024;
+constexpr int RN_V = 8;
+
+template <int NCH>
+__global__ __launch_bounds__(RN_T) void rownorm_f16_kernel(nh_f16* out, const nh_f16* x,
+                                                           const float* __restrict__ gamma,
+                                                           const float* __restrict__ beta, float eps, uint32_t cols,
+                                                           size_t ld, float inv_n) {
+    __shared__ float slots[RN_T / 64];
+    const uint32_t row = blockIdx.x;
+    const int tid = threadIdx.x;
+    const nh_f16* xr = x + (size_t)row * ld;
+    nh_f16* orow = out + (size_t)row * ld;
+
+    // The row stays packed (two halves per register) for the whole kernel;
+    // nh_keep_packed() between sweeps stops the compiler from widening it to
+    // one fp32 register per element, which would not fit the register file.
+    nh_u32 raw[NCH][RN_V / 2];
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+        const uint32_t c = (uint32_t)(k * RN_T + tid) * RN_V;
+        if (c < cols) {
+            nh_load_vec<nh_u32, RN_V / 2>(reinterpret_cast<const nh_u32*>(xr + c), raw[k]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < RN_V / 2; ++j) raw[k][j] = 0u;  // +0.0 pairs
+        }
+    }
+    const float g = gamma[row];
+    const float b = beta[row];
+
+    float s = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NCH; ++k)
+#pragma unroll
+        for (int j = 0; j < RN_V / 2; ++j) {  // padding chunks hold zeros
+            s += nh_f16_lo(raw[k][j]);
+            s += nh_f16_hi(raw[k][j]);
+        }
+    const float mean = nh_block_allreduce<nh_op_sum, RN_T / 64>(s, slots) * inv_n;
+
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) nh_keep_packed(raw[k]);
+    float q = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+        const uint32_t c = (uint32_t)(k * RN_T + tid) * RN_V;
+        if (c < cols) {
+#pragma unroll
+            for (int j = 0; j < RN_V / 2; ++j) {
+                q += nh_sqr(nh_f16_lo(raw[k][j]) - mean);
+                q += nh_sqr(nh_f16_hi(raw[k][j]) - mean);
+            }
+        }
+    }
+    const float var = nh_block_allreduce<nh_op_sum, RN_T / 64>(q, slots) * inv_n;
+    const float denom = sqrtf(var + eps);
+
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) nh_keep_packed(raw[k]);
+#pragma unroll
+    for (int k = 0; k < NCH; ++k) {
+        const uint32_t c = (uint32_t)(k * RN_T + tid) * RN_V;
+        if (c < cols) {
+            nh_u32 o[RN_V / 2];
+#pragma unroll
+            for (int j = 0; j < RN_V / 2; ++j)
+                o[j] = nh_f16_pack((g * (nh_f16_lo(raw[k][j]) - mean)) / denom + b,
+                                   (g * (nh_f16_hi(raw[k][j]) - mean)) / denom + b);
+            nh_store_vec<nh_u32, RN_V / 2>(reinterpret_cast<nh_u32*>(orow + c), o);
+        }
+    }
+}
+
+template <int NCH>
+void launch_rownorm(uint16_t* out, const uint16_t* x, const float* gamma, const float* beta, float eps,
+                    uint32_t rows, uint32_t cols, size_t ld, hipStream_t s) {
+    hipLaunchKernelGGL((rownorm_f16_kernel<NCH>), dim3(rows), dim3(RN_T), 0, s, (nh_f16*)out, (const nh_f16*)x,
+                       gamma, beta, eps, cols, ld, 1.0f / (float)cols);
+}
+
+// ---------------------------------------------------------------------------
+// Column (axis-0) max / argmax.  Lanes run across columns so every load is
+// coalesced; a workgroup is CR_LX column-lanes x CR_LY row-lanes and owns a
+// (rows_per_chunk x CR_LX*V) tile.  Tiles of one column strip leave (value,
+// index) partials in the workspace; the last workgroup of the strip to finish
+// (ticket counter) folds them, in row order, into the result.  No workgroup
+// ever waits for another.
+// ---------------------------------------------------------------------------
+constexpr int CR_LX = 16;
+constexpr int CR_LY = 16;
+constexpr int CR_T = CR_LX * CR_LY;
+constexpr int CR_MAX_STRIPS = 4096;
+constexpr int CR_MAX_CHUNKS = 128;
+
+__device__ unsigned int g_cr_tickets[CR_MAX_STRIPS];  // zero at load; each strip's last workgroup resets its ticket
+
+template <int V>
+__device__ __forceinline__ void cr_fold_rows(nh_pair (&acc)[V], float (*sv)[CR_LX * V + 1], int (*si)[CR_LX * V + 1],
+                                              int tx, int ty) {
+    // join the CR_LY row-lanes of each column through LDS, lowest rows first
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        sv[ty][tx * V + j] = acc[j].v;
+        si[ty][tx * V + j] = acc[j].i;
+    }
+    __syncthreads();
+    if (ty == 0) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            nh_pair r;
+            r.v = sv[0][tx * V + j];
+            r.i = si[0][tx * V + j];
+            for (int y = 1; y < CR_LY; ++y) {
+                nh_pair o;
+                o.v = sv[y][tx * V + j];
+                o.i = si[y][tx * V + j];
+                r = nh_op_argmax::f(r, o);
+            }
+            acc[j] = r;
+        }
+    }
+    __syncthreads();
+}
+
+template <int V>
+__global__ __launch_bounds__(CR_T) void colmax_kernel(const float* __restrict__ x, uint32_t rows, uint32_t cols,
+                                                      size_t ld, uint32_t rows_per_chunk, float* pval, int* pidx,
+                                                      float* __restrict__ outv, int* __restrict__ outi,
+                                                      unsigned int* tickets) {
+    __shared__ float sv[CR_LY][CR_LX * V + 1];
+    __shared__ int si[CR_LY][CR_LX * V + 1];
+    __shared__ int s_last;
+    const int tid = threadIdx.x;
+    const int tx = tid % CR_LX, ty = tid / CR_LX;
+    const uint32_t c = (blockIdx.x * CR_LX + tx) * V;
+    const uint32_t r0 = blockIdx.y * rows_per_chunk;
+    const uint32_t r1 = (r0 + rows_per_chunk < rows) ? r0 + rows_per_chunk : rows;
+    const bool live = c < cols;  // cols % V == 0 is checked on the host
+
+    nh_pair acc[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) acc[j] = nh_op_argmax::init();
+    if (live) {
+        const float* xp = x + c;
+        uint32_t r = r0 + ty;
+        // four independent rows in flight per lane
+        for (; r + 3 * CR_LY < r1; r += 4 * CR_LY) {
+            float a0[V], a1[V], a2[V], a3[V];
+            nh_load_vec<float, V>(xp + (size_t)r * ld, a0);
+            nh_load_vec<float, V>(xp + (size_t)(r + CR_LY) * ld, a1);
+            nh_load_vec<float, V>(xp + (size_t)(r + 2 * CR_LY) * ld, a2);
+            nh_load_vec<float, V>(xp + (size_t)(r + 3 * CR_LY) * ld, a3);
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                nh_op_argmax::step(acc[j], a0[j], (int)r);
+                nh_op_argmax::step(acc[j], a1[j], (int)(r + CR_LY));
+                nh_op_argmax::step(acc[j], a2[j], (int)(r + 2 * CR_LY));
+                nh_op_argmax::step(acc[j], a3[j], (int)(r + 3 * CR_LY));
+            }
+        }
+        for (; r < r1; r += CR_LY) {
+            float a0[V];
+            nh_load_vec<float, V>(xp + (size_t)r * ld, a0);
+#pragma unroll
+            for (int j = 0; j < V; ++j) nh_op_argmax::step(acc[j], a0[j], (int)r);
+        }
+    }
+    cr_fold_rows<V>(acc, sv, si, tx, ty);
+
+    const uint32_t nchunks = gridDim.y;
+    if (nchunks == 1) {
+        if (ty == 0 && live) {
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                if (outv) outv[c + j] = acc[j].v;
+                if (outi) outi[c + j] = acc[j].i;
+            }
+        }
+        return;
+    }
+    if (ty == 0 && live) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            pval[(size_t)blockIdx.y * cols + c + j] = acc[j].v;
+            pidx[(size_t)blockIdx.y * cols + c + j] = acc[j].i;
+        }
+    }
+    __threadfence();  // partials visible device-wide before the ticket is taken
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned int t = atomicAdd(&tickets[blockIdx.x], 1u);
+        s_last = (t == nchunks - 1);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();  // acquire: drop any stale cached copy of the partials
+
+#pragma unroll
+    for (int j = 0; j < V; ++j) acc[j] = nh_op_argmax::init();
+    if (live) {
+        for (uint32_t k = ty; k < nchunks; k += CR_LY) {
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                nh_pair o;
+                o.v = pval[(size_t)k * cols + c + j];
+                o.i = pidx[(size_t)k * cols + c + j];
+                acc[j] = nh_op_argmax::f(acc[j], o);
+            }
+        }
+    }
+    cr_fold_rows<V>(acc, sv, si, tx, ty);
+    if (ty == 0 && live) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            if (outv) outv[c + j] = acc[j].v;
+            if (outi) outi[c + j] = acc[j].i;
+        }
+    }
+    if (tid == 0) tickets[blockIdx.x] = 0;  // ready for the next launch on this stream
+}
+
+struct CrPlan { uint32_t strips, chunks, rows_per_chunk; int v; };
+
+CrPlan cr_plan(uint32_t rows, uint32_t cols, bool vec) {
+    CrPlan p;
+    p.v = vec ? 4 : 1;
+    const uint32_t strip_cols = CR_LX * p.v;
+    p.strips = (cols + strip_cols - 1) / strip_cols;
+    const uint32_t target_groups = 1024;  // about four workgroups per compute unit
+    uint32_t chunks = target_groups / (p.strips ? p.strips : 1);
+    if (chunks < 1) chunks = 1;
+    if (chunks > CR_MAX_CHUNKS) chunks = CR_MAX_CHUNKS;
+    uint32_t rpc = (rows + chunks - 1) / chunks;
+    const uint32_t min_rpc = 4 * CR_LY;
+    if (rpc < min_rpc) rpc = min_rpc;
+    rpc = (rpc + CR_LY - 1) / CR_LY * CR_LY;
+    p.rows_per_chunk = rpc;
+    p.chunks = (rows + rpc - 1) / rpc;
+    if (p.chunks < 1) p.chunks = 1;
+    return p;
+}
+
+}  // namespace
+
+extern "C" {
+
+int nh_ew_axpby_f32(float* out, const float* x, const float* y, float alpha, float beta, size_t n, void* stream) {
+    if (n && (!out || !x || !y)) return nh_internal_fail(NH_EINVAL, "nh_ew_axpby_f32: null pointer");
+    AxpbyF f{out, x, y, alpha, beta};
+    return launch_ew(f, n, aligned16(out) && aligned16(x) && aligned16(y), stream, "nh_ew_axpby_f32");
+}
+
+int nh_ew_sigmoid_f32(float* out, const float* x, size_t n, void* stream) {
+    if (n && (!out || !x)) return nh_internal_fail(NH_EINVAL, "nh_ew_sigmoid_f32: null pointer");
+    SigmoidF f{out, x};
+    return launch_ew(f, n, aligned16(out) && aligned16(x), stream, "nh_ew_sigmoid_f32");
+}
+
+int nh_adam_step_f32(float* param, float* m, float* v, const float* grad, float lr_t, float beta1,
+                     float one_minus_beta1, float beta2, float one_minus_beta2, float eps, size_t n,
+                     void* stream) {
+    if (n && (!param || !m || !v || !grad)) return nh_internal_fail(NH_EINVAL, "nh_adam_step_f32: null pointer");
+    AdamF f{param, m, v, grad, lr_t, beta1, one_minus_beta1, beta2, one_minus_beta2, eps};
+    return launch_ew(f, n, aligned16(param) && aligned16(m) && aligned16(v) && aligned16(grad), stream,
+                     "nh_adam_step_f32");
+}
+
+int nh_rownorm_f16(uint16_t* out, const uint16_t* x, const float* gamma, const float* beta, float eps,
+                   uint32_t rows, uint32_t cols, size_t ld, void* stream) {
+    if (!nh_internal_ready()) return nh_internal_fail(NH_ENOTINIT, "nh_init has not been called");
+    if (rows == 0 || cols == 0) return 0;
+    if (!out || !x || !gamma || !beta) return nh_internal_fail(NH_EINVAL, "nh_rownorm_f16: null pointer");
+    if (cols > NH_ROWNORM_MAX_COLS) return nh_internal_fail(NH_EINVAL, "nh_rownorm_f16: row longer than NH_ROWNORM_MAX_COLS");
+    if (cols % RN_V || ld % RN_V || ld < cols || !aligned16(out) || !aligned16(x))
+        return nh_internal_fail(NH_EINVAL, "nh_rownorm_f16: cols and ld must be multiples of 8 and pointers 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    const uint32_t per_pass = RN_T * RN_V;
+    const uint32_t nch = (cols + per_pass - 1) / per_pass;
+    switch (nch) {
+        case 1: launch_rownorm<1>(out, x, gamma, beta, eps, rows, cols, ld, s); break;
+        case 2: launch_rownorm<2>(out, x, gamma, beta, eps, rows, cols, ld, s); break;
+        case 3: case 4: launch_rownorm<4>(out, x, gamma, beta, eps, rows, cols, ld, s); break;
+        case 5: case 6: launch_rownorm<6>(out, x, gamma, beta, eps, rows, cols, ld, s); break;
+        case 7: case 8: launch_rownorm<8>(out, x, gamma, beta, eps, rows, cols, ld, s); break;
+        case 9: case 10: launch_rownorm<10>(out, x, gamma, beta, eps, rows, cols, ld, s); break;
+        case 11: case 12: case 13: launch_rownorm<13>(out, x, gamma, beta, eps, rows, cols, ld, s); break;
+        default: launch_rownorm<16>(out, x, gamma, beta, eps, rows, cols, ld, s); break;
+    }
+    return launch_status("nh_rownorm_f16");
+}
+
+size_t nh_colreduce_workspace_bytes(uint32_t rows, uint32_t cols) {
+    if (rows == 0 || cols == 0) return 0;
+    const CrPlan p = cr_plan(rows, cols, true);
+    const CrPlan q = cr_plan(rows, cols, false);
+    const size_t chunks = p.chunks > q.chunks ? p.chunks : q.chunks;
+    return chunks * (size_t)cols * (sizeof(float) + sizeof(int)) + 256;
+}
+
+int nh_colmax_argmax_f32(float* maxval, int32_t* argmax, const float* x, uint32_t rows, uint32_t cols, size_t ld,
+                         void* workspace, void* stream) {
+    if (!nh_internal_ready()) return nh_internal_fail(NH_ENOTINIT, "nh_init has not been called");
+    if (rows == 0 || cols == 0) return 0;
+    if (!x || (!maxval && !argmax)) return nh_internal_fail(NH_EINVAL, "nh_colmax_argmax_f32: null pointer");
+    if (ld < cols) return nh_internal_fail(NH_EINVAL, "nh_colmax_argmax_f32: ld < cols");
+    if (rows > 0x7FFFFFFFu) return nh_internal_fail(NH_EINVAL, "nh_colmax_argmax_f32: too many rows for an int32 index");
+    const bool vec = (cols % 4 == 0) && (ld % 4 == 0) && aligned16(x);
+    const CrPlan p = cr_plan(rows, cols, vec);
+    if (p.strips > CR_MAX_STRIPS) return nh_internal_fail(NH_EINVAL, "nh_colmax_argmax_f32: too many columns");
+    if (p.chunks > 1 && !workspace) return nh_internal_fail(NH_EINVAL, "nh_colmax_argmax_f32: workspace required");
+    if (p.chunks > 65535u) return nh_internal_fail(NH_EINVAL, "nh_colmax_argmax_f32: grid too large");
+    float* pval = (float*)workspace;
+    int* pidx = (int*)(pval + (size_t)p.chunks * cols);
+    unsigned int* tickets = nullptr;
+    hipError_t e = hipGetSymbolAddress((void**)&tickets, HIP_SYMBOL(g_cr_tickets));
+    if (e != hipSuccess) return nh_internal_fail((int)e, "nh_colmax_argmax_f32: ticket symbol lookup failed");
+    hipStream_t s = (hipStream_t)stream;
+    dim3 grid(p.strips, p.chunks);
+    if (vec)
+        hipLaunchKernelGGL((colmax_kernel<4>), grid, dim3(CR_T), 0, s, x, rows, cols, ld, p.rows_per_chunk, pval,
+                           pidx, maxval, (int*)argmax, tickets);
+    else
+        hipLaunchKernelGGL((colmax_kernel<1>), grid, dim3(CR_T), 0, s, x, rows, cols, ld, p.rows_per_chunk, pval,
+                           pidx, maxval, (int*)argmax, tickets);
+    return launch_status("nh_colmax_argmax_f32");
+}
+
+}  // extern "C"

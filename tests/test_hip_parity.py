@@ -1,0 +1,325 @@
+"""Parity of the hip backend against the CPU oracle (runs on the GPU box).
+
+Every case evaluates the same function on both backends from identical seeded
+inputs.  Tolerances: integer / index outputs bit-exact; fp32 1e-5 relative;
+fp16 storage 1e-3 relative.
+"""
+import numpy as np
+import pytest
+
+from neon_amd import configs
+from utils import assert_close, call_func, gen_inputs, rel_err
+
+pytestmark = pytest.mark.gpu
+
+RTOL32 = 1e-5
+
+
+def both(pair, f, arrays, out_dtype=None, rtol=RTOL32, atol=1e-6, what=""):
+    cpu, hip = pair
+    want = call_func(f, cpu, arrays, out_dtype)
+    got = call_func(f, hip, arrays, out_dtype)
+    assert_close(got, want, rtol=rtol, atol=atol, what=what)
+    return got, want
+
+
+# ---- elementwise ------------------------------------------------------------------------
+UNARY = ["neg", "abs", "sgn", "sqr", "exp", "exp2", "sig", "sig2", "tanh", "tanh2", "rint"]
+UNARY_POS = ["sqrt", "log", "log2", "safelog"]
+
+
+@pytest.mark.parametrize("shape", [(64, 327), (4, 3), (1, 1023), (64, 1), (4096, 128)])
+def test_unary_ops(pair, shape):
+    rs = np.random.RandomState(1)
+    x = gen_inputs(rs, shape) * 3
+    xp = gen_inputs(rs, shape, "pos_rand") + 0.01
+    table = dict(neg="negative", abs="absolute", sgn="sgn", sqr="square", exp="exp", exp2="exp2",
+                 sig="sig", sig2="sig2", tanh="tanh", tanh2="tanh2", rint="rint", sqrt="sqrt",
+                 log="log", log2="log2", safelog="safelog")
+    for op in UNARY:
+        both(pair, lambda be, a, op=op: getattr(be, table[op])(a), [x], what=op)
+    for op in UNARY_POS:
+        both(pair, lambda be, a, op=op: getattr(be, table[op])(a), [xp], what=op)
+
+
+@pytest.mark.parametrize("shapes", [((64, 327), (64, 327)), ((64, 327), (64, 1)), ((64, 327), (1, 327)),
+                                    ((64, 1), (1, 327)), ((4, 3), (1, 1)), ((1, 1023), (1, 1023))])
+def test_binary_ops_and_broadcast(pair, shapes):
+    rs = np.random.RandomState(2)
+    a = gen_inputs(rs, shapes[0])
+    b = gen_inputs(rs, shapes[1]) + 1.5
+    fns = {
+        "add": lambda be, x, y: x + y, "sub": lambda be, x, y: x - y,
+        "mul": lambda be, x, y: x * y, "div": lambda be, x, y: x / y,
+        "gt": lambda be, x, y: x > y, "ge": lambda be, x, y: x >= y,
+        "lt": lambda be, x, y: x < y, "le": lambda be, x, y: x <= y,
+        "eq": lambda be, x, y: be.equal(x, y), "ne": lambda be, x, y: be.not_equal(x, y),
+        "max": lambda be, x, y: be.maximum(x, y), "min": lambda be, x, y: be.minimum(x, y),
+        "pow": lambda be, x, y: be.power(be.absolute(x) + 0.1, y),
+        "scalar": lambda be, x, y: 0.5 * x + 2.0 * y - 3 + x / 4.0,
+        "clip": lambda be, x, y: be.clip(x, -0.25, 0.5) * y,
+    }
+    for name, f in fns.items():
+        both(pair, f, [a, b], what=name)
+
+
+def test_inplace_and_views(pair):
+    rs = np.random.RandomState(3)
+    a = gen_inputs(rs, (50, 128))
+    b = gen_inputs(rs, (50, 128))
+    outs = []
+    for be in pair:
+        x, y = be.array(a), be.array(b)
+        x[:] = be.sig(x)                       # in place
+        x[2:7, :] = y[10:15, :] * 2.0          # row-slice views
+        x[:, 3:9] = x[:, 3:9] + y[:, 20:26]    # column-slice views, strided
+        x[0] = y[1] - 1.0                      # int index keeps the axis
+        x[:, 5] = 7.5                          # constant into a strided view
+        z = be.empty((128, 50))
+        z[:] = x.T + 1.0                       # transposed view as operand
+        w = x.reshape((100, 64))
+        w[:] = w * 0.5
+        outs.append((x.get(), z.get()))
+    assert_close(outs[1][0], outs[0][0], what="x")
+    assert_close(outs[1][1], outs[0][1], what="z")
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.int32, np.uint8, np.int8, np.int16, np.uint16, np.uint32])
+def test_storage_dtypes(pair, dtype):
+    rs = np.random.RandomState(4)
+    if np.dtype(dtype).kind == "f":
+        a = (rs.rand(33, 40) * 4 - 2).astype(dtype)
+    else:
+        a = rs.randint(0, 100, (33, 40)).astype(dtype)
+    b = (rs.rand(33, 40) * 3).astype(np.float32)
+    outs = []
+    for be in pair:
+        x = be.array(a, dtype=dtype)
+        y = be.array(b)
+        if np.dtype(dtype).kind == "f":
+            # fp16 storage, fp32 arithmetic: the oracle holds the same values in fp32
+            x32 = be.array(a.astype(np.float32)) if be.backend_name == "cpu" else x
+            o = be.empty((33, 40), dtype=dtype)
+            o[:] = x32 * y + 0.25
+        else:
+            o = be.empty((33, 40), dtype=dtype)
+            o[:] = x + y                       # float -> int store truncates
+        outs.append(o.get())
+    if np.dtype(dtype).kind == "f":
+        assert rel_err(outs[1], outs[0]) <= 1e-3
+    else:
+        assert np.array_equal(outs[1], outs[0])
+
+
+# ---- reductions ---------------------------------------------------------------------------
+RED_SHAPES = [(2, 2), (10, 32), (50, 50), (50, 128), (1000, 128), (257, 1000), (3, 5000), (5000, 3)]
+
+
+@pytest.mark.parametrize("shape", RED_SHAPES)
+@pytest.mark.parametrize("axis", [0, 1])
+def test_reductions(pair, shape, axis):
+    rs = np.random.RandomState(5)
+    a = gen_inputs(rs, shape)
+    for name in ("sum", "max", "min", "mean", "var", "std"):
+        both(pair, lambda be, x, n=name: getattr(be, n)(x, axis=axis), [a], rtol=2e-5, atol=2e-6,
+             what="%s axis%d" % (name, axis))
+    for name in ("argmax", "argmin"):
+        got, want = both(pair, lambda be, x, n=name: getattr(be, n)(x, axis=axis), [a],
+                         out_dtype=np.int32, what=name)
+
+
+@pytest.mark.parametrize("axis", [0, 1])
+def test_argmax_ties_take_first(pair, axis):
+    a = np.zeros((37, 41), dtype=np.float32)
+    a[5, :] = 1
+    a[9, :] = 1
+    a[:, 7] = 1
+    a[:, 30] = 1
+    both(pair, lambda be, x: be.argmax(x, axis=axis), [a], out_dtype=np.int32)
+    both(pair, lambda be, x: be.argmin(-x, axis=axis), [a], out_dtype=np.int32)
+
+
+@pytest.mark.parametrize("shape", [(10, 32), (50, 128), (300, 70)])
+def test_reduction_into_slices(pair, shape):
+    """reductions written through row / column views (reference
+    tests/test_backend_reduction.py:39-43, 59-63)"""
+    rs = np.random.RandomState(6)
+    a = gen_inputs(rs, shape)
+    outs = []
+    for be in pair:
+        x = be.array(a)
+        r = be.zeros((4, shape[1]))
+        c = be.zeros((shape[0], 4))
+        r[1] = be.sum(x, axis=0)
+        r[2, :] = be.max(x, axis=0) + be.min(x, axis=0)
+        c[:, 1] = be.mean(x, axis=1)
+        c[:, 3] = be.std(x, axis=1)
+        outs.append((r.get(), c.get()))
+    assert_close(outs[1][0], outs[0][0], rtol=2e-5, what="rows")
+    assert_close(outs[1][1], outs[0][1], rtol=2e-5, what="cols")
+
+
+def test_compound_and_mixed_axes(pair):
+    """whole-tensor reductions and nested mixed-axis trees need several kernels"""
+    rs = np.random.RandomState(7)
+    a = gen_inputs(rs, (50, 128))
+    b = gen_inputs(rs, (50, 128))
+    both(pair, lambda be, x, y: be.sum(x), [a, b], rtol=2e-5)
+    both(pair, lambda be, x, y: be.mean(x * y), [a, b], rtol=2e-5, atol=1e-6)
+    both(pair, lambda be, x, y: be.std(be.var(x, axis=0), axis=1), [a, b], rtol=5e-5)
+    both(pair, lambda be, x, y: be.max(x) + be.min(y), [a, b])
+    both(pair, lambda be, x, y: x - be.mean(x) + be.sum(y, axis=1), [a, b], rtol=2e-5, atol=2e-6)
+    both(pair, lambda be, x, y: (x * y).T + 1.0, [a, b])
+
+
+def test_onehot(pair):
+    rs = np.random.RandomState(8)
+    idx = rs.randint(0, 40, (1, 64)).astype(np.int32)
+    y = (rs.rand(40, 64) + 0.1).astype(np.float32)
+    outs = []
+    for be in pair:
+        i = be.array(idx, dtype=np.int32)
+        t = be.empty((40, 64))
+        t[:] = be.onehot(i, axis=0)              # top-level form
+        p = be.array(y)
+        ce = be.empty((1, 64))
+        ce[:] = be.sum(-be.onehot(i, axis=0) * be.safelog(p), axis=0)   # in-tree form
+        outs.append((t.get(), ce.get()))
+    assert np.array_equal(outs[1][0], outs[0][0])
+    assert_close(outs[1][1], outs[0][1])
+
+
+# ---- the five benchmark configurations -------------------------------------------------------
+def test_config1(pair):
+    x, y = configs.inputs_c1()
+    res = []
+    for be in pair:
+        tx, ty, out = be.array(x), be.array(y), be.empty(configs.C1_SHAPE)
+        configs.c1a(be, out, tx, ty)
+        a = out.get()
+        configs.c1b(be, out)
+        res.append((a, out.get()))
+    assert_close(res[1][0], res[0][0], rtol=RTOL32)
+    assert_close(res[1][1], res[0][1], rtol=RTOL32)
+
+
+def test_config2_softmax(pair):
+    (x,) = configs.inputs_c2()
+    res = []
+    for be in pair:
+        tx, out = be.array(x), be.empty(configs.C2_SHAPE)
+        configs.c2_softmax(be, out, tx)
+        a = out.get()
+        configs.c2_softmax_neon(be, out, tx)
+        res.append((a, out.get()))
+    assert_close(res[1][0], res[0][0], rtol=RTOL32, atol=1e-12)
+    assert_close(res[1][1], res[0][1], rtol=RTOL32, atol=1e-12)
+    assert np.allclose(res[1][0].sum(axis=0), 1.0, atol=1e-5)
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_config3_adam(pair, fused):
+    shape = (1000, 1250)       # the oracle needs seconds at this size; the full size is in test_full_size
+    grad, param = configs.inputs_c3(shape)
+    from neon_amd.backends.backend import Block
+    res = []
+    for be in pair:
+        bsz, be.bsz = be.bsz, 1
+        g, p = be.array(grad), be.array(param)
+        m, v = be.zeros(shape), be.zeros(shape)
+        snap = None
+        for t in range(1, 11):
+            if fused:
+                be.begin(Block.update, t)
+            configs.c3_adam_step(be, p, g, m, v, t)
+            if fused:
+                be.end(Block.update, t)
+            if t == 1:
+                snap = (p.get(), m.get(), v.get())
+        res.append((snap, (p.get(), m.get(), v.get())))
+        be.bsz = bsz
+    for step in (0, 1):
+        for k, name in enumerate(("param", "m", "v")):
+            assert_close(res[1][step][k], res[0][step][k], rtol=RTOL32, atol=1e-12, what="%s step %d" % (name, step))
+
+
+def test_config4_rownorm_fp16(pair):
+    shape = (32, 100352)
+    x, gamma, beta = configs.inputs_c4(shape)
+    cpu, hip = pair
+    # oracle: fp16-quantised inputs held in fp32, fp32 arithmetic, fp16 store
+    o_cpu = cpu.empty(shape, dtype=np.float16)
+    configs.c4_rownorm(cpu, o_cpu, cpu.array(x.astype(np.float32)), cpu.array(gamma), cpu.array(beta))
+    o_hip = hip.empty(shape, dtype=np.float16)
+    configs.c4_rownorm(hip, o_hip, hip.array(x, dtype=np.float16), hip.array(gamma), hip.array(beta))
+    want, got = o_cpu.get().astype(np.float64), o_hip.get().astype(np.float64)
+    # relative error against max(|want|, 1e-3 * max|want|): values near the row
+    # mean are tiny and one fp16 ulp of the store would dominate otherwise
+    assert rel_err(got, want, floor_frac=1e-3) <= 1e-3
+
+
+def test_config5_argmax_max_ce(pair):
+    shape = (4000, 256)
+    x, idx = configs.inputs_c5(shape)
+    cpu, hip = pair
+    res = []
+    for be in pair:
+        tx = be.array(x)
+        ti = be.array(idx, dtype=np.int32)
+        am = be.empty((1, shape[1]), dtype=np.int32)
+        mx = be.empty((1, shape[1]))
+        ce = be.empty((1, shape[1]))
+        configs.c5a_argmax(be, am, tx)
+        configs.c5b_max(be, mx, tx)
+        if be is cpu:
+            t = be.empty(shape)
+            t[:] = be.onehot(ti, axis=0)
+            configs.c5c_cross_entropy(be, ce, tx, t)
+        else:
+            configs.c5c_cross_entropy(be, ce, tx, be.onehot(ti, axis=0))
+        res.append((am.get(), mx.get(), ce.get()))
+    assert np.array_equal(res[1][0], res[0][0])
+    assert np.array_equal(res[1][1], res[0][1])
+    assert_close(res[1][2], res[0][2], rtol=RTOL32)
+    assert np.array_equal(res[1][0].ravel(), np.argmax(x, axis=0))
+
+
+def test_full_size_properties(hip):
+    """size-independent checks at the benchmark shapes"""
+    be = hip
+    x, idx = configs.inputs_c5()
+    tx = be.array(x)
+    am = be.empty((1, configs.C5_SHAPE[1]), dtype=np.int32)
+    mx = be.empty((1, configs.C5_SHAPE[1]))
+    configs.c5a_argmax(be, am, tx)
+    configs.c5b_max(be, mx, tx)
+    assert np.array_equal(am.get().ravel(), np.argmax(x, axis=0))
+    assert np.array_equal(mx.get().ravel(), np.max(x, axis=0))
+    ce = be.empty((1, configs.C5_SHAPE[1]))
+    configs.c5c_cross_entropy(be, ce, tx, be.onehot(be.array(idx, dtype=np.int32), axis=0))
+    x64 = x.astype(np.float64)
+    lse = np.log(np.exp(x64 - x64.max(0)).sum(0)) + x64.max(0)
+    want = lse - x64[idx.ravel(), np.arange(x.shape[1])]
+    assert_close(ce.get().ravel(), want, rtol=2e-5)
+
+    x4, gamma, beta = configs.inputs_c4()
+    o = be.empty(configs.C4_SHAPE, dtype=np.float16)
+    configs.c4_rownorm(be, o, be.array(x4, dtype=np.float16), be.array(gamma), be.array(beta))
+    got = o.get().astype(np.float64)
+    assert np.allclose(got.mean(axis=1), beta.ravel(), atol=2e-3)
+    assert np.allclose(got.std(axis=1), gamma.ravel(), rtol=2e-3)
+
+    grad, param = configs.inputs_c3()
+    from neon_amd.backends.backend import Block
+    bsz, be.bsz = be.bsz, 1
+    g, p, m, v = be.array(grad), be.array(param), be.zeros(configs.C3_SHAPE), be.zeros(configs.C3_SHAPE)
+    be.begin(Block.update, 1)
+    configs.c3_adam_step(be, p, g, m, v, 1)
+    be.end(Block.update, 1)
+    be.bsz = bsz
+    # after one step from m = v = 0: m = 0.1 g, v = 0.001 g^2, |delta p| ~= lr
+    assert_close(m.get(), np.float32(1. - 0.9) * grad, rtol=1e-6, atol=0)
+    d = param - p.get()
+    nz = np.abs(grad) > 1e-4
+    assert np.allclose(np.abs(d[nz]), 1e-3, rtol=2e-3)
+    assert np.array_equal(np.sign(d[nz]), np.sign(grad[nz]))
