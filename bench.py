@@ -1,0 +1,267 @@
+#!/usr/bin/env python
+"""Benchmark of the fused op-tree path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Headline (``value``): the fused Adam update of 25,000,000 fp32 parameters
+(5000 x 5000) -- the three assigns of neon's Adam.optimize run as ONE kernel --
+as whole-job GB/s over K steps: algorithmic bytes (4 tensors read + 3 written =
+700 MB per step) divided by wall-clock time around the K ``be.begin / assigns /
+be.end`` calls, inputs resident in HBM, stream synchronised on both sides.
+
+``roofline`` is that kernel alone, timed with HIP events on the launch stream
+around the same K launches.  ``per_config`` lists every benchmark op-tree
+(elementwise + sigmoid, softmax, Adam fused and as three kernels, fp16 row
+normalisation, argmax / max / cross-entropy over a 32000-row vocabulary) with
+the same event timing, and a scaled-up (>= 256 MB) instance of the trees whose
+working set fits in cache.  ``cpu_baseline`` times the numpy oracle on the same
+Adam step on this machine's host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def _fresh(be, shape, dtype=np.float32, fill=None, rs=None, scale=1.0, shift=0.0):
+    t = be.empty(shape, dtype=dtype)
+    if rs is not None:
+        # generate on the host in row blocks to bound host memory
+        rows = shape[0]
+        step = max(1, (1 << 24) // max(1, shape[1]))
+        for r0 in range(0, rows, step):
+            r1 = min(rows, r0 + step)
+            blk = (rs.standard_normal((r1 - r0, shape[1])) * scale + shift).astype(np.float32).astype(dtype)
+            t[r0:r1, :].set(blk) if (r0, r1) != (0, rows) else t.set(blk)
+    elif fill is not None:
+        t[:] = fill
+    return t
+
+
+def gpu_leg(steps, warmup, detail=True):
+    from neon_amd import configs
+    from neon_amd.backends import gen_backend
+    from neon_amd.backends.backend import Block
+
+    be = gen_backend("hip", rng_seed=0)
+    be.bsz = 1
+    rt = be.rt
+    out = {"device": rt.props.name.decode(), "arch": rt.arch, "compute_units": be.cu_count}
+
+    # ---- headline: fused Adam, full size, through the public API -----------------------
+    grad_h, param_h = configs.inputs_c3()
+    g, p = be.array(grad_h), be.array(param_h)
+    m, v = be.zeros(configs.C3_SHAPE), be.zeros(configs.C3_SHAPE)
+    del grad_h, param_h
+
+    def adam_step(t):
+        be.begin(Block.update, t)
+        configs.c3_adam_step(be, p, g, m, v, t)
+        be.end(Block.update, t)
+
+    t = 0
+    for _ in range(warmup):
+        t += 1
+        adam_step(t)
+    be.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        t += 1
+        adam_step(t)
+    be.synchronize()
+    wall = time.perf_counter() - t0
+    step_bytes = configs.bytes_c3(fused=True)
+    out["ms_per_step"] = wall * 1e3 / steps
+    out["value_gbs"] = step_bytes * steps / wall / 1e9
+    out["elements_per_s"] = configs.C3_SHAPE[0] * configs.C3_SHAPE[1] * steps / wall
+
+    # the same kernel alone, HIP events around `steps` launches
+    with be.capture() as groups:
+        adam_step(t + 1)
+    assert len(groups) == 1 and len(groups[0]) == 3, "Adam did not fuse into one kernel"
+    ms, plan = be.time_group(groups[0], reps=max(steps, 5))
+    out["roofline"] = {"bound": "hbm", "achieved": step_bytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
+                       "unit": "GB/s", "frac": step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                       "traffic": None, "kernel": plan.spec.name, "kernel_ms": ms,
+                       "algorithmic_bytes": step_bytes}
+    if not detail:
+        return out, be
+
+    # ---- every configuration, kernel by kernel -------------------------------------------
+    rows = []
+
+    def api_ms(issue, reps):
+        """wall-clock per call through the public API (host work included)"""
+        issue()
+        be.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            issue()
+        be.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / reps
+
+    def measure(label, issue, nbytes, elements, reps=50):
+        from neon_amd.backends.hip.planner import NeedsSplit
+        from neon_amd.backends.hip.optree_ir import MixedAxes
+        with be.capture() as grp:
+            issue()
+        row = {"config": label, "bytes": nbytes}
+        try:
+            total, names = 0.0, []
+            for trees in grp:
+                ms_k, pl = be.time_group(trees, reps=reps)
+                total += ms_k
+                names.append("%s[%s]" % (pl.spec.family, ",".join(
+                    "%s=%s" % kv for kv in sorted(pl.spec.params.items())
+                    if kv[0] in ("V", "LX", "LY", "NCH", "NR"))))
+            row.update({"kernels": len(grp), "ms": total, "timing": "HIP events around back-to-back launches",
+                        "plan": " + ".join(names)})
+        except (NeedsSplit, MixedAxes):
+            before = be.plan_stats["launches"]
+            issue()
+            row["kernels"] = be.plan_stats["launches"] - before
+            row["ms"] = api_ms(issue, reps)
+            row["timing"] = "wall clock per API call (several kernels through temporaries)"
+        row["api_ms"] = api_ms(issue, reps)
+        row["gbs"] = nbytes / (row["ms"] * 1e-3) / 1e9
+        row["frac_of_hbm_peak"] = row["gbs"] / HBM_PEAK_GBS
+        row["elements_per_s"] = elements / (row["ms"] * 1e-3)
+        rows.append(row)
+
+    rs = np.random.RandomState(11)
+    # C1
+    x1, y1 = (be.array(a) for a in configs.inputs_c1())
+    o1 = be.empty(configs.C1_SHAPE)
+    n1 = configs.C1_SHAPE[0] * configs.C1_SHAPE[1]
+    measure("C1a 0.5x+2y (4096,128) f32 [cache-hot]", lambda: configs.c1a(be, o1, x1, y1), configs.bytes_c1a(), n1)
+    measure("C1b sig in place (4096,128) f32 [cache-hot]", lambda: configs.c1b(be, o1), configs.bytes_c1b(), n1)
+    measure("C1 fused sig(0.5x+2y) (4096,128) f32 [cache-hot]", lambda: configs.c1_fused(be, o1, x1, y1),
+            configs.bytes_c1a(), n1)
+    big = (16384, 4096)   # 256 MiB per tensor
+    xb, yb, ob = _fresh(be, big, rs=rs), _fresh(be, big, rs=rs), be.empty(big)
+    nb = big[0] * big[1]
+    measure("C1a scaled (16384,4096) f32", lambda: configs.c1a(be, ob, xb, yb), configs.bytes_c1a(big), nb, reps=10)
+    measure("C1b scaled (16384,4096) f32", lambda: configs.c1b(be, ob), configs.bytes_c1b(big), nb, reps=10)
+    # C2
+    (x2h,) = configs.inputs_c2()
+    x2, o2 = be.array(x2h), be.empty(configs.C2_SHAPE)
+    measure("C2 softmax axis0 (1000,128) f32 [cache-hot]", lambda: configs.c2_softmax(be, o2, x2),
+            configs.bytes_c2(), x2h.size)
+    wide = (1000, 65536)  # same depth, 512x the columns: 262 MB per tensor
+    del yb
+    xw = be.empty(wide)
+    xw[:] = 0.001
+    ow = ob.share(wide)
+    measure("C2 softmax axis0 scaled (1000,65536) f32", lambda: configs.c2_softmax(be, ow, xw),
+            configs.bytes_c2(wide), wide[0] * wide[1], reps=10)
+    del xw, ow, xb, ob
+    # C3
+    n3 = configs.C3_SHAPE[0] * configs.C3_SHAPE[1]
+    measure("C3 Adam fused, 1 kernel (5000,5000) f32", lambda: adam_step(t + 2), configs.bytes_c3(fused=True), n3,
+            reps=20)
+    measure("C3 Adam as 3 assigns, 3 kernels (5000,5000) f32",
+            lambda: configs.c3_adam_step(be, p, g, m, v, t + 2), configs.bytes_c3(fused=False), n3, reps=20)
+    # C4
+    x4h, gh, bh = configs.inputs_c4()
+    x4, o4 = be.array(x4h, dtype=np.float16), be.empty(configs.C4_SHAPE, dtype=np.float16)
+    g4, b4 = be.array(gh), be.array(bh)
+    measure("C4 rownorm (256,100352) f16", lambda: configs.c4_rownorm(be, o4, x4, g4, b4), configs.bytes_c4(),
+            x4h.size, reps=30)
+    del x4h
+    # C5
+    x5h, i5h = configs.inputs_c5()
+    x5 = be.array(x5h)
+    i5 = be.array(i5h, dtype=np.int32)
+    am = be.empty((1, configs.C5_SHAPE[1]), dtype=np.int32)
+    mx, ce = be.empty((1, configs.C5_SHAPE[1])), be.empty((1, configs.C5_SHAPE[1]))
+    n5 = x5h.size
+    del x5h
+    measure("C5a argmax axis0 (32000,256) f32", lambda: configs.c5a_argmax(be, am, x5), configs.bytes_c5_reduce(), n5)
+    measure("C5b max axis0 (32000,256) f32", lambda: configs.c5b_max(be, mx, x5), configs.bytes_c5_reduce(), n5)
+    measure("C5c cross-entropy axis0 (32000,256) f32, in-kernel one-hot",
+            lambda: configs.c5c_cross_entropy(be, ce, x5, be.onehot(i5, axis=0)), configs.bytes_c5c(), n5)
+    out["per_config"] = rows
+    return out, be
+
+
+def cpu_leg(max_seconds=25.0):
+    """numpy oracle on the headline workload: full-size Adam steps, 1 core"""
+    from neon_amd import configs
+    from neon_amd.backends.backend import Backend
+    from oracle import nervanacpu  # noqa: F401  (cpu_baseline leg only)
+    cpu = Backend.allocate_backend("cpu", rng_seed=0)
+    cpu.bsz = 1
+    grad_h, param_h = configs.inputs_c3()
+    g, p = cpu.array(grad_h), cpu.array(param_h)
+    m, v = cpu.zeros(configs.C3_SHAPE), cpu.zeros(configs.C3_SHAPE)
+    times = []
+    t = 0
+    t_begin = time.perf_counter()
+    while True:
+        t += 1
+        t0 = time.perf_counter()
+        configs.c3_adam_step(cpu, p, g, m, v, t)
+        times.append(time.perf_counter() - t0)
+        if len(times) >= 7 or (time.perf_counter() - t_begin) > max_seconds:
+            break
+    timed = times[1:] if len(times) > 2 else times      # first step pays page faults
+    med = float(np.median(timed))
+    try:
+        with open("/proc/cpuinfo") as f:
+            model = [l.split(":", 1)[1].strip() for l in f if l.startswith("model name")][0]
+    except Exception:
+        model = "unknown"
+    return {"value": configs.bytes_c3(fused=True) / med / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "%d full-size Adam steps (5000x5000 fp32) on the numpy oracle, median step %.3f s; "
+                      "numpy ufuncs are single-threaded" % (len(timed), med),
+            "elements_per_s": configs.C3_SHAPE[0] * configs.C3_SHAPE[1] / med,
+            "host_cpu": model, "host_cpu_count": os.cpu_count()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle leg")
+    ap.add_argument("--no-detail", action="store_true", help="headline only, no per-config table")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one MI355X; --gpus %d is not supported (the op-tree path has no "
+              "cross-device stage; see DESIGN.md on sharding)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    gpu, be = gpu_leg(args.steps, args.warmup, detail=not args.no_detail)
+    cpu = None if args.no_cpu else cpu_leg()
+    line = {
+        "metric": "fused op-tree HBM GB/s (% of MI355X peak) + elements/s vs CPU backend",
+        "value": gpu["value_gbs"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": gpu["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "C3: fused Adam update op-tree, 25,000,000 fp32 params (5000x5000), "
+                               "4 tensors read + 3 written per step, lr=1e-3 b1=0.9 b2=0.999 eps=1e-8",
+                   "algorithmic_bytes_per_step": 700000000, "parallelism": "single GPU"},
+        "frac_of_hbm_peak": gpu["value_gbs"] / HBM_PEAK_GBS,
+        "elements_per_s": gpu["elements_per_s"],
+        "roofline": gpu["roofline"],
+        "cpu_baseline": cpu,
+        "device": gpu["device"], "arch": gpu["arch"],
+    }
+    if cpu:
+        line["gpu_over_cpu"] = gpu["value_gbs"] / cpu["value"]
+    if "per_config" in gpu:
+        line["per_config"] = gpu["per_config"]
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -111,6 +111,15 @@ int nh_module_get_function(void* module, const char* name, void** function);
 int nh_launch(void* function, const uint32_t grid[3], const uint32_t block[3],
               uint32_t lds_bytes, void* stream, const void* args, size_t arg_bytes);
 
+/* Launch the same kernel `reps` times back to back between two events on
+ * `stream`, wait, and return the mean time per launch in milliseconds.
+ * replaces: the event bracket of the reference's bench mode
+ *           (float_ew.py:917-938: start.record / kernel / end.record /
+ *           end.time_since(start)).                                            */
+int nh_launch_timed(void* function, const uint32_t grid[3], const uint32_t block[3],
+                    uint32_t lds_bytes, void* stream, const void* args, size_t arg_bytes,
+                    uint32_t reps, float* mean_ms);
+
 /* ---- prebuilt hand-written gfx950 kernels ------------------------------------
  * Direct entry points for fixed, hot op-trees; the same trees also run through
  * the generated-code path.  All pointers are device pointers; tensors are

@@ -88,12 +88,16 @@ class _Lines(object):
 class _Gen(object):
     """State shared by the family emitters for one program."""
 
-    def __init__(self, prog, V):
+    def __init__(self, prog, V, stream=False):
         self.prog = prog
         self.V = V
         self.R, self.C = prog.domain
         self.axis = prog.axis
         self.L = _Lines()
+        # streaming kernels (working set far beyond the caches) mark their
+        # global accesses non-temporal
+        self.ld = "load_stream" if stream else "load"
+        self.st = "store_stream" if stream else "store"
 
     # -- parameters -----------------------------------------------------------------
     def slot_ctype(self, slot):
@@ -164,7 +168,7 @@ class _Gen(object):
         name = target or self.tile_name(n, sfx)
         if declare:
             self.L("%s %s;" % (self.tile_type(n, V), name))
-        self.L("%s.load(%s);" % (name, self.tile_addr(n, r, c)))
+        self.L("%s.%s(%s);" % (name, self.ld, self.tile_addr(n, r, c)))
 
     # -- expressions -----------------------------------------------------------------
     def leaf_value(self, n, tile, r, c, V):
@@ -221,13 +225,13 @@ def _finish(family, g, head, fmt, block, lds, params):
 # =====================================================================================
 # family: ew
 # =====================================================================================
-def gen_ew(prog, V, LX, LY, UC, UR, tail):
+def gen_ew(prog, V, LX, LY, UC, UR, tail, stream=False):
     """Elementwise kernel.  Workgroup = LX column-lanes x LY row-lanes; a lane
     handles UC column tiles x UR rows per step, all loads issued before the
     first store.  ``tail``: emit a scalar path for a last partial tile
     (only needed when C % V != 0, which the planner allows for single-row
     domains)."""
-    g = _Gen(prog, V)
+    g = _Gen(prog, V, stream)
     L = g.L
     T = LX * LY
     params, fmt = g.param_list([("int row_tiles", "i")])
@@ -269,7 +273,7 @@ def gen_ew(prog, V, LX, LY, UC, UR, tail):
                 L("o%d%s.set(%s, %s);" % (st.out.index, sfx, jj, val))
         L.close()
         for st in prog.statements:
-            L("o%d%s.store(%s);" % (st.out.index, sfx, g.addr(st.out, r, c)))
+            L("o%d%s.%s(%s);" % (st.out.index, sfx, g.st, g.addr(st.out, r, c)))
 
     L.open("")
     L("const int tx = threadIdx.x %% %d, ty = threadIdx.x / %d;" % (LX, LX))
@@ -303,7 +307,7 @@ def gen_ew(prog, V, LX, LY, UC, UR, tail):
     L.close()
     L.close()
     return _finish("ew", g, head, fmt, T, 0,
-                   dict(V=V, LX=LX, LY=LY, UC=UC, UR=UR, tail=bool(tail)))
+                   dict(V=V, LX=LX, LY=LY, UC=UC, UR=UR, tail=bool(tail), stream=bool(stream)))
 
 
 # =====================================================================================
@@ -327,8 +331,8 @@ def _live_reductions(prog):
 class _RedGen(_Gen):
     """Common machinery of row / col / colsplit."""
 
-    def __init__(self, prog, V):
-        super(_RedGen, self).__init__(prog, V)
+    def __init__(self, prog, V, stream=False):
+        super(_RedGen, self).__init__(prog, V, stream)
         self.col_axis = (prog.axis == 0)   # reductions leave one value per column
 
     # value of a finished reduction at element j of the lane's tile
@@ -375,13 +379,13 @@ class _RedGen(_Gen):
 # =====================================================================================
 # family: row  (axis 1)
 # =====================================================================================
-def gen_row(prog, V, LX, LY, NCH):
+def gen_row(prog, V, LX, LY, NCH, stream=False):
     """Axis-1 reductions.  A team of LX lanes (a power of two up to 64, or the
     whole workgroup) owns one row; the workgroup holds LY rows.  A lane visits
     column tiles tx, tx+LX, ...; with ``NCH`` > 0 that loop has a fixed trip
     count and the tiles loaded in the first sweep stay in registers for the
     later ones; with ``NCH`` == 0 every sweep streams the row again."""
-    g = _RedGen(prog, V)
+    g = _RedGen(prog, V, stream)
     L = g.L
     T = LX * LY
     assert LX <= 64 or LY == 1
@@ -435,12 +439,12 @@ def gen_row(prog, V, LX, LY, NCH):
                 name = "keep%d" % n.nid
                 cached[n.nid] = name
                 tiles[n.nid] = "%s[k]" % name
-                L("if (ok) %s[k].load(%s); else %s[k].zero();" % (name, g.tile_addr(n, "rr", "c"), name))
+                L("if (ok) %s[k].%s(%s); else %s[k].zero();" % (name, g.ld, g.tile_addr(n, "rr", "c"), name))
             else:
                 name = g.tile_name(n, "_s")
                 tiles[n.nid] = name
                 L("%s %s; %s.zero();" % (g.tile_type(n, V), name, name))
-                L("if (ok) %s.load(%s);" % (name, g.tile_addr(n, "rr", "c")))
+                L("if (ok) %s.%s(%s);" % (name, g.ld, g.tile_addr(n, "rr", "c")))
         return tiles
 
     def declare_tiles(leaves):
@@ -546,11 +550,11 @@ def gen_row(prog, V, LX, LY, NCH):
                 L("o%d.set(j, %s);" % (st.out.index, ref(st.root)))
         L.close()
         for st in full_out:
-            L("o%d.store(%s);" % (st.out.index, g.addr(st.out, "r", "c")))
+            L("o%d.%s(%s);" % (st.out.index, g.st, g.addr(st.out, "r", "c")))
         L.close()
         L.close()
     L.close()
-    return _finish("row", g, head, fmt, T, 0, dict(V=V, LX=LX, LY=LY, NCH=NCH))
+    return _finish("row", g, head, fmt, T, 0, dict(V=V, LX=LX, LY=LY, NCH=NCH, stream=bool(stream)))
 
 
 # =====================================================================================
@@ -599,6 +603,7 @@ def _emit_col_fold(g, L, n, LX, LY, T, V, src, dst_decl=True):
     L("#pragma unroll")
     L.open("for (int j = 0; j < %d; ++j)" % V)
     L("%s f = %s[0][tx * %d + j];" % (ty_, buf, V))
+    L("#pragma unroll")
     L("for (int y = 1; y < %d; ++y) f = %s::f(f, %s[y][tx * %d + j]);" % (WY, op, buf, V))
     if n.is_index:
         L("ri%d[j] = f.i; %s[j] = f;" % (n.nid, src))
@@ -616,10 +621,10 @@ def _col_lds(L, LX, LY, T, V, any_index):
     return WY * (LX * V + 1) * (4 + (8 if any_index else 0))
 
 
-def gen_col(prog, V, LX, LY, NR):
+def gen_col(prog, V, LX, LY, NR, stream=False):
     """Axis-0 reductions with all rows of a column strip inside one workgroup
     (LX column-lanes x LY row-lanes, NR rows per lane, kept in registers)."""
-    g = _RedGen(prog, V)
+    g = _RedGen(prog, V, stream)
     L = g.L
     T = LX * LY
     params, fmt = g.param_list([])
@@ -664,7 +669,7 @@ def gen_col(prog, V, LX, LY, NR):
                 continue
             if n.nid not in cached:
                 cached[n.nid] = "keep%d" % n.nid
-                L("if (ok) keep%d[i].load(%s); else keep%d[i].zero();" % (n.nid, g.tile_addr(n, "r", "cc"), n.nid))
+                L("if (ok) keep%d[i].%s(%s); else keep%d[i].zero();" % (n.nid, g.ld, g.tile_addr(n, "r", "cc"), n.nid))
             tiles[n.nid] = "keep%d[i]" % n.nid
         return tiles
 
@@ -756,14 +761,17 @@ def gen_col(prog, V, LX, LY, NR):
                 L("o%d.set(j, %s);" % (st.out.index, ref(st.root)))
         L.close()
         for st in full_out:
-            L("o%d.store(%s);" % (st.out.index, g.addr(st.out, "r", "c")))
+            L("o%d.%s(%s);" % (st.out.index, g.st, g.addr(st.out, "r", "c")))
         L.close()
         L.close()
     L.close()
-    return _finish("col", g, head, fmt, T, lds, dict(V=V, LX=LX, LY=LY, NR=NR))
+    return _finish("col", g, head, fmt, T, lds, dict(V=V, LX=LX, LY=LY, NR=NR, stream=bool(stream)))
 
 
-def gen_colsplit(prog, V, LX, LY):
+COLSPLIT_MAX_CHUNKS = 128
+
+
+def gen_colsplit(prog, V, LX, LY, stream=False):
     """One level of axis-0 reductions over a tall matrix.  grid = (column
     strips, row chunks).  Each workgroup reduces its chunk, leaves one partial
     per column in the workspace and takes a ticket; the workgroup that draws
@@ -774,7 +782,7 @@ def gen_colsplit(prog, V, LX, LY):
     Extra parameters: ``rows_per_chunk``, workspace pointer (partials first,
     tickets after ``ticket_offset`` bytes)."""
     assert prog.nlevels == 1
-    g = _RedGen(prog, V)
+    g = _RedGen(prog, V, stream)
     L = g.L
     T = LX * LY
     params, fmt = g.param_list([("int rows_per_chunk", "i"), ("char* ws", "P"),
@@ -849,10 +857,14 @@ def gen_colsplit(prog, V, LX, LY):
                                                      ("acc%d[j].v" % n.nid) if n.is_index else ("rv%d[j]" % n.nid),
                                                      n.nid,
                                                      ("acc%d[j].i" % n.nid) if n.is_index else "0"))
-        L("part%d[(long long)blockIdx.y * C + c + j] = p%d;" % (n.nid, n.nid))
+        L("nh_part_store(&part%d[(long long)blockIdx.y * C + c + j], p%d);" % (n.nid, n.nid))
     L.close()
     L.close()
-    L("__threadfence();")
+    # The partials were written through to device-coherent memory
+    # (nh_part_store); the barrier makes every lane wait for its own stores
+    # before lane 0 takes the ticket, and the last workgroup reads them past
+    # its L2 (nh_part_load).  No device-wide fence is needed, which matters:
+    # a release fence writes back the whole L2 and costs more than the sweep.
     L("__syncthreads();")
     L.open("if (threadIdx.x == 0)")
     L("const unsigned int t = atomicAdd(&tickets[blockIdx.x], 1u);")
@@ -860,26 +872,35 @@ def gen_colsplit(prog, V, LX, LY):
     L.close()
     L("__syncthreads();")
     L("if (!s_last) return;")
-    L("__threadfence();")
+    QMAX = -(-COLSPLIT_MAX_CHUNKS // LY)
     for n in reds:
-        op = _RED_OP[n.op]
-        L("#pragma unroll")
-        if n.is_index:
-            L("for (int j = 0; j < %d; ++j) acc%d[j] = %s::init();" % (V, n.nid, op))
-        else:
-            L("for (int j = 0; j < %d; ++j) acc%d[j] = %s::init();" % (V, n.nid, op))
-    L.open("if (col_ok)")
-    L.open("for (int q = ty; q < nchunks; q += %d)" % LY)
+        L("nh_pair q%d[%d][%d];" % (n.nid, QMAX, V))
+    L("#pragma unroll")
+    L.open("for (int k = 0; k < %d; ++k)" % QMAX)
+    L("const int q = ty + k * %d;" % LY)
+    L("const bool live = col_ok && (q < nchunks);")
     L("#pragma unroll")
     L.open("for (int j = 0; j < %d; ++j)" % V)
     for n in reds:
         op = _RED_OP[n.op]
-        L("const nh_pair p%d = part%d[(long long)q * C + c + j];" % (n.nid, n.nid))
-        if n.is_index:
-            L("acc%d[j] = %s::f(acc%d[j], p%d);" % (n.nid, op, n.nid, n.nid))
-        else:
-            L("acc%d[j] = %s::f(acc%d[j], p%d.v);" % (n.nid, op, n.nid, n.nid))
+        init = ("%s::init()" % op) if n.is_index else ("nh_pair{%s::init(), 0}" % op)
+        L("q%d[k][j] = live ? nh_part_load(&part%d[(long long)q * C + c + j]) : %s;" % (n.nid, n.nid, init))
     L.close()
+    L.close()
+    for n in reds:
+        op = _RED_OP[n.op]
+        L("#pragma unroll")
+        L("for (int j = 0; j < %d; ++j) acc%d[j] = %s::init();" % (V, n.nid, op))
+    L("#pragma unroll")
+    L.open("for (int k = 0; k < %d; ++k)" % QMAX)
+    L("#pragma unroll")
+    L.open("for (int j = 0; j < %d; ++j)" % V)
+    for n in reds:
+        op = _RED_OP[n.op]
+        if n.is_index:
+            L("acc%d[j] = %s::f(acc%d[j], q%d[k][j]);" % (n.nid, op, n.nid, n.nid))
+        else:
+            L("acc%d[j] = %s::f(acc%d[j], q%d[k][j].v);" % (n.nid, op, n.nid, n.nid))
     L.close()
     L.close()
     for n in reds:
@@ -912,4 +933,4 @@ def gen_colsplit(prog, V, LX, LY):
         L("o%d.store(%s);" % (st.out.index, g.addr(st.out, "0", "c")))
     L.close()
     L.close()
-    return _finish("colsplit", g, head, fmt, T, lds, dict(V=V, LX=LX, LY=LY, NRED=len(reds)))
+    return _finish("colsplit", g, head, fmt, T, lds, dict(V=V, LX=LX, LY=LY, NRED=len(reds), stream=bool(stream)))

@@ -53,6 +53,11 @@ class ShapeTensor(Tensor):
     def __len__(self):
         return self.shape[0]
 
+    def __repr__(self):
+        return "ShapeTensor(%s, %s, strides=%s)" % (self.shape, self.dtype, self.strides)
+
+    __str__ = __repr__
+
     @property
     def T(self):
         return ShapeTensor(self.backend, self.shape[::-1], self.dtype, self.name,

@@ -79,6 +79,8 @@ SIGNATURES = {
     "nh_module_get_function": (c_int, [c_void_p, c_char_p, POINTER(c_void_p)]),
     "nh_launch": (c_int, [c_void_p, POINTER(c_uint32), POINTER(c_uint32), c_uint32,
                           c_void_p, c_void_p, c_size_t]),
+    "nh_launch_timed": (c_int, [c_void_p, POINTER(c_uint32), POINTER(c_uint32), c_uint32,
+                                c_void_p, c_void_p, c_size_t, c_uint32, POINTER(c_float)]),
     "nh_ew_axpby_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_float, c_size_t, c_void_p]),
     "nh_ew_sigmoid_f32": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     "nh_adam_step_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_float,
@@ -226,6 +228,17 @@ class Runtime(object):
         args = kernel.packer.pack(*values)
         _check(self.lib.nh_launch(kernel.function, g, b, lds_bytes, self.stream,
                                   args, kernel.arg_bytes))
+
+    def launch_timed(self, kernel, grid, block, lds_bytes, reps, *values):
+        """mean milliseconds per launch over ``reps`` back-to-back launches"""
+        g, b = self._grid, self._block
+        g[0], g[1], g[2] = grid
+        b[0], b[1], b[2] = block
+        args = kernel.packer.pack(*values)
+        ms = c_float()
+        _check(self.lib.nh_launch_timed(kernel.function, g, b, lds_bytes, self.stream,
+                                        args, kernel.arg_bytes, reps, byref(ms)))
+        return ms.value
 
     def shutdown(self):
         self.lib.nh_shutdown()

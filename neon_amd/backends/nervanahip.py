@@ -365,6 +365,21 @@ class _FuseScope(object):
         return False
 
 
+class _CaptureScope(object):
+    def __init__(self, be):
+        self.be = be
+
+    def __enter__(self):
+        self.be._flush()
+        self.be._captured = []
+        return self.be._captured
+
+    def __exit__(self, exc_type, exc, tb):
+        self.be._flush()
+        self.be._captured = None
+        return False
+
+
 class NervanaHIP(Backend):
     """MI355X backend for the op-tree path.
 
@@ -402,6 +417,7 @@ class NervanaHIP(Backend):
         self._pending = []
         self._fusing = False
         self._fuse_depth = 0
+        self._captured = None
         self._temp_pool = {}
         self._live_allocs = 0
 
@@ -508,7 +524,10 @@ class NervanaHIP(Backend):
     def _flush(self):
         if self._pending:
             trees, self._pending = self._pending, []
-            self._run(trees)
+            if self._captured is not None:
+                self._captured.append(trees)
+            else:
+                self._run(trees)
 
     @staticmethod
     def _is_elementwise(tree):
@@ -544,7 +563,10 @@ class NervanaHIP(Backend):
                 self._pending.append(optree)
                 return optree[1]
             self._flush()
-        self._run([optree])
+        if self._captured is not None:
+            self._captured.append([optree])
+        else:
+            self._run([optree])
         return optree[1]
 
     def _run(self, trees):
@@ -572,6 +594,29 @@ class NervanaHIP(Backend):
                 raise
             self.plan_stats["split"] += 1
             self._run_split(trees[0])
+
+    # -- bench mode (the reference brackets launches with events when its
+    #    ``bench`` flag is set, float_ew.py:917-938) -------------------------------------
+    def capture(self):
+        """Context manager: statements issued inside are recorded instead of
+        run; yields the list of statement groups (lists of assign trees, a
+        fused group being one entry) for ``time_group``."""
+        return _CaptureScope(self)
+
+    def time_group(self, trees, reps=20):
+        """Mean milliseconds per launch of the single kernel that runs the
+        statement group ``trees``, measured with events on the launch stream
+        around ``reps`` back-to-back launches.  Returns (ms, plan)."""
+        prog = Program()
+        for t in trees:
+            prog.add_statement(t)
+        prog.finalize()
+        key = prog.key()
+        plan = self.plans.get(key)
+        if plan is None:
+            plan = make_plan(prog, self.rt, self.kernels, self.cu_count)
+            self.plans[key] = plan
+        return plan.launch_timed(prog, reps), plan
 
     def _run_split(self, tree):
         """Evaluate a tree that does not fit one kernel stage by stage through

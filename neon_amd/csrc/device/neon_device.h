@@ -73,6 +73,43 @@ template <typename T, int V> NEON_DEV void nh_store_vec(T* p, const T (&raw)[V])
     *reinterpret_cast<nh_vec<T, V>*>(p) = t;
 }
 
+// NW consecutive 32-bit words, 16 bytes per instruction; NT = streaming access
+// (non-temporal: the line is not kept in cache, for data touched once).
+typedef nh_u32 nh_u32x2 __attribute__((ext_vector_type(2)));
+typedef nh_u32 nh_u32x4 __attribute__((ext_vector_type(4)));
+template <int NW, bool NT> NEON_DEV void nh_load_words(const nh_u32* p, nh_u32 (&w)[NW]) {
+    if constexpr (!NT) {
+        nh_load_vec<nh_u32, NW>(p, w);
+    } else if constexpr (NW == 1) {
+        w[0] = __builtin_nontemporal_load(p);
+    } else if constexpr (NW == 2) {
+        const nh_u32x2 t = __builtin_nontemporal_load(reinterpret_cast<const nh_u32x2*>(p));
+        w[0] = t.x; w[1] = t.y;
+    } else {
+#pragma unroll
+        for (int i = 0; i < NW; i += 4) {
+            const nh_u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const nh_u32x4*>(p + i));
+            w[i] = t.x; w[i + 1] = t.y; w[i + 2] = t.z; w[i + 3] = t.w;
+        }
+    }
+}
+template <int NW, bool NT> NEON_DEV void nh_store_words(nh_u32* p, const nh_u32 (&w)[NW]) {
+    if constexpr (!NT) {
+        nh_store_vec<nh_u32, NW>(p, w);
+    } else if constexpr (NW == 1) {
+        __builtin_nontemporal_store(w[0], p);
+    } else if constexpr (NW == 2) {
+        nh_u32x2 t; t.x = w[0]; t.y = w[1];
+        __builtin_nontemporal_store(t, reinterpret_cast<nh_u32x2*>(p));
+    } else {
+#pragma unroll
+        for (int i = 0; i < NW; i += 4) {
+            nh_u32x4 t; t.x = w[i]; t.y = w[i + 1]; t.z = w[i + 2]; t.w = w[i + 3];
+            __builtin_nontemporal_store(t, reinterpret_cast<nh_u32x4*>(p + i));
+        }
+    }
+}
+
 // Packed 16-bit storage kept in 32-bit registers (two elements per register).
 typedef nh_f16 nh_f16x2 __attribute__((ext_vector_type(2)));
 NEON_DEV float nh_f16_lo(nh_u32 w) { return (float)__builtin_bit_cast(nh_f16x2, w).x; }
@@ -127,6 +164,10 @@ template <typename T, int V> struct nh_raw {
         if constexpr (PACKED) nh_load_vec<nh_u32, NW>(reinterpret_cast<const nh_u32*>(p), w);
         else w[0] = nh_bits_of<T>(*p);
     }
+    NEON_DEV void load_stream(const T* p) {      // touched once: do not keep in cache
+        if constexpr (PACKED) nh_load_words<NW, true>(reinterpret_cast<const nh_u32*>(p), w);
+        else w[0] = nh_bits_of<T>(__builtin_nontemporal_load(p));
+    }
     NEON_DEV void zero() {
 #pragma unroll
         for (int i = 0; i < NW; ++i) w[i] = 0u;
@@ -169,6 +210,10 @@ template <typename T, int V> struct nh_out {
     NEON_DEV void store(T* p) const {
         if constexpr (PACKED) nh_store_vec<nh_u32, NW>(reinterpret_cast<nh_u32*>(p), w);
         else *p = nh_from_bits<T>(w[0]);
+    }
+    NEON_DEV void store_stream(T* p) const {
+        if constexpr (PACKED) nh_store_words<NW, true>(reinterpret_cast<nh_u32*>(p), w);
+        else __builtin_nontemporal_store(nh_from_bits<T>(w[0]), p);
     }
 };
 
@@ -224,7 +269,7 @@ struct nh_op_sum { static NEON_DEV float init() { return 0.0f; }      static NEO
 struct nh_op_max { static NEON_DEV float init() { return -NH_INF; }   static NEON_DEV float f(float a, float b) { return nh_max(a, b); } };
 struct nh_op_min { static NEON_DEV float init() { return NH_INF; }    static NEON_DEV float f(float a, float b) { return nh_min(a, b); } };
 
-struct nh_pair { float v; int i; };
+struct __attribute__((aligned(8))) nh_pair { float v; int i; };
 struct nh_op_argmax {
     static NEON_DEV nh_pair init() { nh_pair p; p.v = -NH_INF; p.i = 0; return p; }
     static NEON_DEV nh_pair f(nh_pair a, nh_pair b) {
@@ -242,6 +287,18 @@ struct nh_op_argmin {
     }
     static NEON_DEV void step(nh_pair& a, float v, int i) { if (v < a.v) { a.v = v; a.i = i; } }
 };
+
+// Partial results handed from one workgroup to another (possibly on another
+// XCD, behind another L2): stored through to device-coherent memory and loaded
+// past the local L2, as single 8-byte relaxed device-scope atomics.
+NEON_DEV void nh_part_store(nh_pair* p, nh_pair v) {
+    __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), __builtin_bit_cast(unsigned long long, v),
+                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+NEON_DEV nh_pair nh_part_load(const nh_pair* p) {
+    return __builtin_bit_cast(nh_pair, __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p),
+                                                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
 
 template <int CTRL> NEON_DEV nh_pair nh_dpp(nh_pair p) { nh_pair r; r.v = nh_dpp<CTRL>(p.v); r.i = nh_dpp<CTRL>(p.i); return r; }
 NEON_DEV nh_pair nh_swz16(nh_pair p) { nh_pair r; r.v = nh_swz16(p.v); r.i = nh_swz16(p.i); return r; }

@@ -24,56 +24,68 @@ int launch_status(const char* what) {
 }
 
 // ---------------------------------------------------------------------------
-// Streaming elementwise kernels: 256 threads, each owning EW_U vectors of V
-// floats spaced a workgroup apart (so every wave touches 1 KiB contiguous per
-// instruction).  All loads of a tile are issued before the first use.
+// Streaming elementwise kernels: 256 threads, one vector of V floats per lane
+// and tensor (every wave touches 1 KiB contiguous per instruction), all loads
+// issued before the first use.  One vector per lane measured fastest for the
+// 7-stream Adam update (more in flight per lane only adds read/write
+// turnarounds); inputs far larger than the caches use non-temporal accesses.
 // ---------------------------------------------------------------------------
 constexpr int EW_T = 256;
-constexpr int EW_U = 4;
+constexpr size_t EW_STREAM_BYTES = (size_t)256 << 20;
 
-template <int V, class F>
+template <int V, bool NT> __device__ __forceinline__ void ew_ld(const float* p, float (&r)[V]) {
+    nh_u32 w[V];
+    nh_load_words<V, NT>(reinterpret_cast<const nh_u32*>(p), w);
+#pragma unroll
+    for (int j = 0; j < V; ++j) r[j] = __builtin_bit_cast(float, w[j]);
+}
+template <int V, bool NT> __device__ __forceinline__ void ew_st(float* p, const float (&r)[V]) {
+    nh_u32 w[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) w[j] = __builtin_bit_cast(nh_u32, r[j]);
+    nh_store_words<V, NT>(reinterpret_cast<nh_u32*>(p), w);
+}
+
+template <int V, bool NT, class F>
 __global__ __launch_bounds__(EW_T) void ew_stream_kernel(F f, size_t n) {
-    const size_t tile = (size_t)blockIdx.x * (EW_T * EW_U * V);
-    const int tid = threadIdx.x;
-    if (tile + (size_t)EW_T * EW_U * V <= n) {
-        typename F::template regs<V> r[EW_U];
-#pragma unroll
-        for (int u = 0; u < EW_U; ++u) f.template load<V>(r[u], tile + (size_t)(u * EW_T + tid) * V);
-#pragma unroll
-        for (int u = 0; u < EW_U; ++u) {
-            f.template compute<V>(r[u]);
-            f.template store<V>(r[u], tile + (size_t)(u * EW_T + tid) * V);
-        }
+    const size_t i = ((size_t)blockIdx.x * EW_T + threadIdx.x) * V;
+    if (i + V <= n) {
+        typename F::template regs<V> r;
+        f.template load<V, NT>(r, i);
+        f.template compute<V>(r);
+        f.template store<V, NT>(r, i);
     } else {
-        for (size_t i = tile + tid; i < n; i += EW_T) {
+        for (size_t e = i; e < n; ++e) {
             typename F::template regs<1> r;
-            f.template load<1>(r, i);
+            f.template load<1, false>(r, e);
             f.template compute<1>(r);
-            f.template store<1>(r, i);
+            f.template store<1, false>(r, e);
         }
     }
 }
 
 struct AxpbyF {
     float* out; const float* x; const float* y; float a, b;
+    static constexpr int TENSORS = 3;
     template <int V> struct regs { float x[V], y[V]; };
-    template <int V> __device__ void load(regs<V>& r, size_t i) const { nh_load_vec<float, V>(x + i, r.x); nh_load_vec<float, V>(y + i, r.y); }
+    template <int V, bool NT> __device__ void load(regs<V>& r, size_t i) const { ew_ld<V, NT>(x + i, r.x); ew_ld<V, NT>(y + i, r.y); }
     template <int V> __device__ void compute(regs<V>& r) const {
 #pragma unroll
         for (int j = 0; j < V; ++j) r.x[j] = a * r.x[j] + b * r.y[j];
     }
-    template <int V> __device__ void store(const regs<V>& r, size_t i) const { nh_store_vec<float, V>(out + i, r.x); }
+    template <int V, bool NT> __device__ void store(const regs<V>& r, size_t i) const { ew_st<V, NT>(out + i, r.x); }
 };
 
 struct SigmoidF {
     float* out; const float* x;
+    static constexpr int TENSORS = 2;
     template <int V> struct regs { float x[V]; };
-    template <int V> __device__ void load(regs<V>& r, size_t i) const { nh_load_vec<float, V>(x + i, r.x); }
+    template <int V, bool NT> __device__ void load(regs<V>& r, size_t i) const { ew_ld<V, NT>(x + i, r.x); }
     template <int V> __device__ void compute(regs<V>& r) const {
 #pragma unroll
         for (int j = 0; j < V; ++j) r.x[j] = nh_sig(r.x[j]);
     }
-    template <int V> __device__ void store(const regs<V>& r, size_t i) const { nh_store_vec<float, V>(out + i, r.x); }
+    template <int V, bool NT> __device__ void store(const regs<V>& r, size_t i) const { ew_st<V, NT>(out + i, r.x); }
 };
 
 // The three assigns of the reference's Adam.optimize
@@ -83,10 +95,10 @@ struct SigmoidF {
 struct AdamF {
     float* p; float* m; float* v; const float* g;
     float lr, b1, omb1, b2, omb2, eps;
+    static constexpr int TENSORS = 7;
     template <int V> struct regs { float p[V], m[V], v[V], g[V]; };
-    template <int V> __device__ void load(regs<V>& r, size_t i) const {
-        nh_load_vec<float, V>(g + i, r.g); nh_load_vec<float, V>(m + i, r.m);
-        nh_load_vec<float, V>(v + i, r.v); nh_load_vec<float, V>(p + i, r.p);
+    template <int V, bool NT> __device__ void load(regs<V>& r, size_t i) const {
+        ew_ld<V, NT>(g + i, r.g); ew_ld<V, NT>(m + i, r.m); ew_ld<V, NT>(v + i, r.v); ew_ld<V, NT>(p + i, r.p);
     }
     template <int V> __device__ void compute(regs<V>& r) const {
 #pragma unroll
@@ -99,8 +111,8 @@ struct AdamF {
             r.p[j] = r.p[j] - (lr * mj) / (sqrtf(vj) + eps);
         }
     }
-    template <int V> __device__ void store(const regs<V>& r, size_t i) const {
-        nh_store_vec<float, V>(m + i, r.m); nh_store_vec<float, V>(v + i, r.v); nh_store_vec<float, V>(p + i, r.p);
+    template <int V, bool NT> __device__ void store(const regs<V>& r, size_t i) const {
+        ew_st<V, NT>(m + i, r.m); ew_st<V, NT>(v + i, r.v); ew_st<V, NT>(p + i, r.p);
     }
 };
 
@@ -108,17 +120,14 @@ template <class F> int launch_ew(const F& f, size_t n, bool vec_ok, void* stream
     if (!nh_internal_ready()) return nh_internal_fail(NH_ENOTINIT, "nh_init has not been called");
     if (n == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
-    if (vec_ok) {
-        const size_t per_block = (size_t)EW_T * EW_U * 4;
-        const size_t blocks = (n + per_block - 1) / per_block;
-        if (blocks > 0x7FFFFFFFull) return nh_internal_fail(NH_EINVAL, "tensor too large for one launch");
-        hipLaunchKernelGGL((ew_stream_kernel<4, F>), dim3((unsigned)blocks), dim3(EW_T), 0, s, f, n);
-    } else {
-        const size_t per_block = (size_t)EW_T * EW_U;
-        const size_t blocks = (n + per_block - 1) / per_block;
-        if (blocks > 0x7FFFFFFFull) return nh_internal_fail(NH_EINVAL, "tensor too large for one launch");
-        hipLaunchKernelGGL((ew_stream_kernel<1, F>), dim3((unsigned)blocks), dim3(EW_T), 0, s, f, n);
-    }
+    const int v = vec_ok ? 4 : 1;
+    const size_t per_block = (size_t)EW_T * v;
+    const size_t blocks = (n + per_block - 1) / per_block;
+    if (blocks > 0x7FFFFFFFull) return nh_internal_fail(NH_EINVAL, "tensor too large for one launch");
+    const bool nt = n * sizeof(float) * F::TENSORS >= EW_STREAM_BYTES;
+    if (vec_ok && nt) hipLaunchKernelGGL((ew_stream_kernel<4, true, F>), dim3((unsigned)blocks), dim3(EW_T), 0, s, f, n);
+    else if (vec_ok) hipLaunchKernelGGL((ew_stream_kernel<4, false, F>), dim3((unsigned)blocks), dim3(EW_T), 0, s, f, n);
+    else hipLaunchKernelGGL((ew_stream_kernel<1, false, F>), dim3((unsigned)blocks), dim3(EW_T), 0, s, f, n);
     return launch_status(what);
 }
 
@@ -132,7 +141,7 @@ template <class F> int launch_ew(const F& f, size_t n, bool vec_ok, void* stream
 constexpr int RN_T = 1024;
 constexpr int RN_V = 8;
 
-template <int NCH>
+template <int NCH, bool NT>
 __global__ __launch_bounds__(RN_T) void rownorm_f16_kernel(nh_f16* out, const nh_f16* x,
                                                            const float* __restrict__ gamma,
                                                            const float* __restrict__ beta, float eps, uint32_t cols,
@@ -151,7 +160,7 @@ __global__ __launch_bounds__(RN_T) void rownorm_f16_kernel(nh_f16* out, const nh
     for (int k = 0; k < NCH; ++k) {
         const uint32_t c = (uint32_t)(k * RN_T + tid) * RN_V;
         if (c < cols) {
-            nh_load_vec<nh_u32, RN_V / 2>(reinterpret_cast<const nh_u32*>(xr + c), raw[k]);
+            nh_load_words<RN_V / 2, NT>(reinterpret_cast<const nh_u32*>(xr + c), raw[k]);
         } else {
 #pragma unroll
             for (int j = 0; j < RN_V / 2; ++j) raw[k][j] = 0u;  // +0.0 pairs
@@ -198,7 +207,7 @@ __global__ __launch_bounds__(RN_T) void rownorm_f16_kernel(nh_f16* out, const nh
             for (int j = 0; j < RN_V / 2; ++j)
                 o[j] = nh_f16_pack((g * (nh_f16_lo(raw[k][j]) - mean)) / denom + b,
                                    (g * (nh_f16_hi(raw[k][j]) - mean)) / denom + b);
-            nh_store_vec<nh_u32, RN_V / 2>(reinterpret_cast<nh_u32*>(orow + c), o);
+            nh_store_words<RN_V / 2, NT>(reinterpret_cast<nh_u32*>(orow + c), o);
         }
     }
 }
@@ -206,8 +215,14 @@ __global__ __launch_bounds__(RN_T) void rownorm_f16_kernel(nh_f16* out, const nh
 template <int NCH>
 void launch_rownorm(uint16_t* out, const uint16_t* x, const float* gamma, const float* beta, float eps,
                     uint32_t rows, uint32_t cols, size_t ld, hipStream_t s) {
-    hipLaunchKernelGGL((rownorm_f16_kernel<NCH>), dim3(rows), dim3(RN_T), 0, s, (nh_f16*)out, (const nh_f16*)x,
-                       gamma, beta, eps, cols, ld, 1.0f / (float)cols);
+    // beyond what the L2 slices hold, the row is touched once: stream it
+    const bool nt = (size_t)rows * cols * 2 * sizeof(uint16_t) >= ((size_t)32 << 20);
+    if (nt)
+        hipLaunchKernelGGL((rownorm_f16_kernel<NCH, true>), dim3(rows), dim3(RN_T), 0, s, (nh_f16*)out,
+                           (const nh_f16*)x, gamma, beta, eps, cols, ld, 1.0f / (float)cols);
+    else
+        hipLaunchKernelGGL((rownorm_f16_kernel<NCH, false>), dim3(rows), dim3(RN_T), 0, s, (nh_f16*)out,
+                           (const nh_f16*)x, gamma, beta, eps, cols, ld, 1.0f / (float)cols);
 }
 
 // ---------------------------------------------------------------------------
@@ -215,52 +230,49 @@ void launch_rownorm(uint16_t* out, const uint16_t* x, const float* gamma, const 
 // coalesced; a workgroup is CR_LX column-lanes x CR_LY row-lanes and owns a
 // (rows_per_chunk x CR_LX*V) tile.  Tiles of one column strip leave (value,
 // index) partials in the workspace; the last workgroup of the strip to finish
-// (ticket counter) folds them, in row order, into the result.  No workgroup
-// ever waits for another.
+// (ticket counter) folds them into the result.  No workgroup ever waits for
+// another.  Partials cross XCDs as write-through stores / L2-bypassing loads,
+// so no device-wide fence (a whole-L2 write-back) is needed.
 // ---------------------------------------------------------------------------
 constexpr int CR_LX = 16;
 constexpr int CR_LY = 16;
 constexpr int CR_T = CR_LX * CR_LY;
+constexpr int CR_WY = CR_T / 64;          // wave groups to join through LDS
 constexpr int CR_MAX_STRIPS = 4096;
 constexpr int CR_MAX_CHUNKS = 128;
+constexpr int CR_QMAX = CR_MAX_CHUNKS / CR_LY;
 
 __device__ unsigned int g_cr_tickets[CR_MAX_STRIPS];  // zero at load; each strip's last workgroup resets its ticket
 
 template <int V>
-__device__ __forceinline__ void cr_fold_rows(nh_pair (&acc)[V], float (*sv)[CR_LX * V + 1], int (*si)[CR_LX * V + 1],
-                                              int tx, int ty) {
-    // join the CR_LY row-lanes of each column through LDS, lowest rows first
+__device__ __forceinline__ void cr_fold_rows(nh_pair (&acc)[V], nh_pair (*sp)[CR_LX * V + 1], int tx) {
+    // lanes of a wave that share a column tile differ in lane bits 4 and 5
 #pragma unroll
-    for (int j = 0; j < V; ++j) {
-        sv[ty][tx * V + j] = acc[j].v;
-        si[ty][tx * V + j] = acc[j].i;
+    for (int j = 0; j < V; ++j) acc[j] = nh_op_argmax::f(acc[j], nh_lane_xor<16>(acc[j]));
+#pragma unroll
+    for (int j = 0; j < V; ++j) acc[j] = nh_op_argmax::f(acc[j], nh_lane_xor<32>(acc[j]));
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) < CR_LX) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) sp[wave][tx * V + j] = acc[j];
     }
     __syncthreads();
-    if (ty == 0) {
 #pragma unroll
-        for (int j = 0; j < V; ++j) {
-            nh_pair r;
-            r.v = sv[0][tx * V + j];
-            r.i = si[0][tx * V + j];
-            for (int y = 1; y < CR_LY; ++y) {
-                nh_pair o;
-                o.v = sv[y][tx * V + j];
-                o.i = si[y][tx * V + j];
-                r = nh_op_argmax::f(r, o);
-            }
-            acc[j] = r;
-        }
+    for (int j = 0; j < V; ++j) {
+        nh_pair r = sp[0][tx * V + j];
+#pragma unroll
+        for (int y = 1; y < CR_WY; ++y) r = nh_op_argmax::f(r, sp[y][tx * V + j]);
+        acc[j] = r;
     }
     __syncthreads();
 }
 
 template <int V>
 __global__ __launch_bounds__(CR_T) void colmax_kernel(const float* __restrict__ x, uint32_t rows, uint32_t cols,
-                                                      size_t ld, uint32_t rows_per_chunk, float* pval, int* pidx,
+                                                      size_t ld, uint32_t rows_per_chunk, nh_pair* part,
                                                       float* __restrict__ outv, int* __restrict__ outi,
                                                       unsigned int* tickets) {
-    __shared__ float sv[CR_LY][CR_LX * V + 1];
-    __shared__ int si[CR_LY][CR_LX * V + 1];
+    __shared__ nh_pair sp[CR_WY][CR_LX * V + 1];
     __shared__ int s_last;
     const int tid = threadIdx.x;
     const int tx = tid % CR_LX, ty = tid / CR_LX;
@@ -297,50 +309,40 @@ __global__ __launch_bounds__(CR_T) void colmax_kernel(const float* __restrict__ 
             for (int j = 0; j < V; ++j) nh_op_argmax::step(acc[j], a0[j], (int)r);
         }
     }
-    cr_fold_rows<V>(acc, sv, si, tx, ty);
+    cr_fold_rows<V>(acc, sp, tx);
 
     const uint32_t nchunks = gridDim.y;
-    if (nchunks == 1) {
+    if (nchunks > 1) {
         if (ty == 0 && live) {
 #pragma unroll
-            for (int j = 0; j < V; ++j) {
-                if (outv) outv[c + j] = acc[j].v;
-                if (outi) outi[c + j] = acc[j].i;
-            }
+            for (int j = 0; j < V; ++j) nh_part_store(&part[(size_t)blockIdx.y * cols + c + j], acc[j]);
         }
-        return;
-    }
-    if (ty == 0 && live) {
-#pragma unroll
-        for (int j = 0; j < V; ++j) {
-            pval[(size_t)blockIdx.y * cols + c + j] = acc[j].v;
-            pidx[(size_t)blockIdx.y * cols + c + j] = acc[j].i;
+        __syncthreads();  // every lane's partial stores have completed before the ticket is taken
+        if (tid == 0) {
+            const unsigned int t = atomicAdd(&tickets[blockIdx.x], 1u);
+            s_last = (t == nchunks - 1);
         }
-    }
-    __threadfence();  // partials visible device-wide before the ticket is taken
-    __syncthreads();
-    if (tid == 0) {
-        const unsigned int t = atomicAdd(&tickets[blockIdx.x], 1u);
-        s_last = (t == nchunks - 1);
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();  // acquire: drop any stale cached copy of the partials
+        __syncthreads();
+        if (!s_last) return;
 
+        nh_pair q[CR_QMAX][V];
 #pragma unroll
-    for (int j = 0; j < V; ++j) acc[j] = nh_op_argmax::init();
-    if (live) {
-        for (uint32_t k = ty; k < nchunks; k += CR_LY) {
+        for (int k = 0; k < CR_QMAX; ++k) {
+            const uint32_t chunk = ty + k * CR_LY;
 #pragma unroll
-            for (int j = 0; j < V; ++j) {
-                nh_pair o;
-                o.v = pval[(size_t)k * cols + c + j];
-                o.i = pidx[(size_t)k * cols + c + j];
-                acc[j] = nh_op_argmax::f(acc[j], o);
-            }
+            for (int j = 0; j < V; ++j)
+                q[k][j] = (live && chunk < nchunks) ? nh_part_load(&part[(size_t)chunk * cols + c + j])
+                                                    : nh_op_argmax::init();
         }
+#pragma unroll
+        for (int j = 0; j < V; ++j) acc[j] = nh_op_argmax::init();
+#pragma unroll
+        for (int k = 0; k < CR_QMAX; ++k)
+#pragma unroll
+            for (int j = 0; j < V; ++j) acc[j] = nh_op_argmax::f(acc[j], q[k][j]);
+        cr_fold_rows<V>(acc, sp, tx);
+        if (tid == 0) tickets[blockIdx.x] = 0;  // ready for the next launch on this stream
     }
-    cr_fold_rows<V>(acc, sv, si, tx, ty);
     if (ty == 0 && live) {
 #pragma unroll
         for (int j = 0; j < V; ++j) {
@@ -348,7 +350,6 @@ __global__ __launch_bounds__(CR_T) void colmax_kernel(const float* __restrict__ 
             if (outi) outi[c + j] = acc[j].i;
         }
     }
-    if (tid == 0) tickets[blockIdx.x] = 0;  // ready for the next launch on this stream
 }
 
 struct CrPlan { uint32_t strips, chunks, rows_per_chunk; int v; };
@@ -358,8 +359,14 @@ CrPlan cr_plan(uint32_t rows, uint32_t cols, bool vec) {
     p.v = vec ? 4 : 1;
     const uint32_t strip_cols = CR_LX * p.v;
     p.strips = (cols + strip_cols - 1) / strip_cols;
-    const uint32_t target_groups = 1024;  // about four workgroups per compute unit
-    uint32_t chunks = target_groups / (p.strips ? p.strips : 1);
+    // one workgroup per compute unit for small inputs, up to eight for large
+    // ones, each with at least ~128 KiB to stream
+    const uint64_t bytes = (uint64_t)rows * cols * sizeof(float);
+    const uint32_t cus = nh_internal_cu_count() > 0 ? (uint32_t)nh_internal_cu_count() : 256u;
+    uint64_t per_cu = bytes / ((uint64_t)cus * (128u << 10));
+    if (per_cu < 1) per_cu = 1;
+    if (per_cu > 8) per_cu = 8;
+    uint32_t chunks = (uint32_t)(per_cu * cus) / (p.strips ? p.strips : 1);
     if (chunks < 1) chunks = 1;
     if (chunks > CR_MAX_CHUNKS) chunks = CR_MAX_CHUNKS;
     uint32_t rpc = (rows + chunks - 1) / chunks;
@@ -423,10 +430,8 @@ int nh_rownorm_f16(uint16_t* out, const uint16_t* x, const float* gamma, const f
 
 size_t nh_colreduce_workspace_bytes(uint32_t rows, uint32_t cols) {
     if (rows == 0 || cols == 0) return 0;
-    const CrPlan p = cr_plan(rows, cols, true);
-    const CrPlan q = cr_plan(rows, cols, false);
-    const size_t chunks = p.chunks > q.chunks ? p.chunks : q.chunks;
-    return chunks * (size_t)cols * (sizeof(float) + sizeof(int)) + 256;
+    // independent of the device and of which variant runs: the most chunks a launch may use
+    return (size_t)CR_MAX_CHUNKS * (size_t)cols * sizeof(nh_pair) + 256;
 }
 
 int nh_colmax_argmax_f32(float* maxval, int32_t* argmax, const float* x, uint32_t rows, uint32_t cols, size_t ld,
@@ -441,19 +446,20 @@ int nh_colmax_argmax_f32(float* maxval, int32_t* argmax, const float* x, uint32_
     if (p.strips > CR_MAX_STRIPS) return nh_internal_fail(NH_EINVAL, "nh_colmax_argmax_f32: too many columns");
     if (p.chunks > 1 && !workspace) return nh_internal_fail(NH_EINVAL, "nh_colmax_argmax_f32: workspace required");
     if (p.chunks > 65535u) return nh_internal_fail(NH_EINVAL, "nh_colmax_argmax_f32: grid too large");
-    float* pval = (float*)workspace;
-    int* pidx = (int*)(pval + (size_t)p.chunks * cols);
+    if (p.chunks > 1 && (reinterpret_cast<uintptr_t>(workspace) & 7u))
+        return nh_internal_fail(NH_EINVAL, "nh_colmax_argmax_f32: workspace must be 8-byte aligned");
+    nh_pair* part = (nh_pair*)workspace;
     unsigned int* tickets = nullptr;
     hipError_t e = hipGetSymbolAddress((void**)&tickets, HIP_SYMBOL(g_cr_tickets));
     if (e != hipSuccess) return nh_internal_fail((int)e, "nh_colmax_argmax_f32: ticket symbol lookup failed");
     hipStream_t s = (hipStream_t)stream;
     dim3 grid(p.strips, p.chunks);
     if (vec)
-        hipLaunchKernelGGL((colmax_kernel<4>), grid, dim3(CR_T), 0, s, x, rows, cols, ld, p.rows_per_chunk, pval,
-                           pidx, maxval, (int*)argmax, tickets);
+        hipLaunchKernelGGL((colmax_kernel<4>), grid, dim3(CR_T), 0, s, x, rows, cols, ld, p.rows_per_chunk, part,
+                           maxval, (int*)argmax, tickets);
     else
-        hipLaunchKernelGGL((colmax_kernel<1>), grid, dim3(CR_T), 0, s, x, rows, cols, ld, p.rows_per_chunk, pval,
-                           pidx, maxval, (int*)argmax, tickets);
+        hipLaunchKernelGGL((colmax_kernel<1>), grid, dim3(CR_T), 0, s, x, rows, cols, ld, p.rows_per_chunk, part,
+                           maxval, (int*)argmax, tickets);
     return launch_status("nh_colmax_argmax_f32");
 }
 

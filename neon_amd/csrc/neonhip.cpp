@@ -368,6 +368,38 @@ int nh_launch(void* function, const uint32_t grid[3], const uint32_t block[3],
     return 0;
 }
 
+int nh_launch_timed(void* function, const uint32_t grid[3], const uint32_t block[3],
+                    uint32_t lds_bytes, void* stream, const void* args, size_t arg_bytes,
+                    uint32_t reps, float* mean_ms) {
+    NH_NEED_INIT();
+    if (!mean_ms || reps == 0) return fail(NH_EINVAL, "nh_launch_timed: bad argument");
+    *mean_ms = 0.0f;
+    hipEvent_t e0, e1;
+    NH_HIP(hipEventCreate(&e0));
+    hipError_t err = hipEventCreate(&e1);
+    if (err != hipSuccess) {
+        hipEventDestroy(e0);
+        return hip_fail(err, "hipEventCreate");
+    }
+    int rc = 0;
+    hipStream_t s = (hipStream_t)stream;
+    err = hipEventRecord(e0, s);
+    if (err != hipSuccess) rc = hip_fail(err, "hipEventRecord");
+    for (uint32_t i = 0; rc == 0 && i < reps; ++i)
+        rc = nh_launch(function, grid, block, lds_bytes, stream, args, arg_bytes);
+    if (rc == 0) {
+        err = hipEventRecord(e1, s);
+        if (err == hipSuccess) err = hipEventSynchronize(e1);
+        float ms = 0.0f;
+        if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
+        if (err != hipSuccess) rc = hip_fail(err, "nh_launch_timed: event timing");
+        else *mean_ms = ms / (float)reps;
+    }
+    hipEventDestroy(e0);
+    hipEventDestroy(e1);
+    return rc;
+}
+
 }  // extern "C"
 
 // Shared with kernels.hip (same library, not part of the ABI).

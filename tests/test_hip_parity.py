@@ -120,8 +120,13 @@ RED_SHAPES = [(2, 2), (10, 32), (50, 50), (50, 128), (1000, 128), (257, 1000), (
 def test_reductions(pair, shape, axis):
     rs = np.random.RandomState(5)
     a = gen_inputs(rs, shape)
+    # A sum of n terms carries an fp32 rounding error of about eps * sum|x| in
+    # either evaluation order (numpy adds rows one after the other along axis
+    # 0, the device adds a tree), so near-zero results are compared with that
+    # absolute allowance on top of the 1e-5 relative one.
+    atol = 2 * np.finfo(np.float32).eps * float(np.abs(a).sum(axis=axis).max())
     for name in ("sum", "max", "min", "mean", "var", "std"):
-        both(pair, lambda be, x, n=name: getattr(be, n)(x, axis=axis), [a], rtol=2e-5, atol=2e-6,
+        both(pair, lambda be, x, n=name: getattr(be, n)(x, axis=axis), [a], rtol=RTOL32, atol=atol,
              what="%s axis%d" % (name, axis))
     for name in ("argmax", "argmin"):
         got, want = both(pair, lambda be, x, n=name: getattr(be, n)(x, axis=axis), [a],
@@ -168,7 +173,8 @@ def test_compound_and_mixed_axes(pair):
     both(pair, lambda be, x, y: be.mean(x * y), [a, b], rtol=2e-5, atol=1e-6)
     both(pair, lambda be, x, y: be.std(be.var(x, axis=0), axis=1), [a, b], rtol=5e-5)
     both(pair, lambda be, x, y: be.max(x) + be.min(y), [a, b])
-    both(pair, lambda be, x, y: x - be.mean(x) + be.sum(y, axis=1), [a, b], rtol=2e-5, atol=2e-6)
+    # row sums of 128 terms of size ~1 carry ~1e-5 absolute fp32 error in either order
+    both(pair, lambda be, x, y: x - be.mean(x) + be.sum(y, axis=1), [a, b], rtol=RTOL32, atol=2e-5)
     both(pair, lambda be, x, y: (x * y).T + 1.0, [a, b])
 
 
@@ -320,6 +326,6 @@ def test_full_size_properties(hip):
     # after one step from m = v = 0: m = 0.1 g, v = 0.001 g^2, |delta p| ~= lr
     assert_close(m.get(), np.float32(1. - 0.9) * grad, rtol=1e-6, atol=0)
     d = param - p.get()
-    nz = np.abs(grad) > 1e-4
+    nz = np.abs(grad) > 1e-3      # eps / sqrt(v) is below 4e-4 there
     assert np.allclose(np.abs(d[nz]), 1e-3, rtol=2e-3)
     assert np.array_equal(np.sign(d[nz]), np.sign(grad[nz]))

@@ -1,0 +1,245 @@
+"""Host-side logic that needs no GPU: the tensor API, the C ABI surface, the
+DAG builder, shape-class selection, code generation and hiprtc compilation for
+gfx950, the kernel cache, and the error behaviour callers rely on."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from neon_amd.backends.backend import Backend, Block, OpCollection, OpTreeNode
+from neon_amd.backends.hip import codegen, planner, prebuild
+from neon_amd.backends.hip import runtime as hiprt
+from neon_amd.backends.hip.optree_ir import MixedAxes, Program
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture()
+def pb(tmp_path):
+    return prebuild.PlanBackend(cache_dir=str(tmp_path / "kc"), compile_kernels=False)
+
+
+def plan_of(pb, issue):
+    n = len(pb.choices)
+    issue()
+    assert len(pb.choices) == n + 1
+    return pb.choices[-1]
+
+
+# ---- API --------------------------------------------------------------------------------
+def test_backend_registry_and_factory():
+    import neon_amd.backends as nb
+    assert "hip" in Backend.backend_choices()
+    with pytest.raises(ValueError):
+        Backend.allocate_backend("no-such-backend")
+    assert nb.gen_backend.__defaults__[0] == "hip"
+
+
+def test_optree_build_rules(pb):
+    a, b = pb.empty((4, 3)), pb.empty((4, 1))
+    f = a + b * 2.0
+    assert f.shape == (4, 3) and f[0]["op"] == "add"
+    assert (a > b).shape == (4, 3)
+    assert pb.sum(a, axis=0).shape == (1, 3) and pb.sum(a, axis=1).shape == (4, 1)
+    assert pb.sum(a).shape == (1, 1)
+    assert pb.mean(a, axis=1)[0]["op"] == "mul"                # sum * (1/N)
+    assert (2.0 - a)[1] == 2.0 and (2.0 - a)[0]["op"] == "sub"
+    assert (-a)[0]["op"] == "neg" and abs(a)[0]["op"] == "abs"
+    stack = (a * b + a).traverse([])
+    assert [s["op"] if isinstance(s, dict) else "t" for s in stack] == ["t", "t", "mul", "t", "add"]
+    k1, t2i, i2t = (a * b + a).intrinsic_key_maps()
+    assert k1 == ((0, (4, 3)), (1, (4, 1)), "mul", (0, (4, 3)), "add") and i2t[0] is a
+    with pytest.raises(TypeError):
+        OpTreeNode.build("bogus", a, b)
+    assert OpTreeNode.build("add", a, "x") is NotImplemented
+    with pytest.raises(ValueError):
+        pb.onehot(pb.empty((1, 4), dtype=np.int32), axis=2)
+    assert OpCollection.reduction_ops == {"sum", "max", "min", "argmax", "argmin"}
+    assert (a + b).pp().startswith("(")
+
+
+# ---- C ABI ------------------------------------------------------------------------------
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "neonhip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(nh_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = hiprt.load_library()
+    names = _declared_symbols()
+    assert len(names) >= 35
+    for n in names:
+        assert hasattr(lib, n), "libneonhip.so does not export %s" % n
+    assert sorted(hiprt.SIGNATURES) == names, "runtime.py binds a different set than the header declares"
+    assert lib.nh_abi_version() == 1
+
+
+def test_abi_errors_without_device():
+    lib = hiprt.load_library()
+    if hiprt.device_count() > 0:
+        pytest.skip("device present")
+    p = ctypes.c_void_p()
+    assert lib.nh_malloc(ctypes.byref(p), 1024) == hiprt.NH_ENOTINIT
+    assert b"nh_init" in lib.nh_last_error()
+    assert lib.nh_init(0, None) != 0
+    with pytest.raises(hiprt.HipError):
+        hiprt.Runtime(0)
+    from neon_amd.backends import gen_backend
+    with pytest.raises(hiprt.HipError):
+        gen_backend("hip")          # no silent CPU fallback
+
+
+def test_rtc_compile_and_error_log():
+    code, _ = hiprt.rtc_compile('extern "C" __global__ void k(float* a){ a[threadIdx.x] *= 2.f; }', "k.hip", "gfx950")
+    assert code[:4] == b"\x7fELF"
+    with pytest.raises(hiprt.HipError) as e:
+        hiprt.rtc_compile('extern "C" __global__ void k(float* a){ a[0] = undefined_symbol; }', "bad.hip", "gfx950")
+    assert "undefined_symbol" in str(e.value) and e.value.code >= hiprt.NH_RTC_ERROR_BASE
+
+
+# ---- DAG --------------------------------------------------------------------------------
+def _prog(pb, issue):
+    got = []
+    pb_exec, pb.execute = pb.execute, lambda t: got.append(t) or t[1]
+    try:
+        issue()
+    finally:
+        pb.execute = pb_exec
+    p = Program()
+    for t in got:
+        p.add_statement(t)
+    return p.finalize()
+
+
+def test_cse_and_levels(pb):
+    x, out = pb.empty((1000, 128)), pb.empty((1000, 128))
+    p = _prog(pb, lambda: out.__setitem__(slice(None), pb.exp(x - pb.max(x, axis=0)) /
+                                          pb.sum(pb.exp(x - pb.max(x, axis=0)), axis=0)))
+    ops = [n.op for n in p.nodes if n.kind in ("E", "R")]
+    assert ops.count("max") == 1 and ops.count("exp") == 1 and ops.count("sub") == 1   # duplicates merged
+    assert p.axis == 0 and p.nlevels == 2 and p.domain == (1000, 128)
+    assert len(p.tensors) == 2 and p.tensors[0].written and p.tensors[1].read
+
+
+def test_constant_folding_and_key(pb):
+    x, out = pb.empty((8, 8)), pb.empty((8, 8))
+
+    def adam_like(t):
+        l = 1e-3 * pb.sqrt(1 - 0.999 ** t) / (1 - 0.9 ** t)
+        out[:] = x - l * x
+
+    p1, p2 = _prog(pb, lambda: adam_like(1)), _prog(pb, lambda: adam_like(7))
+    assert len(p1.consts) == 1 and np.isclose(p1.consts[0], 1e-3 * np.sqrt(1 - 0.999) / 0.1)
+    assert p1.key() == p2.key() and p1.consts != p2.consts          # same kernel, other argument
+    p3 = _prog(pb, lambda: out.__setitem__(slice(None), 0.5 * x + 0.5 * x))
+    p4 = _prog(pb, lambda: out.__setitem__(slice(None), 0.5 * x + 2.0 * x))
+    assert len(p3.consts) == 1 and len(p4.consts) == 2 and p3.key() != p4.key()
+
+
+def test_identity_reduction_of_broadcast_operand(pb):
+    row, out = pb.empty((1, 16)), pb.empty((1, 16))
+    p = _prog(pb, lambda: out.__setitem__(slice(None), pb.sum(row, axis=0) + pb.argmax(row, axis=0)))
+    assert p.axis is None and not any(n.kind == "R" for n in p.nodes)
+
+
+def test_errors_raised_before_any_launch(pb):
+    a, b = pb.empty((4, 3)), pb.empty((5, 3))
+    with pytest.raises(TypeError):
+        _prog(pb, lambda: a.__setitem__(slice(None), a + b))                  # shapes do not broadcast
+    with pytest.raises(ValueError):
+        _prog(pb, lambda: a.__setitem__(slice(None), OpTreeNode({"op": "sum", "shape": (4, 1), "axis": 2}, a, None)))
+    with pytest.raises(MixedAxes):
+        _prog(pb, lambda: pb.empty((1, 1)).__setitem__(slice(None), pb.sum(pb.sum(a, axis=0), axis=1)))
+    with pytest.raises(TypeError):
+        _prog(pb, lambda: pb.empty((1, 3)).__setitem__(slice(None), a * 2.0))  # result larger than target
+    with pytest.raises(TypeError):
+        a[:] = "text"
+
+
+def test_fusion_forwards_written_values(pb):
+    g, m, p_ = pb.empty((64, 64)), pb.empty((64, 64)), pb.empty((64, 64))
+
+    def stmts():
+        m[:] = m * 0.9 + 0.1 * g
+        p_[:] = p_ - m
+
+    prog = _prog(pb, stmts)
+    assert len(prog.statements) == 2
+    # the second statement reads the value written by the first, not memory
+    sub = prog.statements[1].root
+    assert sub.op == "sub" and sub.args[1] is prog.statements[0].root
+    reads = [t.index for t in prog.tensors if t.read]
+    assert len(reads) == 3                      # g, old m, old p
+
+
+# ---- shape classes --------------------------------------------------------------------
+def test_shape_class_selection(pb):
+    f32, f16 = np.float32, np.float16
+    x, y, o = pb.empty((4096, 128)), pb.empty((4096, 128)), pb.empty((4096, 128))
+    ch = plan_of(pb, lambda: o.__setitem__(slice(None), 0.5 * x + 2.0 * y))
+    assert ch.spec.family == "ew" and ch.spec.params["V"] == 4 and ch.grid[0] == 512
+    col, row = pb.empty((4096, 1)), pb.empty((1, 128))
+    ch = plan_of(pb, lambda: o.__setitem__(slice(None), x * col + row))
+    assert ch.spec.family == "ew" and ch.spec.params["LY"] > 1            # 2-d tiling for broadcasts
+    xs = pb.empty((1000, 128))
+    ch = plan_of(pb, lambda: pb.empty((1000, 128)).__setitem__(slice(None), pb.fprop_softmax(xs, 0)))
+    assert ch.spec.family == "col" and ch.spec.params["NR"] * ch.spec.params["LY"] >= 1000
+    x4, o4 = pb.empty((256, 100352), f16), pb.empty((256, 100352), f16)
+    ch = plan_of(pb, lambda: o4.__setitem__(slice(None), (x4 - pb.mean(x4, axis=1)) / pb.sqrt(pb.var(x4, axis=1) + 1e-5)))
+    assert ch.spec.family == "row" and ch.spec.params["V"] == 8 and ch.spec.params["NCH"] == 13
+    assert ch.spec.params["stream"] and ch.grid == (256, 1, 1)
+    x5 = pb.empty((32000, 256))
+    ch = plan_of(pb, lambda: pb.empty((1, 256), np.int32).__setitem__(slice(None), pb.argmax(x5, axis=0)))
+    assert ch.spec.family == "colsplit" and ch.workspace is not None
+    assert ch.grid[0] * ch.grid[1] <= 2 * 256 and ch.grid[1] <= codegen.COLSPLIT_MAX_CHUNKS
+    with pytest.raises(planner.NeedsSplit):        # three sweeps over 32000 rows do not fit one workgroup
+        pb.empty((32000, 256)).__setitem__(slice(None), pb.fprop_softmax(x5, 0))
+    odd = pb.empty((64, 327))
+    ch = plan_of(pb, lambda: pb.empty((64, 1)).__setitem__(slice(None), pb.sum(odd, axis=1)))
+    assert ch.spec.family == "row" and ch.spec.params["V"] == 1           # 327 columns: no vector access
+    xt = pb.empty((128, 4096)).T
+    ch = plan_of(pb, lambda: o.__setitem__(slice(None), xt + 1.0))
+    assert ch.spec.params["V"] == 1                                          # strided operand
+
+
+def test_adam_fuses_into_one_streaming_kernel(pb):
+    from neon_amd import configs
+    p, g, m, v = (pb.empty(configs.C3_SHAPE) for _ in range(4))
+    n = len(pb.choices)
+    pb.begin(Block.update, 0)
+    configs.c3_adam_step(pb, p, g, m, v, 3)
+    pb.end(Block.update, 0)
+    assert len(pb.choices) == n + 1
+    spec = pb.choices[-1].spec
+    assert spec.family == "ew" and spec.params["stream"] and spec.params["V"] == 4
+    assert spec.source.count(".load_stream(") == 4 and spec.source.count(".store_stream(") == 3
+
+
+# ---- compile + cache --------------------------------------------------------------------
+def test_benchmark_kernels_compile_for_gfx950_and_cache(tmp_path):
+    be = prebuild.PlanBackend(cache_dir=str(tmp_path / "kc"))
+    prebuild.benchmark_statements(be)
+    assert be.cache.stats["compiled"] >= 8 and be.cache.stats["hit_disk"] == 0
+    files = os.listdir(str(tmp_path / "kc"))
+    assert len(files) == be.cache.stats["compiled"] and all(f.endswith(".hsaco") for f in files)
+    be2 = prebuild.PlanBackend(cache_dir=str(tmp_path / "kc"))
+    prebuild.benchmark_statements(be2)
+    assert be2.cache.stats["compiled"] == 0 and be2.cache.stats["hit_disk"] >= 8
+    names = [c.spec.name for c in be.choices]
+    assert names == [c.spec.name for c in be2.choices]       # generation is deterministic
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.int32, np.uint8, np.int16])
+@pytest.mark.parametrize("axis", [0, 1])
+def test_generated_kernels_compile_for_every_dtype(tmp_path, dtype, axis):
+    be = prebuild.PlanBackend(cache_dir=str(tmp_path / "kc"))
+    x = be.empty((96, 160), dtype)
+    be.empty((96, 160), dtype)[:] = x * 2.0 + x
+    shape = (1, 160) if axis == 0 else (96, 1)
+    be.empty(shape)[:] = be.max(x, axis=axis) - be.min(x, axis=axis)
+    be.empty(shape, np.int32)[:] = be.argmin(x, axis=axis)
+    be.empty((96, 160), dtype)[:] = x - be.mean(x, axis=axis)
+    assert be.cache.stats["compiled"] == 4
