@@ -227,6 +227,48 @@ def cpu_leg(max_seconds=25.0):
             "host_cpu": model, "host_cpu_count": os.cpu_count()}
 
 
+def counter_pass():
+    """A short, untimed run for hardware-counter collection
+    (``rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --counter-pass``, then the
+    same with WRITE_SIZE): three launches each of a plain copy kernel of known
+    size (the calibration: 100 MB read, 100 MB written) and of the main
+    benchmark kernels."""
+    from neon_amd import configs
+    from neon_amd.backends import gen_backend
+    from neon_amd.backends.backend import Block
+    be = gen_backend("hip", rng_seed=0)
+    be.bsz = 1
+    rs = np.random.RandomState(3)
+    g = _fresh(be, configs.C3_SHAPE, rs=rs, scale=1e-2)
+    p = _fresh(be, configs.C3_SHAPE, rs=rs, scale=0.05)
+    m, v = be.zeros(configs.C3_SHAPE), be.zeros(configs.C3_SHAPE)
+    x4 = _fresh(be, configs.C4_SHAPE, dtype=np.float16, rs=rs, scale=2.0, shift=0.5)
+    o4 = be.empty(configs.C4_SHAPE, dtype=np.float16)
+    g4, b4 = be.ones((configs.C4_SHAPE[0], 1)), be.zeros((configs.C4_SHAPE[0], 1))
+    x5 = _fresh(be, configs.C5_SHAPE, rs=rs, scale=4.0)
+    am = be.empty((1, configs.C5_SHAPE[1]), dtype=np.int32)
+    mx = be.empty((1, configs.C5_SHAPE[1]))
+    be.synchronize()
+    for t in range(1, 4):
+        m[:] = g * 1.0                     # copy kernel: 100 MB in, 100 MB out
+        be.synchronize()
+    v[:] = 0
+    m[:] = 0
+    for t in range(1, 4):
+        be.begin(Block.update, t)
+        configs.c3_adam_step(be, p, g, m, v, t)
+        be.end(Block.update, t)
+        be.synchronize()
+    for _ in range(3):
+        configs.c4_rownorm(be, o4, x4, g4, b4)
+        be.synchronize()
+    for _ in range(3):
+        configs.c5a_argmax(be, am, x5)
+        configs.c5b_max(be, mx, x5)
+        be.synchronize()
+    print(json.dumps({"counter_pass": "done"}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -234,7 +276,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle leg")
     ap.add_argument("--no-detail", action="store_true", help="headline only, no per-config table")
+    ap.add_argument("--counter-pass", action="store_true",
+                    help="short untimed run for rocprofv3 --pmc (see counter_pass)")
     args = ap.parse_args()
+    if args.counter_pass:
+        counter_pass()
+        return
     if args.gpus != 1:
         print("bench.py measures one MI355X; --gpus %d is not supported (the op-tree path has no "
               "cross-device stage; see DESIGN.md on sharding)" % args.gpus, file=sys.stderr)
