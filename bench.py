@@ -30,6 +30,12 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the fused Adam kernel from rocprofv3 counters
+# (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a
+# plain copy kernel of known size); summary and commands under
+# profiles/hbm_traffic_adam_rownorm_colreduce_pmc.txt.  Counters cannot be read
+# from inside this process, so the figure is carried here.
+ADAM_FUSED_TRAFFIC_BYTES = 699.7e6
 
 
 def _fresh(be, shape, dtype=np.float32, fill=None, rs=None, scale=1.0, shift=0.0):
@@ -91,7 +97,7 @@ def gpu_leg(steps, warmup, detail=True):
     ms, plan = be.time_group(groups[0], reps=max(steps, 5))
     out["roofline"] = {"bound": "hbm", "achieved": step_bytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
                        "unit": "GB/s", "frac": step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                       "traffic": None, "kernel": plan.spec.name, "kernel_ms": ms,
+                       "traffic": ADAM_FUSED_TRAFFIC_BYTES, "kernel": plan.spec.name, "kernel_ms": ms,
                        "algorithmic_bytes": step_bytes}
     if not detail:
         return out, be
