@@ -116,6 +116,28 @@ def _fold_binary(op, a, b):
     raise TypeError("unknown binary op %s" % op)
 
 
+class Num(object):
+    """A number on the build stack: its value and how it derives from the raw
+    numbers of the trees (``('r', i)`` = i-th number in postfix order,
+    ``('1', op, e)`` / ``('2', op, a, b)`` = folded on the host), so that a
+    recorded launch can be re-bound to new constants without rebuilding."""
+    __slots__ = ("value", "expr")
+
+    def __init__(self, value, expr):
+        self.value = value
+        self.expr = expr
+
+
+def eval_const(expr, raw):
+    """value of a constant-slot expression for the raw numbers ``raw``"""
+    tag = expr[0]
+    if tag == "r":
+        return raw[expr[1]]
+    if tag == "1":
+        return _fold_unary(expr[1], eval_const(expr[2], raw))
+    return _fold_binary(expr[1], eval_const(expr[2], raw), eval_const(expr[3], raw))
+
+
 class MixedAxes(ValueError):
     """Reductions along both axes in one tree: needs more than one kernel."""
 
@@ -199,6 +221,8 @@ class Program(object):
         self._const_slot = {}
         self._current = {}         # tensor slot index -> node holding its newest value
         self.key_parts = []
+        self.raw_count = 0         # numbers seen so far, in postfix order
+        self.const_exprs = []      # per constant slot: expressions that produced its value
         self.axis = None           # the one reduction axis, if any
         self.domain = None
         self.nlevels = 0
@@ -222,15 +246,17 @@ class Program(object):
         self._tensor_by_id[id(t)] = slot
         return slot
 
-    def const_node(self, value):
-        value = float(value)
+    def const_node(self, num):
+        value = float(num.value)
         # every occurrence of an equal number shares a slot; the *value* is a
         # run-time argument, so the key records only the slot pattern
         slot = self._const_slot.get(value)
         if slot is None:
             slot = len(self.consts)
             self.consts.append(value)
+            self.const_exprs.append([])
             self._const_slot[value] = slot
+        self.const_exprs[slot].append(num.expr)
         self.key_parts.append(("C", slot))
         return self._intern(("C", slot), lambda: Node("C", slot=slot))
 
@@ -265,7 +291,8 @@ class Program(object):
             elif isinstance(p, Tensor):
                 stack.append(self._read_tensor(p))
             elif isinstance(p, (int, float)):
-                stack.append(float(p))          # folded lazily
+                stack.append(Num(float(p), ("r", self.raw_count)))      # folded lazily
+                self.raw_count += 1
             else:
                 raise TypeError("args must be instance of Tensor, int, float, or dict (for operators)")
         if len(stack) != 1:
@@ -303,7 +330,7 @@ class Program(object):
             x = stack.pop()
             if not isinstance(x, Node):
                 self.key_parts.append(("fold1", op))
-                stack.append(_fold_unary(op, x))
+                stack.append(Num(_fold_unary(op, x.value), ("1", op, x.expr)))
                 return
             self.key_parts.append(op)
             stack.append(self._intern(("E", op, x.nid), lambda: Node("E", op=op, args=(x,))))
@@ -312,7 +339,7 @@ class Program(object):
             a = stack.pop()
             if not isinstance(a, Node) and not isinstance(b, Node):
                 self.key_parts.append(("fold2", op))
-                stack.append(_fold_binary(op, a, b))
+                stack.append(Num(_fold_binary(op, a.value, b.value), ("2", op, a.expr, b.expr)))
                 return
             self.key_parts.append(op)
             a, b = self._as_node(a), self._as_node(b)

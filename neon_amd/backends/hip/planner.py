@@ -236,8 +236,18 @@ class Plan(object):
                     vals[i] = float(np.float32(vals[i]))
         return vals
 
+    def pack(self, prog):
+        """argument buffer for ``prog`` (any program with this plan's key)"""
+        return self.kernel.packer.pack(*self._values(prog))
+
+    def const_offsets(self, prog):
+        """byte offset of every constant slot inside the packed arguments"""
+        import struct
+        head = "@" + "Pqq" * len(prog.tensors)
+        return [struct.calcsize(head + "f" * (k + 1)) - 4 for k in range(len(prog.consts))]
+
     def launch(self, prog):
-        self.rt.launch(self.kernel, self.grid, self.block, 0, *self._values(prog))
+        self.rt.launch_packed(self.kernel, self.grid, self.block, self.pack(prog))
 
     def launch_timed(self, prog, reps):
         """mean ms per launch of ``reps`` back-to-back launches (bench mode)"""
@@ -355,20 +365,32 @@ def _plan_col(prog, cu_count):
     words = _words_per_tile(prog, V, 0)
     line_only = all(st.out.shape[0] == 1 and R > 1 for st in prog.statements)
 
-    # (a) whole column strip inside one workgroup, rows resident in registers
-    lx_min = max(1, min(64, 64 // (V * isz)))
-    LX = max(lx_min, min(64, _pow2floor(max(1, nvec // 32))))
-    LX = min(LX, _pow2ceil(nvec))
+    # (a) whole column strip inside one workgroup, rows resident in registers.
+    # Wider strips coalesce better (>= 128 B per row segment wanted), narrower
+    # ones leave more row-lanes, i.e. fewer rows per lane: take the widest
+    # strip for which all rows fit in registers.
+    lx_min = max(1, min(64, 128 // (V * isz)))
+    if R * C * isz <= (4 << 20):
+        lx_min = 1                       # tiny inputs are latency-bound: favour more workgroups
+    lx_pref = max(lx_min, min(64, _pow2floor(max(1, nvec // 32))))
+    lx_pref = min(lx_pref, _pow2ceil(nvec))
+    lx_min = min(lx_min, lx_pref)
     fit = None
-    strips = _ceil_div(nvec, LX)
-    # few strips: spend more lanes on each so the rows-per-lane count drops
-    for T in ((256, 512, 1024) if strips >= cu_count else (1024, 512, 256)):
-        LY = T // LX
-        NR = _ceil_div(R, LY)
-        budget = 64 if T == 1024 else 128
-        if NR <= 16 and NR * words <= budget:
-            fit = (T, LY, NR)
-            break
+    LX = lx_pref
+    while fit is None and LX >= lx_min:
+        strips = _ceil_div(nvec, LX)
+        # few strips: spend more lanes on each so the rows-per-lane count drops
+        for T in ((256, 512, 1024) if strips >= cu_count else (1024, 512, 256)):
+            LY = T // LX
+            NR = _ceil_div(R, LY)
+            budget = 64 if T == 1024 else 128
+            if NR <= 16 and NR * words <= budget:
+                fit = (T, LY, NR)
+                break
+        if fit is None:
+            LX //= 2
+    if fit is None:
+        LX = lx_pref
     single_level = prog.nlevels == 1
     big = R * C >= (1 << 18)
     if fit and not (single_level and line_only and big and R >= 512):

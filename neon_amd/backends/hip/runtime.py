@@ -229,6 +229,15 @@ class Runtime(object):
         _check(self.lib.nh_launch(kernel.function, g, b, lds_bytes, self.stream,
                                   args, kernel.arg_bytes))
 
+    def launch_packed(self, kernel, grid, block, args):
+        """launch with an already packed argument buffer"""
+        g, b = self._grid, self._block
+        g[0], g[1], g[2] = grid
+        b[0], b[1], b[2] = block
+        rc = self.lib.nh_launch(kernel.function, g, b, 0, self.stream, args, kernel.arg_bytes)
+        if rc:
+            _check(rc)
+
     def launch_timed(self, kernel, grid, block, lds_bytes, reps, *values):
         """mean milliseconds per launch over ``reps`` back-to-back launches"""
         g, b = self._grid, self._block

@@ -19,7 +19,7 @@ import numpy as np
 
 from neon_amd.backends.backend import Backend, OpTreeNode, Tensor
 from neon_amd.backends.hip import runtime as hiprt
-from neon_amd.backends.hip.optree_ir import MixedAxes, Program, REDUCE
+from neon_amd.backends.hip.optree_ir import MixedAxes, Program, REDUCE, eval_const
 from neon_amd.backends.hip.planner import KernelCache, NeedsSplit, make_plan
 
 logger = logging.getLogger(__name__)
@@ -99,6 +99,8 @@ class HIPTensor(Tensor):
             self.gpudata = int(gpudata)
         self.is_contiguous = (not take_array and
                               self.strides == _contiguous_strides(self.shape))
+        # identity for the launch cache: same memory + same layout = same kernel arguments
+        self._geom = (self.gpudata, self.shape, self.strides, dtype.char, id(take_array) if take_array else 0)
 
     def __del__(self):
         if getattr(self, "_owns", False) and self.gpudata:
@@ -365,6 +367,41 @@ class _FuseScope(object):
         return False
 
 
+class _Recorded(object):
+    """Launches recorded for one statement group."""
+    __slots__ = ("launches", "temps", "raw", "patch")
+
+    def __init__(self, launches, temps, raw, patch):
+        self.launches = launches
+        self.temps = temps           # temporaries the recorded arguments point into
+        self.raw = raw               # the numbers of the trees when recorded
+        self.patch = patch           # (byte offsets, slot expressions) or None
+
+    def rebind(self, raw):
+        """the launches for the numbers ``raw``; None when they cannot be
+        derived from the recording"""
+        if raw == self.raw:
+            return self.launches
+        if self.patch is None or len(raw) != len(self.raw):
+            return None
+        offsets, exprs = self.patch
+        kernel, grid, block, args = self.launches[0]
+        buf = bytearray(args)
+        for off, slot_exprs in zip(offsets, exprs):
+            value = eval_const(slot_exprs[0], raw)
+            for e in slot_exprs[1:]:
+                if eval_const(e, raw) != value:
+                    return None      # numbers that shared a slot no longer agree
+            try:
+                struct.pack_into("f", buf, off, value)
+            except OverflowError:
+                with np.errstate(over="ignore"):
+                    struct.pack_into("f", buf, off, float(np.float32(value)))
+        self.launches = [(kernel, grid, block, bytes(buf))]
+        self.raw = list(raw)
+        return self.launches
+
+
 class _CaptureScope(object):
     def __init__(self, be):
         self.be = be
@@ -413,11 +450,15 @@ class NervanaHIP(Backend):
         self.cu_count = int(self.rt.props.compute_units)
         self.kernels = KernelCache(self.rt.arch.split(":")[0], cache_dir)
         self.plans = {}
-        self.plan_stats = {"hit": 0, "miss": 0, "split": 0, "launches": 0}
+        self.plan_stats = {"hit": 0, "miss": 0, "split": 0, "launches": 0, "replayed": 0}
         self._pending = []
         self._fusing = False
         self._fuse_depth = 0
         self._captured = None
+        self._launch_cache = {}      # statement-group identity -> recorded launches
+        self._recording = None
+        self._rec_temps = None
+        self._rec_single = None
         self._temp_pool = {}
         self._live_allocs = 0
 
@@ -441,6 +482,7 @@ class NervanaHIP(Backend):
                 for p in (plan if isinstance(plan, list) else [plan]):
                     p.release()
             self.plans = {}
+            self._launch_cache = {}
             self._temp_pool = {}
         except Exception:
             pass
@@ -569,7 +611,86 @@ class NervanaHIP(Backend):
             self._run([optree])
         return optree[1]
 
+    def _launch_key(self, trees):
+        """Cheap identity of a statement group: ops and the memory layout of
+        every tensor in postfix order, plus the numbers on the side.  Equal
+        keys and equal numbers mean the very same launches with the very same
+        arguments."""
+        parts, raw = [], []
+        add = parts.append
+        for tree in trees:
+            for p in tree.traverse([]):
+                if type(p) is dict:
+                    if "axis" in p:
+                        if p["op"] == "onehot":
+                            add(("onehot", p["axis"], p["idx"]._geom))
+                        else:
+                            add((p["op"], p["axis"]))
+                    else:
+                        add(p["op"])
+                elif isinstance(p, HIPTensor):
+                    add(p._geom)
+                else:
+                    add(None)
+                    raw.append(float(p))
+            add("|")
+        return tuple(parts), raw
+
     def _run(self, trees):
+        """Launch a statement group.  The first time, the slow path builds the
+        DAG, picks or compiles kernels and records every launch it makes
+        (packed arguments included); afterwards an identical group -- same
+        tree, same tensors -- replays the recorded launches, re-binding the
+        constant arguments when only numbers changed (Adam's step-dependent
+        learning rate).  The reference re-derived everything on every call
+        (its own TODO at float_ew.py:640-641 asks for exactly this)."""
+        try:
+            key, raw = self._launch_key(trees)
+        except (AttributeError, TypeError):
+            key, raw = None, None
+        entry = self._launch_cache.get(key) if key is not None else None
+        if entry is not None:
+            launches = entry.rebind(raw)
+            if launches is not None:
+                launch = self.rt.launch_packed
+                for kernel, grid, block, args in launches:
+                    launch(kernel, grid, block, args)
+                if self._recording is not None:
+                    self._recording.extend(launches)
+                    self._rec_temps.extend(entry.temps)
+                    self._rec_single = None
+                self.plan_stats["replayed"] += 1
+                self.plan_stats["launches"] += len(launches)
+                return
+        outer = self._recording is None
+        if outer:
+            self._recording, self._rec_temps, self._rec_single = [], [], None
+        ok = False
+        try:
+            self._run_slow(trees)
+            ok = True
+        finally:
+            if outer:
+                rec, temps, single = self._recording, self._rec_temps, self._rec_single
+                self._recording, self._rec_temps, self._rec_single = None, None, None
+                if ok and key is not None:
+                    if len(self._launch_cache) >= 8192:
+                        self._launch_cache.clear()
+                    if len(rec) != 1:
+                        single = None
+                    self._launch_cache[key] = _Recorded(rec, temps, raw, single)
+
+    def _launch_plan(self, plan, prog):
+        args = plan.pack(prog)
+        self.rt.launch_packed(plan.kernel, plan.grid, plan.block, args)
+        if self._recording is not None:
+            self._recording.append((plan.kernel, plan.grid, plan.block, args))
+            # a group that is exactly one launch of one program can be re-bound
+            # to new constants: remember where they sit and how they derive
+            self._rec_single = (plan.const_offsets(prog), prog.const_exprs) if not self._recording[:-1] else None
+        self.plan_stats["launches"] += 1
+
+    def _run_slow(self, trees):
         try:
             prog = Program()
             for t in trees:
@@ -583,8 +704,7 @@ class NervanaHIP(Backend):
                 self.plans[key] = plan
             else:
                 self.plan_stats["hit"] += 1
-            plan.launch(prog)
-            self.plan_stats["launches"] += 1
+            self._launch_plan(plan, prog)
         except (NeedsSplit, MixedAxes, NotImplementedError) as e:
             if len(trees) != 1:
                 for t in trees:
@@ -677,14 +797,15 @@ class NervanaHIP(Backend):
             self.plans[key] = plan
         else:
             self.plan_stats["hit"] += 1
-        plan.launch(prog)
-        self.plan_stats["launches"] += 1
+        self._launch_plan(plan, prog)
 
     def _temp(self, shape, dtype, temps):
         key = (tuple(shape), np.dtype(dtype))
         pool = self._temp_pool.setdefault(key, [])
         t = pool.pop() if pool else HIPTensor(self, shape, dtype=dtype)
         temps.append(t)
+        if self._rec_temps is not None:
+            self._rec_temps.append(t)      # recorded launches point into it: keep it allocated
         return t
 
     def _temp_release(self, t):
