@@ -621,13 +621,26 @@ def _col_lds(L, LX, LY, T, V, any_index):
     return WY * (LX * V + 1) * (4 + (8 if any_index else 0))
 
 
-def gen_col(prog, V, LX, LY, NR, stream=False):
-    """Axis-0 reductions with all rows of a column strip inside one workgroup
-    (LX column-lanes x LY row-lanes, NR rows per lane, kept in registers)."""
+def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1):
+    """Axis-0 reductions with the rows resident in registers (LX column-lanes x
+    LY row-lanes per workgroup, NR rows per lane).
+
+    ``chunks`` == 1: one workgroup owns a column strip and all its rows.
+
+    ``chunks`` > 1 (family ``colcoop``): the rows of a strip are spread over
+    ``chunks`` workgroups that are all resident at once (the planner keeps the
+    grid within one workgroup per compute unit).  After every sweep they
+    exchange their partial results through device-coherent memory: publish,
+    count arrivals on a per-strip counter, wait (bounded) for the others,
+    gather and fold.  The matrix is still read from HBM exactly once however
+    many sweeps the tree needs.  Extra parameters: workspace pointer and the
+    byte offset of the counters (two per strip: arrivals, departures; zero
+    before the first launch, reset by the last workgroup to leave)."""
+    coop = chunks > 1
     g = _RedGen(prog, V, stream)
     L = g.L
     T = LX * LY
-    params, fmt = g.param_list([])
+    params, fmt = g.param_list([("char* ws", "P"), ("long long ctr_offset", "q")] if coop else [])
     head = ('extern "C" __global__ __launch_bounds__(%d) void @NAME@(%s)\n' % (T, params))
     per_level = _levels(prog)
     nsweeps = prog.nlevels
@@ -637,17 +650,92 @@ def gen_col(prog, V, LX, LY, NR, stream=False):
     done, cached = {}, {}
 
     L.open("")
-    lds = _col_lds(L, LX, LY, T, V, any_index)
+    lds = _col_lds(L, LX, LY, T, V, any_index or coop)
     L("const int tx = threadIdx.x %% %d, ty = threadIdx.x / %d;" % (LX, LX))
     L("const long long c = ((long long)blockIdx.x * %d + tx) * %d;" % (LX, V))
     L("const bool col_ok = c < C;")
     L("const long long cc = col_ok ? c : 0;")
+    if coop:
+        L("__shared__ int s_abort;")
+        L("unsigned int* ctr = reinterpret_cast<unsigned int*>(ws + ctr_offset) + 2 * blockIdx.x;")
+    all_reds = [n for lv in sorted(per_level) for n in per_level[lv]]
+    red_slot = dict((n.nid, k) for k, n in enumerate(all_reds))
+    exchanges = [0]
 
     def row_loop_open():
         L("#pragma unroll")
         L.open("for (int i = 0; i < %d; ++i)" % NR)
-        L("const long long r = (long long)i * %d + ty;" % LY)
+        if coop:
+            L("const long long r = ((long long)blockIdx.y * %d + i) * %d + ty;" % (NR, LY))
+        else:
+            L("const long long r = (long long)i * %d + ty;" % LY)
         L("const bool ok = col_ok && (r < R);")
+
+    def exchange(reds):
+        """fold the workgroups of a strip: afterwards acc/rv/ri hold the
+        result over all rows in every lane of every workgroup"""
+        exchanges[0] += 1
+        QMAX = -(-chunks // LY)
+        for n in reds:
+            L("nh_pair* part%d = reinterpret_cast<nh_pair*>(ws) + (long long)%d * C;"
+              % (n.nid, red_slot[n.nid] * chunks))
+        L.open("if (col_ok && ty == 0)")
+        L("#pragma unroll")
+        L.open("for (int j = 0; j < %d; ++j)" % V)
+        for n in reds:
+            if n.is_index:
+                L("nh_part_store(&part%d[(long long)blockIdx.y * C + c + j], acc%d[j]);" % (n.nid, n.nid))
+            else:
+                L("nh_part_store(&part%d[(long long)blockIdx.y * C + c + j], nh_pair{rv%d[j], 0});" % (n.nid, n.nid))
+        L.close()
+        L.close()
+        L("__syncthreads();     // every lane's partial stores have completed")
+        L.open("if (threadIdx.x == 0)")
+        L("__hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
+        L("unsigned int spins = 0; int bad = 0;")
+        L.open("while (__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < %du)" % (chunks * exchanges[0]))
+        L("__builtin_amdgcn_s_sleep(4);")
+        L("if (++spins > NH_SPIN_LIMIT) { bad = 1; break; }")
+        L.close()
+        L("s_abort = bad;")
+        L.close()
+        L("__syncthreads();")
+        L.open("if (s_abort)")
+        L("if (threadIdx.x == 0) __hip_atomic_store(ctr + 1, 0xDEADu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
+        L("return;              // the other workgroups never showed up: give up rather than hang")
+        L.close()
+        for n in reds:
+            L("nh_pair q%d[%d][%d];" % (n.nid, QMAX, V))
+        L("#pragma unroll")
+        L.open("for (int k = 0; k < %d; ++k)" % QMAX)
+        L("const int q = ty + k * %d;" % LY)
+        L("const bool live = col_ok && (q < %d);" % chunks)
+        L("#pragma unroll")
+        L.open("for (int j = 0; j < %d; ++j)" % V)
+        for n in reds:
+            op = _RED_OP[n.op]
+            init = ("%s::init()" % op) if n.is_index else ("nh_pair{%s::init(), 0}" % op)
+            L("q%d[k][j] = live ? nh_part_load(&part%d[(long long)q * C + c + j]) : %s;" % (n.nid, n.nid, init))
+        L.close()
+        L.close()
+        for n in reds:
+            op = _RED_OP[n.op]
+            L("#pragma unroll")
+            L("for (int j = 0; j < %d; ++j) acc%d[j] = %s::init();" % (V, n.nid, op))
+        L("#pragma unroll")
+        L.open("for (int k = 0; k < %d; ++k)" % QMAX)
+        L("#pragma unroll")
+        L.open("for (int j = 0; j < %d; ++j)" % V)
+        for n in reds:
+            op = _RED_OP[n.op]
+            if n.is_index:
+                L("acc%d[j] = %s::f(acc%d[j], q%d[k][j]);" % (n.nid, op, n.nid, n.nid))
+            else:
+                L("acc%d[j] = %s::f(acc%d[j], q%d[k][j].v);" % (n.nid, op, n.nid, n.nid))
+        L.close()
+        L.close()
+        for n in reds:
+            _emit_col_fold(g, L, n, LX, LY, T, V, "acc%d" % n.nid, dst_decl=False)
 
     def keep_all():
         for nid, name in cached.items():
@@ -714,12 +802,14 @@ def gen_col(prog, V, LX, LY, NR, stream=False):
         for n in reds:
             _emit_col_fold(g, L, n, LX, LY, T, V, "acc%d" % n.nid)
             done[n.nid] = n
+        if coop:
+            exchange(reds)
 
     if line_out:
         roots = [st.root for st in line_out]
         nodes = _needed(roots, done)
         leaves = g.leaf_nodes(nodes)
-        L.open("if (col_ok && ty == 0)")
+        L.open("if (col_ok && ty == 0%s)" % (" && blockIdx.y == 0" if coop else ""))
         for n in leaves:
             g.emit_load(n, "0", "c", V, "_l")
         for st in line_out:
@@ -764,8 +854,20 @@ def gen_col(prog, V, LX, LY, NR, stream=False):
             L("o%d.%s(%s);" % (st.out.index, g.st, g.addr(st.out, "r", "c")))
         L.close()
         L.close()
+    if coop:
+        # the last workgroup of the strip to get here has seen everyone pass
+        # the final wait: it re-arms both counters for the next launch
+        L.open("if (threadIdx.x == 0)")
+        L("const unsigned int t = __hip_atomic_fetch_add(ctr + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
+        L.open("if (t == %du)" % (chunks - 1))
+        L("__hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
+        L("__hip_atomic_store(ctr + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
+        L.close()
+        L.close()
     L.close()
-    return _finish("col", g, head, fmt, T, lds, dict(V=V, LX=LX, LY=LY, NR=NR, stream=bool(stream)))
+    return _finish("colcoop" if coop else "col", g, head, fmt, T, lds,
+                   dict(V=V, LX=LX, LY=LY, NR=NR, stream=bool(stream), chunks=chunks,
+                        NRED=len(all_reds)))
 
 
 COLSPLIT_MAX_CHUNKS = 128

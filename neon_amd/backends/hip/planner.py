@@ -398,6 +398,29 @@ def _plan_col(prog, cu_count):
         spec = codegen.gen_col(prog, V, LX, LY, NR, _streams(prog))
         return Choice(spec, (_ceil_div(nvec, LX), 1, 1))
 
+    # (c) deeper trees (or full-shape results) over many rows: the workgroups of a
+    # strip keep their rows in registers and exchange partials between sweeps.
+    # Everything must be resident at once, so the grid stays within one
+    # workgroup per compute unit.
+    if not (single_level and line_only):
+        lxc = max(1, min(16, _pow2ceil(nvec)))
+        strips_c = _ceil_div(nvec, lxc)
+        if strips_c <= cu_count:
+            chunks = max(1, min(128, cu_count // strips_c))
+            rpc0 = _ceil_div(R, chunks)
+            for T, budget in ((1024, 72), (512, 200), (256, 448)):
+                LY = T // lxc
+                NR = _ceil_div(rpc0, LY)
+                if NR <= 64 and NR * words <= budget:
+                    chunks = _ceil_div(R, NR * LY)
+                    if chunks < 2:
+                        break
+                    spec = codegen.gen_col(prog, V, lxc, LY, NR, _streams(prog), chunks=chunks)
+                    part_bytes = spec.params["NRED"] * chunks * C * 8
+                    ctr_off = _ceil_div(part_bytes, 256) * 256
+                    return Choice(spec, (strips_c, chunks, 1),
+                                  workspace=(ctr_off + strips_c * 8, ctr_off, 2 * strips_c))
+
     # (b) one level, one value per column, many rows: split rows over workgroups
     if single_level and line_only:
         LX = max(lx_min, min(16, _pow2ceil(nvec)))

@@ -27,6 +27,10 @@ typedef unsigned short nh_u16;
 typedef int nh_i32;
 typedef unsigned int nh_u32;
 
+// Upper bound on the polls of a bounded wait for other workgroups (each poll
+// is a device-scope load plus a short sleep, roughly a microsecond).
+#define NH_SPIN_LIMIT (1u << 22)
+
 #define NH_INF __builtin_inff()
 #define NH_FLT_MAX 3.402823466e+38f
 

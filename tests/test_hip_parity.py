@@ -178,6 +178,39 @@ def test_compound_and_mixed_axes(pair):
     both(pair, lambda be, x, y: (x * y).T + 1.0, [a, b])
 
 
+@pytest.mark.parametrize("shape", [(32000, 256), (5000, 100), (20000, 1000), (9001, 36)])
+def test_tall_multilevel_axis0(pair, shape):
+    """deep axis-0 trees over more rows than one workgroup holds: the
+    workgroups of a column strip exchange partials between sweeps"""
+    rs = np.random.RandomState(shape[1])
+    a = (rs.standard_normal(shape) * 3).astype(np.float32)
+    cpu, hip = pair
+    # With tens of thousands of rows the oracle's own rounding is no longer
+    # below 1e-5: numpy adds the rows of an axis-0 sum one after the other in
+    # fp32, the device adds a tree.  So both are held against an fp64
+    # evaluation: the device to the 1e-5 bound, the oracle to what a
+    # sequential fp32 sum of that length can lose.
+    a64 = a.astype(np.float64)
+    e64 = np.exp(a64 - a64.max(axis=0))
+    truth = e64 / e64.sum(axis=0)
+    for _ in range(2):          # twice: the arrival counters must have re-armed themselves
+        got = call_func(lambda be, x: be.fprop_softmax(x, 0), hip, [a])
+        assert_close(got, truth, rtol=RTOL32, atol=1e-12, what="softmax vs fp64")
+    want = call_func(lambda be, x: be.fprop_softmax(x, 0), cpu, [a])
+    assert_close(want, truth, rtol=shape[0] * 1.2e-7, atol=1e-12, what="oracle softmax vs fp64")
+    assert np.allclose(got.astype(np.float64).sum(axis=0), 1.0, atol=1e-5)
+    truth = (a64 - a64.mean(axis=0)) / np.sqrt(a64.var(axis=0) + 1e-5)
+    f = lambda be, x: (x - be.mean(x, axis=0)) / be.sqrt(be.var(x, axis=0) + 1e-5)   # noqa: E731
+    assert_close(call_func(f, hip, [a]), truth, rtol=RTOL32, atol=1e-5, what="colnorm vs fp64")
+    assert_close(call_func(f, cpu, [a]), truth, rtol=shape[0] * 1.2e-7, atol=1e-4, what="oracle colnorm vs fp64")
+    # an index reduction feeding a later sweep
+    both(pair, lambda be, x: be.sum(be.equal(x, be.max(x, axis=0)) * be.argmax(x, axis=0), axis=0), [a],
+         what="index in tree")
+    if hip.plan_stats is not None and shape == (32000, 256):
+        fams = set(p.spec.family for p in hip.plans.values())
+        assert "colcoop" in fams
+
+
 def test_onehot(pair):
     rs = np.random.RandomState(8)
     idx = rs.randint(0, 40, (1, 64)).astype(np.int32)
