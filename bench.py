@@ -195,6 +195,40 @@ def gpu_leg(steps, warmup, detail=True):
     measure("C5b max axis0 (32000,256) f32", lambda: configs.c5b_max(be, mx, x5), configs.bytes_c5_reduce(), n5)
     measure("C5c cross-entropy axis0 (32000,256) f32, in-kernel one-hot",
             lambda: configs.c5c_cross_entropy(be, ce, x5, be.onehot(i5, axis=0)), configs.bytes_c5c(), n5)
+    # ---- the prebuilt hand-written kernels behind the direct C-ABI entry points ------------
+    lib = rt.lib
+    e0, e1 = rt.event(), rt.event()
+
+    def measure_abi(label, call, nbytes, elements, reps=30):
+        for _ in range(3):
+            call()
+        rt.synchronize()
+        rt.event_record(e0)
+        for _ in range(reps):
+            rc = call()
+        rt.event_record(e1)
+        rt.event_sync(e1)
+        assert rc == 0, lib.nh_last_error()
+        ms_k = rt.event_elapsed_ms(e0, e1) / reps
+        rows.append({"config": label, "bytes": nbytes, "kernels": 1, "ms": ms_k, "api_ms": ms_k,
+                     "timing": "HIP events around back-to-back C-ABI calls", "plan": "prebuilt (kernels.hip)",
+                     "gbs": nbytes / (ms_k * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ms_k * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "elements_per_s": elements / (ms_k * 1e-3)})
+
+    measure_abi("C3 prebuilt nh_adam_step_f32 (5000,5000) f32",
+                lambda: lib.nh_adam_step_f32(p.ptr, m.ptr, v.ptr, g.ptr, 1e-3, 0.9, 0.1, 0.999, 0.001, 1e-8, n3, None),
+                configs.bytes_c3(fused=True), n3)
+    measure_abi("C4 prebuilt nh_rownorm_f16 (256,100352) f16",
+                lambda: lib.nh_rownorm_f16(o4.ptr, x4.ptr, g4.ptr, b4.ptr, 1e-5, configs.C4_SHAPE[0],
+                                           configs.C4_SHAPE[1], configs.C4_SHAPE[1], None),
+                configs.bytes_c4(), configs.C4_SHAPE[0] * configs.C4_SHAPE[1])
+    ws = rt.malloc(lib.nh_colreduce_workspace_bytes(configs.C5_SHAPE[0], configs.C5_SHAPE[1]))
+    measure_abi("C5a+b prebuilt nh_colmax_argmax_f32 (32000,256) f32",
+                lambda: lib.nh_colmax_argmax_f32(mx.ptr, am.ptr, x5.ptr, configs.C5_SHAPE[0], configs.C5_SHAPE[1],
+                                                 configs.C5_SHAPE[1], ws, None),
+                configs.bytes_c5_reduce() + 4 * configs.C5_SHAPE[1], n5)
+    rt.synchronize()
+    rt.free(ws)
     out["per_config"] = rows
     return out, be
 

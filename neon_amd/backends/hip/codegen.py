@@ -328,6 +328,37 @@ def _live_reductions(prog):
     return [n for n in used_nodes(roots) if n.kind == "R"]
 
 
+_EXPENSIVE = {"exp", "log", "exp2", "log2", "tanh", "tanh2", "sig", "sig2", "pow", "sqrt",
+              "div", "safelog"}
+
+
+def _kept_values(prog, stages, limit):
+    """Elementwise results worth keeping in registers between sweeps: nodes
+    that two or more sweeps need and that cost a transcendental or a division
+    to recompute (softmax's exp(x - max)).  ``stages`` lists the targets of
+    each sweep in order; at most ``limit`` nodes are returned, outermost
+    first."""
+    reductions = set(n.nid for n in prog.nodes if n.kind == "R")
+    costly = {}
+    for n in prog.nodes:            # topological order
+        if n.kind == "E":
+            costly[n.nid] = (n.op in _EXPENSIVE) or any(costly.get(a.nid, False) for a in n.args)
+    kept = []
+    while len(kept) < limit:
+        avail = reductions | set(k.nid for k in kept)
+        count, by_id = {}, {}
+        for targets in stages:
+            for n in _needed(targets, avail):
+                if n.kind == "E" and n.vr and n.vc and costly.get(n.nid):
+                    count[n.nid] = count.get(n.nid, 0) + 1
+                    by_id[n.nid] = n
+        cands = [nid for nid, c in count.items() if c >= 2]
+        if not cands:
+            break
+        kept.append(by_id[max(cands)])
+    return kept
+
+
 class _RedGen(_Gen):
     """Common machinery of row / col / colsplit."""
 
@@ -341,8 +372,10 @@ class _RedGen(_Gen):
             return ("(float)ri%d[j]" % n.nid) if n.is_index else ("rv%d[j]" % n.nid)
         return ("(float)ri%d" % n.nid) if n.is_index else ("rv%d" % n.nid)
 
-    def make_ref(self, sfx, r, c, Vv, tiles=None):
+    def make_ref(self, sfx, r, c, Vv, tiles=None, vals=None):
         def ref(n):
+            if vals and n.nid in vals:
+                return vals[n.nid]
             if n.kind == "C":
                 return "k%d" % n.slot
             if n.kind in ("T", "H"):
@@ -410,42 +443,62 @@ def gen_row(prog, V, LX, LY, NCH, stream=False):
     if not resident:
         L("const int nch = (C + %d - 1) / %d;" % (LX * V, LX * V))
 
-    def chunk_loop_open():
+    SU = 4      # column tiles in flight per lane when the row is streamed
+
+    def chunk_position(k):
+        L("const long long c = ((long long)(%s) * %d + tx) * %d;" % (k, LX, V))
+        L("const bool ok = row_ok && (c < C);")
+
+    def sweep(leaves, emit_body):
+        """Loop over the lane's column tiles.  All loads of a batch of tiles
+        are issued before the first use (a load directly followed by its use
+        would serialise the round trips): resident rows are fetched by a loop
+        of their own ahead of the first sweep, streamed rows SU tiles at a
+        time.  ``emit_body(tiles)`` writes the per-tile work; ``k``, ``c`` and
+        ``ok`` are in scope."""
+        moving = [n for n in leaves if varies_in_loop(n)]
+        tiles = dict((n.nid, line_tiles[n.nid]) for n in leaves if not varies_in_loop(n))
         if resident:
+            fresh = [n for n in moving if n.nid not in cached]
+            if fresh:
+                L("#pragma unroll")
+                L.open("for (int k = 0; k < %d; ++k)" % NCH)
+                chunk_position("k")
+                for n in fresh:
+                    cached[n.nid] = "keep%d" % n.nid
+                    L("if (ok) keep%d[k].%s(%s); else keep%d[k].zero();"
+                      % (n.nid, g.ld, g.tile_addr(n, "rr", "c"), n.nid))
+                L.close()
+            for n in moving:
+                tiles[n.nid] = "%s[k]" % cached[n.nid]
             L("#pragma unroll")
             L.open("for (int k = 0; k < %d; ++k)" % NCH)
-        else:
-            L("#pragma unroll 2")
-            L.open("for (int k = 0; k < nch; ++k)")
-        L("const long long c = ((long long)k * %d + tx) * %d;" % (LX, V))
-        L("const bool ok = row_ok && (c < C);")
+            chunk_position("k")
+            emit_body(tiles)
+            L.close()
+            return
+        L.open("for (int k0 = 0; k0 < nch; k0 += %d)" % SU)
+        for n in moving:
+            L("%s %s[%d];" % (g.tile_type(n, V), g.tile_name(n, "_s"), SU))
+            tiles[n.nid] = "%s[u]" % g.tile_name(n, "_s")
+        L("#pragma unroll")
+        L.open("for (int u = 0; u < %d; ++u)" % SU)
+        chunk_position("k0 + u")
+        for n in moving:
+            L("if (ok) %s[u].%s(%s); else %s[u].zero();"
+              % (g.tile_name(n, "_s"), g.ld, g.tile_addr(n, "rr", "c"), g.tile_name(n, "_s")))
+        L.close()
+        L("#pragma unroll")
+        L.open("for (int u = 0; u < %d; ++u)" % SU)
+        chunk_position("k0 + u")
+        emit_body(tiles)
+        L.close()
+        L.close()
 
     line_tiles = {}   # leaf nid -> tile that does not change along the row
 
     def varies_in_loop(n):
         return g.tile_width(n, 2) == 2      # tile spans columns
-
-    def load_leaves(leaves, first_use):
-        """make tiles for ``leaves`` available inside the chunk loop"""
-        tiles = {}
-        for n in leaves:
-            if not varies_in_loop(n):
-                tiles[n.nid] = line_tiles[n.nid]
-                continue
-            if resident and n.nid in cached:
-                tiles[n.nid] = "%s[k]" % cached[n.nid]
-                continue
-            if resident:
-                name = "keep%d" % n.nid
-                cached[n.nid] = name
-                tiles[n.nid] = "%s[k]" % name
-                L("if (ok) %s[k].%s(%s); else %s[k].zero();" % (name, g.ld, g.tile_addr(n, "rr", "c"), name))
-            else:
-                name = g.tile_name(n, "_s")
-                tiles[n.nid] = name
-                L("%s %s; %s.zero();" % (g.tile_type(n, V), name, name))
-                L("if (ok) %s.%s(%s);" % (name, g.ld, g.tile_addr(n, "rr", "c")))
-        return tiles
 
     def declare_tiles(leaves):
         """function-scope declarations needed before a sweep's loop"""
@@ -478,19 +531,20 @@ def gen_row(prog, V, LX, LY, NCH, stream=False):
         declare_tiles(leaves)
         for n in reds:
             g.declare_acc(n)
-        chunk_loop_open()
-        tiles = load_leaves(leaves, True)
-        L.open("if (ok)")
-        if V > 1:
-            L("#pragma unroll")
-        L.open("for (int j = 0; j < %d; ++j)" % V)
-        ref = g.make_ref("_s", "rr", "c", V, tiles)
-        g.emit_exprs(nodes, ref, done)
-        for n in reds:
-            g.accumulate(n, ref(n.args[0]), "c + j")
-        L.close()
-        L.close()
-        L.close()
+
+        def reduce_body(tiles, nodes=nodes, reds=reds):
+            L.open("if (ok)")
+            if V > 1:
+                L("#pragma unroll")
+            L.open("for (int j = 0; j < %d; ++j)" % V)
+            ref = g.make_ref("_s", "rr", "c", V, tiles)
+            g.emit_exprs(nodes, ref, done)
+            for n in reds:
+                g.accumulate(n, ref(n.args[0]), "c + j")
+            L.close()
+            L.close()
+
+        sweep(leaves, reduce_body)
         for n in reds:
             op = _RED_OP[n.op]
             ty_ = "nh_pair" if n.is_index else "float"
@@ -533,26 +587,27 @@ def gen_row(prog, V, LX, LY, NCH, stream=False):
         nodes = _needed(roots, done)
         leaves = g.leaf_nodes(nodes)
         declare_tiles(leaves)
-        chunk_loop_open()
-        tiles = load_leaves(leaves, False)
-        L.open("if (ok)")
-        for st in full_out:
-            L("nh_out<%s, %d> o%d; o%d.clear();" % (g.slot_ctype(st.out), V, st.out.index, st.out.index))
-        if V > 1:
-            L("#pragma unroll")
-        L.open("for (int j = 0; j < %d; ++j)" % V)
-        ref = g.make_ref("_s", "rr", "c", V, tiles)
-        g.emit_exprs(nodes, ref, done)
-        for st in full_out:
-            if st.root.kind == "R" and st.root.is_index:
-                L("o%d.seti(j, ri%d);" % (st.out.index, st.root.nid))
-            else:
-                L("o%d.set(j, %s);" % (st.out.index, ref(st.root)))
-        L.close()
-        for st in full_out:
-            L("o%d.%s(%s);" % (st.out.index, g.st, g.addr(st.out, "r", "c")))
-        L.close()
-        L.close()
+
+        def store_body(tiles):
+            L.open("if (ok)")
+            for st in full_out:
+                L("nh_out<%s, %d> o%d; o%d.clear();" % (g.slot_ctype(st.out), V, st.out.index, st.out.index))
+            if V > 1:
+                L("#pragma unroll")
+            L.open("for (int j = 0; j < %d; ++j)" % V)
+            ref = g.make_ref("_s", "rr", "c", V, tiles)
+            g.emit_exprs(nodes, ref, done)
+            for st in full_out:
+                if st.root.kind == "R" and st.root.is_index:
+                    L("o%d.seti(j, ri%d);" % (st.out.index, st.root.nid))
+                else:
+                    L("o%d.set(j, %s);" % (st.out.index, ref(st.root)))
+            L.close()
+            for st in full_out:
+                L("o%d.%s(%s);" % (st.out.index, g.st, g.addr(st.out, "r", "c")))
+            L.close()
+
+        sweep(leaves, store_body)
     L.close()
     return _finish("row", g, head, fmt, T, 0, dict(V=V, LX=LX, LY=LY, NCH=NCH, stream=bool(stream)))
 
@@ -621,7 +676,7 @@ def _col_lds(L, LX, LY, T, V, any_index):
     return WY * (LX * V + 1) * (4 + (8 if any_index else 0))
 
 
-def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1):
+def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
     """Axis-0 reductions with the rows resident in registers (LX column-lanes x
     LY row-lanes per workgroup, NR rows per lane).
 
@@ -750,15 +805,19 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1):
         return n.axis == 1           # one-hot along axis 1 reads idx[r]
 
     def load_leaves(leaves):
+        """names of the tiles inside the row loop; rows not yet resident are
+        fetched by a loop of their own first, so that all loads are in flight
+        before the first use"""
         tiles = {}
-        for n in leaves:
-            if not varies_in_loop(n):
-                tiles[n.nid] = line_tiles[n.nid]
-                continue
-            if n.nid not in cached:
+        fresh = [n for n in leaves if varies_in_loop(n) and n.nid not in cached]
+        if fresh:
+            row_loop_open()
+            for n in fresh:
                 cached[n.nid] = "keep%d" % n.nid
                 L("if (ok) keep%d[i].%s(%s); else keep%d[i].zero();" % (n.nid, g.ld, g.tile_addr(n, "r", "cc"), n.nid))
-            tiles[n.nid] = "keep%d[i]" % n.nid
+            L.close()
+        for n in leaves:
+            tiles[n.nid] = ("keep%d[i]" % n.nid) if varies_in_loop(n) else line_tiles[n.nid]
         return tiles
 
     def declare_tiles(leaves):
@@ -776,29 +835,58 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1):
     declare_tiles([n for n in g.leaf_nodes(used_nodes([st.root for st in prog.statements]))
                    if not varies_in_loop(n)])
 
+    stages = [[n.args[0] for n in per_level.get(s, [])] for s in range(nsweeps)]
+    stages = [t for t in stages if t]
+    if full_out:
+        stages.append([st.root for st in full_out])
+    kept = _kept_values(prog, stages, max_vals)
+    kept_ids = set(n.nid for n in kept)
+    vals = {}          # nid -> expression of a value kept from an earlier sweep
+
+    def stops():
+        d = set(done)
+        d.update(vals)
+        return d
+
+    def stash_new_values(nodes):
+        """inside the j loop: keep the values later sweeps will want"""
+        fresh = [n for n in nodes if n.nid in kept_ids and n.nid not in vals]
+        for n in fresh:
+            L("val%d[i][j] = t%d;" % (n.nid, n.nid))
+        return fresh
+
+    def declare_values(nodes):
+        for n in nodes:
+            if n.nid in kept_ids and n.nid not in vals:
+                L("float val%d[%d][%d];" % (n.nid, NR, V))
+
     for s in range(nsweeps):
         reds = per_level.get(s, [])
         if not reds:
             continue
         args = [n.args[0] for n in reds]
-        nodes = _needed(args, done)
+        nodes = _needed(args, stops())
         leaves = g.leaf_nodes(nodes)
         declare_tiles(leaves)
+        declare_values(nodes)
         for n in reds:
             g.declare_acc(n)
-        row_loop_open()
         tiles = load_leaves(leaves)
+        row_loop_open()
         L.open("if (ok)")
         if V > 1:
             L("#pragma unroll")
         L.open("for (int j = 0; j < %d; ++j)" % V)
-        ref = g.make_ref("_s", "r", "cc", V, tiles)
-        g.emit_exprs(nodes, ref, done)
+        ref = g.make_ref("_s", "r", "cc", V, tiles, vals)
+        g.emit_exprs(nodes, ref, stops())
         for n in reds:
             g.accumulate(n, ref(n.args[0]), "r")
+        fresh = stash_new_values(nodes)
         L.close()
         L.close()
         L.close()
+        for n in fresh:
+            vals[n.nid] = "val%d[i][j]" % n.nid
         for n in reds:
             _emit_col_fold(g, L, n, LX, LY, T, V, "acc%d" % n.nid)
             done[n.nid] = n
@@ -831,19 +919,19 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1):
 
     if full_out:
         roots = [st.root for st in full_out]
-        nodes = _needed(roots, done)
+        nodes = _needed(roots, stops())
         leaves = g.leaf_nodes(nodes)
         declare_tiles(leaves)
-        row_loop_open()
         tiles = load_leaves(leaves)
+        row_loop_open()
         L.open("if (ok)")
         for st in full_out:
             L("nh_out<%s, %d> o%d; o%d.clear();" % (g.slot_ctype(st.out), V, st.out.index, st.out.index))
         if V > 1:
             L("#pragma unroll")
         L.open("for (int j = 0; j < %d; ++j)" % V)
-        ref = g.make_ref("_s", "r", "cc", V, tiles)
-        g.emit_exprs(nodes, ref, done)
+        ref = g.make_ref("_s", "r", "cc", V, tiles, vals)
+        g.emit_exprs(nodes, ref, stops())
         for st in full_out:
             if st.root.kind == "R" and st.root.is_index:
                 L("o%d.seti(j, ri%d[j]);" % (st.out.index, st.root.nid))
@@ -867,7 +955,7 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1):
     L.close()
     return _finish("colcoop" if coop else "col", g, head, fmt, T, lds,
                    dict(V=V, LX=LX, LY=LY, NR=NR, stream=bool(stream), chunks=chunks,
-                        NRED=len(all_reds)))
+                        NRED=len(all_reds), kept=len(kept)))
 
 
 COLSPLIT_MAX_CHUNKS = 128

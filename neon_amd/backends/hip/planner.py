@@ -357,6 +357,13 @@ def _plan_row(prog, cu_count):
     return Choice(spec, (gx, 1, 1))
 
 
+# 32-bit registers per lane that resident tiles (and kept values) may occupy,
+# by workgroup size: what is left of the 512 / (waves per SIMD) budget after
+# the temporaries that full unrolling keeps live (measured: beyond these the
+# compiler spills)
+_COL_BUDGET = {1024: 40, 512: 120, 256: 300}
+
+
 def _plan_col(prog, cu_count):
     R, C = prog.domain
     V = _vector_width(prog, single_row_tail_ok=False)
@@ -383,7 +390,7 @@ def _plan_col(prog, cu_count):
         for T in ((256, 512, 1024) if strips >= cu_count else (1024, 512, 256)):
             LY = T // LX
             NR = _ceil_div(R, LY)
-            budget = 64 if T == 1024 else 128
+            budget = _COL_BUDGET[T]
             if NR <= 16 and NR * words <= budget:
                 fit = (T, LY, NR)
                 break
@@ -395,7 +402,9 @@ def _plan_col(prog, cu_count):
     big = R * C >= (1 << 18)
     if fit and not (single_level and line_only and big and R >= 512):
         T, LY, NR = fit
-        spec = codegen.gen_col(prog, V, LX, LY, NR, _streams(prog))
+        budget = _COL_BUDGET[T]
+        spare = max(0, (budget - NR * words) // (NR * V))
+        spec = codegen.gen_col(prog, V, LX, LY, NR, _streams(prog), max_vals=min(2, spare))
         return Choice(spec, (_ceil_div(nvec, LX), 1, 1))
 
     # (c) deeper trees (or full-shape results) over many rows: the workgroups of a
@@ -408,14 +417,19 @@ def _plan_col(prog, cu_count):
         if strips_c <= cu_count:
             chunks = max(1, min(128, cu_count // strips_c))
             rpc0 = _ceil_div(R, chunks)
-            for T, budget in ((1024, 72), (512, 200), (256, 448)):
+            options = ((1024, 40), (512, 120), (256, 300))
+            if os.environ.get("NEON_HIP_COOP_T"):          # tuning aid
+                options = tuple(o for o in options if o[0] == int(os.environ["NEON_HIP_COOP_T"]))
+            for T, budget in options:
                 LY = T // lxc
                 NR = _ceil_div(rpc0, LY)
                 if NR <= 64 and NR * words <= budget:
                     chunks = _ceil_div(R, NR * LY)
                     if chunks < 2:
                         break
-                    spec = codegen.gen_col(prog, V, lxc, LY, NR, _streams(prog), chunks=chunks)
+                    spare = max(0, (budget - NR * words) // (NR * V))
+                    spec = codegen.gen_col(prog, V, lxc, LY, NR, _streams(prog), chunks=chunks,
+                                           max_vals=min(2, spare))
                     part_bytes = spec.params["NRED"] * chunks * C * 8
                     ctr_off = _ceil_div(part_bytes, 256) * 256
                     return Choice(spec, (strips_c, chunks, 1),

@@ -230,8 +230,10 @@ template <typename T> NEON_DEV float nh_quant(float x) { return (float)nh_store_
 // reference differ: safelog clamps its argument, sign(nan) is nan,
 // minimum/maximum and max/min reductions propagate nan like numpy)
 // ---------------------------------------------------------------------------
-NEON_DEV float nh_max(float a, float b) { return (a != a) ? a : ((b != b) ? b : __builtin_fmaxf(a, b)); }
-NEON_DEV float nh_min(float a, float b) { return (a != a) ? a : ((b != b) ? b : __builtin_fminf(a, b)); }
+// IEEE-754-2019 maximum / minimum: NaN if either operand is NaN, which is what
+// numpy's maximum / max do; one v_maximum3_f32 / v_minimum3_f32 on gfx950.
+NEON_DEV float nh_max(float a, float b) { return __builtin_elementwise_maximum(a, b); }
+NEON_DEV float nh_min(float a, float b) { return __builtin_elementwise_minimum(a, b); }
 NEON_DEV float nh_sgn(float x) { return (x != x) ? x : (float)((x > 0.0f) - (x < 0.0f)); }
 NEON_DEV float nh_sqr(float x) { return x * x; }
 NEON_DEV float nh_safelog(float x) { return logf(nh_max(x, 1.9287498479639178e-22f)); }  // exp(-50)

@@ -195,8 +195,13 @@ def test_shape_class_selection(pb):
     ch = plan_of(pb, lambda: pb.empty((1, 256), np.int32).__setitem__(slice(None), pb.argmax(x5, axis=0)))
     assert ch.spec.family == "colsplit" and ch.workspace is not None
     assert ch.grid[0] * ch.grid[1] <= 2 * 256 and ch.grid[1] <= codegen.COLSPLIT_MAX_CHUNKS
-    with pytest.raises(planner.NeedsSplit):        # three sweeps over 32000 rows do not fit one workgroup
-        pb.empty((32000, 256)).__setitem__(slice(None), pb.fprop_softmax(x5, 0))
+    # three sweeps over 32000 rows do not fit one workgroup: the workgroups of a strip cooperate
+    ch = plan_of(pb, lambda: pb.empty((32000, 256)).__setitem__(slice(None), pb.fprop_softmax(x5, 0)))
+    assert ch.spec.family == "colcoop" and ch.grid[0] * ch.grid[1] <= 256 and ch.workspace is not None
+    assert ch.spec.source.count("nh_part_store") == 2 and "NH_SPIN_LIMIT" in ch.spec.source
+    huge = pb.empty((4000000, 256))
+    with pytest.raises(planner.NeedsSplit):        # too many rows to keep on chip: evaluated stage by stage
+        pb.empty((4000000, 256)).__setitem__(slice(None), pb.fprop_softmax(huge, 0))
     odd = pb.empty((64, 327))
     ch = plan_of(pb, lambda: pb.empty((64, 1)).__setitem__(slice(None), pb.sum(odd, axis=1)))
     assert ch.spec.family == "row" and ch.spec.params["V"] == 1           # 327 columns: no vector access
