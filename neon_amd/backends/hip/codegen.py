@@ -477,20 +477,20 @@ def gen_row(prog, V, LX, LY, NCH, stream=False):
             emit_body(tiles)
             L.close()
             return
-        L.open("for (int k0 = 0; k0 < nch; k0 += %d)" % SU)
+        L.open("for (int kb = 0; kb < nch; kb += %d)" % SU)
         for n in moving:
             L("%s %s[%d];" % (g.tile_type(n, V), g.tile_name(n, "_s"), SU))
             tiles[n.nid] = "%s[u]" % g.tile_name(n, "_s")
         L("#pragma unroll")
         L.open("for (int u = 0; u < %d; ++u)" % SU)
-        chunk_position("k0 + u")
+        chunk_position("kb + u")
         for n in moving:
             L("if (ok) %s[u].%s(%s); else %s[u].zero();"
               % (g.tile_name(n, "_s"), g.ld, g.tile_addr(n, "rr", "c"), g.tile_name(n, "_s")))
         L.close()
         L("#pragma unroll")
         L.open("for (int u = 0; u < %d; ++u)" % SU)
-        chunk_position("k0 + u")
+        chunk_position("kb + u")
         emit_body(tiles)
         L.close()
         L.close()

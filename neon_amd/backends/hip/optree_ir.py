@@ -371,6 +371,12 @@ class Program(object):
     def finalize(self):
         """Infer the iteration domain, per-node variance and reduction levels;
         verify broadcast compatibility."""
+        # a tensor assigned more than once in the group is stored once, with its
+        # final value; readers in between were given the value in registers
+        last = {}
+        for st in self.statements:
+            last[st.out.index] = st
+        self.statements = [st for st in self.statements if last[st.out.index] is st]
         index_only = set(n.slot for n in self.nodes if n.kind == "H")
         index_only -= set(n.slot for n in self.nodes if n.kind == "T")
         index_only -= set(st.out.index for st in self.statements)

@@ -211,6 +211,80 @@ def test_tall_multilevel_axis0(pair, shape):
         assert "colcoop" in fams
 
 
+@pytest.mark.parametrize("shape,axis", [((3, 300000), 1), ((2, 150000), 1), ((40000, 33), 0), ((70000, 8), 0),
+                                        ((6, 70000), 0), ((70000, 6), 1)])
+def test_extreme_aspect_ratios(pair, shape, axis):
+    """rows too long to stay in registers (streamed on every sweep), odd
+    column counts on the split-row path, very flat and very tall inputs"""
+    rs = np.random.RandomState(shape[0] % 91)
+    a = gen_inputs(rs, shape)
+    atol = 4 * np.finfo(np.float32).eps * float(np.abs(a).sum(axis=axis).max())
+    both(pair, lambda be, x: be.sum(x, axis=axis), [a], rtol=RTOL32, atol=atol, what="sum")
+    both(pair, lambda be, x: be.max(x, axis=axis) - be.min(x, axis=axis), [a], what="range")
+    both(pair, lambda be, x: be.argmax(x, axis=axis), [a], out_dtype=np.int32, what="argmax")
+    a64 = a.astype(np.float64)
+    truth = (a64 - a64.mean(axis=axis, keepdims=True)) / np.sqrt(a64.var(axis=axis, keepdims=True) + 1e-5)
+    got = call_func(lambda be, x: (x - be.mean(x, axis=axis)) / be.sqrt(be.var(x, axis=axis) + 1e-5), pair[1], [a])
+    assert_close(got, truth, rtol=RTOL32, atol=1e-5, what="normalise vs fp64")
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.int32, np.uint8, np.int16])
+@pytest.mark.parametrize("axis", [0, 1])
+def test_reductions_over_storage_dtypes(pair, dtype, axis):
+    rs = np.random.RandomState(12)
+    shape = (96, 160)
+    if np.dtype(dtype).kind == "f":
+        a = (rs.rand(*shape) * 4 - 2).astype(dtype)
+    else:
+        a = rs.randint(0, 100, shape).astype(dtype)
+    cpu, hip = pair
+    res = []
+    for be in pair:
+        # the oracle holds the same values in fp32 so that it, too, computes in fp32
+        x = be.array(a.astype(np.float32)) if be is cpu else be.array(a, dtype=dtype)
+        red = (1, shape[1]) if axis == 0 else (shape[0], 1)
+        o1, o2, o3 = be.empty(red), be.empty(red, dtype=np.int32), be.empty(shape, dtype=dtype)
+        o1[:] = be.max(x, axis=axis) - be.min(x, axis=axis) + be.sum(x, axis=axis)
+        o2[:] = be.argmin(x, axis=axis)
+        o3[:] = x - be.min(x, axis=axis)
+        res.append((o1.get(), o2.get(), o3.get()))
+    assert_close(res[1][0], res[0][0], rtol=RTOL32, atol=1e-3, what="stats")
+    assert np.array_equal(res[1][1], res[0][1])
+    if np.dtype(dtype).kind == "f":
+        assert rel_err(res[1][2], res[0][2], floor_frac=1e-3) <= 1e-3
+    else:
+        assert np.array_equal(res[1][2], res[0][2])
+
+
+def test_fused_update_rules(pair):
+    """optimizer-style statement groups between begin/end(Block.update): same
+    results as one kernel per statement (reference optimizer.py: momentum SGD
+    :382-426, RMSProp :589-606)"""
+    from neon_amd.backends.backend import Block
+    rs = np.random.RandomState(13)
+    shape = (300, 130)
+    g0, p0 = gen_inputs(rs, shape) * 0.1, gen_inputs(rs, shape)
+    res = []
+    for be in pair:
+        for fused in (False, True):
+            grad, param = be.array(g0), be.array(p0)
+            vel, state = be.zeros(shape), be.zeros(shape)
+            for step in range(3):
+                if fused:
+                    be.begin(Block.update, step)
+                vel[:] = vel * 0.9 - 0.01 * (grad + 0.0005 * param)          # momentum + weight decay
+                param[:] = param + vel
+                state[:] = 0.95 * state + be.square(grad) * (1.0 - 0.95)     # RMSProp state
+                param[:] = param - (grad * 0.002) / (be.sqrt(state + 1e-6) + 1e-6)
+                if fused:
+                    be.end(Block.update, step)
+            res.append((param.get(), vel.get(), state.get()))
+    for k in range(3):
+        assert np.array_equal(res[2][k], res[3][k]), "fused and unfused device results differ"
+        assert_close(res[3][k], res[1][k], rtol=RTOL32, atol=1e-7)
+        assert_close(res[2][k], res[0][k], rtol=RTOL32, atol=1e-7)
+
+
 def test_onehot(pair):
     rs = np.random.RandomState(8)
     idx = rs.randint(0, 40, (1, 64)).astype(np.int32)
