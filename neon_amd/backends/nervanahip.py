@@ -813,6 +813,65 @@ class NervanaHIP(Backend):
         # soon as its last consumer has been enqueued
         self._temp_pool.setdefault((t.shape, t.dtype), []).append(t)
 
+    # -- batch normalisation as fused statement groups -------------------------------------------
+    @staticmethod
+    def _stmt(out, value):
+        """an assign tree that has not been executed"""
+        return OpTreeNode({"op": "assign"}, out, value)
+
+    def _run_group(self, trees):
+        """run statements as one kernel when the families allow it, otherwise
+        one by one in order (same results either way)"""
+        self._flush()
+        if self._captured is not None:
+            self._captured.append(list(trees))
+        else:
+            self._run(list(trees))
+
+    def compound_fprop_bn(self, x, xsum, xvar, gmean, gvar, gamma, beta, y, eps, rho,
+                          compute_batch_sum, accumbeta=0.0, relu=False, threads=None, repeat=1,
+                          binary=False, inference=False, outputs=None, layer=None):
+        """Batch-norm forward over axis 1 (reference nervanagpu.py:2463-2522;
+        statement-for-statement the CPU backend's version,
+        nervanacpu.py:1688-1728).  All statements -- batch sum, variance,
+        running-statistics updates and the normalised output -- are handed
+        over as ONE group, which the row family turns into a single kernel
+        that reads ``x`` once and keeps each row in registers."""
+        if binary:
+            raise NotImplementedError("shift-based batch norm is outside the op-tree path")
+        if inference:
+            xhat = (x - gmean) / self.sqrt(gvar + eps)
+            y[:] = y * accumbeta + xhat * gamma + beta
+            return
+        st, n = self._stmt, float(x.shape[1])
+        trees = []
+        if compute_batch_sum:
+            trees.append(st(xsum, self.sum(x, axis=1)))
+        trees.append(st(xvar, self.var(x, axis=1)))
+        trees.append(st(xsum, xsum / n))
+        trees.append(st(gmean, gmean * rho + (1.0 - rho) * xsum))
+        trees.append(st(gvar, gvar * rho + (1.0 - rho) * xvar))
+        xhat = (x - xsum) / self.sqrt(xvar + eps)
+        out = y.reshape(x.shape)
+        trees.append(st(out, xhat * gamma + beta + accumbeta * out))
+        self._run_group(trees)
+
+    def compound_bprop_bn(self, delta_out, grad_gamma, grad_beta, delta_in, x, xsum, xvar,
+                          gamma, eps, threads=None, repeat=1, binary=False, layer=None):
+        """Batch-norm backward (reference nervanagpu.py:2524-2588;
+        nervanacpu.py:1730-1760): both parameter gradients and the input
+        deltas from one pass over ``x`` and ``delta_in``."""
+        if binary:
+            raise NotImplementedError("shift-based batch norm is outside the op-tree path")
+        st = self._stmt
+        inv_v = 1.0 / self.sqrt(xvar + eps)
+        xhat = (x - xsum) * inv_v
+        trees = [st(grad_gamma, self.sum(xhat * delta_in, axis=1)),
+                 st(grad_beta, self.sum(delta_in, axis=1))]
+        xtmp = (xhat * grad_gamma + grad_beta) / float(x.shape[1])
+        trees.append(st(delta_out.reshape(delta_in.shape), ((delta_in - xtmp) * gamma) * inv_v))
+        self._run_group(trees)
+
     # -- layer-level helpers that are plain op-trees ----------------------------------------
     def consume(self, buf_index, hostlist, devlist):
         assert 0 <= buf_index < 2, "Can only double buffer"

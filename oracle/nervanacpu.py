@@ -397,6 +397,35 @@ class NervanaCPU(Backend):
     def zeros_like(self, ary, dtype=None, name=None, persist_values=True):
         return self.empty_like(ary, dtype, name, persist_values)
 
+    # -- batch normalisation (reference nervanacpu.py:1688-1760), non-binary path ---
+    def compound_fprop_bn(self, x, xsum, xvar, gmean, gvar, gamma, beta, y, eps, rho,
+                          compute_batch_sum, accumbeta=0.0, relu=False, binary=False,
+                          inference=False, outputs=None, layer=None):
+        assert not binary
+        if inference:
+            xhat = (x - gmean) / self.sqrt(gvar + eps)
+            y[:] = y * accumbeta + xhat * gamma + beta
+            return
+        if compute_batch_sum:
+            xsum[:] = self.sum(x, axis=1)
+        xvar[:] = self.var(x, axis=1)
+        xsum[:] = xsum / x.shape[1]
+        gmean[:] = gmean * rho + (1.0 - rho) * xsum
+        gvar[:] = gvar * rho + (1.0 - rho) * xvar
+        xhat = (x - xsum) / self.sqrt(xvar + eps)
+        outputs = y.reshape(xhat.shape)
+        outputs[:] = xhat * gamma + beta + accumbeta * outputs
+
+    def compound_bprop_bn(self, delta_out, grad_gamma, grad_beta, delta_in, x, xsum, xvar,
+                          gamma, eps, binary=False, layer=None):
+        assert not binary
+        inv_v = 1.0 / self.sqrt(xvar + eps)
+        xhat = (x - xsum) * inv_v
+        grad_gamma[:] = self.sum(xhat * delta_in, axis=1)
+        grad_beta[:] = self.sum(delta_in, axis=1)
+        xtmp = (xhat * grad_gamma + grad_beta) / float(x.shape[1])
+        delta_out.reshape(delta_in.shape)[:] = ((delta_in - xtmp) * gamma) * inv_v
+
     # -- timing marks (reference nervanacpu.py:1865-1905) -------------------------
     def init_mark(self):
         return {"time": 0}

@@ -436,3 +436,39 @@ def test_full_size_properties(hip):
     nz = np.abs(grad) > 1e-3      # eps / sqrt(v) is below 4e-4 there
     assert np.allclose(np.abs(d[nz]), 1e-3, rtol=2e-3)
     assert np.array_equal(np.sign(d[nz]), np.sign(grad[nz]))
+
+
+# ---- batch normalisation entry points (fused statement groups) -----------------------------------
+@pytest.mark.parametrize("shape,dtype", [((32, 128), np.float32), ((64, 6272), np.float32),
+                                         ((16, 100352), np.float16), ((5, 77), np.float32)])
+def test_compound_batchnorm(pair, shape, dtype):
+    cpu, hip = pair
+    rs = np.random.RandomState(shape[1] % 89)
+    x0 = (rs.standard_normal(shape) * 2 + 0.5).astype(np.float32).astype(dtype)
+    d0 = rs.standard_normal(shape).astype(np.float32).astype(dtype)
+    gam0 = rs.uniform(0.5, 1.5, (shape[0], 1)).astype(np.float32)
+    bet0 = (rs.standard_normal((shape[0], 1)) * 0.1).astype(np.float32)
+    res = []
+    for be in pair:
+        # the oracle holds fp16 data as fp32 values so that it computes in fp32 as well
+        sdt = np.float32 if be is cpu else dtype
+        x, din = be.array(x0.astype(sdt), dtype=sdt), be.array(d0.astype(sdt), dtype=sdt)
+        y, dout = be.empty(shape, dtype=dtype), be.empty(shape, dtype=dtype)
+        vec = lambda: be.zeros((shape[0], 1))     # noqa: E731
+        xsum, xvar, gmean, gvar, gg, gb = vec(), vec(), vec(), vec(), vec(), vec()
+        gamma, beta = be.array(gam0), be.array(bet0)
+        for _ in range(2):                        # running statistics accumulate over two calls
+            be.compound_fprop_bn(x, xsum, xvar, gmean, gvar, gamma, beta, y, 1e-3, 0.9, True)
+        be.compound_bprop_bn(dout, gg, gb, din, x, xsum, xvar, gamma, 1e-3)
+        yi = be.empty(shape, dtype=dtype)
+        be.compound_fprop_bn(x, xsum, xvar, gmean, gvar, gamma, beta, yi, 1e-3, 0.9, True, inference=True)
+        res.append([t.get().astype(np.float64) for t in (y, xsum, xvar, gmean, gvar, dout, gg, gb, yi)])
+    names = ("y", "xmean", "xvar", "gmean", "gvar", "delta", "grad_gamma", "grad_beta", "y_inference")
+    tol = 1e-3 if dtype == np.float16 else 2e-5
+    for got, want, name in zip(res[1], res[0], names):
+        scale = np.abs(want).max() + 1e-30
+        assert np.abs(got - want).max() <= tol * scale, (name, np.abs(got - want).max(), scale)
+    if hip.plan_stats is not None and shape[1] >= 128:
+        # forward ran as one row kernel: x read once
+        fams = [p.spec.family for p in hip.plans.values() if len(p.spec.source) and "row" == p.spec.family]
+        assert fams
