@@ -167,6 +167,15 @@ int nh_colmax_argmax_f32(float* maxval, int32_t* argmax, const float* x,
                          uint32_t rows, uint32_t cols, size_t ld,
                          void* workspace, void* stream);
 
+/* 64-bin (nbins <= 256) histogram of rint(log2|x|) over n contiguous fp32
+ * (itemsize 4) or fp16 (itemsize 2) elements into hist[nbins] (cleared
+ * first): bin 0 reaches down to -inf, bin k >= 1 holds offset+k, the last bin
+ * also offset+nbins, larger magnitudes and NaN are not counted -- the binning
+ * of Tensor.hist on the CPU backend (neon/backends/nervanacpu.py:424-445);
+ * replaces kernel_histo / _compute_hist (neon/backends/float_ew.py:1070-1158). */
+int nh_hist_log2(int32_t* hist, const void* x, int itemsize, size_t n, int nbins,
+                 int offset, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -129,12 +129,17 @@ class _Gen(object):
 
     # -- addresses ------------------------------------------------------------------
     def addr(self, slot, r, c):
-        """Element address of (r, c) in a slot, honouring broadcast dims."""
+        """Element address of (r, c) in a slot, honouring broadcast dims and
+        index vectors of gather / scatter views."""
         parts = ["a%d" % slot.index]
         if slot.shape[0] > 1:
+            if slot.take_axis == 0:
+                r = "a%d[(long long)(%s)]" % (slot.take_slot, r)
             parts.append("(long long)(%s) * sr%d" % (r, slot.index))
         if slot.shape[1] > 1:
-            if self.col_unit(slot):
+            if slot.take_axis == 1:
+                parts.append("(long long)a%d[(long long)(%s)] * sc%d" % (slot.take_slot, c, slot.index))
+            elif self.col_unit(slot):
                 parts.append("(long long)(%s)" % c)
             else:
                 parts.append("(long long)(%s) * sc%d" % (c, slot.index))

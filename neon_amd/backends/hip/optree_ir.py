@@ -167,9 +167,11 @@ class Node(object):
 class TensorSlot(object):
     """One kernel pointer argument: a distinct (memory, geometry, dtype)."""
     __slots__ = ("index", "tensor", "dtype", "shape", "strides", "ptr", "written",
-                 "read", "geom")
+                 "read", "geom", "take_axis", "take_slot")
 
     def __init__(self, index, tensor, shape, strides):
+        self.take_axis = None      # gather / scatter view: indexed axis ...
+        self.take_slot = None      # ... and the slot of its int32 index vector
         self.index = index
         self.tensor = tensor
         self.dtype = np.dtype(tensor.dtype)
@@ -221,6 +223,7 @@ class Program(object):
         self._const_slot = {}
         self._current = {}         # tensor slot index -> node holding its newest value
         self.key_parts = []
+        self.index_slots = set()   # slots used only as index vectors of gather views
         self.raw_count = 0         # numbers seen so far, in postfix order
         self.const_exprs = []      # per constant slot: expressions that produced its value
         self.axis = None           # the one reduction axis, if any
@@ -232,15 +235,30 @@ class Program(object):
         slot = self._tensor_by_id.get(id(t))
         if slot is not None:
             return slot
-        if getattr(t, "take_array", None):
-            raise NotImplementedError("fancy-indexed views inside op-trees")
+        take = getattr(t, "take_array", None)
+        take_slot = take_axis = None
+        if take:
+            # a view through an index vector (the reference's in1/in2/out1/out2
+            # argument kinds, cuda_templates.py:448-483): position i along the
+            # indexed axis addresses element idx[i] of the base
+            idx, take_axis = take
+            if len(t.shape) != 2 or take_axis not in (0, 1):
+                raise NotImplementedError("fancy-indexed views with more than 2 dimensions")
+            if idx.dtype != np.dtype(np.int32) or not idx.is_contiguous:
+                raise TypeError("index vector of a fancy-indexed view must be contiguous int32")
+            take_slot = self.tensor_slot(idx)
+            self.index_slots.add(take_slot.index)
         shape, strides = view_2d(t)
-        geom = (t.ptr, shape, strides, np.dtype(t.dtype))
+        geom = (t.ptr, shape, strides, np.dtype(t.dtype),
+                take_axis, take_slot.index if take_slot else None)
         slot = self._tensor_by_geom.get(geom)
         if slot is None:
             if np.dtype(t.dtype) not in DTYPE_CODE:
                 raise TypeError("unsupported tensor dtype %s" % t.dtype)
             slot = TensorSlot(len(self.tensors), t, shape, strides)
+            slot.take_axis = take_axis
+            slot.take_slot = take_slot.index if take_slot else None
+            slot.geom = geom
             self.tensors.append(slot)
             self._tensor_by_geom[geom] = slot
         self._tensor_by_id[id(t)] = slot
@@ -377,7 +395,7 @@ class Program(object):
         for st in self.statements:
             last[st.out.index] = st
         self.statements = [st for st in self.statements if last[st.out.index] is st]
-        index_only = set(n.slot for n in self.nodes if n.kind == "H")
+        index_only = set(n.slot for n in self.nodes if n.kind == "H") | set(self.index_slots)
         index_only -= set(n.slot for n in self.nodes if n.kind == "T")
         index_only -= set(st.out.index for st in self.statements)
         shaped = [t for t in self.tensors if t.index not in index_only]
@@ -433,8 +451,8 @@ class Program(object):
 
     def key(self):
         """Hashable identity of the program's structure and operand geometry."""
-        geo = tuple((DTYPE_CODE[t.dtype], t.shape, t.strides, t.ptr % 16 == 0, t.written)
-                    for t in self.tensors)
+        geo = tuple((DTYPE_CODE[t.dtype], t.shape, t.strides, t.ptr % 16 == 0, t.written,
+                     t.take_axis, t.take_slot) for t in self.tensors)
         return (tuple(self.key_parts), geo, self._alias_signature())
 
     def _alias_signature(self):
@@ -446,6 +464,8 @@ class Program(object):
             extent = 1 + sum((s - 1) * abs(st) for s, st in zip(t.shape, t.strides) if s > 0)
             spans.append((t.ptr, t.ptr + extent * isz))
         sig = []
+        if any(t.take_axis is not None for t in self.tensors):
+            sig.append(("gather",))      # extent of a gather view is data dependent: assume overlap
         for i in range(len(spans)):
             for j in range(i + 1, len(spans)):
                 if spans[i][0] < spans[j][1] and spans[j][0] < spans[i][1]:

@@ -143,7 +143,7 @@ def _vector_width(prog, single_row_tail_ok):
     hot0 = [prog.tensors[n.slot] for n in used if n.kind == "H" and n.axis == 0]
     if not cols and not hot0:
         return 1
-    if any(t.strides[1] != 1 for t in cols):
+    if any(t.strides[1] != 1 or t.take_axis == 1 for t in cols):
         return 1
     isz_min = min([t.dtype.itemsize for t in cols] + [4 for _ in hot0])
     V = min(8, 16 // isz_min)
@@ -184,6 +184,8 @@ def _try_flatten(prog):
     if R == 1:
         return
     for t in prog.tensors:
+        if t.take_axis is not None or t.index in prog.index_slots:
+            return
         if t.shape == (1, 1):
             continue
         if t.shape != (R, C) or t.strides != (C, 1):

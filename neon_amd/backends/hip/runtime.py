@@ -87,6 +87,7 @@ SIGNATURES = {
                                  c_float, c_float, c_float, c_float, c_size_t, c_void_p]),
     "nh_rownorm_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_uint32,
                                c_uint32, c_size_t, c_void_p]),
+    "nh_hist_log2": (c_int, [c_void_p, c_void_p, c_int, c_size_t, c_int, c_int, c_void_p]),
     "nh_colreduce_workspace_bytes": (c_size_t, [c_uint32, c_uint32]),
     "nh_colmax_argmax_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_uint32, c_uint32,
                                      c_size_t, c_void_p, c_void_p]),
@@ -248,6 +249,10 @@ class Runtime(object):
         _check(self.lib.nh_launch_timed(kernel.function, g, b, lds_bytes, self.stream,
                                         args, kernel.arg_bytes, reps, byref(ms)))
         return ms.value
+
+    def hist_log2(self, hist_ptr, x_ptr, itemsize, n, nbins, offset):
+        _check(self.lib.nh_hist_log2(c_void_p(hist_ptr), c_void_p(x_ptr), itemsize, n, nbins, offset,
+                                     self.stream))
 
     def shutdown(self):
         self.lib.nh_shutdown()

@@ -100,7 +100,8 @@ class HIPTensor(Tensor):
         self.is_contiguous = (not take_array and
                               self.strides == _contiguous_strides(self.shape))
         # identity for the launch cache: same memory + same layout = same kernel arguments
-        self._geom = (self.gpudata, self.shape, self.strides, dtype.char, id(take_array) if take_array else 0)
+        self._geom = (self.gpudata, self.shape, self.strides, dtype.char,
+                      (take_array[0]._geom, take_array[1]) if take_array else 0)
 
     def __del__(self):
         if getattr(self, "_owns", False) and self.gpudata:
@@ -332,6 +333,19 @@ class HIPTensor(Tensor):
             return OpTreeNode.build("assign", out, self.T)
         return self.T
 
+    def hist(self, tag):
+        """log2-magnitude histogram of the tensor into the backend's buffer row
+        for ``tag`` (reference nervanagpu.py:620-638)"""
+        be = self.backend
+        src = self
+        if not self.is_contiguous or self.dtype.itemsize not in (2, 4) or self.dtype.kind != "f":
+            src = be.empty(self.shape, np.float32)
+            src.copy(self)
+        out = be._hist_tensor(tag)
+        be._flush()
+        be.rt.hist_log2(out.gpudata, src.gpudata, src.dtype.itemsize, src.size, be.hist_bins, be.hist_offset)
+        return out
+
     def share(self, shape, dtype=None, name=None):
         """New tensor over the first ``prod(shape)`` elements of this one's
         memory (reference nervanagpu.py:589-618)."""
@@ -447,6 +461,7 @@ class NervanaHIP(Backend):
         self.stream = None
         self.use_pinned_mem = False
         self.hist_bins, self.hist_offset = hist_bins, hist_offset
+        self.hist_base, self.hist_map, self.hist_idx, self.hist_max = None, dict(), 0, 4 * 4096
         self.cu_count = int(self.rt.props.compute_units)
         self.kernels = KernelCache(self.rt.arch.split(":")[0], cache_dir)
         self.plans = {}
@@ -880,8 +895,37 @@ class NervanaHIP(Backend):
             devlist[buf_index] = self.empty_like(hostlist[buf_index])
         devlist[buf_index].set(hostlist[buf_index])
 
+    # -- histograms (reference nervanagpu.py:620-638, 826-841, 1077-1097) --------------------
     def set_hist_buffers(self, hist_bins, hist_offset):
-        self.hist_bins, self.hist_offset = hist_bins, hist_offset
+        """(re)allocate the contiguous buffer that holds one row of bins per
+        tagged tensor"""
+        if (hist_bins != self.hist_bins or hist_offset != self.hist_offset or self.hist_base is None):
+            self.hist_bins, self.hist_offset = hist_bins, hist_offset
+            self.hist_map = dict()
+            self.hist_idx = 0
+            self.hist_max = 4 * 4096
+            self.hist_base = HIPTensor(self, (self.hist_max, self.hist_bins), dtype=np.int32)
+            self.hist_base._assign(0)
+
+    def _hist_tensor(self, tag):
+        """row of the histogram buffer for ``tag``"""
+        if self.hist_base is None:
+            self.set_hist_buffers(self.hist_bins, self.hist_offset)
+        assert self.hist_idx < self.hist_max
+        self.hist_map[tag] = self.hist_idx
+        row = self.hist_base[self.hist_idx]
+        self.hist_idx += 1
+        row.name = tag
+        return row
+
+    def dump_hist_data(self):
+        """all histograms recorded so far as a host array + the tag -> row map;
+        recording starts over"""
+        data = self.hist_base[0:max(self.hist_idx, 1)].get()[:self.hist_idx]
+        hist_map = self.hist_map
+        self.hist_map = dict()
+        self.hist_idx = 0
+        return data, hist_map
 
 
 def _splittable(tree):

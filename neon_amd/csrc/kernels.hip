@@ -352,6 +352,38 @@ __global__ __launch_bounds__(CR_T) void colmax_kernel(const float* __restrict__ 
     }
 }
 
+// ---------------------------------------------------------------------------
+// log2-magnitude histogram (the reference's kernel_histo, float_ew.py:1070-1131,
+// with the binning of its CPU backend, nervanacpu.py:424-445): value v lands in
+// bin clamp(rint(log2|v|) - offset, 0, ...); bin 0 extends to -inf (zeros), the
+// last bin is closed at offset+nbins, anything larger is not counted.
+// Integer counts, LDS atomics per workgroup, one global atomic per bin and
+// workgroup: the result does not depend on scheduling.
+// ---------------------------------------------------------------------------
+constexpr int HIST_T = 256;
+constexpr int HIST_MAX_BINS = 256;
+
+template <typename T>
+__global__ __launch_bounds__(HIST_T) void hist_log2_kernel(const T* __restrict__ x, size_t n, int nbins, int offset,
+                                                           int* __restrict__ hist) {
+    __shared__ int bins[HIST_MAX_BINS];
+    for (int b = threadIdx.x; b < nbins; b += HIST_T) bins[b] = 0;
+    __syncthreads();
+    const size_t stride = (size_t)gridDim.x * HIST_T;
+    for (size_t i = (size_t)blockIdx.x * HIST_T + threadIdx.x; i < n; i += stride) {
+        const float v = rintf(log2f(__builtin_fabsf((float)x[i])));
+        const float b = v - (float)offset;           // nan compares false everywhere: not counted
+        if (b <= (float)nbins) {
+            int bin = b < 1.0f ? 0 : (int)b;
+            if (bin > nbins - 1) bin = nbins - 1;
+            atomicAdd(&bins[bin], 1);
+        }
+    }
+    __syncthreads();
+    for (int b = threadIdx.x; b < nbins; b += HIST_T)
+        if (bins[b]) atomicAdd(&hist[b], bins[b]);
+}
+
 struct CrPlan { uint32_t strips, chunks, rows_per_chunk; int v; };
 
 CrPlan cr_plan(uint32_t rows, uint32_t cols, bool vec) {
@@ -426,6 +458,28 @@ int nh_rownorm_f16(uint16_t* out, const uint16_t* x, const float* gamma, const f
         default: launch_rownorm<16>(out, x, gamma, beta, eps, rows, cols, ld, s); break;
     }
     return launch_status("nh_rownorm_f16");
+}
+
+int nh_hist_log2(int32_t* hist, const void* x, int itemsize, size_t n, int nbins, int offset, void* stream) {
+    if (!nh_internal_ready()) return nh_internal_fail(NH_ENOTINIT, "nh_init has not been called");
+    if (!hist || (n && !x)) return nh_internal_fail(NH_EINVAL, "nh_hist_log2: null pointer");
+    if (nbins < 1 || nbins > HIST_MAX_BINS) return nh_internal_fail(NH_EINVAL, "nh_hist_log2: nbins out of range");
+    if (itemsize != 4 && itemsize != 2) return nh_internal_fail(NH_EINVAL, "nh_hist_log2: fp32 or fp16 input only");
+    hipStream_t s = (hipStream_t)stream;
+    hipError_t e = hipMemsetAsync(hist, 0, sizeof(int32_t) * (size_t)nbins, s);
+    if (e != hipSuccess) return nh_internal_fail((int)e, "nh_hist_log2: clearing the bins failed");
+    if (n == 0) return 0;
+    size_t blocks = (n + HIST_T * 16 - 1) / ((size_t)HIST_T * 16);
+    const size_t cap = (size_t)(nh_internal_cu_count() > 0 ? nh_internal_cu_count() : 256) * 8;
+    if (blocks > cap) blocks = cap;
+    if (blocks < 1) blocks = 1;
+    if (itemsize == 4)
+        hipLaunchKernelGGL((hist_log2_kernel<float>), dim3((unsigned)blocks), dim3(HIST_T), 0, s, (const float*)x, n,
+                           nbins, offset, (int*)hist);
+    else
+        hipLaunchKernelGGL((hist_log2_kernel<nh_f16>), dim3((unsigned)blocks), dim3(HIST_T), 0, s, (const nh_f16*)x, n,
+                           nbins, offset, (int*)hist);
+    return launch_status("nh_hist_log2");
 }
 
 size_t nh_colreduce_workspace_bytes(uint32_t rows, uint32_t cols) {

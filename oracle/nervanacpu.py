@@ -212,6 +212,21 @@ class CPUTensor(Tensor):
                               dtype=self._tensor.dtype, base=self)
 
 
+def _cpu_hist(self, tag):
+    """log2-magnitude histogram (reference nervanacpu.py:424-445): log2 is taken
+    in fp32 whatever the dtype; the lowest bin reaches down to -inf"""
+    nbins, offset = self.backend.hist_bins, self.backend.hist_offset
+    bins = np.arange(nbins + 1) + float(offset)
+    bins[0] = -float("Inf")
+    with np.errstate(divide="ignore"):
+        log_abs = np.rint(np.log2(np.abs(self._tensor.astype(np.float32))))
+    counts, _ = np.histogram(log_abs, density=False, bins=bins)
+    return self.backend._hist_tensor(tag)._assign(counts.astype(np.int32).reshape(1, nbins))
+
+
+CPUTensor.hist = _cpu_hist
+
+
 def _arg_keepdims(fn):
     """np.argmax/np.argmin with the reduced axis kept
     (reference nervanacpu.py:453-473): first occurrence, int64."""
@@ -425,6 +440,23 @@ class NervanaCPU(Backend):
         grad_beta[:] = self.sum(delta_in, axis=1)
         xtmp = (xhat * grad_gamma + grad_beta) / float(x.shape[1])
         delta_out.reshape(delta_in.shape)[:] = ((delta_in - xtmp) * gamma) * inv_v
+
+    # -- histogram buffers (reference nervanacpu.py:1767-1800) ------------------------
+    def set_hist_buffers(self, hist_bins, hist_offset):
+        self.hist_bins, self.hist_offset = hist_bins, hist_offset
+        self.hist_max = 4 * 4096
+        self.hist_buf = self.empty((self.hist_max, hist_bins), dtype=np.int32)
+        self.hist_idx = 0
+        self.hist_map = dict()
+
+    def _hist_tensor(self, tag):
+        if getattr(self, "hist_buf", None) is None:
+            self.set_hist_buffers(self.hist_bins, self.hist_offset)
+        assert self.hist_idx < self.hist_max
+        self.hist_map[tag] = self.hist_idx
+        row = self.hist_buf[self.hist_idx]
+        self.hist_idx += 1
+        return row
 
     # -- timing marks (reference nervanacpu.py:1865-1905) -------------------------
     def init_mark(self):

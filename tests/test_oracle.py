@@ -285,6 +285,25 @@ def test_onehot_forms_agree(cpu, axis):
     assert np.array_equal(a.get(), b.get())
 
 
+def test_hist_bruteforce(cpu):
+    """Tensor.hist (tests/test_backend_hist.py:24-40): per-element binning done
+    here with math.log2 and Python's round-half-even"""
+    vals = [0.0, 1.0, 2.0, 3.0, -4.0, 1e-20, 1e30, 2.0 ** -48, 2.0 ** 16, 2.0 ** 15.4, -0.75, 6.0, 2.0 ** -47]
+    a = np.array(vals, dtype=np.float32).reshape(1, -1)
+    want = [0] * 64
+    for v in a.ravel():
+        v = abs(float(v))
+        if v == 0.0:
+            want[0] += 1
+            continue
+        b = round(math.log2(v)) + 48
+        if b > 64:
+            continue                    # beyond the last (closed) bin edge
+        want[min(max(b, 0), 63)] += 1
+    got = cpu.array(a).hist("t").get()
+    assert got.shape == (1, 64) and got.ravel().tolist() == want
+
+
 # ---------------------------------------------------------------------------
 # views (tests/test_backend_tensor.py:252-315)
 # ---------------------------------------------------------------------------
