@@ -96,6 +96,7 @@ class _Gen(object):
         self.L = _Lines()
         # streaming kernels (working set far beyond the caches) mark their
         # global accesses non-temporal
+        self.pos = ("0", "0")      # (row, column) expressions of the element being emitted
         self.ld = "load_stream" if stream else "load"
         self.st = "store_stream" if stream else "store"
 
@@ -122,6 +123,9 @@ class _Gen(object):
             fmt += "f"
         ps += ["int R", "int C"]
         fmt += "ii"
+        if self.prog.rand_count:
+            ps += ["unsigned int rng_seed", "unsigned long long rng_base"]
+            fmt += "IQ"
         for decl, f in extras:
             ps.append(decl)
             fmt += f
@@ -196,6 +200,10 @@ class _Gen(object):
                 e = "nh_quant<%s>(%s)" % (CTYPE[n.op.split(":")[1]], a[0])
             elif n.op == "zero_index":
                 e = "0.0f"
+            elif n.op == "rand":
+                r, c = self.pos
+                e = ("nh_rand01(rng_seed, rng_base + ((unsigned long long)(%s) * (unsigned long long)C + "
+                     "(unsigned long long)((%s) + j)) * %dull + %dull)" % (r, c, self.prog.rand_count, n.slot))
             elif len(a) == 1:
                 e = _UN[n.op].format(*a)
             else:
@@ -246,6 +254,8 @@ def gen_ew(prog, V, LX, LY, UC, UR, tail, stream=False):
     leaves = g.leaf_nodes(nodes)
 
     def ref_for(sfx, r, c, Vv):
+        g.pos = (r, c)
+
         def ref(n):
             if n.kind == "C":
                 return "k%d" % n.slot
@@ -378,6 +388,8 @@ class _RedGen(_Gen):
         return ("(float)ri%d" % n.nid) if n.is_index else ("rv%d" % n.nid)
 
     def make_ref(self, sfx, r, c, Vv, tiles=None, vals=None):
+        self.pos = (r, c)
+
         def ref(n):
             if vals and n.nid in vals:
                 return vals[n.nid]

@@ -224,6 +224,8 @@ class Program(object):
         self._current = {}         # tensor slot index -> node holding its newest value
         self.key_parts = []
         self.index_slots = set()   # slots used only as index vectors of gather views
+        self.rand_count = 0        # number of rand nodes (each draws its own stream)
+        self.rng_args = (0, 0)     # (seed, first counter) bound by the backend before a launch
         self.raw_count = 0         # numbers seen so far, in postfix order
         self.const_exprs = []      # per constant slot: expressions that produced its value
         self.axis = None           # the one reduction axis, if any
@@ -380,7 +382,13 @@ class Program(object):
             self.key_parts.append(("onehot", slot.index, axis))
             stack.append(self._intern(("H", slot.index, axis),
                                       lambda: Node("H", op="onehot", slot=slot.index, axis=axis)))
-        elif op in ("dot", "transpose", "rand", "binarize", "shift", "assign"):
+        elif op == "rand":
+            # uniform [0, 1): every occurrence is its own stream (never merged)
+            ordinal = self.rand_count
+            self.rand_count += 1
+            self.key_parts.append("rand")
+            stack.append(self._intern(("rand", ordinal), lambda: Node("E", op="rand", slot=ordinal)))
+        elif op in ("dot", "transpose", "binarize", "shift", "assign"):
             raise NotImplementedError("op '%s' cannot be part of a fused op-tree kernel" % op)
         else:
             raise TypeError("%s is not a valid operation" % op)
@@ -420,6 +428,8 @@ class Program(object):
             elif n.kind == "H":
                 # one-hot of a vector of indices: full variance wherever the
                 # index vector and the hot axis have extent
+                n.vr, n.vc, n.level = R > 1, C > 1, 0
+            elif n.kind == "E" and not n.args:       # rand: varies wherever the domain has extent
                 n.vr, n.vc, n.level = R > 1, C > 1, 0
             elif n.kind == "E":
                 n.vr = any(a.vr for a in n.args)

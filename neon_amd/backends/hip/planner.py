@@ -227,6 +227,8 @@ class Plan(object):
         vals.extend(prog.consts)
         vals.append(self.domain[0])
         vals.append(self.domain[1])
+        if prog.rand_count:
+            vals.extend(prog.rng_args)
         if self.extras_fn is not None:
             vals.extend(self.extras_fn())
         try:

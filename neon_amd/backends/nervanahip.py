@@ -506,6 +506,55 @@ class NervanaHIP(Backend):
         self._flush()
         self.rt.synchronize()
 
+    # -- random numbers (reference nervanagpu.py:901-1049, 1825-1861) ---------------------
+    def gen_rng(self, seed=None):
+        """host RandomState plus the device generator's (seed, counter).  The
+        device generator is counter based (nh_rand01): no state on the device,
+        so get/set/reset are a pair of integers."""
+        self.rng = np.random.RandomState(seed)
+        self.init_rng_state = self.rng.get_state()
+        if seed is None:
+            dev_seed = int(np.random.randint(0, 2 ** 31 - 1))
+        else:
+            dev_seed = int(seed) & 0xFFFFFFFF
+        self._rng_dev_seed, self._rng_dev_counter = dev_seed, 0
+        self.init_rng_state_dev = (dev_seed, 0)
+        return self.rng
+
+    def rng_reset(self):
+        self.rng_set_state((self.init_rng_state, self.init_rng_state_dev))
+
+    def rng_get_state(self):
+        return (self.rng.get_state(), (self._rng_dev_seed, self._rng_dev_counter))
+
+    def rng_set_state(self, rng_states):
+        if len(rng_states) != 2 or not isinstance(rng_states[1], tuple) or len(rng_states[1]) != 2:
+            # a host-only state (e.g. saved by the CPU backend)
+            self.rng_reset()
+            self.rng.set_state(rng_states)
+            return
+        self.rng.set_state(rng_states[0])
+        self._rng_dev_seed, self._rng_dev_counter = int(rng_states[1][0]), int(rng_states[1][1])
+
+    def rand(self, out=None):
+        """uniform [0, 1) as an op-tree leaf"""
+        return OpTreeNode.build("rand", None, None, out=out)
+
+    def dropout(self, keep=0.5, out=None):
+        """keep mask: 1 where a uniform draw is <= ``keep``"""
+        return self.less_equal(self.rand(), keep, out=out)
+
+    def make_binary_mask(self, out, keepthresh=0.5):
+        self.dropout(keep=keepthresh, out=out)
+
+    def fill_normal(self, ary, mean=0, stdv=1):
+        """normally distributed values from the host generator"""
+        vals = (self.rng.standard_normal(ary.shape) * stdv + mean).astype(ary.dtype)
+        if ary.is_contiguous:
+            ary.set(vals)
+        else:
+            ary[:] = self.array(vals, dtype=ary.dtype)
+
     # -- allocation API (reference nervanagpu.py:1285-1439) --------------------------
     def empty(self, shape, dtype=None, name=None, persist_values=True,
               parallel=False, distributed=False, allocator=None):
@@ -636,6 +685,8 @@ class NervanaHIP(Backend):
         for tree in trees:
             for p in tree.traverse([]):
                 if type(p) is dict:
+                    if p["op"] == "rand":
+                        raise TypeError("random trees are never replayed")
                     if "axis" in p:
                         if p["op"] == "onehot":
                             add(("onehot", p["axis"], p["idx"]._geom))
@@ -696,6 +747,11 @@ class NervanaHIP(Backend):
                     self._launch_cache[key] = _Recorded(rec, temps, raw, single)
 
     def _launch_plan(self, plan, prog):
+        if prog.rand_count:
+            # counter-based generator: this launch owns the next R*C*streams counters
+            n = plan.domain[0] * plan.domain[1] * prog.rand_count
+            prog.rng_args = (self._rng_dev_seed, self._rng_dev_counter)
+            self._rng_dev_counter += n
         args = plan.pack(prog)
         self.rt.launch_packed(plan.kernel, plan.grid, plan.block, args)
         if self._recording is not None:

@@ -242,6 +242,19 @@ NEON_DEV float nh_sig2(float x) { return 1.0f / (1.0f + exp2f(-x)); }
 NEON_DEV float nh_tanh2(float x) { const float e = exp2f(2.0f * x); return (e - 1.0f) / (e + 1.0f); }
 NEON_DEV float nh_finite(float x) { return (__builtin_fabsf(x) <= NH_FLT_MAX) ? 1.0f : 0.0f; }
 
+// Counter-based uniform random numbers in [0, 1): element `counter` of the
+// stream `seed` (splitmix64 finaliser, top 24 bits).  Stateless, so a tensor
+// filled twice from the same (seed, counter) gets the same values and no
+// generator state lives on the device (the reference kept a pool of LFSR
+// states, cuda_templates.py:138-186).
+NEON_DEV float nh_rand01(nh_u32 seed, unsigned long long counter) {
+    unsigned long long z = counter + ((unsigned long long)seed + 1ull) * 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    return (float)(nh_u32)(z >> 40) * 5.9604644775390625e-8f;      // 2^-24
+}
+
 // ---------------------------------------------------------------------------
 // DPP lane permutations.  Every lane of the wave must be active at the call.
 // ---------------------------------------------------------------------------
