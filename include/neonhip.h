@@ -176,6 +176,17 @@ int nh_colmax_argmax_f32(float* maxval, int32_t* argmax, const float* x,
 int nh_hist_log2(int32_t* hist, const void* x, int itemsize, size_t n, int nbins,
                  int offset, void* stream);
 
+/* Dense contraction hand-off: C[m,n] = alpha * op(A) * op(B) + beta * C on
+ * row-major operands; op(X) = X^T when trans_x != 0; lda/ldb/ldc = elements
+ * between consecutive stored rows; itemsize 4 = fp32, 2 = fp16 storage with
+ * fp32 accumulation.  Forwards to rocBLAS (opened on first use).  Replaces the
+ * library GEMM behind NervanaGPU.compound_dot / cublas_dot
+ * (neon/backends/nervanagpu.py:1441-1470, 3012-3044), which `dot` nodes inside
+ * op-trees are staged through (nervanagpu.py:1099-1237).                      */
+int nh_gemm(int itemsize, int trans_a, int trans_b, uint32_t m, uint32_t n, uint32_t k,
+            float alpha, const void* a, size_t lda, const void* b, size_t ldb,
+            float beta, void* c, size_t ldc, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -88,6 +88,8 @@ SIGNATURES = {
     "nh_rownorm_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_uint32,
                                c_uint32, c_size_t, c_void_p]),
     "nh_hist_log2": (c_int, [c_void_p, c_void_p, c_int, c_size_t, c_int, c_int, c_void_p]),
+    "nh_gemm": (c_int, [c_int, c_int, c_int, c_uint32, c_uint32, c_uint32, c_float, c_void_p, c_size_t,
+                        c_void_p, c_size_t, c_float, c_void_p, c_size_t, c_void_p]),
     "nh_colreduce_workspace_bytes": (c_size_t, [c_uint32, c_uint32]),
     "nh_colmax_argmax_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_uint32, c_uint32,
                                      c_size_t, c_void_p, c_void_p]),
@@ -253,6 +255,10 @@ class Runtime(object):
     def hist_log2(self, hist_ptr, x_ptr, itemsize, n, nbins, offset):
         _check(self.lib.nh_hist_log2(c_void_p(hist_ptr), c_void_p(x_ptr), itemsize, n, nbins, offset,
                                      self.stream))
+
+    def gemm(self, itemsize, trans_a, trans_b, m, n, k, alpha, a_ptr, lda, b_ptr, ldb, beta, c_ptr, ldc):
+        _check(self.lib.nh_gemm(itemsize, int(trans_a), int(trans_b), m, n, k, alpha, c_void_p(a_ptr), lda,
+                                c_void_p(b_ptr), ldb, beta, c_void_p(c_ptr), ldc, self.stream))
 
     def shutdown(self):
         self.lib.nh_shutdown()

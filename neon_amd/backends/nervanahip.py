@@ -473,6 +473,7 @@ class NervanaHIP(Backend):
         self._launch_cache = {}      # statement-group identity -> recorded launches
         self._recording = None
         self._rec_temps = None
+        self._rec_foreign = False     # the group being recorded made a call that is not a kernel launch
         self._rec_single = None
         self._temp_pool = {}
         self._live_allocs = 0
@@ -731,6 +732,7 @@ class NervanaHIP(Backend):
         outer = self._recording is None
         if outer:
             self._recording, self._rec_temps, self._rec_single = [], [], None
+            self._rec_foreign = False
         ok = False
         try:
             self._run_slow(trees)
@@ -739,7 +741,7 @@ class NervanaHIP(Backend):
             if outer:
                 rec, temps, single = self._recording, self._rec_temps, self._rec_single
                 self._recording, self._rec_temps, self._rec_single = None, None, None
-                if ok and key is not None:
+                if ok and key is not None and not self._rec_foreign:
                     if len(self._launch_cache) >= 8192:
                         self._launch_cache.clear()
                     if len(rec) != 1:
@@ -823,10 +825,27 @@ class NervanaHIP(Backend):
             if not isinstance(node, OpTreeNode):
                 return node
             op = node[0]["op"]
-            if op == "dot":
-                raise NotImplementedError("dot inside an op-tree is outside the hip backend's scope")
             left = lower(node[1])
             right = lower(node[2])
+            if op == "dot":
+                # operands that are themselves expressions are evaluated into
+                # temporaries, the product goes through the GEMM hand-off
+                ops = []
+                for side in (left, right):
+                    if isinstance(side, OpTreeNode):
+                        tmp = self._temp(side.shape, np.float32, temps)
+                        self._run([OpTreeNode({"op": "assign"}, tmp, side)])
+                        side = tmp
+                    ops.append(side)
+                if ops[0].dtype != ops[1].dtype:
+                    for i, side in enumerate(ops):
+                        if side.dtype != np.float32:
+                            tmp = self._temp(side.shape, np.float32, temps)
+                            self._run([OpTreeNode({"op": "assign"}, tmp, side)])
+                            ops[i] = tmp
+                tmp = self._temp(node[0]["shape"], ops[0].dtype, temps)
+                self._gemm(ops[0], ops[1], tmp, 1.0, 0.0, temps)
+                return tmp
             if op == "transpose":
                 if isinstance(left, HIPTensor):
                     return left.T
@@ -883,6 +902,68 @@ class NervanaHIP(Backend):
         # kernels run in stream order, so the buffer may be handed out again as
         # soon as its last consumer has been enqueued
         self._temp_pool.setdefault((t.shape, t.dtype), []).append(t)
+
+    # -- dense contraction: handed to the library GEMM ---------------------------------------------
+    def _gemm_operand(self, t, temps):
+        """(tensor, transposed?, leading dimension) for a 2-D operand the GEMM
+        can read in place; anything else (gather views, doubly strided views)
+        is first copied into a dense temporary"""
+        rows, cols = t.shape
+        sr, sc = t.strides
+        if not t.take_array:
+            if cols == 1 or sc == 1:
+                if rows == 1 or sr >= cols:
+                    return t, False, max(sr, cols, 1)
+            if rows == 1 or sr == 1:
+                if cols == 1 or sc >= rows:
+                    return t, True, max(sc, rows, 1)
+        tmp = self._temp(t.shape, t.dtype, temps)
+        self._run([OpTreeNode({"op": "assign"}, tmp, t)])
+        return tmp, False, max(cols, 1)
+
+    def _gemm(self, A, B, C, alpha, beta, temps):
+        """C = alpha * A.B + beta * C for dense 2-D C (unit column stride)"""
+        m, k = A.shape
+        n = B.shape[1]
+        a, ta, lda = self._gemm_operand(A, temps)
+        b, tb, ldb = self._gemm_operand(B, temps)
+        self._rec_foreign = True      # a library call cannot be replayed from recorded launches
+        self.rt.gemm(C.dtype.itemsize, ta, tb, m, n, k, float(alpha), a.gpudata, lda,
+                     b.gpudata, ldb, float(beta), C.gpudata, max(C.strides[0], n, 1))
+
+    def compound_dot(self, A, B, C, alpha=1.0, beta=0.0, relu=False, bsum=None):
+        """C = alpha * A.B + beta * C; ``relu`` clamps the product term before
+        the beta term is added; ``bsum`` receives the row sums of the final C
+        (reference nervanagpu.py:1441-1470 with its cublas branch :3012-3044;
+        CPU statement order nervanacpu.py:906-960).  The product is the library
+        GEMM's, the ReLU / beta / row-sum epilogues are op-tree kernels."""
+        for t in (A, B, C):
+            assert isinstance(t, HIPTensor) and len(t.shape) == 2, "compound_dot takes 2-D tensors"
+        assert A.dtype == B.dtype == C.dtype
+        assert C.dtype.type in (np.float32, np.float16), "compound_dot takes float32 or float16 tensors"
+        assert A.shape[0] == C.shape[0]
+        assert B.shape[1] == C.shape[1]
+        assert A.shape[1] == B.shape[0]
+        self._flush()
+        temps = []
+        try:
+            dense = (not C.take_array and (C.shape[1] == 1 or C.strides[1] == 1) and
+                     (C.shape[0] == 1 or C.strides[0] >= C.shape[1]))
+            if dense and not (relu and beta != 0):
+                self._gemm(A, B, C, alpha, beta, temps)
+                if relu:
+                    self._run([self._stmt(C, self.maximum(C, 0))])
+            else:
+                prod = self._temp(C.shape, C.dtype, temps)
+                self._gemm(A, B, prod, alpha, 0.0, temps)
+                term = self.maximum(prod, 0) if relu else prod
+                self._run([self._stmt(C, term + beta * C if beta != 0 else term)])
+            if bsum is not None:
+                self._run([self._stmt(bsum, self.sum(C, 1))])
+        finally:
+            for t in temps:
+                self._temp_release(t)
+        return C
 
     # -- batch normalisation as fused statement groups -------------------------------------------
     @staticmethod
@@ -986,6 +1067,6 @@ class NervanaHIP(Backend):
 
 def _splittable(tree):
     for p in tree.traverse(list()):
-        if isinstance(p, dict) and p["op"] == "transpose":
+        if isinstance(p, dict) and p["op"] in ("transpose", "dot"):
             return True
     return False

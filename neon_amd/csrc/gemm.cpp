@@ -1,0 +1,104 @@
+// Dense contraction hand-off of libneonhip.so: nh_gemm forwards one row-major
+// GEMM to rocBLAS.  The library is opened on the first call, so processes that
+// only run op-trees never load it.
+#include "neonhip.h"
+
+#include <hip/hip_runtime.h>
+#include <rocblas/rocblas.h>
+
+#include <dlfcn.h>
+
+#include <mutex>
+#include <string>
+
+bool nh_internal_ready();
+int nh_internal_fail(int code, const char* msg);
+
+namespace {
+
+struct Blas {
+    void* lib = nullptr;
+    rocblas_handle handle = nullptr;
+    decltype(&rocblas_create_handle) create = nullptr;
+    decltype(&rocblas_destroy_handle) destroy = nullptr;
+    decltype(&rocblas_set_stream) set_stream = nullptr;
+    decltype(&rocblas_set_pointer_mode) set_pointer_mode = nullptr;
+    decltype(&rocblas_gemm_ex) gemm_ex = nullptr;
+    std::string error;
+    bool tried = false;
+};
+
+Blas g_blas;
+std::mutex g_blas_mutex;
+
+template <typename F>
+bool bind(F& fn, const char* name) {
+    fn = reinterpret_cast<F>(dlsym(g_blas.lib, name));
+    if (!fn) g_blas.error = std::string("librocblas lacks ") + name;
+    return fn != nullptr;
+}
+
+// caller holds g_blas_mutex
+bool blas_ready() {
+    if (g_blas.handle) return true;
+    if (g_blas.tried) return false;
+    g_blas.tried = true;
+    for (const char* name : {"librocblas.so.5", "librocblas.so", "/opt/rocm/lib/librocblas.so"}) {
+        g_blas.lib = dlopen(name, RTLD_NOW | RTLD_LOCAL);
+        if (g_blas.lib) break;
+    }
+    if (!g_blas.lib) {
+        const char* why = dlerror();
+        g_blas.error = std::string("cannot open librocblas: ") + (why ? why : "unknown");
+        return false;
+    }
+    if (!bind(g_blas.create, "rocblas_create_handle") || !bind(g_blas.destroy, "rocblas_destroy_handle") ||
+        !bind(g_blas.set_stream, "rocblas_set_stream") ||
+        !bind(g_blas.set_pointer_mode, "rocblas_set_pointer_mode") || !bind(g_blas.gemm_ex, "rocblas_gemm_ex"))
+        return false;
+    rocblas_status st = g_blas.create(&g_blas.handle);
+    if (st != rocblas_status_success) {
+        g_blas.handle = nullptr;
+        g_blas.error = "rocblas_create_handle failed with status " + std::to_string((int)st);
+        return false;
+    }
+    g_blas.set_pointer_mode(g_blas.handle, rocblas_pointer_mode_host);
+    return true;
+}
+
+}  // namespace
+
+extern "C" int nh_gemm(int itemsize, int trans_a, int trans_b, uint32_t m, uint32_t n, uint32_t k,
+                       float alpha, const void* a, size_t lda, const void* b, size_t ldb,
+                       float beta, void* c, size_t ldc, void* stream) {
+    if (!nh_internal_ready()) return nh_internal_fail(NH_ENOTINIT, "nh_init has not been called");
+    if (itemsize != 4 && itemsize != 2) return nh_internal_fail(NH_EINVAL, "nh_gemm: itemsize must be 4 (fp32) or 2 (fp16)");
+    if (m == 0 || n == 0) return 0;
+    if (!a || !b || !c) return nh_internal_fail(NH_EINVAL, "nh_gemm: null operand");
+    const size_t int_max = 0x7fffffff;
+    if (m > int_max || n > int_max || k > int_max || lda > int_max || ldb > int_max || ldc > int_max)
+        return nh_internal_fail(NH_EINVAL, "nh_gemm: extent beyond 2^31-1");
+    // leading dimensions are elements per stored row
+    const size_t need_a = trans_a ? m : k, need_b = trans_b ? k : n;
+    if (lda < (need_a ? need_a : 1) || ldb < (need_b ? need_b : 1) || ldc < n)
+        return nh_internal_fail(NH_EINVAL, "nh_gemm: leading dimension shorter than a stored row");
+
+    std::lock_guard<std::mutex> hold(g_blas_mutex);
+    if (!blas_ready()) return nh_internal_fail(NH_EINVAL, ("nh_gemm: " + g_blas.error).c_str());
+    rocblas_status st = g_blas.set_stream(g_blas.handle, (hipStream_t)stream);
+    if (st != rocblas_status_success) return nh_internal_fail(NH_EINVAL, "nh_gemm: rocblas_set_stream failed");
+    // A row-major matrix is its transpose in column-major storage, so
+    // C = op(A) op(B) becomes C^T = op(B)^T op(A)^T: operands swap places and
+    // keep their flags.
+    const rocblas_datatype t = itemsize == 4 ? rocblas_datatype_f32_r : rocblas_datatype_f16_r;
+    st = g_blas.gemm_ex(g_blas.handle,
+                        trans_b ? rocblas_operation_transpose : rocblas_operation_none,
+                        trans_a ? rocblas_operation_transpose : rocblas_operation_none,
+                        (rocblas_int)n, (rocblas_int)m, (rocblas_int)k, &alpha,
+                        b, t, (rocblas_int)ldb, a, t, (rocblas_int)lda, &beta,
+                        c, t, (rocblas_int)ldc, c, t, (rocblas_int)ldc,
+                        rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+    if (st != rocblas_status_success)
+        return nh_internal_fail(NH_EINVAL, ("nh_gemm: rocblas_gemm_ex failed with status " + std::to_string((int)st)).c_str());
+    return 0;
+}

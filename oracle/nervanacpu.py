@@ -412,6 +412,33 @@ class NervanaCPU(Backend):
     def zeros_like(self, ary, dtype=None, name=None, persist_values=True):
         return self.empty_like(ary, dtype, name, persist_values)
 
+    # -- dense contraction (reference nervanacpu.py:906-960) ------------------------
+    def compound_dot(self, A, B, C, alpha=1.0, beta=0.0, relu=False, bsum=None):
+        """C = alpha * A.B + beta * C, ReLU (if asked) on the product term before
+        the beta term is added, ``bsum`` = row sums of the final C.
+
+        One deliberate difference from nervanacpu.py:939-948: with beta == 0 that
+        code stores the bare product and drops ``alpha``; its own docstring
+        (:915-916) and the GPU backend (nervanagpu.py:1441-1470) apply it, and so
+        does this."""
+        assert A.dtype == B.dtype == C.dtype
+        assert A.shape[0] == C.shape[0]
+        assert B.shape[1] == C.shape[1]
+        assert A.shape[1] == B.shape[0]
+        prod = np.dot(A._tensor, B._tensor)
+        if alpha != 1.0:
+            prod = np.multiply(prod, np.asarray(alpha, dtype=prod.dtype))
+        if relu:
+            prod = np.maximum(prod, 0)
+        if beta == 0:
+            C._tensor[:] = prod
+        else:
+            np.multiply(C._tensor, np.asarray(beta, dtype=C._tensor.dtype), C._tensor)
+            np.add(C._tensor, prod, C._tensor)
+        if bsum is not None:
+            bsum[:] = self.sum(C, 1)
+        return C
+
     # -- batch normalisation (reference nervanacpu.py:1688-1760), non-binary path ---
     def compound_fprop_bn(self, x, xsum, xvar, gmean, gvar, gamma, beta, y, eps, rho,
                           compute_batch_sum, accumbeta=0.0, relu=False, binary=False,

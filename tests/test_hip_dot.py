@@ -1,0 +1,156 @@
+"""Dense contraction hand-off: compound_dot and `dot` nodes inside op-trees.
+
+The product itself is the library GEMM's; what is checked here is the operand
+plumbing (transposed views, strided views, leading dimensions), the alpha /
+beta / ReLU / row-sum epilogues and the staging of `dot` nodes through
+temporaries -- against the oracle backend and a float64 numpy product.
+"""
+import numpy as np
+import pytest
+
+from neon_amd.backends.autodiff import Autodiff
+from utils import assert_close
+
+
+def _rand(rs, shape, dtype=np.float32):
+    return (-1 + 2 * rs.rand(*shape)).astype(dtype)
+
+
+def _want(a, b, c, alpha, beta, relu):
+    prod = alpha * (a.astype(np.float64) @ b.astype(np.float64))
+    if relu:
+        prod = np.maximum(prod, 0)
+    return prod + beta * c.astype(np.float64)
+
+
+CASES = [
+    # m, n, k, transA, transB, alpha, beta, relu
+    (64, 48, 32, False, False, 1.0, 0.0, False),
+    (65, 47, 33, True, False, 1.0, 0.0, False),
+    (65, 47, 33, False, True, 1.0, 0.0, False),
+    (128, 256, 512, False, False, 0.5, 0.0, False),
+    (128, 256, 512, True, False, 2.0, 0.75, False),
+    (100, 30, 70, False, True, 1.5, -0.5, True),
+    (100, 30, 70, False, False, 1.0, 0.0, True),
+    (1, 40, 50, False, False, 1.0, 0.0, False),
+    (40, 1, 50, False, False, 1.0, 1.0, False),
+    (40, 1, 50, True, False, 1.0, 0.0, False),
+    (7, 9, 1, False, False, 1.0, 0.0, False),
+]
+
+
+def test_compound_dot_oracle(cpu):
+    rs = np.random.RandomState(0)
+    for m, n, k, ta, tb, alpha, beta, relu in CASES:
+        a = _rand(rs, (k, m) if ta else (m, k))
+        b = _rand(rs, (n, k) if tb else (k, n))
+        c = _rand(rs, (m, n))
+        A, B, C = cpu.array(a), cpu.array(b), cpu.array(c)
+        bsum = cpu.empty((m, 1))
+        cpu.compound_dot(A.T if ta else A, B.T if tb else B, C, alpha=alpha, beta=beta, relu=relu, bsum=bsum)
+        want = _want(a.T if ta else a, b.T if tb else b, c, alpha, beta, relu)
+        assert_close(C.get(), want.astype(np.float32), rtol=1e-4, atol=1e-4 * k)
+        assert_close(bsum.get(), want.sum(axis=1, keepdims=True).astype(np.float32), rtol=1e-4, atol=1e-4 * k * n)
+
+
+def test_dot_gradients_oracle(cpu):
+    """d sum(A.B * E) / dA = E.B^T and / dB = A^T.E"""
+    rs = np.random.RandomState(1)
+    a, b, e = _rand(rs, (6, 5)), _rand(rs, (5, 7)), _rand(rs, (6, 7))
+    A, B = cpu.array(a), cpu.array(b)
+    ga, gb = Autodiff(cpu.dot(A, B), cpu, next_error=cpu.array(e)).get_grad_asnumpyarray([A, B])
+    assert_close(ga, e @ b.T, rtol=1e-5, atol=1e-5)
+    assert_close(gb, a.T @ e, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-5), (np.float16, 2e-3)], ids=["f32", "f16"])
+@pytest.mark.parametrize("case", CASES, ids=[str(i) for i in range(len(CASES))])
+def test_compound_dot_hip(hip, case, dtype, tol):
+    m, n, k, ta, tb, alpha, beta, relu = case
+    rs = np.random.RandomState(m * 7 + n)
+    a = _rand(rs, (k, m) if ta else (m, k), dtype)
+    b = _rand(rs, (n, k) if tb else (k, n), dtype)
+    c = _rand(rs, (m, n), dtype)
+    A, B, C = hip.array(a, dtype=dtype), hip.array(b, dtype=dtype), hip.array(c, dtype=dtype)
+    bsum = hip.empty((m, 1), dtype=np.float32)
+    out = hip.compound_dot(A.T if ta else A, B.T if tb else B, C, alpha=alpha, beta=beta, relu=relu, bsum=bsum)
+    assert out is C
+    want = _want(a.T if ta else a, b.T if tb else b, c, alpha, beta, relu)
+    scale = max(1.0, np.abs(want).max())
+    got = C.get()
+    assert_close(got, want.astype(dtype), rtol=tol, atol=tol * scale)
+    # the row sums are those of the stored C
+    assert_close(bsum.get(), got.astype(np.float64).sum(axis=1, keepdims=True).astype(np.float32),
+                 rtol=1e-5, atol=1e-5 * scale * n)
+
+
+@pytest.mark.gpu
+def test_compound_dot_views_hip(pair):
+    cpu, hip = pair
+    rs = np.random.RandomState(5)
+    a, b, c = _rand(rs, (96, 80)), _rand(rs, (80, 72)), _rand(rs, (96, 100))
+    res = []
+    for be in pair:
+        A, B, C = be.array(a), be.array(b), be.array(c)
+        # row/column windows of the operands, a column window of the output
+        be.compound_dot(A[8:72, 16:64], B[16:64, 4:44], C[8:72, 30:70], alpha=1.0, beta=0.5)
+        # every second row of A is neither dense nor transposed: staged through a copy
+        be.compound_dot(A[0:64:2, :], B, C[0:32, 0:72])
+        res.append(C.get())
+    assert_close(res[1], res[0], rtol=1e-5, atol=1e-5 * 80)
+    assert np.array_equal(res[1][72:, :], c[72:, :])
+
+
+@pytest.mark.gpu
+def test_compound_dot_rejects_bad_operands(hip):
+    A, B, C = hip.zeros((4, 5)), hip.zeros((6, 3)), hip.zeros((4, 3))
+    with pytest.raises(AssertionError):
+        hip.compound_dot(A, B, C)
+    with pytest.raises(AssertionError):
+        hip.compound_dot(hip.zeros((4, 6), dtype=np.float16), B, C)
+
+
+def _func_dot(be, x0, x1, x2, x3, x4):
+    # reference tests/test_backend_autodiff.py Funcs.func_dot
+    return (x0 + x3) + be.dot(x1, x2) - (x1 - x2) - be.dot(x3, x4)
+
+
+def _func_dot_reduction_mix(be, x0, x1, x2, x3, x4):
+    # reference tests/test_backend_autodiff.py Funcs.func_dot_reduction_mix
+    f1 = be.max(x0, axis=1, keepdims=True)
+    f2 = be.min(x1, axis=0, keepdims=True)
+    f3 = be.dot(1. / x3, x2 + x4)
+    f4 = be.min(x3, axis=0, keepdims=True)
+    return f1 + f2 + f3 + f4
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("f", [_func_dot, _func_dot_reduction_mix], ids=["dot", "dot_reduction_mix"])
+@pytest.mark.parametrize("dim", [2, 48])
+def test_dot_in_optree_hip(pair, f, dim):
+    rs = np.random.RandomState(dim)
+    arrays = [(0.5 + rs.rand(dim, dim)).astype(np.float32) for _ in range(5)]
+    vals, grads = [], []
+    for be in pair:
+        tensors = [be.array(a) for a in arrays]
+        out = be.empty((dim, dim))
+        for _ in range(2):                       # second pass: nothing stale is replayed
+            out[:] = f(be, *tensors)
+        vals.append(out.get())
+        ad = Autodiff(f(be, *tensors), be)
+        grads.append(ad.get_grad_asnumpyarray(tensors))
+    assert_close(vals[1], vals[0], rtol=1e-5, atol=1e-5 * dim)
+    for g, w in zip(grads[1], grads[0]):
+        assert_close(g, w, rtol=1e-4, atol=1e-4 * max(1.0, np.abs(w).max()))
+
+
+@pytest.mark.gpu
+def test_dot_tree_sees_new_values_on_second_run(hip):
+    rs = np.random.RandomState(3)
+    a, b = _rand(rs, (32, 16)), _rand(rs, (16, 24))
+    A, B, out = hip.array(a), hip.array(b), hip.empty((32, 24))
+    out[:] = hip.dot(A, B) + 1.0
+    A[:] = A * 2.0
+    out[:] = hip.dot(A, B) + 1.0
+    assert_close(out.get(), (2 * a.astype(np.float64) @ b + 1.0).astype(np.float32), rtol=1e-5, atol=1e-5 * 16)
