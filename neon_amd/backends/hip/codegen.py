@@ -200,10 +200,15 @@ class _Gen(object):
                 e = "nh_quant<%s>(%s)" % (CTYPE[n.op.split(":")[1]], a[0])
             elif n.op == "zero_index":
                 e = "0.0f"
-            elif n.op == "rand":
+            elif n.op == "rand" or n.op.startswith("sround:"):
+                # counter = element index * streams + this node's stream
                 r, c = self.pos
-                e = ("nh_rand01(rng_seed, rng_base + ((unsigned long long)(%s) * (unsigned long long)C + "
-                     "(unsigned long long)((%s) + j)) * %dull + %dull)" % (r, c, self.prog.rand_count, n.slot))
+                counter = ("rng_base + ((unsigned long long)(%s) * (unsigned long long)C + "
+                           "(unsigned long long)((%s) + j)) * %dull + %dull" % (r, c, self.prog.rand_count, n.slot))
+                if n.op == "rand":
+                    e = "nh_rand01(rng_seed, %s)" % counter
+                else:
+                    e = "nh_sround(%s, %s, rng_seed, %s)" % (a[0], n.op.split(":")[1], counter)
             elif len(a) == 1:
                 e = _UN[n.op].format(*a)
             else:

@@ -142,6 +142,23 @@ class MixedAxes(ValueError):
     """Reductions along both axes in one tree: needs more than one kernel."""
 
 
+def stochastic_bits(tensor):
+    """Mantissa bits a store into ``tensor`` rounds to stochastically, 0 for
+    the ordinary round-to-nearest store (reference float_ew.py:832-844: True
+    means 10, at most 15 for float32 and 10 for float16 targets)."""
+    rounding = getattr(tensor, "rounding", 0)
+    if not rounding:
+        return 0
+    dtype = np.dtype(tensor.dtype)
+    if dtype == np.float32:
+        cap = 15
+    elif dtype == np.float16:
+        cap = 10
+    else:
+        raise NotImplementedError("stochastic rounding into %s tensors" % dtype)
+    return 10 if rounding is True else max(1, min(int(rounding), cap))
+
+
 class Node(object):
     """DAG node.  kind: 'T' tensor leaf, 'C' constant slot, 'E' elementwise op,
     'R' reduction, 'H' one-hot of an index tensor."""
@@ -320,6 +337,17 @@ class Program(object):
         root = stack[0]
         if not isinstance(root, Node):
             root = self.const_node(root)
+        bits = stochastic_bits(out_t)
+        if bits:
+            # the store rounds stochastically: one more random stream, applied
+            # to the value before it is converted to the storage type
+            ordinal = self.rand_count
+            self.rand_count += 1
+            self.key_parts.append(("sround", bits))
+            value_node = root
+            root = self._intern(("sround", ordinal),
+                                lambda: Node("E", op="sround:%d" % bits, args=(value_node,), slot=ordinal,
+                                             axis=out_slot.index))     # axis field: the slot stored to
         out_slot.written = True
         st = Statement(out_slot, root)
         self.statements.append(st)
@@ -431,6 +459,11 @@ class Program(object):
                 n.vr, n.vc, n.level = R > 1, C > 1, 0
             elif n.kind == "E" and not n.args:       # rand: varies wherever the domain has extent
                 n.vr, n.vc, n.level = R > 1, C > 1, 0
+            elif n.kind == "E" and n.op.startswith("sround:"):
+                # every stored element draws its own random number
+                if self.tensors[n.axis].shape != (R, C):
+                    raise NotImplementedError("stochastic rounding of an output narrower than the kernel's domain")
+                n.vr, n.vc, n.level = R > 1, C > 1, n.args[0].level
             elif n.kind == "E":
                 n.vr = any(a.vr for a in n.args)
                 n.vc = any(a.vc for a in n.args)

@@ -435,8 +435,9 @@ class NervanaHIP(Backend):
     """MI355X backend for the op-tree path.
 
     Arguments mirror ``gen_backend``'s keyword set (reference
-    neon/backends/__init__.py:107-114).  ``stochastic_round`` is accepted and
-    must be falsy: rounding is to nearest even.
+    neon/backends/__init__.py:107-114).  ``stochastic_round`` must be False,
+    as the reference insists: stochastic rounding is requested per tensor
+    through its ``rounding`` attribute (mantissa bits, or True for 10).
     """
     backend_name = "hip"
 
@@ -446,8 +447,9 @@ class NervanaHIP(Backend):
                  cache_dir=None):
         if default_dtype not in (np.float16, np.float32):
             raise ValueError("Default data type for the hip backend must be float16 or 32")
-        if stochastic_round:
-            raise NotImplementedError("stochastic rounding is not implemented by the hip backend")
+        # as in the reference (nervanagpu.py:768): rounding is a property of
+        # individual tensors (``tensor.rounding = bits``), never of the backend
+        assert stochastic_round is False, "Are you sure about using SR globally in the backend?"
         self.rt = None
         self.rt = hiprt.Runtime(device_id or 0)       # raises if library or device is missing
         if not self.rt.arch.startswith("gfx950"):
@@ -684,6 +686,8 @@ class NervanaHIP(Backend):
         parts, raw = [], []
         add = parts.append
         for tree in trees:
+            if tree[1].rounding:
+                raise TypeError("stochastically rounded stores are never replayed")
             for p in tree.traverse([]):
                 if type(p) is dict:
                     if p["op"] == "rand":
@@ -782,6 +786,20 @@ class NervanaHIP(Backend):
             if len(trees) != 1:
                 for t in trees:
                     self._run([t])
+                return
+            out, expr = trees[0][1], trees[0][2]
+            if out.rounding and isinstance(expr, OpTreeNode):
+                # a stochastically rounded store needs one value per element of
+                # the kernel's domain: evaluate into a float32 temporary of the
+                # output's shape first, then round while copying
+                temps = []
+                try:
+                    tmp = self._temp(out.shape, np.float32, temps)
+                    self._run([OpTreeNode({"op": "assign"}, tmp, expr)])
+                    self._run([OpTreeNode({"op": "assign"}, out, tmp)])
+                finally:
+                    for t in temps:
+                        self._temp_release(t)
                 return
             if isinstance(e, NotImplementedError) and not _splittable(trees[0]):
                 raise

@@ -247,12 +247,31 @@ NEON_DEV float nh_finite(float x) { return (__builtin_fabsf(x) <= NH_FLT_MAX) ? 
 // filled twice from the same (seed, counter) gets the same values and no
 // generator state lives on the device (the reference kept a pool of LFSR
 // states, cuda_templates.py:138-186).
-NEON_DEV float nh_rand01(nh_u32 seed, unsigned long long counter) {
+NEON_DEV nh_u32 nh_rand_u32(nh_u32 seed, unsigned long long counter) {
     unsigned long long z = counter + ((unsigned long long)seed + 1ull) * 0x9E3779B97F4A7C15ull;
     z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
     z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
     z ^= z >> 31;
-    return (float)(nh_u32)(z >> 40) * 5.9604644775390625e-8f;      // 2^-24
+    return (nh_u32)(z >> 32);
+}
+NEON_DEV float nh_rand01(nh_u32 seed, unsigned long long counter) {
+    return (float)(nh_rand_u32(seed, counter) >> 8) * 5.9604644775390625e-8f;      // 2^-24
+}
+
+// Stochastic rounding to `bits` (1..22) mantissa bits: the value moves to the
+// neighbour of larger magnitude with probability equal to the fraction of the
+// spacing it sits above the neighbour of smaller magnitude, so the result is
+// unbiased (the reference adds a uniform fraction of the spacing with
+// round-toward-zero and masks, cuda_templates.py:148-152, 193-235).  Done on
+// the bit pattern: random bits added below the kept mantissa bits carry into
+// them (and on into the exponent) with exactly that probability.  Infinities
+// and NaN pass through.
+NEON_DEV float nh_sround(float x, int bits, nh_u32 seed, unsigned long long counter) {
+    const nh_u32 b = __builtin_bit_cast(nh_u32, x);
+    if ((b & 0x7f800000u) == 0x7f800000u) return x;
+    const int drop = 23 - bits;
+    const nh_u32 noise = nh_rand_u32(seed, counter) >> (32 - drop);
+    return __builtin_bit_cast(float, (b + noise) & (0xffffffffu << drop));
 }
 
 // ---------------------------------------------------------------------------

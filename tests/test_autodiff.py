@@ -36,6 +36,18 @@ class _NP(object):
     def var(a, axis=None):
         return np.var(a, axis=axis, keepdims=True)
 
+    @staticmethod
+    def std(a, axis=None):
+        return np.std(a, axis=axis, keepdims=True)
+
+    @staticmethod
+    def argmax(a, axis=1):
+        return np.argmax(a, axis=axis).reshape((-1, 1) if axis == 1 else (1, -1))
+
+    @staticmethod
+    def argmin(a, axis=1):
+        return np.argmin(a, axis=axis).reshape((-1, 1) if axis == 1 else (1, -1))
+
     exp = staticmethod(np.exp)
     log = staticmethod(np.log)
     tanh = staticmethod(np.tanh)
@@ -81,6 +93,11 @@ FUNCS = [
      [(8, 12)] * 2, "rand"),
     ("softmax", lambda ns, a: ns.exp(a - ns.max(a, axis=0)) / ns.sum(ns.exp(a - ns.max(a, axis=0)), axis=0)
      * ns.exp(a), [(10, 6)], "rand"),
+    # reference tests/test_backend_autodiff_extra.py test_reduction: every reduction, with and without an axis
+    ("reduction_mix", lambda ns, a, b, c, d: (a + c) + ns.sum(a, axis=0) - (a - b) - ns.mean(d, axis=1)
+     + (c + d) + ns.var(a, axis=0) + (c + d) + ns.std(a) - (c - d) - ns.max(d, axis=1)
+     - (c - d) - ns.min(d, axis=0) - (c - d) - ns.argmax(d, axis=1) - (c - d) - ns.argmin(d, axis=0),
+     [(5, 7)] * 4, "rand"),
     # transposes of op-trees (a transposed *tensor* is a view and is keyed by its base)
     ("transpose", lambda ns, a, b: _T(ns, a * 2.0) * b + _T(ns, _T(ns, b * b) * a), [(5, 8), (8, 5)], "rand"),
 ]

@@ -154,3 +154,85 @@ def test_dot_tree_sees_new_values_on_second_run(hip):
     A[:] = A * 2.0
     out[:] = hip.dot(A, B) + 1.0
     assert_close(out.get(), (2 * a.astype(np.float64) @ b + 1.0).astype(np.float32), rtol=1e-5, atol=1e-5 * 16)
+
+
+class _Np(object):
+    """numpy float64 evaluation of the same builders"""
+    dot = staticmethod(np.dot)
+
+    @staticmethod
+    def var(a, axis=None, keepdims=True):
+        return np.var(a, axis=axis, keepdims=True)
+
+    @staticmethod
+    def std(a, axis=None, keepdims=True):
+        return np.std(a, axis=axis, keepdims=True)
+
+    @staticmethod
+    def max(a, axis=None, keepdims=True):
+        return np.max(a, axis=axis, keepdims=True)
+
+    @staticmethod
+    def min(a, axis=None, keepdims=True):
+        return np.min(a, axis=axis, keepdims=True)
+
+
+def _compound_mix(be, x0, x1, x2, x3, x4):
+    # reference tests/test_backend_compound_optree.py func_dot_reduction_mix
+    f1 = be.std(be.var(x0, axis=0, keepdims=True), axis=1, keepdims=True)
+    f2 = be.max(x1, axis=0, keepdims=True) + be.min(x1, axis=0, keepdims=True)
+    f3 = be.std(x2, keepdims=True)
+    f4 = be.dot(1.0 / x3, x4 / x2)
+    f5 = be.dot(x3, x4 - x0)
+    f6 = be.dot(x2 / f4, f5 + x3)
+    return f1 + f2 + f3 + f4 + 1.0 / (be.dot(f5, f6))
+
+
+def _compound_transpose_mix(be, x0, x1, x2, x3, x4):
+    # reference tests/test_backend_compound_optree.py func_dot_reduction_transpose_mix
+    f1 = be.std(be.var(x0, axis=0, keepdims=True), axis=1, keepdims=True)
+    f2 = be.max(x1, axis=0, keepdims=True) + be.min(x1, axis=0, keepdims=True)
+    f3 = be.std(x2, keepdims=True).T
+    f4 = be.dot(1.0 / x3, (x4 / x2).T).T
+    f5 = be.dot(x3, (x4 - x0).T)
+    f6 = be.dot(x2 / f4.T, f5 + x3).T
+    return f1 + f2 + f3 + f4 + 1.0 / (be.dot(f5, f6))
+
+
+def _compound_inputs(flag, dim):
+    rs = np.random.RandomState(17)
+    lo, hi = {"pos_rand": (0.5, 1.5), "neg_rand": (-1.5, -0.5), "rand": (0.5, 1.5)}[flag]
+    xs = [(lo + (hi - lo) * rs.rand(dim, dim)).astype(np.float32) for _ in range(5)]
+    if flag == "rand":           # mixed signs, kept away from the poles of the divisions
+        xs = [x * np.where(rs.rand(dim, dim) < 0.5, -1, 1).astype(np.float32) for x in xs]
+    return xs
+
+
+@pytest.mark.parametrize("f", [_compound_mix, _compound_transpose_mix], ids=["mix", "transpose_mix"])
+@pytest.mark.parametrize("flag", ["pos_rand", "neg_rand", "rand"])
+def test_compound_optree_oracle_vs_numpy(cpu, f, flag):
+    xs = _compound_inputs(flag, 2)
+    want = f(_Np(), *[x.astype(np.float64) for x in xs])
+    out = cpu.empty((2, 2))
+    out[:] = f(cpu, *[cpu.array(x) for x in xs])
+    # the reference's own bar for these trees (rtol = atol = 1e-2)
+    assert_close(out.get(), want.astype(np.float32), rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("f", [_compound_mix, _compound_transpose_mix], ids=["mix", "transpose_mix"])
+@pytest.mark.parametrize("flag", ["pos_rand", "neg_rand", "rand"])
+@pytest.mark.parametrize("dim", [2, 40])
+def test_compound_optree_hip(pair, f, flag, dim):
+    xs = _compound_inputs(flag, dim)
+    want = f(_Np(), *[x.astype(np.float64) for x in xs])
+    got = []
+    for be in pair:
+        out = be.empty((dim, dim))
+        out[:] = f(be, *[be.array(x) for x in xs])
+        got.append(out.get())
+    # chained products and reciprocals amplify rounding: compare both backends
+    # with float64 at a tolerance scaled by the condition of the final division
+    scale = max(1.0, np.abs(want).max())
+    assert_close(got[0], want.astype(np.float32), rtol=1e-2, atol=1e-2 * scale)
+    assert_close(got[1], want.astype(np.float32), rtol=1e-2, atol=1e-2 * scale)

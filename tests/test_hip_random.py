@@ -77,3 +77,97 @@ def test_reproducibility(hip):
     assert abs(d.mean()) < 0.02 and 0.1 < d.var() < 0.25
     be.fill_normal(a, mean=2.0, stdv=0.5)
     assert abs(a.get().mean() - 2.0) < 0.05
+
+
+# ---- stochastic rounding of stores (tensor.rounding = mantissa bits) --------------------------
+
+def _on_grid(values, bits):
+    """every value has at most `bits` mantissa bits set"""
+    b = np.asarray(values, dtype=np.float32).view(np.uint32)
+    return bool(np.all((b & np.uint32((1 << (23 - bits)) - 1)) == 0))
+
+
+def test_sr_one_bit_fp16(hip):
+    """reference tests/test_backend_sr.py test_sr: 1 + 0.1 stored with one
+    mantissa bit is 1.0 or 1.5, mostly 1.0"""
+    n = 10
+    A = hip.ones((n, n), dtype=np.float16)
+    B = hip.ones((n, n), dtype=np.float16)
+    hip.multiply(B, 0.1, out=B)
+    C = hip.ones((n, n), dtype=np.float16)
+    C.rounding = 1
+    C[:] = A + B
+    got = C.get().ravel()
+    assert np.all((got == 1.0) | (got == 1.5))
+    assert (got == 1.5).sum() > .1 * n ** 2
+    assert (got == 1.0).sum() > .7 * n ** 2
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
+@pytest.mark.parametrize("bits", [1, 3, 8, True])
+def test_sr_unbiased_neighbours(hip, dtype, bits):
+    rs = np.random.RandomState(11)
+    rows, cols = 64, 8192
+    x = ((0.25 + rs.rand(rows, 1)) * np.where(rs.rand(rows, 1) < 0.5, -1, 1)).astype(np.float32)
+    X = hip.array(x)
+    out = hip.empty((rows, cols), dtype=dtype)
+    out.rounding = bits
+    out[:] = X + hip.zeros((1, cols))                      # each row: one value, 8192 draws
+    got = out.get().astype(np.float32)
+    m = 10 if bits is True else bits
+    assert _on_grid(got, m)
+    ulp = 2.0 ** (np.floor(np.log2(np.abs(x))) - m)
+    lo = np.trunc(x / ulp) * ulp                           # neighbour toward zero
+    hi = lo + np.sign(x) * ulp
+    assert np.all((got == lo) | (got == hi))
+    # unbiased: the mean over many draws approaches the value (5 sigma of a
+    # two-point distribution with spread ulp)
+    err = np.abs(got.astype(np.float64).mean(axis=1, keepdims=True) - x)
+    assert np.all(err <= 5 * 0.5 * ulp / np.sqrt(cols) + 1e-7)
+
+
+def test_sr_leaves_representable_values_and_specials(hip):
+    x = np.array([[0.0, 1.0, -2.5, 0.75, np.inf, -np.inf, np.nan, 1024.0]], dtype=np.float32)
+    out = hip.empty(x.shape, dtype=np.float32)
+    out.rounding = 2
+    out[:] = hip.array(x) * 1.0
+    got = out.get()
+    assert np.array_equal(got[:, :4], x[:, :4])
+    assert got[0, 4] == np.inf and got[0, 5] == -np.inf and np.isnan(got[0, 6]) and got[0, 7] == 1024.0
+
+
+def test_sr_fresh_draws_each_time_and_reproducible_state(hip):
+    x = hip.array(np.full((64, 256), 1.3, dtype=np.float32))
+    out = hip.empty((64, 256), dtype=np.float16)
+    out.rounding = 2
+    state = hip.rng_get_state()
+    out[:] = x * 1.0
+    first = out.get()
+    out[:] = x * 1.0
+    second = out.get()
+    assert not np.array_equal(first, second)               # not a replay of the first launch
+    hip.rng_set_state(state)
+    out[:] = x * 1.0
+    assert np.array_equal(out.get(), first)
+
+
+def test_sr_reduced_output_and_fused_group(hip):
+    rs = np.random.RandomState(2)
+    x = rs.rand(128, 300).astype(np.float32)
+    X = hip.array(x)
+    sums = hip.empty((128, 1), dtype=np.float32)
+    sums.rounding = 4
+    sums[:] = hip.sum(X, axis=1)                           # staged: reduce, then round while copying
+    got = sums.get()
+    want = x.astype(np.float64).sum(axis=1, keepdims=True)
+    assert _on_grid(got, 4)
+    assert np.all(np.abs(got - want) <= 2.0 ** (np.floor(np.log2(want)) - 4) * 1.001)
+    # inside a fused group: the rounded tensor feeds the next statement rounded
+    a = hip.empty((128, 300), dtype=np.float16)
+    a.rounding = 3
+    b = hip.empty((128, 300), dtype=np.float32)
+    with hip.fused():
+        a[:] = X * 1.0
+        b[:] = a * 2.0
+    assert _on_grid(a.get().astype(np.float32), 3)
+    assert np.array_equal(b.get(), a.get().astype(np.float32) * 2.0)

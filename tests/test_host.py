@@ -248,3 +248,25 @@ def test_generated_kernels_compile_for_every_dtype(tmp_path, dtype, axis):
     be.empty(shape, np.int32)[:] = be.argmin(x, axis=axis)
     be.empty((96, 160), dtype)[:] = x - be.mean(x, axis=axis)
     assert be.cache.stats["compiled"] == 4
+
+
+def test_stochastic_rounding_store_compiles_and_changes_the_plan(tmp_path):
+    be = prebuild.PlanBackend(cache_dir=str(tmp_path / "kc"))
+    x = be.empty((96, 160))
+    plain = be.empty((96, 160), np.float16)
+    rounded = be.empty((96, 160), np.float16)
+    rounded.rounding = 3
+    plain[:] = x * 2.0
+    rounded[:] = x * 2.0
+    soft = be.empty((96, 160), np.float16)
+    soft.rounding = 3
+    soft[:] = x - be.max(x, axis=1)               # full-size output of a reduction tree
+    assert be.cache.stats["compiled"] == 3
+    narrow = be.empty((96, 1))
+    narrow.rounding = 3
+    with pytest.raises(NotImplementedError):      # the hip backend stages this one through a temporary
+        narrow[:] = be.sum(x, axis=1)
+    with pytest.raises(NotImplementedError):
+        bad = be.empty((4, 4), np.int32)
+        bad.rounding = 2
+        bad[:] = x[:4, :4] * 1.0
