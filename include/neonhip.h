@@ -187,6 +187,18 @@ int nh_gemm(int itemsize, int trans_a, int trans_b, uint32_t m, uint32_t n, uint
             float alpha, const void* a, size_t lda, const void* b, size_t ldb,
             float beta, void* c, size_t ldc, void* stream);
 
+/* Dimension shuffle, numpy.transpose(in, axes) written into `out`: `ndim`
+ * dimensions listed in OUTPUT order -- shape[i] is the extent of output
+ * dimension i, out_strides[i] its stride in `out` and in_strides[i] the stride
+ * of the input dimension it comes from (axes[i]), all in elements and
+ * non-negative.  Elements are moved as opaque `itemsize`-byte values (1, 2, 4
+ * or 8).  `out` and `in` must not overlap.  Replaces
+ * NervanaGPU.copy_transpose / _get_copy_transpose_kernel
+ * (neon/backends/nervanagpu.py:3077-3118).                                      */
+#define NH_TRANSPOSE_MAX_DIMS 8
+int nh_copy_transpose(void* out, const void* in, int itemsize, int ndim, const uint32_t* shape,
+                      const int64_t* out_strides, const int64_t* in_strides, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

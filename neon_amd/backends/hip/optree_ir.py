@@ -242,6 +242,9 @@ class Program(object):
         self.key_parts = []
         self.index_slots = set()   # slots used only as index vectors of gather views
         self.rand_count = 0        # number of rand nodes (each draws its own stream)
+        # ids of tensor objects whose reads mean "the value before this group
+        # ran" even after a statement of the group has assigned that memory
+        self.originals = frozenset()
         self.rng_args = (0, 0)     # (seed, first counter) bound by the backend before a launch
         self.raw_count = 0         # numbers seen so far, in postfix order
         self.const_exprs = []      # per constant slot: expressions that produced its value
@@ -357,8 +360,9 @@ class Program(object):
 
     def _read_tensor(self, t):
         slot = self.tensor_slot(t)
-        self.key_parts.append(("T", slot.index))
-        cur = self._current.get(slot.index)
+        original = id(t) in self.originals
+        self.key_parts.append(("T0" if original else "T", slot.index))
+        cur = None if original else self._current.get(slot.index)
         if cur is not None:
             # value written by an earlier statement of this program: forward it,
             # rounded the way the store rounds it

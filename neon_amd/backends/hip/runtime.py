@@ -90,6 +90,7 @@ SIGNATURES = {
     "nh_hist_log2": (c_int, [c_void_p, c_void_p, c_int, c_size_t, c_int, c_int, c_void_p]),
     "nh_gemm": (c_int, [c_int, c_int, c_int, c_uint32, c_uint32, c_uint32, c_float, c_void_p, c_size_t,
                         c_void_p, c_size_t, c_float, c_void_p, c_size_t, c_void_p]),
+    "nh_copy_transpose": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "nh_colreduce_workspace_bytes": (c_size_t, [c_uint32, c_uint32]),
     "nh_colmax_argmax_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_uint32, c_uint32,
                                      c_size_t, c_void_p, c_void_p]),
@@ -259,6 +260,14 @@ class Runtime(object):
     def gemm(self, itemsize, trans_a, trans_b, m, n, k, alpha, a_ptr, lda, b_ptr, ldb, beta, c_ptr, ldc):
         _check(self.lib.nh_gemm(itemsize, int(trans_a), int(trans_b), m, n, k, alpha, c_void_p(a_ptr), lda,
                                 c_void_p(b_ptr), ldb, beta, c_void_p(c_ptr), ldc, self.stream))
+
+    def copy_transpose(self, out_ptr, in_ptr, itemsize, shape, out_strides, in_strides):
+        n = len(shape)
+        c_shape = (c_uint32 * n)(*shape)
+        c_os = (ctypes.c_int64 * n)(*out_strides)
+        c_is = (ctypes.c_int64 * n)(*in_strides)
+        _check(self.lib.nh_copy_transpose(c_void_p(out_ptr), c_void_p(in_ptr), itemsize, n, c_shape, c_os, c_is,
+                                          self.stream))
 
     def shutdown(self):
         self.lib.nh_shutdown()

@@ -890,9 +890,12 @@ class NervanaHIP(Backend):
             for t in temps:
                 self._temp_release(t)
 
-    def _run_leaf(self, tree):
+    def _run_leaf(self, tree, more=(), originals=()):
         prog = Program()
+        prog.originals = frozenset(id(t) for t in originals)
         prog.add_statement(tree)
+        for t in more:
+            prog.add_statement(t)
         prog.finalize()
         key = prog.key()
         plan = self.plans.get(key)
@@ -982,6 +985,73 @@ class NervanaHIP(Backend):
             for t in temps:
                 self._temp_release(t)
         return C
+
+    # -- dimension shuffle -------------------------------------------------------------------
+    def copy_transpose(self, a, out, axes=None, repeat=1):
+        """``out[...] = numpy.transpose(a, axes)`` for tensors of any rank
+        (reference nervanagpu.py:3077-3118; CPU form nervanacpu.py:1046-1051).
+        Dimensions of extent 1 are dropped and dimensions that stay adjacent on
+        both sides are merged before the tiled kernel is launched."""
+        assert a.dtype == out.dtype
+        assert a.size == out.size
+        assert a.gpudata != out.gpudata
+        assert not a.take_array and not out.take_array, "copy_transpose takes strided tensors"
+        if axes is None:
+            axes = tuple(range(len(a.shape) - 1, -1, -1))
+        elif type(axes) is not tuple:
+            axes = tuple(axes)
+        assert sorted(axes) == list(range(len(a.shape))), "axes must be a permutation"
+        assert all(out.shape[i] == a.shape[x] for i, x in enumerate(axes))
+        self._flush()
+        if a.size == 0:
+            return
+        dims = [[out.shape[i], out.strides[i], a.strides[x]] for i, x in enumerate(axes) if out.shape[i] != 1]
+        merged = []
+        for d in dims:
+            if merged and merged[-1][1] == d[1] * d[0] and merged[-1][2] == d[2] * d[0]:
+                merged[-1] = [merged[-1][0] * d[0], d[1], d[2]]
+            else:
+                merged.append(d)
+        if not merged:
+            merged = [[1, 1, 1]]
+        for _ in range(max(int(repeat), 1)):
+            if len(merged) == 1 and merged[0][1] == 1 and merged[0][2] == 1:
+                self.rt.memcpy_d2d(out.gpudata, a.gpudata, a.size * a.dtype.itemsize)
+            else:
+                self.rt.copy_transpose(out.gpudata, a.gpudata, a.dtype.itemsize,
+                                       [d[0] for d in merged], [d[1] for d in merged], [d[2] for d in merged])
+
+    # -- compensated (Kahan) accumulation -------------------------------------------------------
+    def compensated_sum(self, sum_tensor, cmp_tensor, add_tensor, cmp_scale=1.0, add_scale=1.0):
+        """sum += add * add_scale, carrying the rounding error of each step in
+        ``cmp_tensor`` (reference nervanagpu.py:1896-1917, kernel
+        float_ew.py:943-1037):
+
+            y   = add * add_scale - cmp * cmp_scale
+            t   = store(sum + y)         # rounded to the storage type, stochastically
+                                         # if sum_tensor.rounding is set
+            cmp = (t - sum) - y          # what the store lost
+            sum = t
+
+        One fused kernel; ``cmp_tensor.kahan_reset`` restarts the compensation
+        every that many calls, as in the reference."""
+        if cmp_tensor.kahan_reset and cmp_tensor.kahan_count > cmp_tensor.kahan_reset:
+            cmp_scale = 0
+            cmp_tensor.kahan_count = 0
+        assert sum_tensor.dtype.type == cmp_tensor.dtype.type == add_tensor.dtype.type
+        assert sum_tensor.shape == cmp_tensor.shape == add_tensor.shape
+        cmp_tensor.kahan_count += 1
+        self._flush()
+        # second handles on the same memory: reads through them see the values
+        # from before the update even after `sum_tensor` has been assigned
+        def alias(t):
+            return HIPTensor(backend=self, shape=t.shape, dtype=t.dtype, base=t, gpudata=t.gpudata,
+                             strides=t.strides, name=t.name)
+        old_sum, old_cmp = alias(sum_tensor), alias(cmp_tensor)
+        y = add_tensor * add_scale - old_cmp * cmp_scale
+        self._run_leaf(self._stmt(sum_tensor, old_sum + y),
+                       more=[self._stmt(cmp_tensor, (sum_tensor - old_sum) - y)],
+                       originals=(old_sum, old_cmp))
 
     # -- batch normalisation as fused statement groups -------------------------------------------
     @staticmethod

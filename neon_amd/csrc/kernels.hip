@@ -411,6 +411,84 @@ CrPlan cr_plan(uint32_t rows, uint32_t cols, bool vec) {
     return p;
 }
 
+// ---------------------------------------------------------------------------
+// Dimension shuffle (numpy.transpose into a destination tensor).  Dimensions
+// are given in OUTPUT order, each with its output and its input stride.  A
+// workgroup moves one 64 x 64 tile spanned by axis `ax` (the output's
+// fastest-moving dimension) and axis `ay`; all other dimensions are decoded
+// once per workgroup from the block index.
+//   SWAP = true:  `ay` is the dimension that moves fastest in the INPUT: the
+//     tile is read with lanes along `ay`, turned in LDS (row pitch 65 words:
+//     conflict-free for 4- and 8-byte elements) and written with lanes along
+//     `ax`, so both sides see 64-element contiguous runs.
+//   SWAP = false: the fastest dimension is the same on both sides; lanes run
+//     along it for the read and the write and LDS is not used.
+// ---------------------------------------------------------------------------
+constexpr int TR_TILE = 64;
+constexpr int TR_T = 256;
+
+struct TrGeom {
+    uint32_t n[NH_TRANSPOSE_MAX_DIMS];
+    long long os[NH_TRANSPOSE_MAX_DIMS];
+    long long is[NH_TRANSPOSE_MAX_DIMS];
+    int nd, ax, ay;
+    uint32_t tiles_x, tiles_y;
+};
+
+template <typename T, bool SWAP>
+__global__ __launch_bounds__(TR_T) void transpose_tile_kernel(T* __restrict__ out, const T* __restrict__ in, TrGeom g) {
+    __shared__ T tile[SWAP ? TR_TILE : 1][TR_TILE + 1];
+    unsigned long long b = blockIdx.x;
+    const uint32_t tx = (uint32_t)(b % g.tiles_x);
+    b /= g.tiles_x;
+    const uint32_t ty = (uint32_t)(b % g.tiles_y);
+    b /= g.tiles_y;
+    long long ibase = 0, obase = 0;
+    for (int k = g.nd - 1; k >= 0; --k) {
+        if (k == g.ax || k == g.ay) continue;
+        const unsigned long long idx = b % g.n[k];
+        b /= g.n[k];
+        ibase += (long long)idx * g.is[k];
+        obase += (long long)idx * g.os[k];
+    }
+    const uint32_t nx = g.n[g.ax], ny = g.ay >= 0 ? g.n[g.ay] : 1u;
+    const long long isx = g.is[g.ax], osx = g.os[g.ax];
+    const long long isy = g.ay >= 0 ? g.is[g.ay] : 0, osy = g.ay >= 0 ? g.os[g.ay] : 0;
+    const uint32_t x0 = tx * TR_TILE, y0 = ty * TR_TILE;
+    const uint32_t lane = threadIdx.x & (TR_TILE - 1), row = threadIdx.x / TR_TILE;
+    constexpr uint32_t ROWS = TR_T / TR_TILE;
+    if constexpr (SWAP) {
+        for (uint32_t i = row; i < TR_TILE; i += ROWS) {
+            const uint32_t x = x0 + i, y = y0 + lane;
+            if (x < nx && y < ny) tile[i][lane] = in[ibase + (long long)x * isx + (long long)y * isy];
+        }
+        __syncthreads();
+        for (uint32_t i = row; i < TR_TILE; i += ROWS) {
+            const uint32_t x = x0 + lane, y = y0 + i;
+            if (x < nx && y < ny) out[obase + (long long)x * osx + (long long)y * osy] = tile[lane][i];
+        }
+    } else {
+        const uint32_t x = x0 + lane;
+        if (x < nx) {
+            for (uint32_t i = row; i < TR_TILE; i += ROWS) {
+                const uint32_t y = y0 + i;
+                if (y < ny)
+                    out[obase + (long long)x * osx + (long long)y * osy] =
+                        in[ibase + (long long)x * isx + (long long)y * isy];
+            }
+        }
+    }
+}
+
+template <typename T>
+void launch_transpose(void* out, const void* in, const TrGeom& g, bool swap, unsigned blocks, hipStream_t s) {
+    if (swap)
+        hipLaunchKernelGGL((transpose_tile_kernel<T, true>), dim3(blocks), dim3(TR_T), 0, s, (T*)out, (const T*)in, g);
+    else
+        hipLaunchKernelGGL((transpose_tile_kernel<T, false>), dim3(blocks), dim3(TR_T), 0, s, (T*)out, (const T*)in, g);
+}
+
+
 }  // namespace
 
 extern "C" {
@@ -480,6 +558,63 @@ int nh_hist_log2(int32_t* hist, const void* x, int itemsize, size_t n, int nbins
         hipLaunchKernelGGL((hist_log2_kernel<nh_f16>), dim3((unsigned)blocks), dim3(HIST_T), 0, s, (const nh_f16*)x, n,
                            nbins, offset, (int*)hist);
     return launch_status("nh_hist_log2");
+}
+
+int nh_copy_transpose(void* out, const void* in, int itemsize, int ndim, const uint32_t* shape,
+                      const int64_t* out_strides, const int64_t* in_strides, void* stream) {
+    if (!nh_internal_ready()) return nh_internal_fail(NH_ENOTINIT, "nh_init has not been called");
+    if (ndim < 1 || ndim > NH_TRANSPOSE_MAX_DIMS)
+        return nh_internal_fail(NH_EINVAL, "nh_copy_transpose: ndim must be 1..NH_TRANSPOSE_MAX_DIMS");
+    if (!shape || !out_strides || !in_strides) return nh_internal_fail(NH_EINVAL, "nh_copy_transpose: null geometry");
+    if (itemsize != 1 && itemsize != 2 && itemsize != 4 && itemsize != 8)
+        return nh_internal_fail(NH_EINVAL, "nh_copy_transpose: itemsize must be 1, 2, 4 or 8");
+    TrGeom g;
+    unsigned long long total = 1;
+    for (int k = 0; k < ndim; ++k) {
+        if (out_strides[k] < 0 || in_strides[k] < 0)
+            return nh_internal_fail(NH_EINVAL, "nh_copy_transpose: negative stride");
+        g.n[k] = shape[k];
+        g.os[k] = out_strides[k];
+        g.is[k] = in_strides[k];
+        total *= shape[k];
+    }
+    if (total == 0) return 0;
+    if (!out || !in) return nh_internal_fail(NH_EINVAL, "nh_copy_transpose: null pointer");
+    g.nd = ndim;
+    // ax: the dimension the output walks fastest; ay: the one the input walks
+    // fastest (extent-1 dimensions never matter)
+    int ax = -1, ay = -1;
+    for (int k = 0; k < ndim; ++k) {
+        if (g.n[k] == 1) continue;
+        if (ax < 0 || g.os[k] < g.os[ax]) ax = k;
+        if (ay < 0 || g.is[k] < g.is[ay]) ay = k;
+    }
+    if (ax < 0) ax = ay = ndim - 1;             // a single element
+    bool swap = ax != ay;
+    if (!swap) {
+        // same fastest dimension on both sides: pair it with the next-fastest output dimension
+        ay = -1;
+        for (int k = 0; k < ndim; ++k) {
+            if (k == ax || g.n[k] == 1) continue;
+            if (ay < 0 || g.os[k] < g.os[ay]) ay = k;
+        }
+    }
+    g.ax = ax;
+    g.ay = ay;
+    g.tiles_x = (g.n[ax] + TR_TILE - 1) / TR_TILE;
+    g.tiles_y = ay >= 0 ? (g.n[ay] + TR_TILE - 1) / TR_TILE : 1u;
+    unsigned long long blocks = (unsigned long long)g.tiles_x * g.tiles_y;
+    for (int k = 0; k < ndim; ++k)
+        if (k != ax && k != ay) blocks *= g.n[k];
+    if (blocks > 0x7fffffffull) return nh_internal_fail(NH_EINVAL, "nh_copy_transpose: too many tiles for one launch");
+    hipStream_t s = (hipStream_t)stream;
+    switch (itemsize) {
+        case 1: launch_transpose<uint8_t>(out, in, g, swap, (unsigned)blocks, s); break;
+        case 2: launch_transpose<uint16_t>(out, in, g, swap, (unsigned)blocks, s); break;
+        case 4: launch_transpose<uint32_t>(out, in, g, swap, (unsigned)blocks, s); break;
+        default: launch_transpose<unsigned long long>(out, in, g, swap, (unsigned)blocks, s); break;
+    }
+    return launch_status("nh_copy_transpose");
 }
 
 size_t nh_colreduce_workspace_bytes(uint32_t rows, uint32_t cols) {

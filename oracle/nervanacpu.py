@@ -439,6 +439,36 @@ class NervanaCPU(Backend):
             bsum[:] = self.sum(C, 1)
         return C
 
+    # -- dimension shuffle (reference nervanacpu.py:1046-1051) ------------------------
+    def copy_transpose(self, a, out, axes=None, repeat=1):
+        out._tensor[:] = np.transpose(a._tensor, axes).copy()
+
+    # -- compensated accumulation ---------------------------------------------------
+    def compensated_sum(self, sum_tensor, cmp_tensor, add_tensor, cmp_scale=1.0, add_scale=1.0):
+        """The reference's CPU backend has no such method; this restates, in
+        numpy float32 arithmetic, the element loop of the accelerator kernel
+        (neon/backends/float_ew.py:966-992, round-to-nearest stores) with the
+        host-side reset logic of nervanagpu.py:1896-1905.  Pinned in
+        tests/test_oracle.py by the defining property of compensated summation
+        (many small addends into a float16 accumulator stay within one unit in
+        the last place of the exact sum, where plain accumulation stalls)."""
+        reset = getattr(cmp_tensor, "kahan_reset", 0)
+        count = getattr(cmp_tensor, "kahan_count", 0)
+        if reset and count > reset:
+            cmp_scale = 0
+            count = 0
+        assert sum_tensor.dtype.type == cmp_tensor.dtype.type == add_tensor.dtype.type
+        cmp_tensor.kahan_count = count + 1
+        store = sum_tensor.dtype.type
+        s32 = sum_tensor._tensor.astype(np.float32)
+        c32 = cmp_tensor._tensor.astype(np.float32)
+        a32 = add_tensor._tensor.astype(np.float32)
+        y32 = a32 * np.float32(add_scale) - c32 * np.float32(cmp_scale)
+        t = (s32 + y32).astype(store)
+        c = ((t.astype(np.float32) - s32) - y32).astype(store)
+        sum_tensor._tensor[:] = t
+        cmp_tensor._tensor[:] = c
+
     # -- batch normalisation (reference nervanacpu.py:1688-1760), non-binary path ---
     def compound_fprop_bn(self, x, xsum, xvar, gmean, gvar, gamma, beta, y, eps, rho,
                           compute_batch_sum, accumbeta=0.0, relu=False, binary=False,
