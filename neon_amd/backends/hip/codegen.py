@@ -983,6 +983,9 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
 COLSPLIT_MAX_CHUNKS = 128
 
 
+COLSPLIT_ROWS_IN_FLIGHT = 4
+
+
 def gen_colsplit(prog, V, LX, LY, stream=False):
     """One level of axis-0 reductions over a tall matrix.  grid = (column
     strips, row chunks).  Each workgroup reduces its chunk, leaves one partial
@@ -1021,7 +1024,7 @@ def gen_colsplit(prog, V, LX, LY, stream=False):
     leaves = g.leaf_nodes(nodes)
     for n in reds:
         g.declare_acc(n)
-    U = 4
+    U = COLSPLIT_ROWS_IN_FLIGHT
     # main loop: U independent rows in flight per lane
     L.open("if (col_ok)")
     L("long long r = r0 + ty;")

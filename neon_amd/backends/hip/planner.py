@@ -368,6 +368,9 @@ def _plan_row(prog, cu_count):
 _COL_BUDGET = {1024: 40, 512: 120, 256: 300}
 
 
+COLSPLIT_THREADS = 256
+
+
 def _plan_col(prog, cu_count):
     R, C = prog.domain
     V = _vector_width(prog, single_row_tail_ok=False)
@@ -442,7 +445,7 @@ def _plan_col(prog, cu_count):
     # (b) one level, one value per column, many rows: split rows over workgroups
     if single_level and line_only:
         LX = max(lx_min, min(16, _pow2ceil(nvec)))
-        LY = 256 // LX
+        LY = COLSPLIT_THREADS // LX
         strips = _ceil_div(nvec, LX)
         # Workgroups are cheap to run but not free to start: give each one at
         # least ~128 KiB to stream, one per compute unit for small inputs and
@@ -451,7 +454,7 @@ def _plan_col(prog, cu_count):
         per_cu = max(1, min(8, bytes_total // (cu_count * (128 << 10))))
         target = per_cu * cu_count
         chunks = max(1, min(codegen.COLSPLIT_MAX_CHUNKS, target // strips))
-        rpc = max(4 * LY, _ceil_div(R, chunks))
+        rpc = max(codegen.COLSPLIT_ROWS_IN_FLIGHT * LY, _ceil_div(R, chunks))
         rpc = _ceil_div(rpc, LY) * LY
         chunks = _ceil_div(R, rpc)
         if chunks > 65535:
