@@ -35,7 +35,7 @@ HBM_PEAK_GBS = 8000.0
 # plain copy kernel of known size); summary and commands under
 # profiles/hbm_traffic_adam_rownorm_colreduce_pmc.txt.  Counters cannot be read
 # from inside this process, so the figure is carried here.
-ADAM_FUSED_TRAFFIC_BYTES = 699.6e6
+ADAM_FUSED_TRAFFIC_BYTES = 699.9e6
 
 
 def _fresh(be, shape, dtype=np.float32, fill=None, rs=None, scale=1.0, shift=0.0):

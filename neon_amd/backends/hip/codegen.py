@@ -29,6 +29,7 @@ tensor slot ``(pointer, row stride, column stride)`` in elements, one float per
 constant slot, ``R``, ``C``, then family-specific extras.
 """
 import hashlib
+import os
 
 from neon_amd.backends.hip.optree_ir import DTYPE_CODE, used_nodes
 
@@ -50,6 +51,16 @@ _UN = {"neg": "(-{0})", "abs": "__builtin_fabsf({0})", "sgn": "nh_sgn({0})",
        "rint": "rintf({0})", "finite": "nh_finite({0})", "ident": "({0})"}
 _RED_OP = {"sum": "nh_op_sum", "max": "nh_op_max", "min": "nh_op_min",
            "argmax": "nh_op_argmax", "argmin": "nh_op_argmin"}
+
+
+# Streaming kernels (working set far beyond the caches) read with non-temporal
+# loads.  Their stores are ordinary ones, except in the row family: measured
+# on the 7-stream fused Adam update, non-temporal loads with ordinary stores
+# run at 6.5-6.7 TB/s against 5.9-6.2 TB/s with both non-temporal (axpby,
+# in-place sigmoid and the column softmax gain 3-7 % the same way), whereas the
+# row kernels, whose workgroups all read, then all write, lose 20 % without
+# non-temporal stores.
+STREAM_STORES = {"ew": False, "row": True, "col": False, "colsplit": False}
 
 
 class Spec(object):
@@ -88,7 +99,7 @@ class _Lines(object):
 class _Gen(object):
     """State shared by the family emitters for one program."""
 
-    def __init__(self, prog, V, stream=False):
+    def __init__(self, prog, V, stream=False, family="ew"):
         self.prog = prog
         self.V = V
         self.R, self.C = prog.domain
@@ -98,7 +109,7 @@ class _Gen(object):
         # global accesses non-temporal
         self.pos = ("0", "0")      # (row, column) expressions of the element being emitted
         self.ld = "load_stream" if stream else "load"
-        self.st = "store_stream" if stream else "store"
+        self.st = "store_stream" if (stream and STREAM_STORES[family]) else "store"
 
     # -- parameters -----------------------------------------------------------------
     def slot_ctype(self, slot):
@@ -382,8 +393,8 @@ def _kept_values(prog, stages, limit):
 class _RedGen(_Gen):
     """Common machinery of row / col / colsplit."""
 
-    def __init__(self, prog, V, stream=False):
-        super(_RedGen, self).__init__(prog, V, stream)
+    def __init__(self, prog, V, stream=False, family="row"):
+        super(_RedGen, self).__init__(prog, V, stream, family)
         self.col_axis = (prog.axis == 0)   # reductions leave one value per column
 
     # value of a finished reduction at element j of the lane's tile
@@ -440,7 +451,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False):
     column tiles tx, tx+LX, ...; with ``NCH`` > 0 that loop has a fixed trip
     count and the tiles loaded in the first sweep stay in registers for the
     later ones; with ``NCH`` == 0 every sweep streams the row again."""
-    g = _RedGen(prog, V, stream)
+    g = _RedGen(prog, V, stream, "row")
     L = g.L
     T = LX * LY
     assert LX <= 64 or LY == 1
@@ -714,7 +725,7 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
     byte offset of the counters (two per strip: arrivals, departures; zero
     before the first launch, reset by the last workgroup to leave)."""
     coop = chunks > 1
-    g = _RedGen(prog, V, stream)
+    g = _RedGen(prog, V, stream, "col")
     L = g.L
     T = LX * LY
     params, fmt = g.param_list([("char* ws", "P"), ("long long ctr_offset", "q")] if coop else [])
@@ -997,7 +1008,7 @@ def gen_colsplit(prog, V, LX, LY, stream=False):
     Extra parameters: ``rows_per_chunk``, workspace pointer (partials first,
     tickets after ``ticket_offset`` bytes)."""
     assert prog.nlevels == 1
-    g = _RedGen(prog, V, stream)
+    g = _RedGen(prog, V, stream, "colsplit")
     L = g.L
     T = LX * LY
     params, fmt = g.param_list([("int rows_per_chunk", "i"), ("char* ws", "P"),

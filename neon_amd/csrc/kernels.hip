@@ -28,7 +28,9 @@ int launch_status(const char* what) {
 // and tensor (every wave touches 1 KiB contiguous per instruction), all loads
 // issued before the first use.  One vector per lane measured fastest for the
 // 7-stream Adam update (more in flight per lane only adds read/write
-// turnarounds); inputs far larger than the caches use non-temporal accesses.
+// turnarounds); inputs far larger than the caches are read with non-temporal
+// loads and written with ordinary stores (measured: 6.7 TB/s on the Adam
+// update against 5.9 TB/s with non-temporal stores as well).
 // ---------------------------------------------------------------------------
 constexpr int EW_T = 256;
 constexpr size_t EW_STREAM_BYTES = (size_t)256 << 20;
@@ -73,7 +75,7 @@ struct AxpbyF {
 #pragma unroll
         for (int j = 0; j < V; ++j) r.x[j] = a * r.x[j] + b * r.y[j];
     }
-    template <int V, bool NT> __device__ void store(const regs<V>& r, size_t i) const { ew_st<V, NT>(out + i, r.x); }
+    template <int V, bool NT> __device__ void store(const regs<V>& r, size_t i) const { ew_st<V, false>(out + i, r.x); }
 };
 
 struct SigmoidF {
@@ -85,7 +87,7 @@ struct SigmoidF {
 #pragma unroll
         for (int j = 0; j < V; ++j) r.x[j] = nh_sig(r.x[j]);
     }
-    template <int V, bool NT> __device__ void store(const regs<V>& r, size_t i) const { ew_st<V, NT>(out + i, r.x); }
+    template <int V, bool NT> __device__ void store(const regs<V>& r, size_t i) const { ew_st<V, false>(out + i, r.x); }
 };
 
 // The three assigns of the reference's Adam.optimize
@@ -112,7 +114,7 @@ struct AdamF {
         }
     }
     template <int V, bool NT> __device__ void store(const regs<V>& r, size_t i) const {
-        ew_st<V, NT>(m + i, r.m); ew_st<V, NT>(v + i, r.v); ew_st<V, NT>(p + i, r.p);
+        ew_st<V, false>(m + i, r.m); ew_st<V, false>(v + i, r.v); ew_st<V, false>(p + i, r.p);
     }
 };
 
