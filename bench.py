@@ -324,7 +324,7 @@ def main():
         return
     if args.gpus != 1:
         print("bench.py measures one MI355X; --gpus %d is not supported (the op-tree path has no "
-              "cross-device stage; see DESIGN.md on sharding)" % args.gpus, file=sys.stderr)
+              "cross-device stage: every figure here is one GPU's)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
     gpu, be = gpu_leg(args.steps, args.warmup, detail=not args.no_detail)
