@@ -327,6 +327,8 @@ def main():
               "cross-device stage: every figure here is one GPU's)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
+    import __graft_entry__
+    __graft_entry__.ensure_built()
     gpu, be = gpu_leg(args.steps, args.warmup, detail=not args.no_detail)
     cpu = None if args.no_cpu else cpu_leg()
     line = {

@@ -17,6 +17,10 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs an MI355X (run on the GPU box)")
+    # the tests load the library the build left in the tree; build it only if
+    # there is none
+    import __graft_entry__
+    __graft_entry__.ensure_built()
 
 
 def _device_count():
