@@ -13,8 +13,9 @@ be.end`` calls, inputs resident in HBM, stream synchronised on both sides.
 around the same K launches.  ``per_config`` lists every benchmark op-tree
 (elementwise + sigmoid, softmax, Adam fused and as three kernels, fp16 row
 normalisation, argmax / max / cross-entropy over a 32000-row vocabulary) with
-the same event timing, and a scaled-up (>= 256 MB) instance of the trees whose
-working set fits in cache.  ``cpu_baseline`` times the numpy oracle on the same
+the same event timing, a scaled-up (>= 256 MB) instance of the trees whose
+working set fits in cache, and cold-cache timings of those trees (launches
+rotating over >= 768 MB of distinct tensors).  ``cpu_baseline`` times the numpy oracle on the same
 Adam step on this machine's host cores.
 """
 import argparse
@@ -36,6 +37,7 @@ HBM_PEAK_GBS = 8000.0
 # profiles/hbm_traffic_adam_rownorm_colreduce_pmc.txt.  Counters cannot be read
 # from inside this process, so the figure is carried here.
 ADAM_FUSED_TRAFFIC_BYTES = 699.9e6
+COLD_BYTES = 768 << 20         # tensor sets rotated through by the cold-cache rows
 
 
 def _fresh(be, shape, dtype=np.float32, fill=None, rs=None, scale=1.0, shift=0.0):
@@ -195,6 +197,46 @@ def gpu_leg(steps, warmup, detail=True):
     measure("C5b max axis0 (32000,256) f32", lambda: configs.c5b_max(be, mx, x5), configs.bytes_c5_reduce(), n5)
     measure("C5c cross-entropy axis0 (32000,256) f32, in-kernel one-hot",
             lambda: configs.c5c_cross_entropy(be, ce, x5, be.onehot(i5, axis=0)), configs.bytes_c5c(), n5)
+    # ---- the same trees with cold caches: each launch works on another set of tensors, enough
+    #      sets (>= 768 MB in total) that neither the L2s nor the 256 MB memory-side cache hold them
+    def measure_cold(label, make_set, issue, nbytes, elements):
+        nsets = max(3, min(600, -(-COLD_BYTES // nbytes)))
+        sets = [make_set() for _ in range(nsets)]
+        groups = []
+        for tensors in sets:
+            with be.capture() as grp:
+                issue(*tensors)
+            assert len(grp) == 1, "cold rows are single-kernel trees"
+            groups.append(grp[0])
+        be.time_group_sets(groups, reps=nsets)                    # touch every buffer once
+        ms_k, pl = be.time_group_sets(groups, reps=max(2 * nsets, 60))
+        rows.append({"config": label, "bytes": nbytes, "kernels": 1, "ms": ms_k, "api_ms": None,
+                     "timing": "HIP events around launches rotating over %d tensor sets" % nsets,
+                     "plan": pl.spec.family, "gbs": nbytes / (ms_k * 1e-3) / 1e9,
+                     "frac_of_hbm_peak": nbytes / (ms_k * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "elements_per_s": elements / (ms_k * 1e-3)})
+        del sets, groups
+
+    f16, i32 = np.float16, np.int32
+    measure_cold("C1 fused sig(0.5x+2y) (4096,128) f32 [cold]",
+                 lambda: (be.empty(configs.C1_SHAPE), be.zeros(configs.C1_SHAPE), be.zeros(configs.C1_SHAPE)),
+                 lambda o, x, y: configs.c1_fused(be, o, x, y), configs.bytes_c1a(), n1)
+    measure_cold("C2 softmax axis0 (1000,128) f32 [cold]",
+                 lambda: (be.empty(configs.C2_SHAPE), be.zeros(configs.C2_SHAPE)),
+                 lambda o, x: configs.c2_softmax(be, o, x), configs.bytes_c2(), configs.C2_SHAPE[0] * configs.C2_SHAPE[1])
+    measure_cold("C4 rownorm (256,100352) f16 [cold]",
+                 lambda: (be.empty(configs.C4_SHAPE, dtype=f16), be.zeros(configs.C4_SHAPE, dtype=f16)),
+                 lambda o, x: configs.c4_rownorm(be, o, x, g4, b4), configs.bytes_c4(),
+                 configs.C4_SHAPE[0] * configs.C4_SHAPE[1])
+    measure_cold("C5a argmax axis0 (32000,256) f32 [cold]",
+                 lambda: (be.empty((1, configs.C5_SHAPE[1]), dtype=i32), be.zeros(configs.C5_SHAPE)),
+                 lambda o, x: configs.c5a_argmax(be, o, x), configs.bytes_c5_reduce(), n5)
+    measure_cold("C5b max axis0 (32000,256) f32 [cold]",
+                 lambda: (be.empty((1, configs.C5_SHAPE[1])), be.zeros(configs.C5_SHAPE)),
+                 lambda o, x: configs.c5b_max(be, o, x), configs.bytes_c5_reduce(), n5)
+    measure_cold("C5c cross-entropy axis0 (32000,256) f32 [cold]",
+                 lambda: (be.empty((1, configs.C5_SHAPE[1])), be.zeros(configs.C5_SHAPE)),
+                 lambda o, x: configs.c5c_cross_entropy(be, o, x, be.onehot(i5, axis=0)), configs.bytes_c5c(), n5)
     # ---- the prebuilt hand-written kernels behind the direct C-ABI entry points ------------
     lib = rt.lib
     e0, e1 = rt.event(), rt.event()

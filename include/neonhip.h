@@ -120,6 +120,15 @@ int nh_launch_timed(void* function, const uint32_t grid[3], const uint32_t block
                     uint32_t lds_bytes, void* stream, const void* args, size_t arg_bytes,
                     uint32_t reps, float* mean_ms);
 
+/* The same, cycling through `nsets` argument buffers (launch i uses
+ * arg_sets[i % nsets]): with enough distinct tensors behind the sets every
+ * launch finds its operands in HBM rather than in a cache.  The reference has
+ * no counterpart; it is the cold-cache companion of the bench-mode bracket
+ * above.                                                                       */
+int nh_launch_timed_sets(void* function, const uint32_t grid[3], const uint32_t block[3],
+                         uint32_t lds_bytes, void* stream, const void* const* arg_sets, size_t arg_bytes,
+                         uint32_t nsets, uint32_t reps, float* mean_ms);
+
 /* ---- prebuilt hand-written gfx950 kernels ------------------------------------
  * Direct entry points for fixed, hot op-trees; the same trees also run through
  * the generated-code path.  All pointers are device pointers; tensors are

@@ -257,6 +257,12 @@ class Plan(object):
         """mean ms per launch of ``reps`` back-to-back launches (bench mode)"""
         return self.rt.launch_timed(self.kernel, self.grid, self.block, 0, reps, *self._values(prog))
 
+    def launch_timed_sets(self, progs, reps):
+        """the same over several programs of this plan's shape (identical
+        structure, different tensors), launched in rotation"""
+        return self.rt.launch_timed_sets(self.kernel, self.grid, self.block, 0, reps,
+                                         [self._values(prog) for prog in progs])
+
     def release(self):
         if self.workspace:
             self.rt.free(self.workspace)

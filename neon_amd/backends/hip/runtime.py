@@ -81,6 +81,9 @@ SIGNATURES = {
                           c_void_p, c_void_p, c_size_t]),
     "nh_launch_timed": (c_int, [c_void_p, POINTER(c_uint32), POINTER(c_uint32), c_uint32,
                                 c_void_p, c_void_p, c_size_t, c_uint32, POINTER(c_float)]),
+    "nh_launch_timed_sets": (c_int, [c_void_p, POINTER(c_uint32), POINTER(c_uint32), c_uint32,
+                                     c_void_p, POINTER(c_void_p), c_size_t, c_uint32, c_uint32,
+                                     POINTER(c_float)]),
     "nh_ew_axpby_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_float, c_size_t, c_void_p]),
     "nh_ew_sigmoid_f32": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     "nh_adam_step_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_float,
@@ -251,6 +254,20 @@ class Runtime(object):
         ms = c_float()
         _check(self.lib.nh_launch_timed(kernel.function, g, b, lds_bytes, self.stream,
                                         args, kernel.arg_bytes, reps, byref(ms)))
+        return ms.value
+
+    def launch_timed_sets(self, kernel, grid, block, lds_bytes, reps, value_sets):
+        """mean milliseconds per launch over ``reps`` launches that cycle
+        through the argument tuples in ``value_sets``"""
+        g, b = self._grid, self._block
+        g[0], g[1], g[2] = grid
+        b[0], b[1], b[2] = block
+        bufs = [ctypes.create_string_buffer(bytes(kernel.packer.pack(*values)), kernel.arg_bytes)
+                for values in value_sets]
+        ptrs = (c_void_p * len(bufs))(*[ctypes.addressof(buf) for buf in bufs])
+        ms = c_float()
+        _check(self.lib.nh_launch_timed_sets(kernel.function, g, b, lds_bytes, self.stream, ptrs,
+                                             kernel.arg_bytes, len(bufs), reps, byref(ms)))
         return ms.value
 
     def hist_log2(self, hist_ptr, x_ptr, itemsize, n, nbins, offset):

@@ -829,6 +829,26 @@ class NervanaHIP(Backend):
             self.plans[key] = plan
         return plan.launch_timed(prog, reps), plan
 
+    def time_group_sets(self, groups, reps=20):
+        """As ``time_group`` for several statement groups that are the same
+        computation on different tensors: one kernel, launched ``reps`` times
+        in rotation over the groups' tensors, so that with enough groups no
+        launch finds its operands in a cache.  Returns (ms per launch, plan)."""
+        progs = []
+        for trees in groups:
+            prog = Program()
+            for t in trees:
+                prog.add_statement(t)
+            prog.finalize()
+            progs.append(prog)
+        key = progs[0].key()
+        assert all(prog.key() == key for prog in progs), "groups differ in more than their tensors"
+        plan = self.plans.get(key)
+        if plan is None:
+            plan = make_plan(progs[0], self.rt, self.kernels, self.cu_count)
+            self.plans[key] = plan
+        return plan.launch_timed_sets(progs, reps), plan
+
     def _run_split(self, tree):
         """Evaluate a tree that does not fit one kernel stage by stage through
         temporaries: every reduction (innermost first) and every transposed

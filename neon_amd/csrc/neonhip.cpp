@@ -368,17 +368,17 @@ int nh_launch(void* function, const uint32_t grid[3], const uint32_t block[3],
     return 0;
 }
 
-int nh_launch_timed(void* function, const uint32_t grid[3], const uint32_t block[3],
-                    uint32_t lds_bytes, void* stream, const void* args, size_t arg_bytes,
-                    uint32_t reps, float* mean_ms) {
+int nh_launch_timed_sets(void* function, const uint32_t grid[3], const uint32_t block[3],
+                         uint32_t lds_bytes, void* stream, const void* const* arg_sets, size_t arg_bytes,
+                         uint32_t nsets, uint32_t reps, float* mean_ms) {
     NH_NEED_INIT();
-    if (!mean_ms || reps == 0) return fail(NH_EINVAL, "nh_launch_timed: bad argument");
+    if (!mean_ms || reps == 0 || nsets == 0 || !arg_sets) return fail(NH_EINVAL, "nh_launch_timed_sets: bad argument");
     *mean_ms = 0.0f;
     hipEvent_t e0, e1;
     NH_HIP(hipEventCreate(&e0));
     hipError_t err = hipEventCreate(&e1);
     if (err != hipSuccess) {
-        hipEventDestroy(e0);
+        (void)hipEventDestroy(e0);
         return hip_fail(err, "hipEventCreate");
     }
     int rc = 0;
@@ -386,18 +386,25 @@ int nh_launch_timed(void* function, const uint32_t grid[3], const uint32_t block
     err = hipEventRecord(e0, s);
     if (err != hipSuccess) rc = hip_fail(err, "hipEventRecord");
     for (uint32_t i = 0; rc == 0 && i < reps; ++i)
-        rc = nh_launch(function, grid, block, lds_bytes, stream, args, arg_bytes);
+        rc = nh_launch(function, grid, block, lds_bytes, stream, arg_sets[i % nsets], arg_bytes);
     if (rc == 0) {
         err = hipEventRecord(e1, s);
         if (err == hipSuccess) err = hipEventSynchronize(e1);
         float ms = 0.0f;
         if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
-        if (err != hipSuccess) rc = hip_fail(err, "nh_launch_timed: event timing");
+        if (err != hipSuccess) rc = hip_fail(err, "nh_launch_timed_sets: event timing");
         else *mean_ms = ms / (float)reps;
     }
-    hipEventDestroy(e0);
-    hipEventDestroy(e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
     return rc;
+}
+
+int nh_launch_timed(void* function, const uint32_t grid[3], const uint32_t block[3],
+                    uint32_t lds_bytes, void* stream, const void* args, size_t arg_bytes,
+                    uint32_t reps, float* mean_ms) {
+    const void* one[1] = {args};
+    return nh_launch_timed_sets(function, grid, block, lds_bytes, stream, one, arg_bytes, 1, reps, mean_ms);
 }
 
 }  // extern "C"
