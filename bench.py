@@ -271,8 +271,109 @@ def gpu_leg(steps, warmup, detail=True):
                 configs.bytes_c5_reduce() + 4 * configs.C5_SHAPE[1], n5)
     rt.synchronize()
     rt.free(ws)
+    del x5, x4, o4
+    next_rows(be, rows)
     out["per_config"] = rows
     return out, be
+
+
+def next_rows(be, rows):
+    """Callers either side of the op-tree path (batch norm, random numbers and
+    rounding, indexing and layout, compensated accumulation, the GEMM
+    hand-off), each on a shape of the benchmark configurations, timed like the
+    rows above and priced by the bytes (or flops) the operation has to move."""
+    rt = be.rt
+    f32, f16, i32 = np.float32, np.float16, np.int32
+    rs = np.random.RandomState(5)
+    e0, e1 = rt.event(), rt.event()
+
+    def add(label, ms_k, nbytes, plan, kernels=1, flops=None):
+        row = {"config": label, "bytes": nbytes, "kernels": kernels, "ms": ms_k, "api_ms": None,
+               "timing": "HIP events around back-to-back launches", "plan": plan,
+               "gbs": nbytes / (ms_k * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ms_k * 1e-3) / 1e9 / HBM_PEAK_GBS,
+               "elements_per_s": None}
+        if flops:
+            row["tflops"] = flops / (ms_k * 1e-3) / 1e12
+        rows.append(row)
+
+    def trees(label, issue, nbytes, reps=30):
+        with be.capture() as grp:
+            issue()
+        total, names = 0.0, []
+        for group in grp:
+            ms_k, pl = be.time_group(group, reps=reps)
+            total += ms_k
+            names.append(pl.spec.family)
+        add(label, total, nbytes, " + ".join(names), kernels=len(grp))
+
+    def calls(label, call, nbytes, plan, reps=30, flops=None):
+        for _ in range(3):
+            call()
+        rt.synchronize()
+        rt.event_record(e0)
+        for _ in range(reps):
+            call()
+        rt.event_record(e1)
+        rt.event_sync(e1)
+        add(label, rt.event_elapsed_ms(e0, e1) / reps, nbytes, plan, flops=flops)
+
+    # batch norm over (256 feature maps, 100352 = N*H*W) fp16, as one fused kernel each way
+    K, N = 256, 100352
+    x = _fresh(be, (K, N), dtype=f16, rs=rs, scale=2.0, shift=0.5)
+    y = be.empty((K, N), dtype=f16)
+    vec = lambda fill: _fresh(be, (K, 1), fill=fill)
+    xsum, xvar, gmean, gvar, gamma, beta = vec(0.0), vec(0.0), vec(0.0), vec(1.0), vec(1.0), vec(0.0)
+    trees("BN fprop fused (256,100352) f16", lambda: be.compound_fprop_bn(
+        x, xsum, xvar, gmean, gvar, gamma, beta, y, 1e-5, 0.9, True), 2 * K * N * 2)
+    delta = _fresh(be, (K, N), dtype=f16, rs=rs, scale=0.1)
+    dout = be.empty((K, N), dtype=f16)
+    gg, gb = vec(0.0), vec(0.0)
+    trees("BN bprop fused (256,100352) f16", lambda: be.compound_bprop_bn(
+        dout, gg, gb, delta, x, xsum, xvar, gamma, 1e-5), 3 * K * N * 2)
+    del x, y, delta, dout
+
+    # random numbers and rounding on the Adam shape
+    shape = (5000, 5000)
+    n = shape[0] * shape[1]
+    a32, b32 = _fresh(be, shape, rs=rs), be.empty(shape)
+    trees("dropout mask (5000,5000) f32", lambda: be.make_binary_mask(b32, 0.5), n * 4)
+    trees("dropout applied x*mask/keep (5000,5000) f32",
+          lambda: b32.__setitem__(slice(None), a32 * be.dropout(0.5) * 2.0), 2 * n * 4)
+    r16 = be.empty(shape, dtype=f16)
+    r16.rounding = 8
+    trees("stochastic-rounding store f32 -> f16, 8 bits (5000,5000)",
+          lambda: r16.__setitem__(slice(None), a32 * 1.0), n * 6)
+    s16, c16, a16 = be.zeros(shape, dtype=f16), be.zeros(shape, dtype=f16), _fresh(be, shape, dtype=f16, rs=rs)
+    calls("compensated_sum (5000,5000) f16", lambda: be.compensated_sum(s16, c16, a16), 5 * n * 2, "ew")
+    del r16, s16, c16, a16
+
+    # indexing and layout
+    calls("hist log2 (5000,5000) f32", lambda: a32.hist("bench"), n * 4, "prebuilt (kernels.hip)")
+    table = _fresh(be, (32000, 256), rs=rs)
+    idx = be.array(rs.randint(0, 32000, size=(65536, 1)).astype(i32), dtype=i32)
+    rows_out = be.empty((65536, 256))
+    trees("gather 65536 rows of a (32000,256) f32 table", lambda: rows_out.__setitem__(slice(None), table[idx]),
+          2 * 65536 * 256 * 4 + 65536 * 4)
+    del table, rows_out, b32
+    sq = (8192, 8192)
+    t_in, t_out = _fresh(be, sq, rs=rs), be.empty(sq)
+    calls("copy_transpose (8192,8192) f32", lambda: be.copy_transpose(t_in, t_out), 2 * sq[0] * sq[1] * 4,
+          "prebuilt (kernels.hip)", reps=10)
+    t3_in = t_in.reshape((64, 512, 2048))
+    t3_out = t_out.reshape((2048, 64, 512))
+    calls("copy_transpose (64,512,2048) f32 axes (2,0,1)", lambda: be.copy_transpose(t3_in, t3_out, axes=(2, 0, 1)),
+          2 * sq[0] * sq[1] * 4, "prebuilt (kernels.hip)", reps=10)
+    del t_in, t_out, t3_in, t3_out, a32
+
+    # the GEMM hand-off (library kernel; flops, not bytes, bound it)
+    m = 4096
+    for dt, label in ((f32, "f32"), (f16, "f16")):
+        A, B, C = (_fresh(be, (m, m), dtype=dt, rs=rs, scale=0.1) for _ in range(3))
+        calls("compound_dot (4096,4096)x(4096,4096) %s [library GEMM]" % label,
+              lambda: be.compound_dot(A, B, C), 3 * m * m * np.dtype(dt).itemsize, "rocBLAS", reps=10,
+              flops=2.0 * m * m * m)
+        del A, B, C
+    rt.synchronize()
 
 
 def cpu_leg(max_seconds=25.0):

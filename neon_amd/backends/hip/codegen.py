@@ -108,6 +108,7 @@ class _Gen(object):
         # streaming kernels (working set far beyond the caches) mark their
         # global accesses non-temporal
         self.pos = ("0", "0")      # (row, column) expressions of the element being emitted
+        self.pos_v = 1             # ... the column expression is a multiple of this
         self.ld = "load_stream" if stream else "load"
         self.st = "store_stream" if (stream and STREAM_STORES[family]) else "store"
 
@@ -212,14 +213,19 @@ class _Gen(object):
             elif n.op == "zero_index":
                 e = "0.0f"
             elif n.op == "rand" or n.op.startswith("sround:"):
-                # counter = element index * streams + this node's stream
+                # random word number = launch base + element index * streams + this node's stream
                 r, c = self.pos
-                counter = ("rng_base + ((unsigned long long)(%s) * (unsigned long long)C + "
-                           "(unsigned long long)((%s) + j)) * %dull + %dull" % (r, c, self.prog.rand_count, n.slot))
+                streams = self.prog.rand_count
+                # the launch base is even; the words of a lane's tile pair up
+                # on shared evaluations when its first word is even as well
+                aligned = streams % 2 == 0 or (self.pos_v % 2 == 0 and (self.C % 2 == 0 or self.R == 1))
+                word = ("nh_rand_word<%d, %d, %s>(rng_seed, rng_base + ((unsigned long long)(%s) * "
+                        "(unsigned long long)C + (unsigned long long)(%s)) * %dull, j)"
+                        % (streams, n.slot, "true" if aligned else "false", r, c, streams))
                 if n.op == "rand":
-                    e = "nh_rand01(rng_seed, %s)" % counter
+                    e = "nh_rand01(%s)" % word
                 else:
-                    e = "nh_sround(%s, %s, rng_seed, %s)" % (a[0], n.op.split(":")[1], counter)
+                    e = "nh_sround(%s, %s, %s)" % (a[0], n.op.split(":")[1], word)
             elif len(a) == 1:
                 e = _UN[n.op].format(*a)
             else:
@@ -271,6 +277,7 @@ def gen_ew(prog, V, LX, LY, UC, UR, tail, stream=False):
 
     def ref_for(sfx, r, c, Vv):
         g.pos = (r, c)
+        g.pos_v = Vv
 
         def ref(n):
             if n.kind == "C":
@@ -405,6 +412,7 @@ class _RedGen(_Gen):
 
     def make_ref(self, sfx, r, c, Vv, tiles=None, vals=None):
         self.pos = (r, c)
+        self.pos_v = Vv
 
         def ref(n):
             if vals and n.nid in vals:

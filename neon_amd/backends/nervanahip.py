@@ -756,6 +756,7 @@ class NervanaHIP(Backend):
         if prog.rand_count:
             # counter-based generator: this launch owns the next R*C*streams counters
             n = plan.domain[0] * plan.domain[1] * prog.rand_count
+            self._rng_dev_counter += self._rng_dev_counter & 1       # kernels pair words from an even base
             prog.rng_args = (self._rng_dev_seed, self._rng_dev_counter)
             self._rng_dev_counter += n
         args = plan.pack(prog)

@@ -242,35 +242,52 @@ NEON_DEV float nh_sig2(float x) { return 1.0f / (1.0f + exp2f(-x)); }
 NEON_DEV float nh_tanh2(float x) { const float e = exp2f(2.0f * x); return (e - 1.0f) / (e + 1.0f); }
 NEON_DEV float nh_finite(float x) { return (__builtin_fabsf(x) <= NH_FLT_MAX) ? 1.0f : 0.0f; }
 
-// Counter-based uniform random numbers in [0, 1): element `counter` of the
-// stream `seed` (splitmix64 finaliser, top 24 bits).  Stateless, so a tensor
-// filled twice from the same (seed, counter) gets the same values and no
+// Counter-based random numbers.  Word `w` of the stream `seed` is one half of
+// splitmix64(w >> 1): stateless, so a tensor filled twice from the same
+// (seed, counter) gets the same values whatever the kernel's tiling, and no
 // generator state lives on the device (the reference kept a pool of LFSR
-// states, cuda_templates.py:138-186).
-NEON_DEV nh_u32 nh_rand_u32(nh_u32 seed, unsigned long long counter) {
-    unsigned long long z = counter + ((unsigned long long)seed + 1ull) * 0x9E3779B97F4A7C15ull;
+// states, cuda_templates.py:138-186).  The two 64-bit multiplies dominate the
+// cost of a dropout mask, hence two words per evaluation.
+NEON_DEV unsigned long long nh_splitmix64(nh_u32 seed, unsigned long long index) {
+    unsigned long long z = index + ((unsigned long long)seed + 1ull) * 0x9E3779B97F4A7C15ull;
     z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
     z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
-    z ^= z >> 31;
-    return (nh_u32)(z >> 32);
+    return z ^ (z >> 31);
 }
-NEON_DEV float nh_rand01(nh_u32 seed, unsigned long long counter) {
-    return (float)(nh_rand_u32(seed, counter) >> 8) * 5.9604644775390625e-8f;      // 2^-24
+// Word w0 + j * STRIDE + OFF.  With ALIGNED the caller guarantees that w0 is
+// even: the pair index then is (w0 >> 1) plus a compile-time constant once j
+// is unrolled, and neighbouring words share one evaluation.
+template <int STRIDE, int OFF, bool ALIGNED>
+NEON_DEV nh_u32 nh_rand_word(nh_u32 seed, unsigned long long w0, int j) {
+    const int rel = j * STRIDE + OFF;
+    unsigned long long z;
+    bool high;
+    if constexpr (ALIGNED) {
+        z = nh_splitmix64(seed, (w0 >> 1) + (unsigned long long)(rel >> 1));
+        high = (rel & 1) != 0;
+    } else {
+        const unsigned long long w = w0 + (unsigned long long)rel;
+        z = nh_splitmix64(seed, w >> 1);
+        high = (w & 1ull) != 0;
+    }
+    return high ? (nh_u32)(z >> 32) : (nh_u32)z;
 }
+// uniform in [0, 1) from the top 24 bits of a random word
+NEON_DEV float nh_rand01(nh_u32 word) { return (float)(word >> 8) * 5.9604644775390625e-8f; }      // 2^-24
 
-// Stochastic rounding to `bits` (1..22) mantissa bits: the value moves to the
-// neighbour of larger magnitude with probability equal to the fraction of the
-// spacing it sits above the neighbour of smaller magnitude, so the result is
-// unbiased (the reference adds a uniform fraction of the spacing with
-// round-toward-zero and masks, cuda_templates.py:148-152, 193-235).  Done on
-// the bit pattern: random bits added below the kept mantissa bits carry into
-// them (and on into the exponent) with exactly that probability.  Infinities
-// and NaN pass through.
-NEON_DEV float nh_sround(float x, int bits, nh_u32 seed, unsigned long long counter) {
+// Stochastic rounding to `bits` (1..22) mantissa bits with the random word
+// `rnd`: the value moves to the neighbour of larger magnitude with probability
+// equal to the fraction of the spacing it sits above the neighbour of smaller
+// magnitude, so the result is unbiased (the reference adds a uniform fraction
+// of the spacing with round-toward-zero and masks, cuda_templates.py:148-152,
+// 193-235).  Done on the bit pattern: random bits added below the kept
+// mantissa bits carry into them (and on into the exponent) with exactly that
+// probability.  Infinities and NaN pass through.
+NEON_DEV float nh_sround(float x, int bits, nh_u32 rnd) {
     const nh_u32 b = __builtin_bit_cast(nh_u32, x);
     if ((b & 0x7f800000u) == 0x7f800000u) return x;
     const int drop = 23 - bits;
-    const nh_u32 noise = nh_rand_u32(seed, counter) >> (32 - drop);
+    const nh_u32 noise = rnd >> (32 - drop);
     return __builtin_bit_cast(float, (b + noise) & (0xffffffffu << drop));
 }
 
