@@ -476,6 +476,7 @@ class NervanaHIP(Backend):
         self._recording = None
         self._rec_temps = None
         self._rec_foreign = False     # the group being recorded made a call that is not a kernel launch
+        self._originals = frozenset() # ids of handles whose reads mean "before the running group" (compensated_sum)
         self._rec_single = None
         self._temp_pool = {}
         self._live_allocs = 0
@@ -717,6 +718,8 @@ class NervanaHIP(Backend):
         (its own TODO at float_ew.py:640-641 asks for exactly this)."""
         try:
             key, raw = self._launch_key(trees)
+            if self._originals:
+                key = key + ("reads-before-group",)
         except (AttributeError, TypeError):
             key, raw = None, None
         entry = self._launch_cache.get(key) if key is not None else None
@@ -771,6 +774,7 @@ class NervanaHIP(Backend):
     def _run_slow(self, trees):
         try:
             prog = Program()
+            prog.originals = self._originals
             for t in trees:
                 prog.add_statement(t)
             prog.finalize()
@@ -784,6 +788,8 @@ class NervanaHIP(Backend):
                 self.plan_stats["hit"] += 1
             self._launch_plan(plan, prog)
         except (NeedsSplit, MixedAxes, NotImplementedError) as e:
+            if self._originals:
+                raise          # statements that read pre-group values only make sense as one kernel
             if len(trees) != 1:
                 for t in trees:
                     self._run([t])
@@ -911,12 +917,9 @@ class NervanaHIP(Backend):
             for t in temps:
                 self._temp_release(t)
 
-    def _run_leaf(self, tree, more=(), originals=()):
+    def _run_leaf(self, tree):
         prog = Program()
-        prog.originals = frozenset(id(t) for t in originals)
         prog.add_statement(tree)
-        for t in more:
-            prog.add_statement(t)
         prog.finalize()
         key = prog.key()
         plan = self.plans.get(key)
@@ -1070,9 +1073,11 @@ class NervanaHIP(Backend):
                              strides=t.strides, name=t.name)
         old_sum, old_cmp = alias(sum_tensor), alias(cmp_tensor)
         y = add_tensor * add_scale - old_cmp * cmp_scale
-        self._run_leaf(self._stmt(sum_tensor, old_sum + y),
-                       more=[self._stmt(cmp_tensor, (sum_tensor - old_sum) - y)],
-                       originals=(old_sum, old_cmp))
+        self._originals = frozenset((id(old_sum), id(old_cmp)))
+        try:
+            self._run([self._stmt(sum_tensor, old_sum + y), self._stmt(cmp_tensor, (sum_tensor - old_sum) - y)])
+        finally:
+            self._originals = frozenset()
 
     # -- batch normalisation as fused statement groups -------------------------------------------
     @staticmethod
