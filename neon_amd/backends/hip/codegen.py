@@ -453,17 +453,25 @@ class _RedGen(_Gen):
 # =====================================================================================
 # family: row  (axis 1)
 # =====================================================================================
-def gen_row(prog, V, LX, LY, NCH, stream=False):
+def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None):
     """Axis-1 reductions.  A team of LX lanes (a power of two up to 64, or the
     whole workgroup) owns one row; the workgroup holds LY rows.  A lane visits
     column tiles tx, tx+LX, ...; with ``NCH`` > 0 that loop has a fixed trip
     count and the tiles loaded in the first sweep stay in registers for the
-    later ones; with ``NCH`` == 0 every sweep streams the row again."""
+    later ones; with ``NCH`` == 0 every sweep streams the row again.
+
+    ``keep_words`` (with ``NCH`` > 0) limits the 32-bit registers per lane that
+    resident tiles may take: operands are made resident in order of first use
+    while they fit, the others are fetched again, a few tiles at a time, in
+    every sweep that reads them (batch-norm backward keeps ``x`` and re-reads
+    the deltas: four passes over HBM instead of five)."""
     g = _RedGen(prog, V, stream, "row")
     L = g.L
     T = LX * LY
     assert LX <= 64 or LY == 1
     resident = NCH > 0
+    words_left = [keep_words]       # None: everything is kept
+    transient = set()               # nids of row operands that are not kept
     params, fmt = g.param_list([])
     head = ('extern "C" __global__ __launch_bounds__(%d) void @NAME@(%s)\n' % (T, params))
     per_level = _levels(prog)
@@ -485,6 +493,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False):
         L("const int nch = (C + %d - 1) / %d;" % (LX * V, LX * V))
 
     SU = 4      # column tiles in flight per lane when the row is streamed
+    NCHP = -(-NCH // SU) * SU
 
     def chunk_position(k):
         L("const long long c = ((long long)(%s) * %d + tx) * %d;" % (k, LX, V))
@@ -500,7 +509,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False):
         moving = [n for n in leaves if varies_in_loop(n)]
         tiles = dict((n.nid, line_tiles[n.nid]) for n in leaves if not varies_in_loop(n))
         if resident:
-            fresh = [n for n in moving if n.nid not in cached]
+            fresh = [n for n in moving if n.nid not in cached and n.nid not in transient]
             if fresh:
                 L("#pragma unroll")
                 L.open("for (int k = 0; k < %d; ++k)" % NCH)
@@ -510,12 +519,37 @@ def gen_row(prog, V, LX, LY, NCH, stream=False):
                     L("if (ok) keep%d[k].%s(%s); else keep%d[k].zero();"
                       % (n.nid, g.ld, g.tile_addr(n, "rr", "c"), n.nid))
                 L.close()
+            passing = [n for n in moving if n.nid in transient]
             for n in moving:
-                tiles[n.nid] = "%s[k]" % cached[n.nid]
+                if n.nid not in transient:
+                    tiles[n.nid] = "%s[k]" % cached[n.nid]
+            if not passing:
+                L("#pragma unroll")
+                L.open("for (int k = 0; k < %d; ++k)" % NCH)
+                chunk_position("k")
+                emit_body(tiles)
+                L.close()
+                return
+            # kept tiles come from registers, the others SU tiles at a time
             L("#pragma unroll")
-            L.open("for (int k = 0; k < %d; ++k)" % NCH)
+            L.open("for (int kb = 0; kb < %d; kb += %d)" % (NCH, SU))
+            for n in passing:
+                L("%s %s[%d];" % (g.tile_type(n, V), g.tile_name(n, "_s"), SU))
+                tiles[n.nid] = "%s[u]" % g.tile_name(n, "_s")
+            L("#pragma unroll")
+            L.open("for (int u = 0; u < %d; ++u)" % SU)
+            L("const int k = kb + u;")
+            chunk_position("k")         # k beyond the row: c >= C, so ok is false
+            for n in passing:
+                L("if (ok) %s[u].%s(%s); else %s[u].zero();"
+                  % (g.tile_name(n, "_s"), g.ld, g.tile_addr(n, "rr", "c"), g.tile_name(n, "_s")))
+            L.close()
+            L("#pragma unroll")
+            L.open("for (int u = 0; u < %d; ++u)" % SU)
+            L("const int k = kb + u;")
             chunk_position("k")
             emit_body(tiles)
+            L.close()
             L.close()
             return
         L.open("for (int kb = 0; kb < nch; kb += %d)" % SU)
@@ -550,8 +584,15 @@ def gen_row(prog, V, LX, LY, NCH, stream=False):
                     line_tiles[n.nid] = name
                     L("%s %s;" % (g.tile_type(n, V), name))
                     L("%s.load(%s);" % (name, g.tile_addr(n, "rr", "0")))
-            elif resident and n.nid not in cached:
-                L("%s keep%d[%d];" % (g.tile_type(n, V), n.nid, NCH))
+            elif resident and n.nid not in cached and n.nid not in transient:
+                need = NCH * max(1, (g.tile_width(n, V) * prog.tensors[n.slot].dtype.itemsize + 3) // 4)
+                if words_left[0] is not None and need > words_left[0]:
+                    transient.add(n.nid)
+                    continue
+                if words_left[0] is not None:
+                    words_left[0] -= need
+                # (rounded up to whole batches so that batch loops index within bounds)
+                L("%s keep%d[%d];" % (g.tile_type(n, V), n.nid, NCHP))
         if resident:
             for nid, name in cached.items():
                 L("#pragma unroll")
@@ -650,7 +691,8 @@ def gen_row(prog, V, LX, LY, NCH, stream=False):
 
         sweep(leaves, store_body)
     L.close()
-    return _finish("row", g, head, fmt, T, 0, dict(V=V, LX=LX, LY=LY, NCH=NCH, stream=bool(stream)))
+    return _finish("row", g, head, fmt, T, 0, dict(V=V, LX=LX, LY=LY, NCH=NCH, stream=bool(stream),
+                                                   passing=len(transient)))
 
 
 # =====================================================================================

@@ -1105,9 +1105,11 @@ class NervanaHIP(Backend):
         that reads ``x`` once and keeps each row in registers."""
         if binary:
             raise NotImplementedError("shift-based batch norm is outside the op-tree path")
+        # like the reference's kernel (cuda_batchnorm.py:176-188) the previous
+        # output is only read when it is accumulated into
         if inference:
             xhat = (x - gmean) / self.sqrt(gvar + eps)
-            y[:] = y * accumbeta + xhat * gamma + beta
+            y[:] = (y * accumbeta + xhat * gamma + beta) if accumbeta != 0 else (xhat * gamma + beta)
             return
         st, n = self._stmt, float(x.shape[1])
         trees = []
@@ -1119,7 +1121,7 @@ class NervanaHIP(Backend):
         trees.append(st(gvar, gvar * rho + (1.0 - rho) * xvar))
         xhat = (x - xsum) / self.sqrt(xvar + eps)
         out = y.reshape(x.shape)
-        trees.append(st(out, xhat * gamma + beta + accumbeta * out))
+        trees.append(st(out, (xhat * gamma + beta + accumbeta * out) if accumbeta != 0 else (xhat * gamma + beta)))
         self._run_group(trees)
 
     def compound_bprop_bn(self, delta_out, grad_gamma, grad_beta, delta_in, x, xsum, xvar,

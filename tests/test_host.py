@@ -272,3 +272,24 @@ def test_stochastic_rounding_store_compiles_and_changes_the_plan(tmp_path):
         bad = be.empty((4, 4), np.int32)
         bad.rounding = 2
         bad[:] = x[:4, :4] * 1.0
+
+
+def test_long_rows_of_two_tensors_keep_one_resident(pb):
+    """batch-norm backward shape: x and the deltas, 100352 fp16 columns each --
+    one row fits the registers of a 1024-lane workgroup, two do not"""
+    K, N = 256, 100352
+    x, d, out = (pb.empty((K, N), np.float16) for _ in range(3))
+    mean, scale = pb.empty((K, 1)), pb.empty((K, 1))
+    gg, gb = pb.empty((K, 1)), pb.empty((K, 1))
+    n = len(pb.choices)
+    pb.begin(Block.update, 0)
+    xhat = (x - mean) * scale
+    gg[:] = pb.sum(xhat * d, axis=1)
+    gb[:] = pb.sum(d, axis=1)
+    out[:] = (d - (xhat * gg + gb) / float(N)) * scale
+    pb.end(Block.update, 0)
+    assert len(pb.choices) == n + 1
+    spec = pb.choices[-1].spec
+    assert spec.family == "row" and spec.params["NCH"] == 13 and spec.params["passing"] == 1
+    # x is loaded once, the deltas once per sweep
+    assert spec.source.count(".load_stream(") == 3
