@@ -365,25 +365,114 @@ __global__ __launch_bounds__(CR_T) void colmax_kernel(const float* __restrict__ 
 constexpr int HIST_T = 256;
 constexpr int HIST_MAX_BINS = 256;
 
-template <typename T>
+// Bin of one value: rint(log2|v|) - offset, clamped below into bin 0 and (one
+// past the end only) above into the last bin; -1 = not counted (larger
+// magnitudes, NaN).
+__device__ __forceinline__ int hist_bin(float v, int nbins, int offset) {
+    const float b = rintf(log2f(__builtin_fabsf(v))) - (float)offset;    // nan compares false everywhere
+    if (!(b <= (float)nbins)) return -1;
+    const int bin = b < 1.0f ? 0 : (int)b;
+    return bin > nbins - 1 ? nbins - 1 : bin;
+}
+
+// Magnitudes of real tensors fall into a handful of bins, so LDS atomics on a
+// shared histogram serialise (64 lanes, a few addresses).  Two ways round it:
+//
+// PRIVATE (nbins <= 64): every lane counts into its own 16-bit counters --
+// word [bin][tid % 128] holds lane tid's count in its low half and lane
+// tid + 128's in its high half, so the lanes of a wave always hit distinct
+// banks whatever the data; the host sizes the grid so that no lane sees more
+// than 65535 elements.  32 KiB of LDS per workgroup.
+//
+// otherwise: the wave agrees on one bin at a time (ballot) and a single lane
+// adds the number of lanes that hold it to the wave's own histogram.
+constexpr int HIST_PRIVATE_BINS = 64;
+
+template <typename T, bool PRIVATE>
 __global__ __launch_bounds__(HIST_T) void hist_log2_kernel(const T* __restrict__ x, size_t n, int nbins, int offset,
                                                            int* __restrict__ hist) {
-    __shared__ int bins[HIST_MAX_BINS];
-    for (int b = threadIdx.x; b < nbins; b += HIST_T) bins[b] = 0;
+    constexpr int V = 16 / (int)sizeof(T);                 // elements per 16-byte load
+    constexpr int WAVES = HIST_T / 64;
+    constexpr int WORDS = PRIVATE ? HIST_PRIVATE_BINS * (HIST_T / 2) : WAVES * HIST_MAX_BINS;
+    __shared__ int bins[WORDS];
+    for (int b = threadIdx.x; b < WORDS; b += HIST_T) bins[b] = 0;
     __syncthreads();
-    const size_t stride = (size_t)gridDim.x * HIST_T;
-    for (size_t i = (size_t)blockIdx.x * HIST_T + threadIdx.x; i < n; i += stride) {
-        const float v = rintf(log2f(__builtin_fabsf((float)x[i])));
-        const float b = v - (float)offset;           // nan compares false everywhere: not counted
-        if (b <= (float)nbins) {
-            int bin = b < 1.0f ? 0 : (int)b;
-            if (bin > nbins - 1) bin = nbins - 1;
-            atomicAdd(&bins[bin], 1);
+    const int lane = threadIdx.x & 63;
+    int* mine = PRIVATE ? bins + (threadIdx.x & (HIST_T / 2 - 1)) : bins + (threadIdx.x / 64) * HIST_MAX_BINS;
+    const int one = (PRIVATE && threadIdx.x >= HIST_T / 2) ? 0x10000 : 1;
+    const size_t stride = (size_t)gridDim.x * HIST_T * V;
+    // same trip count for every lane of the grid: the wave-wide counting needs all lanes
+    const size_t trips = (n + stride - 1) / stride;
+    const bool vec_ok = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
+    size_t i0 = ((size_t)blockIdx.x * HIST_T + threadIdx.x) * V;
+    constexpr int U = 4;                                   // loads in flight per lane
+    for (size_t t = 0; t < trips; t += U, i0 += U * stride) {
+        nh_u32 w[U][4];
+        bool whole[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const size_t i = i0 + u * stride;
+            whole[u] = vec_ok && t + u < trips && i + V <= n;
+            if (whole[u]) nh_load_words<4, true>(reinterpret_cast<const nh_u32*>(x + i), w[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const size_t i = i0 + u * stride;
+            float v[V];
+            int live = 0;
+            if (whole[u]) {
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    if constexpr (sizeof(T) == 4) v[j] = __builtin_bit_cast(float, w[u][j]);
+                    else v[j] = (j & 1) ? nh_f16_hi(w[u][j / 2]) : nh_f16_lo(w[u][j / 2]);
+                }
+                live = V;
+            } else if (t + u < trips) {
+#pragma unroll
+                for (int j = 0; j < V; ++j)
+                    if (i + j < n) { v[j] = (float)x[i + j]; live = j + 1; }
+            }
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                const int bin = j < live ? hist_bin(v[j], nbins, offset) : -1;
+                if constexpr (PRIVATE) {
+                    if (bin >= 0) atomicAdd(&mine[bin * (HIST_T / 2)], one);     // LDS; only lane tid +- 128 shares the word
+                } else {
+                    unsigned long long todo = __ballot(bin >= 0);
+                    while (todo) {
+                        const int leader = __ffsll((long long)todo) - 1;
+                        const int b = __builtin_amdgcn_readlane(bin, leader);
+                        const unsigned long long same = __ballot(bin == b);
+                        if (lane == leader) mine[b] += __popcll(same);
+                        todo &= ~same;
+                    }
+                }
+            }
         }
     }
     __syncthreads();
-    for (int b = threadIdx.x; b < nbins; b += HIST_T)
-        if (bins[b]) atomicAdd(&hist[b], bins[b]);
+    if constexpr (PRIVATE) {
+        // four lanes per bin, 32 words each, both halves of every word
+        const int b = threadIdx.x / 4, part = threadIdx.x % 4;
+        int total = 0;
+        if (b < nbins) {
+            const int* row = bins + b * (HIST_T / 2) + part * (HIST_T / 8);
+            for (int k = 0; k < HIST_T / 8; ++k) {
+                const unsigned int w = (unsigned int)row[(k + lane) % (HIST_T / 8)];
+                total += (int)(w & 0xffffu) + (int)(w >> 16);
+            }
+        }
+        total += __shfl_xor(total, 1);
+        total += __shfl_xor(total, 2);
+        if (part == 0 && b < nbins && total) atomicAdd(&hist[b], total);
+    } else {
+        for (int b = threadIdx.x; b < nbins; b += HIST_T) {
+            int total = 0;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) total += bins[w * HIST_MAX_BINS + b];
+            if (total) atomicAdd(&hist[b], total);
+        }
+    }
 }
 
 struct CrPlan { uint32_t strips, chunks, rows_per_chunk; int v; };
@@ -550,15 +639,19 @@ int nh_hist_log2(int32_t* hist, const void* x, int itemsize, size_t n, int nbins
     if (e != hipSuccess) return nh_internal_fail((int)e, "nh_hist_log2: clearing the bins failed");
     if (n == 0) return 0;
     size_t blocks = (n + HIST_T * 16 - 1) / ((size_t)HIST_T * 16);
-    const size_t cap = (size_t)(nh_internal_cu_count() > 0 ? nh_internal_cu_count() : 256) * 8;
+    const size_t cap = (size_t)(nh_internal_cu_count() > 0 ? nh_internal_cu_count() : 256) * 4;
     if (blocks > cap) blocks = cap;
     if (blocks < 1) blocks = 1;
-    if (itemsize == 4)
-        hipLaunchKernelGGL((hist_log2_kernel<float>), dim3((unsigned)blocks), dim3(HIST_T), 0, s, (const float*)x, n,
-                           nbins, offset, (int*)hist);
-    else
-        hipLaunchKernelGGL((hist_log2_kernel<nh_f16>), dim3((unsigned)blocks), dim3(HIST_T), 0, s, (const nh_f16*)x, n,
-                           nbins, offset, (int*)hist);
+    // private 16-bit counters: at most 65535 elements per lane
+    const bool priv = nbins <= HIST_PRIVATE_BINS && n / (blocks * HIST_T) < 60000;
+    const dim3 grid((unsigned)blocks), block(HIST_T);
+    if (itemsize == 4) {
+        if (priv) hipLaunchKernelGGL((hist_log2_kernel<float, true>), grid, block, 0, s, (const float*)x, n, nbins, offset, (int*)hist);
+        else hipLaunchKernelGGL((hist_log2_kernel<float, false>), grid, block, 0, s, (const float*)x, n, nbins, offset, (int*)hist);
+    } else {
+        if (priv) hipLaunchKernelGGL((hist_log2_kernel<nh_f16, true>), grid, block, 0, s, (const nh_f16*)x, n, nbins, offset, (int*)hist);
+        else hipLaunchKernelGGL((hist_log2_kernel<nh_f16, false>), grid, block, 0, s, (const nh_f16*)x, n, nbins, offset, (int*)hist);
+    }
     return launch_status("nh_hist_log2");
 }
 

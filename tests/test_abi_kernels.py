@@ -129,3 +129,30 @@ def test_launch_validation(hip):
     assert lib.nh_malloc(byref(p), 0) == hiprt.NH_EINVAL
     assert lib.nh_malloc(byref(p), c_size_t(1 << 60)) != 0          # far beyond device memory
     assert b"exceeds" in lib.nh_last_error()
+
+
+@pytest.mark.parametrize("nbins,offset", [(64, -48), (100, -60), (256, -130), (7, -3)])
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
+@pytest.mark.parametrize("n,skew", [(1, 0), (4099, 0), (1 << 20, 0), (3 * 1000 * 1000 + 5, 1)])
+def test_hist_log2_entry_point(dev, n, skew, dtype, nbins, offset):
+    """both counting schemes (private counters up to 64 bins, wave-agreed bins
+    beyond), vector body and scalar tail, aligned and unaligned start, against
+    numpy's histogram of rint(log2|x|) (the binning of nervanacpu.py:424-445)"""
+    rs = np.random.RandomState(n % 89 + nbins)
+    # magnitudes 2^(k + f), |f| <= 0.4: rint(log2|x|) = k whatever the last bit of log2f
+    lo, hi = (-20, 8) if dtype == np.float32 else (-12, 8)
+    a = (np.exp2(rs.randint(lo, hi, size=n + skew) + rs.uniform(-0.4, 0.4, size=n + skew)) *
+         rs.choice([-1.0, 1.0], size=n + skew)).astype(dtype)
+    a[rs.randint(0, n + skew, size=min(n, 5))] = 0
+    if n > 16:
+        a[3], a[7], a[11] = np.nan, np.inf, -np.inf
+    base = dev.put(a)
+    x = base + skew * a.dtype.itemsize               # skew: not 16-byte aligned
+    hist = dev.alloc(4 * nbins)
+    ok(dev.lib, dev.lib.nh_hist_log2(c_void_p(hist), c_void_p(x), a.dtype.itemsize, n, nbins, offset, None))
+    got = dev.get(hist, (nbins,), np.int32)
+    edges = np.arange(nbins + 1) + float(offset)
+    edges[0] = -np.inf
+    with np.errstate(divide="ignore", invalid="ignore"):
+        want, _ = np.histogram(np.rint(np.log2(np.abs(a[skew:].astype(np.float32)))), bins=edges)
+    assert np.array_equal(got, want.astype(np.int32))
