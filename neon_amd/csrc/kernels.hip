@@ -571,6 +571,69 @@ __global__ __launch_bounds__(TR_T) void transpose_tile_kernel(T* __restrict__ ou
     }
 }
 
+// The same tile walk for 4-byte elements with 16-byte global accesses: 16
+// lanes cover a 64-element run, the workgroup moves 16 runs per pass.  Needs
+// both tile extents, the strides of every other dimension and the base
+// addresses to be multiples of 4 elements.  LDS is still accessed word by word
+// (row pitch 65: the four words a lane turns into an output vector come from
+// four tile rows), two-way bank conflicts at worst.
+template <bool SWAP>
+__global__ __launch_bounds__(TR_T) void transpose_tile_v4_kernel(uint32_t* __restrict__ out,
+                                                                 const uint32_t* __restrict__ in, TrGeom g) {
+    __shared__ uint32_t tile[SWAP ? TR_TILE : 1][TR_TILE + 1];
+    unsigned long long b = blockIdx.x;
+    const uint32_t tx = (uint32_t)(b % g.tiles_x);
+    b /= g.tiles_x;
+    const uint32_t ty = (uint32_t)(b % g.tiles_y);
+    b /= g.tiles_y;
+    long long ibase = 0, obase = 0;
+    for (int k = g.nd - 1; k >= 0; --k) {
+        if (k == g.ax || k == g.ay) continue;
+        const unsigned long long idx = b % g.n[k];
+        b /= g.n[k];
+        ibase += (long long)idx * g.is[k];
+        obase += (long long)idx * g.os[k];
+    }
+    const uint32_t nx = g.n[g.ax], ny = g.ay >= 0 ? g.n[g.ay] : 1u;
+    const long long isx = g.is[g.ax], osx = g.os[g.ax];
+    const long long isy = g.ay >= 0 ? g.is[g.ay] : 0, osy = g.ay >= 0 ? g.os[g.ay] : 0;
+    const uint32_t x0 = tx * TR_TILE, y0 = ty * TR_TILE;
+    const uint32_t quad = (threadIdx.x & 15u) * 4u, run = threadIdx.x >> 4;     // 16 runs of 16 quads
+    constexpr uint32_t RUNS = TR_T / 16;
+    if constexpr (SWAP) {
+        // input runs along y (isy == 1): run index = x
+        for (uint32_t i = run; i < TR_TILE; i += RUNS) {
+            const uint32_t x = x0 + i, y = y0 + quad;
+            if (x < nx && y < ny) {
+                nh_u32 w[4];
+                nh_load_words<4, true>(in + ibase + (long long)x * isx + (long long)y, w);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) tile[i][quad + j] = w[j];
+            }
+        }
+        __syncthreads();
+        // output runs along x (osx == 1): run index = y
+        for (uint32_t i = run; i < TR_TILE; i += RUNS) {
+            const uint32_t x = x0 + quad, y = y0 + i;
+            if (x < nx && y < ny) {
+                nh_u32 w[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) w[j] = tile[quad + j][i];
+                nh_store_words<4, false>(out + obase + (long long)x + (long long)y * osy, w);
+            }
+        }
+    } else {
+        for (uint32_t i = run; i < TR_TILE; i += RUNS) {
+            const uint32_t x = x0 + quad, y = y0 + i;
+            if (x < nx && y < ny) {
+                nh_u32 w[4];
+                nh_load_words<4, true>(in + ibase + (long long)x + (long long)y * isy, w);
+                nh_store_words<4, false>(out + obase + (long long)x + (long long)y * osy, w);
+            }
+        }
+    }
+}
+
 template <typename T>
 void launch_transpose(void* out, const void* in, const TrGeom& g, bool swap, unsigned blocks, hipStream_t s) {
     if (swap)
@@ -703,6 +766,25 @@ int nh_copy_transpose(void* out, const void* in, int itemsize, int ndim, const u
         if (k != ax && k != ay) blocks *= g.n[k];
     if (blocks > 0x7fffffffull) return nh_internal_fail(NH_EINVAL, "nh_copy_transpose: too many tiles for one launch");
     hipStream_t s = (hipStream_t)stream;
+    if (itemsize == 4 && ay >= 0) {
+        // 16-byte accesses when every run of four elements is aligned on both sides
+        bool v4 = aligned16(out) && aligned16(in) && g.n[ax] % 4 == 0 && g.os[ax] == 1 &&
+                  (swap ? (g.n[ay] % 4 == 0 && g.is[ay] == 1) : g.is[ax] == 1);
+        for (int k = 0; k < ndim && v4; ++k) {
+            if (g.n[k] == 1) continue;
+            if (k != ax && g.os[k] % 4) v4 = false;
+            if (k != (swap ? ay : ax) && g.is[k] % 4) v4 = false;
+        }
+        if (v4) {
+            if (swap)
+                hipLaunchKernelGGL((transpose_tile_v4_kernel<true>), dim3((unsigned)blocks), dim3(TR_T), 0, s,
+                                   (uint32_t*)out, (const uint32_t*)in, g);
+            else
+                hipLaunchKernelGGL((transpose_tile_v4_kernel<false>), dim3((unsigned)blocks), dim3(TR_T), 0, s,
+                                   (uint32_t*)out, (const uint32_t*)in, g);
+            return launch_status("nh_copy_transpose");
+        }
+    }
     switch (itemsize) {
         case 1: launch_transpose<uint8_t>(out, in, g, swap, (unsigned)blocks, s); break;
         case 2: launch_transpose<uint16_t>(out, in, g, swap, (unsigned)blocks, s); break;
