@@ -1,0 +1,254 @@
+"""Activations, costs and metrics (neon_amd/transforms): the known answers the
+reference's own tests hold (tests/test_activations.py, tests/test_costs.py) on
+the oracle backend, then the hip backend against the oracle at sizes where the
+reductions run as column kernels."""
+import contextlib
+
+import numpy as np
+import pytest
+
+from neon_amd import NervanaObject
+from neon_amd.transforms import (Accuracy, CrossEntropyBinary, CrossEntropyMulti, Explin, Identity,
+                                 LogLoss, Logistic, MeanSquared, Misclassification, Normalizer,
+                                 PrecisionRecall, Rectlin, Rectlinclip, SmoothL1Loss, Softmax,
+                                 SquareHingeLoss, SumSquared, Tanh, TopKMisclassification)
+from utils import assert_close
+
+
+@contextlib.contextmanager
+def using(be, bsz=None):
+    """make `be` the process-wide backend, as gen_backend would"""
+    old, old_bsz = NervanaObject.be, be.bsz
+    NervanaObject.be = be
+    if bsz is not None:
+        be.bsz = bsz
+    try:
+        yield be
+    finally:
+        NervanaObject.be, be.bsz = old, old_bsz
+
+
+def _eval(be, tree, shape):
+    if isinstance(tree, (int, float)):
+        return np.full((1, 1), tree, dtype=np.float32)
+    out = be.empty(shape)
+    out[:] = tree
+    return out.get()
+
+
+def _act(be, func, inputs, deriv=False):
+    x = be.array(np.asarray(inputs, dtype=np.float32))
+    with using(be):
+        tree = func.bprop(x) if deriv else func(x)
+        return _eval(be, tree, np.asarray(inputs).shape)
+
+
+def _cost(be, func, y, t, deriv=False):
+    yt, tt = be.array(np.asarray(y, dtype=np.float32)), be.array(np.asarray(t, dtype=np.float32))
+    with using(be):
+        tree = func.bprop(yt, tt) if deriv else func(yt, tt)
+        return _eval(be, tree, tree.shape)
+
+
+col = lambda *v: np.array(v, dtype=np.float64).reshape((-1, 1))
+EPS = np.exp(-50)
+
+ACT_CASES = [
+    # (name, transform, inputs, expected, derivative?, tolerance)  -- reference tests/test_activations.py
+    ("identity", lambda: Identity(), col(0, 1, -2), col(0, 1, -2), False, 0),
+    ("identity_d", lambda: Identity(), col(0, 1, -2), np.ones((1, 1)), True, 0),
+    ("rectlin_pos", lambda: Rectlin(), col(1, 3, 2), col(1, 3, 2), False, 0),
+    ("rectlin_neg", lambda: Rectlin(), [[-1, -3], [-2, -4]], [[0, 0], [0, 0]], False, 0),
+    ("rectlin_mixed", lambda: Rectlin(), [[4, 0], [-2, 9]], [[4, 0], [0, 9]], False, 0),
+    ("rectlin_d_pos", lambda: Rectlin(), col(1, 3, 2), col(1, 1, 1), True, 0),
+    ("rectlin_d_neg", lambda: Rectlin(), [[-1, -3], [-2, -4]], [[0, 0], [0, 0]], True, 0),
+    ("rectlin_d_mixed", lambda: Rectlin(), [[4, 0], [-2, 9]], [[1, 0], [0, 1]], True, 0),
+    ("leaky_neg", lambda: Rectlin(slope=0.2), [[-1, -3], [-2, -4]], np.array([[-1, -3], [-2, -4]]) * 0.2, False, 1e-7),
+    ("leaky_mixed", lambda: Rectlin(slope=0.2), [[4, 0], [-2, 9]], [[4, 0], [-0.4, 9]], False, 1e-7),
+    ("leaky_d_mixed", lambda: Rectlin(slope=0.2), [[4, 0], [-2, 9]], [[1, 0], [0.2, 1]], True, 1e-7),
+    ("softmax", lambda: Softmax(), col(0, 1, -2), np.exp(col(0, 1, -2) - 1) / np.sum(np.exp(col(0, 1, -2) - 1)), False, 1e-7),
+    ("softmax_d", lambda: Softmax(), col(0, 1, -2), np.ones((1, 1)), True, 0),
+    ("tanh", lambda: Tanh(), col(0, 1, -2), np.tanh(col(0, 1, -2)), False, 1e-7),
+    ("tanh_d", lambda: Tanh(), np.tanh(col(0, 1, -2)), 1 - np.tanh(col(0, 1, -2)) ** 2, True, 1e-7),
+    ("logistic", lambda: Logistic(), col(0, 1, -2), 1 / (1 + np.exp(-col(0, 1, -2))), False, 1e-7),
+    ("logistic_d", lambda: Logistic(shortcut=False), 1 / (1 + np.exp(-col(0, 1, -2))),
+     (1 / (1 + np.exp(-col(0, 1, -2)))) * (1 - 1 / (1 + np.exp(-col(0, 1, -2)))), True, 1e-7),
+    ("logistic_shortcut", lambda: Logistic(shortcut=True), col(0.5, 0.7), np.ones((1, 1)), True, 0),
+    # closed forms for the ones the reference's tests do not cover
+    ("explin", lambda: Explin(alpha=0.5), col(2, 0, -1), col(2, 0, 0.5 * (np.exp(-1) - 1)), False, 1e-7),
+    ("explin_d", lambda: Explin(alpha=0.5), col(2, -0.25), col(1, -0.25 + 0.5), True, 1e-7),
+    ("rectlinclip", lambda: Rectlinclip(slope=0.1, xcut=3.0), col(5, 2, -2), col(3, 2, -0.2), False, 1e-7),
+    ("rectlinclip_d", lambda: Rectlinclip(slope=0.1, xcut=3.0), col(5, 2, -2), col(0, 1, 0.1), True, 1e-7),
+    ("normalizer", lambda: Normalizer(divisor=4.0), col(2, -8), col(0.5, -2), False, 0),
+]
+
+
+@pytest.mark.parametrize("name,make,inputs,expected,deriv,tol", ACT_CASES, ids=[c[0] for c in ACT_CASES])
+def test_activation_known_answers(cpu, name, make, inputs, expected, deriv, tol):
+    got = _act(cpu, make(), inputs, deriv)
+    want = np.asarray(expected, dtype=np.float64)
+    assert got.shape == want.shape or want.shape == (1, 1)
+    assert np.all(np.abs(got - want) <= tol + 1e-12), (got, want)
+
+
+def test_softmax_big_inputs(cpu):
+    """reference tests/test_activations.py:156-184: 1000 classes, large logits"""
+    rs = np.random.RandomState(1)
+    x = rs.random_sample((1000, 128)) * 100
+    got = _act(cpu, Softmax(), x)
+    m = x.max(axis=0, keepdims=True)
+    want = np.exp(x - m) / np.exp(x - m).sum(axis=0, keepdims=True)
+    assert_close(got, want.astype(np.float32), rtol=1e-5, atol=1e-7)
+
+
+Y1, T1 = col(0.5, 0.9, 0.1, 0.0001), col(0.5, 0.99, 0.01, 0.2)
+Y2, T2 = col(0.5, 1.0, 0.0, 0.0001), col(0.5, 0.0, 1.0, 0.2)
+
+
+def _ceb(y, t):
+    return np.sum(-t * np.log(np.maximum(y, EPS)) - (1 - t) * np.log(np.maximum(1 - y, EPS)), keepdims=True)
+
+
+def _cem(y, t):
+    return np.sum(-t * np.log(np.maximum(y, EPS)), axis=0, keepdims=True)
+
+
+COST_CASES = [
+    # reference tests/test_costs.py:66-184
+    ("ce_binary", lambda: CrossEntropyBinary(), Y1, T1, _ceb(Y1, T1), False, 1e-6),
+    ("ce_binary_limits", lambda: CrossEntropyBinary(), Y2, T2, _ceb(Y2, T2), False, 1e-5),
+    ("ce_binary_d", lambda: CrossEntropyBinary(), Y2, T2, (Y2 - T2), True, 1e-6),
+    ("ce_multi", lambda: CrossEntropyMulti(), Y1, T1, _cem(Y1, T1), False, 1e-6),
+    ("ce_multi_limits", lambda: CrossEntropyMulti(), Y2, T2, _cem(Y2, T2), False, 1e-5),
+    ("ce_multi_d", lambda: CrossEntropyMulti(), Y2, T2, (Y2 - T2), True, 1e-6),
+    ("ce_multi_bits", lambda: CrossEntropyMulti(usebits=True), Y1, T1, _cem(Y1, T1) / np.log(2), False, 1e-6),
+    ("sum_squared", lambda: SumSquared(), Y1, T1, np.sum((Y1 - T1) ** 2, axis=0, keepdims=True) / 2, False, 1e-7),
+    ("sum_squared_d", lambda: SumSquared(), Y2, T2, (Y2 - T2), True, 1e-7),
+    ("mean_squared", lambda: MeanSquared(), Y1, T1, np.mean((Y1 - T1) ** 2, axis=0, keepdims=True) / 2, False, 1e-7),
+    ("mean_squared_d", lambda: MeanSquared(), Y2, T2, (Y2 - T2) / 4, True, 1e-7),
+    ("hinge", lambda: SquareHingeLoss(), col(0.5, -2, 3), col(1, -1, -1),
+     np.mean(np.maximum(1 - col(1, -1, -1) * col(0.5, -2, 3), 0) ** 2, axis=0, keepdims=True), False, 1e-6),
+]
+
+
+@pytest.mark.parametrize("name,make,y,t,expected,deriv,tol", COST_CASES, ids=[c[0] for c in COST_CASES])
+def test_cost_known_answers(cpu, name, make, y, t, expected, deriv, tol):
+    got = _cost(cpu, make(), y, t, deriv)
+    assert got.shape == np.asarray(expected).shape
+    assert np.all(np.abs(got - expected) <= tol), (got, expected)
+
+
+@pytest.mark.parametrize("sigma", [1.0, 0.5, 2.0])
+@pytest.mark.parametrize("magnitude", [0.1, 10.0])
+def test_smooth_l1(cpu, sigma, magnitude):
+    """reference tests/test_costs.py:243-300 (value and derivative)"""
+    rs = np.random.RandomState(3)
+    y, t = (rs.random_sample((7, 5)) - 0.5) * magnitude, rs.random_sample((7, 5))
+    x, s2 = y - t, sigma ** 2
+    small = np.abs(x) < 1.0 / s2
+    want = np.where(small, 0.5 * x ** 2 * s2, np.abs(x) - 0.5 / s2).sum(axis=0, keepdims=True)
+    assert_close(_cost(cpu, SmoothL1Loss(sigma=sigma), y, t), want.astype(np.float32), rtol=1e-5, atol=1e-6)
+    dwant = np.where(small, x * s2, np.sign(x))
+    assert_close(_cost(cpu, SmoothL1Loss(sigma=sigma), y, t, deriv=True), dwant.astype(np.float32), rtol=1e-5, atol=1e-6)
+
+
+def test_cross_entropy_shape_check(cpu):
+    with using(cpu):
+        with pytest.raises(ValueError):
+            CrossEntropyMulti()(cpu.zeros((4, 2)), cpu.zeros((4, 3)))
+
+
+def _metrics(be):
+    """the reference's metric known answers (tests/test_costs.py:200-235) plus
+    log loss / accuracy / top-k on the same small case"""
+    out = {}
+    y = np.array([[0.25, 0.99, 0.33], [0.5, 0.005, 0.32], [0.25, 0.005, 0.34]], dtype=np.float32)
+    t = np.array([[0, 1, 0], [1, 0, 1], [0, 0, 0]], dtype=np.float32)
+    with using(be, bsz=3):
+        out["mis"] = Misclassification()(be.array(y), be.array(t))
+        out["acc"] = Accuracy()(be.array(y), be.array(t))
+        out["logloss"] = LogLoss()(be.array(y), be.array(t))
+        out["top2"] = TopKMisclassification(2)(be.array(y), be.array(t))
+    preds = np.array([[0, 1, 0, 1], [1, 0, 0, 0], [0, 0, 1, 0]], dtype=np.float32)
+    soft = np.array([[0.2, 0.9, 0.01, 1], [0.75, 0.05, 0.44, 0], [0.05, 0.05, 0.55, 0]], dtype=np.float32)
+    targ = np.array([[0, 1, 0, 1], [1, 0, 1, 0], [0, 0, 0, 0]], dtype=np.float32)
+    with using(be, bsz=4):
+        out["pr"] = PrecisionRecall(3)(be.array(preds), be.array(targ))
+        out["pr_bin"] = PrecisionRecall(3, binarize=True)(be.array(soft), be.array(targ))
+    return out
+
+
+def _check_metrics(m):
+    assert abs(m["mis"] - 1.0 / 3) < 1e-7
+    assert abs(m["acc"] - 2.0 / 3) < 1e-7
+    assert abs(float(m["logloss"]) - (-np.log([0.5, 0.99, 0.32]).mean())) < 1e-6
+    assert_close(m["pr"], np.array([2, 1.5]) / 3, rtol=1e-5, atol=1e-6)
+    assert_close(m["pr_bin"], np.array([2, 1.5]) / 3, rtol=1e-5, atol=1e-6)
+    # sample 3: the true class (0.32) is the third largest of (0.33, 0.32, 0.34): a top-2 miss
+    assert_close(m["top2"], np.array([-np.log([0.5, 0.99, 0.32]).mean(), 1.0 / 3, 1.0 / 3]), rtol=1e-5, atol=1e-6)
+
+
+def test_metric_known_answers(cpu):
+    _check_metrics(_metrics(cpu))
+
+
+# ---- GPU --------------------------------------------------------------------------------
+@pytest.mark.gpu
+def test_metric_known_answers_hip(hip):
+    _check_metrics(_metrics(hip))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,make", [
+    ("rectlin", lambda: Rectlin(slope=0.1)), ("rectlinclip", lambda: Rectlinclip(slope=0.1, xcut=1.5)),
+    ("explin", lambda: Explin(alpha=0.7)), ("tanh", lambda: Tanh()), ("logistic", lambda: Logistic()),
+    ("softmax0", lambda: Softmax()), ("softmax1", lambda: Softmax(axis=1)), ("normalizer", lambda: Normalizer(divisor=3.0)),
+])
+def test_activations_hip_match_oracle(pair, name, make):
+    x = (np.random.RandomState(8).standard_normal((1000, 384)) * 2).astype(np.float32)
+    for deriv in (False, True):
+        got = [_act(be, make(), x, deriv) for be in pair]
+        assert_close(got[1], got[0], rtol=1e-5, atol=1e-6, what="%s deriv=%s" % (name, deriv))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,make", [
+    ("ce_binary", lambda: CrossEntropyBinary()), ("ce_multi", lambda: CrossEntropyMulti()),
+    ("ce_multi_bits", lambda: CrossEntropyMulti(usebits=True, scale=0.5)), ("sum_squared", lambda: SumSquared()),
+    ("mean_squared", lambda: MeanSquared()), ("smooth_l1", lambda: SmoothL1Loss(sigma=1.5)),
+    ("hinge", lambda: SquareHingeLoss(margin=0.8)),
+])
+def test_costs_hip_match_oracle(pair, name, make):
+    rs = np.random.RandomState(9)
+    logits = rs.standard_normal((1000, 256)) * 3
+    y = np.exp(logits - logits.max(axis=0)) / np.exp(logits - logits.max(axis=0)).sum(axis=0)
+    t = np.zeros_like(y)
+    t[rs.randint(0, 1000, size=256), np.arange(256)] = 1
+    y[0, :4] = 0.0                                                    # exercises the clamp of safelog
+    for deriv in (False, True):
+        got = [_cost(be, make(), y, t, deriv) for be in pair]
+        # sums over 1000 classes: absolute floor scaled by the magnitude of the result
+        assert_close(got[1], got[0], rtol=2e-5, atol=1e-6 * max(1.0, np.abs(got[0]).max()),
+                     what="%s deriv=%s" % (name, deriv))
+
+
+@pytest.mark.gpu
+def test_classification_metrics_hip_match_oracle(pair):
+    rs = np.random.RandomState(10)
+    nclass, batch = 1000, 512
+    logits = rs.standard_normal((nclass, batch)) * 2
+    y = (np.exp(logits) / np.exp(logits).sum(axis=0)).astype(np.float32)
+    labels = np.where(rs.rand(batch) < 0.5, y.argmax(axis=0), rs.randint(0, nclass, size=batch))
+    t = np.zeros_like(y)
+    t[labels, np.arange(batch)] = 1
+    res = []
+    for be in pair:
+        with using(be, bsz=batch):
+            yt, tt = be.array(y), be.array(t)
+            res.append((Misclassification()(yt, tt), Accuracy()(yt, tt), float(LogLoss()(yt, tt)),
+                        TopKMisclassification(5)(yt, tt), PrecisionRecall(nclass, binarize=True)(be.array(y), tt)))
+    assert res[1][0] == res[0][0] == np.float32((y.argmax(axis=0) != labels).mean())
+    assert res[1][1] == res[0][1]
+    assert abs(res[1][2] - res[0][2]) < 1e-5
+    assert_close(res[1][3], res[0][3], rtol=1e-5, atol=1e-6)
+    assert_close(res[1][4], res[0][4], rtol=1e-5, atol=1e-6)
