@@ -208,6 +208,22 @@ int nh_gemm(int itemsize, int trans_a, int trans_b, uint32_t m, uint32_t n, uint
 int nh_copy_transpose(void* out, const void* in, int itemsize, int ndim, const uint32_t* shape,
                       const int64_t* out_strides, const int64_t* in_strides, void* stream);
 
+/* Lookup-table (embedding) backward pass: dW[w, 0:embed] = sum over the
+ * positions j with ids[j] == w of error_t[j, 0:embed], positions in ascending
+ * order (deterministic); rows of words that do not occur, of `pad_idx` and of
+ * ids >= vocab are left untouched.  `ids` holds nin int32 word ids, error_t is
+ * the (nin, embed) transposed error, dW the (vocab, embed) gradient, both of
+ * `itemsize` 4 (fp32) or 2 (fp16, fp32 accumulation) with leading dimensions
+ * in elements.  `workspace` is device scratch of nh_lut_workspace_bytes(nin,
+ * vocab) bytes (0 from that call means the size query failed).  Replaces the
+ * sorting + _get_lut_bprop_kernel sequence of NervanaGPU.compound_bprop_lut
+ * (neon/backends/nervanagpu.py:2591-2660); semantics of the CPU backend
+ * (neon/backends/nervanacpu.py:1762-1782).                                     */
+size_t nh_lut_workspace_bytes(uint32_t nin, uint32_t vocab);
+int nh_lut_bprop(void* dW, const void* error_t, const int32_t* ids, int itemsize, uint32_t nin, uint32_t embed,
+                 uint32_t vocab, size_t ld_dw, size_t ld_err, int32_t pad_idx, void* workspace, size_t workspace_bytes,
+                 void* stream);
+
 #ifdef __cplusplus
 }
 #endif

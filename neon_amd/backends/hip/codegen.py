@@ -148,14 +148,17 @@ class _Gen(object):
         """Element address of (r, c) in a slot, honouring broadcast dims and
         index vectors of gather / scatter views."""
         parts = ["a%d" % slot.index]
-        if slot.shape[0] > 1:
-            if slot.take_axis == 0:
-                r = "a%d[(long long)(%s)]" % (slot.take_slot, r)
+        if slot.take_axis == 0:
+            # (a view of a single gathered row still has to look its index up)
+            parts.append("(long long)a%d[(long long)(%s)] * sr%d"
+                         % (slot.take_slot, r if slot.shape[0] > 1 else "0", slot.index))
+        elif slot.shape[0] > 1:
             parts.append("(long long)(%s) * sr%d" % (r, slot.index))
-        if slot.shape[1] > 1:
-            if slot.take_axis == 1:
-                parts.append("(long long)a%d[(long long)(%s)] * sc%d" % (slot.take_slot, c, slot.index))
-            elif self.col_unit(slot):
+        if slot.take_axis == 1:
+            parts.append("(long long)a%d[(long long)(%s)] * sc%d"
+                         % (slot.take_slot, c if slot.shape[1] > 1 else "0", slot.index))
+        elif slot.shape[1] > 1:
+            if self.col_unit(slot):
                 parts.append("(long long)(%s)" % c)
             else:
                 parts.append("(long long)(%s) * sc%d" % (c, slot.index))

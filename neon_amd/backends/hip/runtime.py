@@ -94,6 +94,9 @@ SIGNATURES = {
     "nh_gemm": (c_int, [c_int, c_int, c_int, c_uint32, c_uint32, c_uint32, c_float, c_void_p, c_size_t,
                         c_void_p, c_size_t, c_float, c_void_p, c_size_t, c_void_p]),
     "nh_copy_transpose": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "nh_lut_workspace_bytes": (c_size_t, [c_uint32, c_uint32]),
+    "nh_lut_bprop": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_uint32, c_uint32, c_uint32, c_size_t,
+                             c_size_t, c_int32, c_void_p, c_size_t, c_void_p]),
     "nh_colreduce_workspace_bytes": (c_size_t, [c_uint32, c_uint32]),
     "nh_colmax_argmax_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_uint32, c_uint32,
                                      c_size_t, c_void_p, c_void_p]),
@@ -285,6 +288,14 @@ class Runtime(object):
         c_is = (ctypes.c_int64 * n)(*in_strides)
         _check(self.lib.nh_copy_transpose(c_void_p(out_ptr), c_void_p(in_ptr), itemsize, n, c_shape, c_os, c_is,
                                           self.stream))
+
+    def lut_workspace_bytes(self, nin, vocab):
+        return self.lib.nh_lut_workspace_bytes(nin, vocab)
+
+    def lut_bprop(self, dw_ptr, err_t_ptr, ids_ptr, itemsize, nin, embed, vocab, ld_dw, ld_err, pad_idx,
+                  ws_ptr, ws_bytes):
+        _check(self.lib.nh_lut_bprop(c_void_p(dw_ptr), c_void_p(err_t_ptr), c_void_p(ids_ptr), itemsize, nin, embed,
+                                     vocab, ld_dw, ld_err, pad_idx, c_void_p(ws_ptr), ws_bytes, self.stream))
 
     def shutdown(self):
         self.lib.nh_shutdown()

@@ -476,6 +476,7 @@ class NervanaHIP(Backend):
         self._recording = None
         self._rec_temps = None
         self._rec_foreign = False     # the group being recorded made a call that is not a kernel launch
+        self._lut_ws = None           # (pointer, bytes) scratch of compound_bprop_lut
         self._originals = frozenset() # ids of handles whose reads mean "before the running group" (compensated_sum)
         self._rec_single = None
         self._temp_pool = {}
@@ -503,6 +504,9 @@ class NervanaHIP(Backend):
             self.plans = {}
             self._launch_cache = {}
             self._temp_pool = {}
+            if getattr(self, "_lut_ws", None):
+                rt.free(self._lut_ws[0])
+                self._lut_ws = None
         except Exception:
             pass
 
@@ -1009,6 +1013,34 @@ class NervanaHIP(Backend):
             for t in temps:
                 self._temp_release(t)
         return C
+
+    # -- lookup table backward -----------------------------------------------------------------
+    def compound_bprop_lut(self, nin, inputs, error, error_t, dW, pad_idx, alpha=1.0, beta=0):
+        """Gradient of an embedding table: ``dW[w, :]`` = sum of the columns of
+        ``error`` (embedding_dim, positions) whose word id in ``inputs`` is
+        ``w``; rows of words that do not occur and of ``pad_idx`` keep their
+        values (the layer clears ``dW`` first).  Semantics of the CPU backend
+        (nervanacpu.py:1762-1782, which like this ignores alpha / beta); done
+        as the reference's deterministic path does it (nervanagpu.py:2591-2660):
+        transpose the error, sort the positions by word id, sum every run."""
+        assert isinstance(inputs, HIPTensor) and inputs.dtype == np.int32, "word ids must be an int32 tensor"
+        assert error.dtype == error_t.dtype == dW.dtype and dW.dtype.type in (np.float32, np.float16)
+        count = inputs.size
+        embed, vocab = dW.shape[1], dW.shape[0]
+        assert error.shape == (embed, count) and error_t.shape == (count, embed)
+        assert inputs.is_contiguous and error_t.is_contiguous and dW.strides[1] == 1 and not dW.take_array
+        self.copy_transpose(error, error_t)
+        need = self.rt.lut_workspace_bytes(count, vocab)
+        if need == 0:
+            raise hiprt.HipError(hiprt.NH_EINVAL, "size query for the position sort failed")
+        if self._lut_ws is None or self._lut_ws[1] < need:
+            if self._lut_ws is not None:
+                self.synchronize()
+                self.rt.free(self._lut_ws[0])
+            self._lut_ws = (self.rt.malloc(need), need)
+        self.rt.lut_bprop(dW.gpudata, error_t.gpudata, inputs.gpudata, dW.dtype.itemsize, count, embed, vocab,
+                          dW.strides[0], embed, -1 if pad_idx is None else int(pad_idx),
+                          self._lut_ws[0], self._lut_ws[1])
 
     # -- dimension shuffle -------------------------------------------------------------------
     def copy_transpose(self, a, out, axes=None, repeat=1):

@@ -439,6 +439,17 @@ class NervanaCPU(Backend):
             bsum[:] = self.sum(C, 1)
         return C
 
+    # -- lookup table backward (reference nervanacpu.py:1762-1782) -------------------
+    def compound_bprop_lut(self, nin, inputs, error, error_t, dW, pad_idx, alpha=1.0, beta=0):
+        wrd_ids = inputs._tensor.reshape(-1)
+        unqidx, inv = np.unique(wrd_ids, return_inverse=True)
+        for k, wrd_id in enumerate(unqidx):
+            if wrd_id != pad_idx:
+                group = np.where(inv == k)[0]
+                # (the reference assigns self.sum(error.take(group, axis=1), axis=1) through a
+                # row view; the same numpy sum, written into the row directly)
+                dW._tensor[int(wrd_id), :] = np.sum(error._tensor.take(group, axis=1), axis=1)
+
     # -- dimension shuffle (reference nervanacpu.py:1046-1051) ------------------------
     def copy_transpose(self, a, out, axes=None, repeat=1):
         out._tensor[:] = np.transpose(a._tensor, axes).copy()

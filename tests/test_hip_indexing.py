@@ -78,3 +78,21 @@ def test_hist_matches_oracle(pair, shape, dtype):
         assert np.array_equal(hv, want)
     data, tags = hip.dump_hist_data()
     assert "w" in tags and data.shape[1] == 64
+
+
+
+def test_single_index_gather_and_scatter(hip):
+    """a gather view of exactly one row / column still goes through its index"""
+    rs = np.random.RandomState(12)
+    w = rs.standard_normal((40, 9)).astype(np.float32)
+    W = hip.array(w)
+    one = hip.array(np.array([[17]], dtype=np.int32), dtype=np.int32)
+    col = hip.array(np.array([[5]], dtype=np.int32), dtype=np.int32)
+    row_out, col_out = hip.empty((1, 9)), hip.empty((40, 1))
+    row_out[:] = W.take(one, axis=0) * 2.0
+    col_out[:] = W.take(col, axis=1) + 1.0
+    assert np.array_equal(row_out.get(), w[17:18] * 2.0)
+    assert np.array_equal(col_out.get(), w[:, 5:6] + 1.0)
+    W[one] = row_out                                   # scatter into the single indexed row
+    w[17] = w[17] * 2.0
+    assert np.array_equal(W.get(), w)
