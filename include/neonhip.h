@@ -196,6 +196,16 @@ int nh_gemm(int itemsize, int trans_a, int trans_b, uint32_t m, uint32_t n, uint
             float alpha, const void* a, size_t lda, const void* b, size_t ldb,
             float beta, void* c, size_t ldc, void* stream);
 
+/* `batch` such products in one call: product i reads a + i * stride_a and
+ * b + i * stride_b and updates c + i * stride_c (strides in elements; 0 for an
+ * operand shared by the whole batch; the outputs must not overlap).  Replaces
+ * the batched sgemm/hgemm kernels behind NervanaGPU.batched_dot
+ * (neon/backends/nervanagpu.py:1623-1760).                                      */
+int nh_gemm_batched(int itemsize, int trans_a, int trans_b, uint32_t m, uint32_t n, uint32_t k,
+                    float alpha, const void* a, size_t lda, long long stride_a, const void* b, size_t ldb,
+                    long long stride_b, float beta, void* c, size_t ldc, long long stride_c,
+                    uint32_t batch, void* stream);
+
 /* Dimension shuffle, numpy.transpose(in, axes) written into `out`: `ndim`
  * dimensions listed in OUTPUT order -- shape[i] is the extent of output
  * dimension i, out_strides[i] its stride in `out` and in_strides[i] the stride

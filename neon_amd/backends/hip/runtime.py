@@ -93,6 +93,9 @@ SIGNATURES = {
     "nh_hist_log2": (c_int, [c_void_p, c_void_p, c_int, c_size_t, c_int, c_int, c_void_p]),
     "nh_gemm": (c_int, [c_int, c_int, c_int, c_uint32, c_uint32, c_uint32, c_float, c_void_p, c_size_t,
                         c_void_p, c_size_t, c_float, c_void_p, c_size_t, c_void_p]),
+    "nh_gemm_batched": (c_int, [c_int, c_int, c_int, c_uint32, c_uint32, c_uint32, c_float, c_void_p, c_size_t,
+                                ctypes.c_longlong, c_void_p, c_size_t, ctypes.c_longlong, c_float, c_void_p,
+                                c_size_t, ctypes.c_longlong, c_uint32, c_void_p]),
     "nh_copy_transpose": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "nh_lut_workspace_bytes": (c_size_t, [c_uint32, c_uint32]),
     "nh_lut_bprop": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_uint32, c_uint32, c_uint32, c_size_t,
@@ -288,6 +291,12 @@ class Runtime(object):
         c_is = (ctypes.c_int64 * n)(*in_strides)
         _check(self.lib.nh_copy_transpose(c_void_p(out_ptr), c_void_p(in_ptr), itemsize, n, c_shape, c_os, c_is,
                                           self.stream))
+
+    def gemm_batched(self, itemsize, trans_a, trans_b, m, n, k, alpha, a_ptr, lda, stride_a, b_ptr, ldb, stride_b,
+                     beta, c_ptr, ldc, stride_c, batch):
+        _check(self.lib.nh_gemm_batched(itemsize, int(trans_a), int(trans_b), m, n, k, alpha, c_void_p(a_ptr), lda,
+                                        stride_a, c_void_p(b_ptr), ldb, stride_b, beta, c_void_p(c_ptr), ldc,
+                                        stride_c, batch, self.stream))
 
     def lut_workspace_bytes(self, nin, vocab):
         return self.lib.nh_lut_workspace_bytes(nin, vocab)

@@ -957,15 +957,10 @@ class NervanaHIP(Backend):
         """(tensor, transposed?, leading dimension) for a 2-D operand the GEMM
         can read in place; anything else (gather views, doubly strided views)
         is first copied into a dense temporary"""
-        rows, cols = t.shape
-        sr, sc = t.strides
         if not t.take_array:
-            if cols == 1 or sc == 1:
-                if rows == 1 or sr >= cols:
-                    return t, False, max(sr, cols, 1)
-            if rows == 1 or sr == 1:
-                if cols == 1 or sc >= rows:
-                    return t, True, max(sc, rows, 1)
+            geom = _matrix_geometry(t.shape[0], t.shape[1], t.strides[0], t.strides[1])
+            if geom is not None:
+                return t, geom[0], geom[1]
         tmp = self._temp(t.shape, t.dtype, temps)
         self._run([OpTreeNode({"op": "assign"}, tmp, t)])
         return tmp, False, max(cols, 1)
@@ -1012,6 +1007,57 @@ class NervanaHIP(Backend):
         finally:
             for t in temps:
                 self._temp_release(t)
+        return C
+
+    def batched_dot(self, A, B, C, alpha=1.0, beta=0.0, relu=False):
+        """Products over a leading batch dimension (reference
+        nervanagpu.py:1624-1760, CPU semantics nervanacpu.py:962-1017):
+
+            forward   A (K,C),   B (X,C,N), C (X,K,N):  C[i] = A . B[i]
+            backward  A.T,       B (X,K,N), C (X,C,N):  C[i] = A.T . B[i]
+            update    A (X,K,N), B.T (X,N,C), C (K,C):  C    = sum_i A[i] . B.T[i]
+
+        each as ``C = alpha * product + beta * C``; one strided-batched library
+        call for a 3-D ``C``, an accumulating sequence for the 2-D one."""
+        assert A.dtype == B.dtype == C.dtype and C.dtype.type in (np.float32, np.float16)
+        dima, dimb, dimc = int(len(A.shape) == 3), int(len(B.shape) == 3), int(len(C.shape) == 3)
+        assert dima or dimb, "Tensor A or B must have 3 dims to use batched_dot"
+        batch = A.shape[0] if dima else B.shape[0]
+        assert not (dima and dimb) or A.shape[0] == B.shape[0]
+        assert not dimc or C.shape[0] == batch
+        m, k, n = A.shape[0 + dima], A.shape[1 + dima], B.shape[1 + dimb]
+        assert m == C.shape[0 + dimc] and n == C.shape[1 + dimc] and k == B.shape[0 + dimb]
+        if relu and (beta != 0 or not dimc):
+            raise NotImplementedError("batched_dot with relu is limited to beta == 0 and a batched output")
+        self._flush()
+
+        def geometry(t, three):
+            if t.take_array:
+                raise NotImplementedError("batched_dot on gather views")
+            g = _matrix_geometry(t.shape[-2], t.shape[-1], t.strides[-2], t.strides[-1])
+            if g is None:
+                raise NotImplementedError("batched_dot operands need a unit stride along rows or columns")
+            return g[0], g[1], (t.strides[0] if three else 0)
+
+        ta, lda, sa = geometry(A, dima)
+        tb, ldb, sb = geometry(B, dimb)
+        tc, ldc, sc = geometry(C, dimc)
+        if tc:
+            raise NotImplementedError("batched_dot into a transposed output")
+        isz = C.dtype.itemsize
+        self._rec_foreign = True
+        if dimc:
+            self.rt.gemm_batched(isz, ta, tb, m, n, k, float(alpha), A.gpudata, lda, sa, B.gpudata, ldb, sb,
+                                 float(beta), C.gpudata, ldc, sc, batch)
+            if relu:
+                flat = C.reshape((batch * m, n)) if C.is_contiguous else None
+                if flat is None:
+                    raise NotImplementedError("relu on a strided batched output")
+                self._run([self._stmt(flat, self.maximum(flat, 0))])
+        else:
+            for i in range(batch):
+                self.rt.gemm(isz, ta, tb, m, n, k, float(alpha), A.gpudata + i * sa * isz, lda,
+                             B.gpudata + i * sb * isz, ldb, float(beta) if i == 0 else 1.0, C.gpudata, ldc)
         return C
 
     # -- lookup table backward -----------------------------------------------------------------
@@ -1211,6 +1257,18 @@ class NervanaHIP(Backend):
         self.hist_map = dict()
         self.hist_idx = 0
         return data, hist_map
+
+
+def _matrix_geometry(rows, cols, sr, sc):
+    """(transposed?, leading dimension) under which a library GEMM can read a
+    strided 2-D operand in place, or None"""
+    if cols == 1 or sc == 1:
+        if rows == 1 or sr >= cols:
+            return False, max(sr, cols, 1)
+    if rows == 1 or sr == 1:
+        if cols == 1 or sc >= rows:
+            return True, max(sc, rows, 1)
+    return None
 
 
 def _splittable(tree):

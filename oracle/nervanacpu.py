@@ -439,6 +439,33 @@ class NervanaCPU(Backend):
             bsum[:] = self.sum(C, 1)
         return C
 
+    # -- products over a batch dimension (reference nervanacpu.py:962-1017) ----------
+    def batched_dot(self, A, B, C, alpha=1.0, beta=0.0, relu=False):
+        assert A.dtype == B.dtype == C.dtype
+        dima, dimb, dimc = int(len(A.shape) == 3), int(len(B.shape) == 3), int(len(C.shape) == 3)
+        assert dima or dimb, "Tensor A or B must have 3 dims to use batched_dot"
+        if dimc:
+            assert not dima or A.shape[0] == C.shape[0]
+            assert not dimb or B.shape[0] == C.shape[0]
+        loops = A.shape[0] if dima else B.shape[0]
+        assert not (dima and dimb) or A.shape[0] == B.shape[0]
+        assert A.shape[0 + dima] == C.shape[0 + dimc]
+        assert B.shape[1 + dimb] == C.shape[1 + dimc]
+        assert A.shape[1 + dima] == B.shape[0 + dimb]
+        tmp = np.zeros(C.shape)
+        for i in range(loops):
+            a = A._tensor[i] if dima else A._tensor
+            b = B._tensor[i] if dimb else B._tensor
+            if dimc:
+                tmp[i] = np.dot(a, b)
+            else:
+                tmp += np.dot(a, b)
+        np.multiply(tmp, alpha, tmp)
+        if relu:
+            np.maximum(tmp, 0, tmp)
+        C._tensor[:] = C._tensor * beta + tmp
+        return C
+
     # -- lookup table backward (reference nervanacpu.py:1762-1782) -------------------
     def compound_bprop_lut(self, nin, inputs, error, error_t, dW, pad_idx, alpha=1.0, beta=0):
         wrd_ids = inputs._tensor.reshape(-1)

@@ -236,3 +236,67 @@ def test_compound_optree_hip(pair, f, flag, dim):
     scale = max(1.0, np.abs(want).max())
     assert_close(got[0], want.astype(np.float32), rtol=1e-2, atol=1e-2 * scale)
     assert_close(got[1], want.astype(np.float32), rtol=1e-2, atol=1e-2 * scale)
+
+
+# ---- batched_dot (reference tests/test_backend_batched_dot.py) -----------------------------------
+
+def _batched_case(be, I, E, W, dtype):
+    devI, devE, devW = (be.array(a.astype(dtype), dtype=dtype) for a in (I, E, W))
+    devO, devB, devU = be.zeros(E.shape, dtype=dtype), be.zeros(I.shape, dtype=dtype), be.zeros(W.shape, dtype=dtype)
+    be.batched_dot(devW, devI, devO)            # fprop
+    be.batched_dot(devW.T, devE, devB)          # bprop
+    be.batched_dot(devE, devI.T, devU)          # update
+    return devO.get(), devB.get(), devU.get()
+
+
+def _batched_data(X, N, C, K, seed=0):
+    rs = np.random.RandomState(seed)
+    return (rs.uniform(-1, 1, (X, C, N)), rs.uniform(-1, 1, (X, K, N)), rs.uniform(-1, 1, (K, C)))
+
+
+def _batched_numpy(I, E, W):
+    O = np.stack([W @ I[i] for i in range(I.shape[0])])
+    B = np.stack([W.T @ E[i] for i in range(I.shape[0])])
+    U = sum(E[i] @ I[i].T for i in range(I.shape[0]))
+    return O, B, U
+
+
+def test_batched_dot_oracle():
+    from oracle import nervanacpu  # noqa: F401
+    from neon_amd.backends.backend import Backend
+    cpu = Backend.allocate_backend("cpu", rng_seed=0)
+    I, E, W = _batched_data(5, 8, 24, 12)
+    for got, want in zip(_batched_case(cpu, I, E, W, np.float32), _batched_numpy(I, E, W)):
+        assert_close(got, want.astype(np.float32), rtol=0, atol=1e-4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,atol", [(np.float32, 1e-3), (np.float16, 0.25)], ids=["f32", "f16"])
+@pytest.mark.parametrize("X,N,C,K", [(100, 32, 1536, 768), (3, 5, 7, 9), (1, 64, 64, 64)])
+def test_batched_dot_hip(hip, X, N, C, K, dtype, atol):
+    I, E, W = _batched_data(X, N, C, K, seed=X)
+    q = lambda a: a.astype(dtype).astype(np.float64)
+    want = _batched_numpy(q(I), q(E), q(W))
+    got = _batched_case(hip, I, E, W, dtype)
+    for g, w in zip(got, want):
+        # the reference's bar for fp32 (tests/test_backend_batched_dot.py: atol 1e-3); fp16 stores
+        # sums of up to X*N = 3200 products
+        assert_close(g.astype(np.float64), w, rtol=2e-3 if dtype == np.float16 else 0, atol=atol)
+
+
+@pytest.mark.gpu
+def test_batched_dot_alpha_beta_relu_hip(pair):
+    I, E, W = _batched_data(4, 16, 40, 24, seed=2)
+    res = []
+    for be in pair:
+        devI, devE, devW = (be.array(a.astype(np.float32)) for a in (I, E, W))
+        O = be.array(E.astype(np.float32))
+        U = be.array(W.astype(np.float32))
+        be.batched_dot(devW, devI, O, alpha=0.5, beta=2.0)
+        be.batched_dot(devE, devI.T, U, alpha=-1.5, beta=0.25)
+        R = be.zeros(E.shape)
+        be.batched_dot(devW, devI, R, relu=True)
+        res.append((O.get(), U.get(), R.get()))
+    for g, w in zip(res[1], res[0]):
+        assert_close(g, w, rtol=1e-4, atol=1e-4)
+    assert res[1][2].min() == 0.0
