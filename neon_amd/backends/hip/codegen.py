@@ -231,9 +231,25 @@ class _Gen(object):
                     e = "nh_sround(%s, %s, %s)" % (a[0], n.op.split(":")[1], word)
             elif len(a) == 1:
                 e = _UN[n.op].format(*a)
+            elif n.op == "div" and RECIPROCAL_OF_BROADCAST and _broadcast_under(n.args[1], n.args[0]):
+                # The divisor is constant along an axis the dividend varies on
+                # (a row's standard deviation, a column's softmax sum): one
+                # reciprocal per row / column, hoisted out of the element loop
+                # by the compiler, and a multiply per element instead of an
+                # IEEE division (about ten instructions).  At most 1.5 units in
+                # the last place away from the quotient.
+                e = "({0} * (1.0f / {1}))".format(*a)
             else:
                 e = _BIN[n.op].format(*a)
             self.L("const float t%d = %s;" % (n.nid, e))
+
+
+RECIPROCAL_OF_BROADCAST = os.environ.get("NEON_HIP_RCP", "1") != "0"
+
+
+def _broadcast_under(b, a):
+    """b is constant along at least one axis on which a varies, and varies on none that a does not"""
+    return (b.vr <= a.vr and b.vc <= a.vc) and (b.vr < a.vr or b.vc < a.vc)
 
 
 def _needed(targets, available):
