@@ -44,6 +44,15 @@ bool blas_ready() {
     if (g_blas.handle) return true;
     if (g_blas.tried) return false;
     g_blas.tried = true;
+    if (g_blas.lib && g_blas.create) {            // library already bound: only the handle was released
+        if (g_blas.create(&g_blas.handle) != rocblas_status_success) {
+            g_blas.handle = nullptr;
+            g_blas.error = "rocblas_create_handle failed";
+            return false;
+        }
+        g_blas.set_pointer_mode(g_blas.handle, rocblas_pointer_mode_host);
+        return true;
+    }
     for (const char* name : {"librocblas.so.5", "librocblas.so", "/opt/rocm/lib/librocblas.so"}) {
         g_blas.lib = dlopen(name, RTLD_NOW | RTLD_LOCAL);
         if (g_blas.lib) break;
@@ -67,6 +76,18 @@ bool blas_ready() {
     g_blas.set_pointer_mode(g_blas.handle, rocblas_pointer_mode_host);
     return true;
 }
+
+}  // namespace
+
+// called by nh_shutdown: the handle belongs to the device context being left
+void nh_internal_blas_release() {
+    std::lock_guard<std::mutex> hold(g_blas_mutex);
+    if (g_blas.handle && g_blas.destroy) g_blas.destroy(g_blas.handle);
+    g_blas.handle = nullptr;
+    g_blas.tried = false;
+}
+
+namespace {
 
 // batch == 0: one product through gemm_ex; otherwise `batch` products whose
 // operands lie stride_x elements apart (0 = the same matrix every time)

@@ -14,6 +14,8 @@
 #include <string>
 #include <vector>
 
+void nh_internal_blas_release();      // gemm.cpp: drops the rocBLAS handle, if one was created
+
 namespace {
 
 thread_local std::string g_err;
@@ -95,6 +97,7 @@ int nh_init(int device, nh_props* props) {
 int nh_shutdown(void) {
     if (!g_init) return 0;
     NH_HIP(hipDeviceSynchronize());
+    nh_internal_blas_release();
     g_init = false;
     return 0;
 }
