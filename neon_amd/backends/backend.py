@@ -736,3 +736,34 @@ class Backend(metaclass=_BackendRegistry):
 
     def make_binary_mask(self, out, keepthresh=0.5):
         raise NotImplementedError()
+
+    # -- binary-network helpers: compositions of ordinary ops (reference
+    #    nervanacpu.py:1823-1863) ------------------------------------------------
+    def _uniform_like(self, ary):
+        """uniform [0, 1) values of ``ary``'s shape, as a tensor or an op-tree"""
+        raise NotImplementedError()
+
+    def binarize(self, ary, out, stochastic=True):
+        """``out`` = +1 / -1: the sign of ``ary`` (zero counts as positive), or,
+        with ``stochastic``, +1 with probability clip((ary + 1) / 2, 0, 1)"""
+        if stochastic:
+            out[:] = (ary + 1) / 2.0
+            self.clip(out, 0, 1, out)
+            self.less_equal(self._uniform_like(ary), out, out)
+        else:
+            self.greater_equal(ary, 0, out)
+        out[:] = 2 * out - 1
+        return out
+
+    def shift(self, ary, shift_ary, value=True, out=None):
+        """``ary`` times a power of two: 2 ** shift_ary, or (``value``) the power
+        of two nearest to ``shift_ary`` in the log domain, with its sign"""
+        if value:
+            exponent = self.rint(self.safelog(self.absolute(shift_ary)) / self.log(2))
+            ap2 = self.multiply(self.sgn(shift_ary), self.exp2(exponent))
+        else:
+            ap2 = self.exp2(shift_ary)
+        if out is None:
+            out = self.empty_like(ary) if hasattr(ary, "shape") else self.empty((1, 1))
+        out[:] = self.multiply(ary, ap2)
+        return out

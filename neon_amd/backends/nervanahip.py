@@ -548,6 +548,9 @@ class NervanaHIP(Backend):
         """uniform [0, 1) as an op-tree leaf"""
         return OpTreeNode.build("rand", None, None, out=out)
 
+    def _uniform_like(self, ary):
+        return self.rand()          # drawn inside the kernel that consumes it
+
     def dropout(self, keep=0.5, out=None):
         """keep mask: 1 where a uniform draw is <= ``keep``"""
         return self.less_equal(self.rand(), keep, out=out)

@@ -3,4 +3,4 @@
 from neon_amd.optimizers.optimizer import (Adadelta, Adagrad, Adam, ExpSchedule,  # noqa: F401
                                            GradientDescentMomentum, MultiOptimizer, Optimizer,
                                            PolySchedule, PowerSchedule, RMSProp, Schedule,
-                                           StepSchedule, get_param_list)
+                                           ShiftAdaMax, ShiftSchedule, StepSchedule, get_param_list)

@@ -111,6 +111,18 @@ class PolySchedule(Schedule):
         return float(learning_rate * (1. - epoch // self.total_epochs) ** self.power)
 
 
+class ShiftSchedule(Schedule):
+    """rate halved (``shift_size`` binary places) every ``interval`` epochs"""
+
+    def __init__(self, interval, shift_size=1):
+        self.interval = interval
+        self.shift_size = shift_size
+
+    def get_learning_rate(self, learning_rate, epoch):
+        total_shift = -1 * self.shift_size * int(epoch / self.interval)
+        return float(self.be.shift(learning_rate, total_shift, value=False).get().reshape(-1)[0])
+
+
 # ---------------------------------------------------------------------------------------
 # update rules
 # ---------------------------------------------------------------------------------------
@@ -293,6 +305,37 @@ class Adam(Optimizer):
             v[:] = v * self.beta_2 + (1. - self.beta_2) * grad * grad
             param[:] = self.clip_value(param - (scale * step * m) / (be.sqrt(v) + self.epsilon),
                                        self.param_clip_value)
+
+
+class ShiftAdaMax(Optimizer):
+    """AdaMax whose scalings are rounded to powers of two (binary networks):
+    ``m = b1 m + (1-b1) g;  v = max(b2 v, |g|);  W -= shift(shift(m, 1/(v+eps)), lr / (1 - b1^t))``,
+    ``W`` kept in [-1, 1] (reference optimizer.py:933-990)."""
+
+    def __init__(self, stochastic_round=False, learning_rate=0.002, beta_1=0.9, beta_2=0.999,
+                 epsilon=1e-8, schedule=None, name="ShiftAdaMax"):
+        super(ShiftAdaMax, self).__init__(name=name)
+        self.beta_1, self.beta_2, self.epsilon = beta_1, beta_2, epsilon
+        self.learning_rate = learning_rate
+        self.stochastic_round = stochastic_round
+        self.schedule = schedule if schedule is not None else Schedule()
+
+    def optimize(self, layer_list, epoch):
+        be = self.be
+        t = epoch + 1
+        lrate = self.schedule.get_learning_rate(self.learning_rate, epoch)
+        step = lrate / (1 - self.beta_1 ** t)
+        for (param, grad), states in get_param_list(layer_list):
+            param.rounding = self.stochastic_round
+            if len(states) == 0:
+                states.extend(be.zeros_like(grad) for _ in range(3))
+            grad = grad / be.bsz
+            m, v, inv_v = states
+            m[:] = m * self.beta_1 + (1. - self.beta_1) * grad
+            v[:] = be.maximum(v * self.beta_2, be.absolute(grad))
+            inv_v[:] = 1.0 / (v + self.epsilon)
+            param[:] = param - be.shift(be.shift(m, inv_v), step)
+            be.clip(param, -1, 1, param)
 
 
 class MultiOptimizer(Optimizer):

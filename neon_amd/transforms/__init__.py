@@ -1,7 +1,7 @@
 """Activation functions, cost functions and metrics: callers of the op-tree
 path (each returns an op-tree, or assigns a few into small buffers)."""
 from neon_amd.transforms.activation import (Explin, Identity, Logistic, Normalizer, Rectlin,  # noqa: F401
-                                            Rectlinclip, Softmax, Tanh)
+                                            Rectlinclip, Sign, Softmax, Tanh)
 from neon_amd.transforms.cost import (Accuracy, Cost, CrossEntropyBinary, CrossEntropyMulti,  # noqa: F401
                                       LogLoss, MeanSquared, Metric, Misclassification,
                                       PrecisionRecall, SmoothL1Loss, SquareHingeLoss, SumSquared,

@@ -125,3 +125,15 @@ class Logistic(Transform):
 
     def bprop(self, y):
         return self.bprop_func(y)
+
+
+class Sign(Transform):
+    """+1 / -1 by the sign of x, in place (binary networks; reference
+    activation.py:363-377); the straight-through derivative passes gradients
+    where the stored input lies in [-1, 1]"""
+
+    def __call__(self, x):
+        return self.be.binarize(x, x, stochastic=False)
+
+    def bprop(self, x):
+        return self.be.less_equal(self.be.absolute(self.inputs), 1)

@@ -439,6 +439,10 @@ class NervanaCPU(Backend):
             bsum[:] = self.sum(C, 1)
         return C
 
+    def _uniform_like(self, ary):
+        # host draws, as in the reference's binarize (nervanacpu.py:1835)
+        return self.array(self.rng.uniform(0, 1, size=ary.shape))
+
     # -- products over a batch dimension (reference nervanacpu.py:962-1017) ----------
     def batched_dot(self, A, B, C, alpha=1.0, beta=0.0, relu=False):
         assert A.dtype == B.dtype == C.dtype
