@@ -33,6 +33,9 @@ class OpCollection(object):
     ew_ops = float_ops - {"dot", "transpose"}
 
 
+_EW_NOT_ASSIGN = frozenset(OpCollection.ew_ops) - {"assign"}
+
+
 class Block(object):
     """Kinds of repeated computation announced through ``Backend.begin/end``
     (reference backend.py:2076-2088)."""
@@ -41,6 +44,32 @@ class Block(object):
 
 def _operand_ok(x):
     return x is None or isinstance(x, (int, float, Tensor, OpTreeNode))
+
+
+_NO_OPERAND, _SCALAR_SHAPE = (0, 0), (1, 1)
+
+
+def _shape_of_operand(x):
+    """2-d shape an operand contributes to shape inference, None for a type
+    that cannot be an operand"""
+    if x is None:
+        return _NO_OPERAND
+    tx = type(x)
+    if tx is float or tx is int:
+        return _SCALAR_SHAPE
+    if tx is OpTreeNode:
+        shp = x[0]["shape"]
+    elif isinstance(x, Tensor):
+        shp = x.shape
+    elif isinstance(x, (int, float)):
+        return _SCALAR_SHAPE
+    elif isinstance(x, OpTreeNode):
+        shp = x[0]["shape"]
+    else:
+        return None
+    if len(shp) == 1:
+        return (shp[0], 1)
+    return shp if type(shp) is tuple else tuple(shp)
 
 
 def _operand_shape(x):
@@ -293,11 +322,17 @@ class OpTreeNode(_LazyOperators, tuple):
         surfaces in ``execute``); reduction with ``axis`` = operand shape with
         that axis set to 1; numbers are 1x1; 1-d shapes are padded to 2-d.
         """
-        if not (_operand_ok(a) and _operand_ok(b)):
+        sa, sb = _shape_of_operand(a), _shape_of_operand(b)
+        if sa is None or sb is None:
             return NotImplemented
-        sa, sb = _operand_shape(a), _operand_shape(b)
-        if op in OpCollection.ew_ops and op != "assign":
-            shape = (max(sa[0], sb[0]), max(sa[1], sb[1]))
+        if op in _EW_NOT_ASSIGN:
+            # (this branch runs for every arithmetic operator a caller writes: kept short)
+            if sa == sb:
+                shape = sa
+            else:
+                shape = (sa[0] if sa[0] > sb[0] else sb[0], sa[1] if sa[1] > sb[1] else sb[1])
+            if not kwargs and out is None:
+                return OpTreeNode({"op": op, "shape": shape}, a, b)
         elif op in OpCollection.reduction_ops:
             if "axis" in kwargs:
                 shape = list(sa)

@@ -377,7 +377,7 @@ class _FuseScope(object):
             if exc_type is None:
                 self.be._flush()
             else:
-                self.be._pending = []
+                self.be._pending, self.be._pending_post = [], []
         return False
 
 
@@ -469,6 +469,7 @@ class NervanaHIP(Backend):
         self.plans = {}
         self.plan_stats = {"hit": 0, "miss": 0, "split": 0, "launches": 0, "replayed": 0}
         self._pending = []
+        self._pending_post = []       # postfix walks of the pending statements
         self._fusing = False
         self._fuse_depth = 0
         self._captured = None
@@ -496,7 +497,7 @@ class NervanaHIP(Backend):
         if rt is None:
             return
         try:
-            self._pending = []
+            self._pending, self._pending_post = [], []
             rt.synchronize()
             for plan in self.plans.values():
                 for p in (plan if isinstance(plan, list) else [plan]):
@@ -641,62 +642,66 @@ class NervanaHIP(Backend):
     def _flush(self):
         if self._pending:
             trees, self._pending = self._pending, []
+            posts, self._pending_post = self._pending_post, []
             if self._captured is not None:
                 self._captured.append(trees)
             else:
-                self._run(trees)
+                self._run(trees, posts)
 
-    @staticmethod
-    def _is_elementwise(tree):
-        for p in tree.traverse(list()):
-            if isinstance(p, dict) and (p["op"] in REDUCE or p["op"] in ("dot", "transpose", "onehot")):
-                return False
-        return True
+    _NOT_FUSABLE = frozenset(REDUCE) | {"dot", "transpose", "onehot"}
 
-    def _can_join(self, tree):
+    def _can_join(self, tree, post):
         """A statement joins the pending group when it is purely elementwise,
         every tensor in it has the group's shape and is contiguous (or is
-        1x1), so each lane only ever touches its own elements."""
-        if not self._is_elementwise(tree):
-            return False
-        shape = tree[1].shape
-        for p in [tree[1]] + [q for q in tree.traverse(list()) if isinstance(q, Tensor)]:
-            if p.size == 1 and p.is_contiguous:
-                if any(p.ptr == q[1].ptr for q in self._pending + [tree]):
-                    return False        # a scalar that is also written: order matters
-                continue
-            if p.shape != shape or not p.is_contiguous:
-                return False
+        1x1), so each lane only ever touches its own elements.  ``post`` is
+        the statement's postfix walk."""
+        out = tree[1]
+        shape = out.shape
         if self._pending and self._pending[0][1].shape != shape:
             return False
+        not_fusable = self._NOT_FUSABLE
+        for p in post:
+            tp = type(p)
+            if tp is dict:
+                if p["op"] in not_fusable:
+                    return False
+            elif tp is HIPTensor:
+                if p.size == 1 and p.is_contiguous:
+                    ptr = p.gpudata
+                    if ptr == out.gpudata or any(ptr == q[1].gpudata for q in self._pending):
+                        return False        # a scalar that is also written: order matters
+                elif p.shape != shape or not p.is_contiguous:
+                    return False
         return True
 
     # -- execution -----------------------------------------------------------------------
     def execute(self, optree):
         """Run ``assign(out, expr)`` (reference nervanagpu.py:1255-1283)."""
         assert optree[0]["op"] == "assign"
+        post = optree.traverse([])
         if self._fusing:
-            if self._can_join(optree):
+            if self._can_join(optree, post):
                 self._pending.append(optree)
+                self._pending_post.append(post)
                 return optree[1]
             self._flush()
         if self._captured is not None:
             self._captured.append([optree])
         else:
-            self._run([optree])
+            self._run([optree], [post])
         return optree[1]
 
-    def _launch_key(self, trees):
+    def _launch_key(self, trees, posts=None):
         """Cheap identity of a statement group: ops and the memory layout of
         every tensor in postfix order, plus the numbers on the side.  Equal
         keys and equal numbers mean the very same launches with the very same
         arguments."""
         parts, raw = [], []
         add = parts.append
-        for tree in trees:
+        for k, tree in enumerate(trees):
             if tree[1].rounding:
                 raise TypeError("stochastically rounded stores are never replayed")
-            for p in tree.traverse([]):
+            for p in (posts[k] if posts is not None else tree.traverse([])):
                 if type(p) is dict:
                     if p["op"] == "rand":
                         raise TypeError("random trees are never replayed")
@@ -707,7 +712,7 @@ class NervanaHIP(Backend):
                             add((p["op"], p["axis"]))
                     else:
                         add(p["op"])
-                elif isinstance(p, HIPTensor):
+                elif type(p) is HIPTensor:
                     add(p._geom)
                 else:
                     add(None)
@@ -715,7 +720,7 @@ class NervanaHIP(Backend):
             add("|")
         return tuple(parts), raw
 
-    def _run(self, trees):
+    def _run(self, trees, posts=None):
         """Launch a statement group.  The first time, the slow path builds the
         DAG, picks or compiles kernels and records every launch it makes
         (packed arguments included); afterwards an identical group -- same
@@ -724,7 +729,7 @@ class NervanaHIP(Backend):
         learning rate).  The reference re-derived everything on every call
         (its own TODO at float_ew.py:640-641 asks for exactly this)."""
         try:
-            key, raw = self._launch_key(trees)
+            key, raw = self._launch_key(trees, posts)
             if self._originals:
                 key = key + ("reads-before-group",)
         except (AttributeError, TypeError):
