@@ -380,6 +380,10 @@ def next_rows(be, rows):
     calls("copy_transpose (64,512,2048) f32 axes (2,0,1)", lambda: be.copy_transpose(t3_in, t3_out, axes=(2, 0, 1)),
           2 * sq[0] * sq[1] * 4, "prebuilt (kernels.hip)", reps=10)
     del t_in, t_out, t3_in, t3_out, a32
+    h_in, h_out = _fresh(be, sq, dtype=f16, rs=rs), be.empty(sq, dtype=f16)
+    calls("copy_transpose (8192,8192) f16", lambda: be.copy_transpose(h_in, h_out), 2 * sq[0] * sq[1] * 2,
+          "prebuilt (kernels.hip)", reps=10)
+    del h_in, h_out
 
     # the GEMM hand-off (library kernel; flops, not bytes, bound it)
     m = 4096

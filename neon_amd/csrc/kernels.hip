@@ -574,16 +574,19 @@ __global__ __launch_bounds__(TR_T) void transpose_tile_kernel(T* __restrict__ ou
     }
 }
 
-// The same tile walk for 4-byte elements with 16-byte global accesses: 16
-// lanes cover a 64-element run, the workgroup moves 16 runs per pass.  Needs
-// both tile extents, the strides of every other dimension and the base
-// addresses to be multiples of 4 elements.  LDS is still accessed word by word
-// (row pitch 65: the four words a lane turns into an output vector come from
-// four tile rows), two-way bank conflicts at worst.
-template <bool SWAP>
-__global__ __launch_bounds__(TR_T) void transpose_tile_v4_kernel(uint32_t* __restrict__ out,
-                                                                 const uint32_t* __restrict__ in, TrGeom g) {
-    __shared__ uint32_t tile[SWAP ? TR_TILE : 1][TR_TILE + 1];
+// The same tile walk for 2- and 4-byte elements with 16-byte global accesses:
+// VE = 16 / sizeof(T) elements per lane, 64 / VE lanes cover a 64-element run.
+// Needs both tile extents, the strides of every other dimension and the base
+// addresses to be multiples of VE elements.  LDS is still accessed element by
+// element (the VE elements a lane turns into an output vector come from VE
+// tile rows; odd row pitch in 32-bit words), two-way bank conflicts at worst.
+template <typename T, bool SWAP>
+__global__ __launch_bounds__(TR_T) void transpose_tile_vec_kernel(T* __restrict__ out, const T* __restrict__ in,
+                                                                  TrGeom g) {
+    constexpr int VE = 16 / (int)sizeof(T);
+    constexpr int PITCH = TR_TILE + 4 / (int)sizeof(T);          // 65 words (4-byte) or 33 words (2-byte) per row
+    constexpr uint32_t LANES = TR_TILE / VE, RUNS = TR_T / LANES;
+    __shared__ T tile[SWAP ? TR_TILE : 1][PITCH];
     unsigned long long b = blockIdx.x;
     const uint32_t tx = (uint32_t)(b % g.tiles_x);
     b /= g.tiles_x;
@@ -598,43 +601,51 @@ __global__ __launch_bounds__(TR_T) void transpose_tile_v4_kernel(uint32_t* __res
         obase += (long long)idx * g.os[k];
     }
     const uint32_t nx = g.n[g.ax], ny = g.ay >= 0 ? g.n[g.ay] : 1u;
-    const long long isx = g.is[g.ax], osx = g.os[g.ax];
+    const long long isx = g.is[g.ax];
     const long long isy = g.ay >= 0 ? g.is[g.ay] : 0, osy = g.ay >= 0 ? g.os[g.ay] : 0;
     const uint32_t x0 = tx * TR_TILE, y0 = ty * TR_TILE;
-    const uint32_t quad = (threadIdx.x & 15u) * 4u, run = threadIdx.x >> 4;     // 16 runs of 16 quads
-    constexpr uint32_t RUNS = TR_T / 16;
+    const uint32_t first = (threadIdx.x % LANES) * VE, run = threadIdx.x / LANES;
+    union Vec { nh_u32 w[4]; T e[VE]; };
     if constexpr (SWAP) {
         // input runs along y (isy == 1): run index = x
         for (uint32_t i = run; i < TR_TILE; i += RUNS) {
-            const uint32_t x = x0 + i, y = y0 + quad;
+            const uint32_t x = x0 + i, y = y0 + first;
             if (x < nx && y < ny) {
-                nh_u32 w[4];
-                nh_load_words<4, true>(in + ibase + (long long)x * isx + (long long)y, w);
+                Vec v;
+                nh_load_words<4, true>(reinterpret_cast<const nh_u32*>(in + ibase + (long long)x * isx + (long long)y), v.w);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) tile[i][quad + j] = w[j];
+                for (int j = 0; j < VE; ++j) tile[i][first + j] = v.e[j];
             }
         }
         __syncthreads();
-        // output runs along x (osx == 1): run index = y
+        // output runs along x (stride 1): run index = y
         for (uint32_t i = run; i < TR_TILE; i += RUNS) {
-            const uint32_t x = x0 + quad, y = y0 + i;
+            const uint32_t x = x0 + first, y = y0 + i;
             if (x < nx && y < ny) {
-                nh_u32 w[4];
+                Vec v;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) w[j] = tile[quad + j][i];
-                nh_store_words<4, false>(out + obase + (long long)x + (long long)y * osy, w);
+                for (int j = 0; j < VE; ++j) v.e[j] = tile[first + j][i];
+                nh_store_words<4, false>(reinterpret_cast<nh_u32*>(out + obase + (long long)x + (long long)y * osy), v.w);
             }
         }
     } else {
         for (uint32_t i = run; i < TR_TILE; i += RUNS) {
-            const uint32_t x = x0 + quad, y = y0 + i;
+            const uint32_t x = x0 + first, y = y0 + i;
             if (x < nx && y < ny) {
-                nh_u32 w[4];
-                nh_load_words<4, true>(in + ibase + (long long)x + (long long)y * isy, w);
-                nh_store_words<4, false>(out + obase + (long long)x + (long long)y * osy, w);
+                Vec v;
+                nh_load_words<4, true>(reinterpret_cast<const nh_u32*>(in + ibase + (long long)x + (long long)y * isy), v.w);
+                nh_store_words<4, false>(reinterpret_cast<nh_u32*>(out + obase + (long long)x + (long long)y * osy), v.w);
             }
         }
     }
+}
+
+template <typename T>
+void launch_transpose_vec(void* out, const void* in, const TrGeom& g, bool swap, unsigned blocks, hipStream_t s) {
+    if (swap)
+        hipLaunchKernelGGL((transpose_tile_vec_kernel<T, true>), dim3(blocks), dim3(TR_T), 0, s, (T*)out, (const T*)in, g);
+    else
+        hipLaunchKernelGGL((transpose_tile_vec_kernel<T, false>), dim3(blocks), dim3(TR_T), 0, s, (T*)out, (const T*)in, g);
 }
 
 template <typename T>
@@ -769,22 +780,19 @@ int nh_copy_transpose(void* out, const void* in, int itemsize, int ndim, const u
         if (k != ax && k != ay) blocks *= g.n[k];
     if (blocks > 0x7fffffffull) return nh_internal_fail(NH_EINVAL, "nh_copy_transpose: too many tiles for one launch");
     hipStream_t s = (hipStream_t)stream;
-    if (itemsize == 4 && ay >= 0) {
-        // 16-byte accesses when every run of four elements is aligned on both sides
-        bool v4 = aligned16(out) && aligned16(in) && g.n[ax] % 4 == 0 && g.os[ax] == 1 &&
-                  (swap ? (g.n[ay] % 4 == 0 && g.is[ay] == 1) : g.is[ax] == 1);
-        for (int k = 0; k < ndim && v4; ++k) {
+    if ((itemsize == 4 || itemsize == 2) && ay >= 0) {
+        // 16-byte accesses when every run of VE elements is aligned on both sides
+        const uint32_t ve = 16u / (uint32_t)itemsize;
+        bool vec = aligned16(out) && aligned16(in) && g.n[ax] % ve == 0 && g.os[ax] == 1 &&
+                   (swap ? (g.n[ay] % ve == 0 && g.is[ay] == 1) : g.is[ax] == 1);
+        for (int k = 0; k < ndim && vec; ++k) {
             if (g.n[k] == 1) continue;
-            if (k != ax && g.os[k] % 4) v4 = false;
-            if (k != (swap ? ay : ax) && g.is[k] % 4) v4 = false;
+            if (k != ax && g.os[k] % ve) vec = false;
+            if (k != (swap ? ay : ax) && g.is[k] % ve) vec = false;
         }
-        if (v4) {
-            if (swap)
-                hipLaunchKernelGGL((transpose_tile_v4_kernel<true>), dim3((unsigned)blocks), dim3(TR_T), 0, s,
-                                   (uint32_t*)out, (const uint32_t*)in, g);
-            else
-                hipLaunchKernelGGL((transpose_tile_v4_kernel<false>), dim3((unsigned)blocks), dim3(TR_T), 0, s,
-                                   (uint32_t*)out, (const uint32_t*)in, g);
+        if (vec) {
+            if (itemsize == 4) launch_transpose_vec<uint32_t>(out, in, g, swap, (unsigned)blocks, s);
+            else launch_transpose_vec<uint16_t>(out, in, g, swap, (unsigned)blocks, s);
             return launch_status("nh_copy_transpose");
         }
     }
