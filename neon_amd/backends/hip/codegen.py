@@ -389,20 +389,69 @@ _EXPENSIVE = {"exp", "log", "exp2", "log2", "tanh", "tanh2", "sig", "sig2", "pow
               "div", "safelog"}
 
 
-def _kept_values(prog, stages, limit):
-    """Elementwise results worth keeping in registers between sweeps: nodes
-    that two or more sweeps need and that cost a transcendental or a division
-    to recompute (softmax's exp(x - max)).  ``stages`` lists the targets of
-    each sweep in order; at most ``limit`` nodes are returned, outermost
-    first."""
-    reductions = set(n.nid for n in prog.nodes if n.kind == "R")
+def _costly_nodes(prog):
     costly = {}
     for n in prog.nodes:            # topological order
         if n.kind == "E":
             costly[n.nid] = (n.op in _EXPENSIVE) or any(costly.get(a.nid, False) for a in n.args)
+    return costly
+
+
+def _overwriting_values(prog, stages, resident_ok):
+    """Kept values that cost no registers: (node, leaf) pairs where ``node`` is
+    an expensive elementwise result that two or more sweeps need and ``leaf``
+    is a resident float32 operand that nothing after the node's first sweep
+    reads except through the node (softmax: once the maximum is known
+    exp(x - max) can take x's place).  The node's value is written over the
+    leaf's registers at the end of the sweep that first computes it.
+    ``resident_ok(leaf)`` says whether the leaf's tile is one 32-bit word per
+    element."""
+    reductions = set(n.nid for n in prog.nodes if n.kind == "R")
+    costly = _costly_nodes(prog)
+    pairs = []                      # (node, leaf, first sweep that computes node)
+
+    def avail_at(t, extra=()):
+        # a kept value exists from the sweep after the one that computes it
+        return reductions | set(n.nid for n, _, f in list(pairs) + list(extra) if f < t)
+
+    while True:
+        taken = set(leaf.nid for _, leaf, _ in pairs)
+        first, count, by_id = {}, {}, {}
+        for s, targets in enumerate(stages):
+            for n in _needed(targets, avail_at(s)):
+                if n.kind == "E" and n.vr and n.vc and costly.get(n.nid):
+                    first.setdefault(n.nid, s)
+                    count[n.nid] = count.get(n.nid, 0) + 1
+                    by_id[n.nid] = n
+        found = None
+        for nid in sorted((k for k, c in count.items() if c >= 2), reverse=True):
+            n, f = by_id[nid], first[nid]
+            later = set()
+            for t in range(f + 1, len(stages)):
+                later.update(m.nid for m in _needed(stages[t], avail_at(t, [(n, None, f)])))
+            for leaf in _needed([n], avail_at(f)):
+                if (leaf.kind == "T" and leaf.nid not in taken and leaf.nid not in later
+                        and resident_ok(leaf)):
+                    found = (n, leaf, f)
+                    break
+            if found:
+                break
+        if not found:
+            return [(n, leaf) for n, leaf, _ in pairs]
+        pairs.append(found)
+
+
+def _kept_values(prog, stages, limit, already=()):
+    """Elementwise results worth keeping in registers between sweeps: nodes
+    that two or more sweeps need and that cost a transcendental or a division
+    to recompute (softmax's exp(x - max)).  ``stages`` lists the targets of
+    each sweep in order; at most ``limit`` nodes are returned, outermost
+    first.  ``already``: nodes kept by other means."""
+    reductions = set(n.nid for n in prog.nodes if n.kind == "R")
+    costly = _costly_nodes(prog)
     kept = []
     while len(kept) < limit:
-        avail = reductions | set(k.nid for k in kept)
+        avail = reductions | set(k.nid for k in kept) | set(n.nid for n in already)
         count, by_id = {}, {}
         for targets in stages:
             for n in _needed(targets, avail):
@@ -622,30 +671,55 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None):
     declare_tiles([n for n in g.leaf_nodes(used_nodes([st.root for st in prog.statements]))
                    if not varies_in_loop(n)])
 
+    # expensive values that later sweeps need again take over the registers of
+    # a resident float32 operand nothing else reads afterwards
+    over, vals = {}, {}
+    if resident:
+        stages = [[n.args[0] for n in per_level.get(s, [])] for s in range(nsweeps)]
+        stages = [t for t in stages if t]
+        if full_out:
+            stages.append([st.root for st in full_out])
+
+        def one_word_per_element(leaf):
+            return varies_in_loop(leaf) and DTYPE_CODE[prog.tensors[leaf.slot].dtype] == "f4"
+
+        over = dict((n.nid, leaf) for n, leaf in _overwriting_values(prog, stages, one_word_per_element))
+
+    def stops():
+        d = set(done)
+        d.update(vals)
+        return d
+
     for s in range(nsweeps):
         reds = [n for n in per_level.get(s, [])]
         if not reds:
             continue
         args = [n.args[0] for n in reds]
-        nodes = _needed(args, done)
+        nodes = _needed(args, stops())
         leaves = g.leaf_nodes(nodes)
         declare_tiles(leaves)
         for n in reds:
             g.declare_acc(n)
+        # (an operand that did not get registers cannot lend them)
+        fresh = [n for n in nodes if n.nid in over and n.nid not in vals and over[n.nid].nid not in transient]
 
-        def reduce_body(tiles, nodes=nodes, reds=reds):
+        def reduce_body(tiles, nodes=nodes, reds=reds, fresh=fresh):
             L.open("if (ok)")
             if V > 1:
                 L("#pragma unroll")
             L.open("for (int j = 0; j < %d; ++j)" % V)
-            ref = g.make_ref("_s", "rr", "c", V, tiles)
-            g.emit_exprs(nodes, ref, done)
+            ref = g.make_ref("_s", "rr", "c", V, tiles, vals)
+            g.emit_exprs(nodes, ref, stops())
             for n in reds:
                 g.accumulate(n, ref(n.args[0]), "c + j")
+            for n in fresh:
+                L("keep%d[k].put(j, t%d);" % (over[n.nid].nid, n.nid))
             L.close()
             L.close()
 
         sweep(leaves, reduce_body)
+        for n in fresh:
+            vals[n.nid] = "keep%d[k].get(j)" % over[n.nid].nid
         for n in reds:
             op = _RED_OP[n.op]
             ty_ = "nh_pair" if n.is_index else "float"
@@ -685,7 +759,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None):
     # outputs with the full shape: one more sweep
     if full_out:
         roots = [st.root for st in full_out]
-        nodes = _needed(roots, done)
+        nodes = _needed(roots, stops())
         leaves = g.leaf_nodes(nodes)
         declare_tiles(leaves)
 
@@ -696,8 +770,8 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None):
             if V > 1:
                 L("#pragma unroll")
             L.open("for (int j = 0; j < %d; ++j)" % V)
-            ref = g.make_ref("_s", "rr", "c", V, tiles)
-            g.emit_exprs(nodes, ref, done)
+            ref = g.make_ref("_s", "rr", "c", V, tiles, vals)
+            g.emit_exprs(nodes, ref, stops())
             for st in full_out:
                 if st.root.kind == "R" and st.root.is_index:
                     L("o%d.seti(j, ri%d);" % (st.out.index, st.root.nid))
@@ -711,7 +785,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None):
         sweep(leaves, store_body)
     L.close()
     return _finish("row", g, head, fmt, T, 0, dict(V=V, LX=LX, LY=LY, NCH=NCH, stream=bool(stream),
-                                                   passing=len(transient)))
+                                                   passing=len(transient), over=len(vals)))
 
 
 # =====================================================================================
@@ -941,8 +1015,14 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
     stages = [t for t in stages if t]
     if full_out:
         stages.append([st.root for st in full_out])
-    kept = _kept_values(prog, stages, max_vals)
-    kept_ids = set(n.nid for n in kept)
+    def one_word_per_element(leaf):
+        t = prog.tensors[leaf.slot]
+        return varies_in_loop(leaf) and t.shape[1] > 1 and DTYPE_CODE[t.dtype] == "f4"
+
+    over = dict((n.nid, leaf) for n, leaf in _overwriting_values(prog, stages, one_word_per_element))
+    by_nid = dict((n.nid, n) for n in prog.nodes)
+    kept = _kept_values(prog, stages, max_vals, already=[by_nid[k] for k in over])
+    kept_ids = set(n.nid for n in kept) | set(over)
     vals = {}          # nid -> expression of a value kept from an earlier sweep
 
     def stops():
@@ -954,12 +1034,15 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
         """inside the j loop: keep the values later sweeps will want"""
         fresh = [n for n in nodes if n.nid in kept_ids and n.nid not in vals]
         for n in fresh:
-            L("val%d[i][j] = t%d;" % (n.nid, n.nid))
+            if n.nid in over:
+                L("keep%d[i].put(j, t%d);" % (over[n.nid].nid, n.nid))
+            else:
+                L("val%d[i][j] = t%d;" % (n.nid, n.nid))
         return fresh
 
     def declare_values(nodes):
         for n in nodes:
-            if n.nid in kept_ids and n.nid not in vals:
+            if n.nid in kept_ids and n.nid not in vals and n.nid not in over:
                 L("float val%d[%d][%d];" % (n.nid, NR, V))
 
     for s in range(nsweeps):
@@ -988,7 +1071,7 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
         L.close()
         L.close()
         for n in fresh:
-            vals[n.nid] = "val%d[i][j]" % n.nid
+            vals[n.nid] = ("keep%d[i].get(j)" % over[n.nid].nid) if n.nid in over else ("val%d[i][j]" % n.nid)
         for n in reds:
             _emit_col_fold(g, L, n, LX, LY, T, V, "acc%d" % n.nid)
             done[n.nid] = n
@@ -1057,7 +1140,7 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
     L.close()
     return _finish("colcoop" if coop else "col", g, head, fmt, T, lds,
                    dict(V=V, LX=LX, LY=LY, NR=NR, stream=bool(stream), chunks=chunks,
-                        NRED=len(all_reds), kept=len(kept)))
+                        NRED=len(all_reds), kept=len(kept), over=len(over)))
 
 
 COLSPLIT_MAX_CHUNKS = 128

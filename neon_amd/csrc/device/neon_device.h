@@ -192,6 +192,11 @@ template <typename T, int V> struct nh_raw {
 #pragma unroll
         for (int i = 0; i < NW; ++i) asm volatile("" : "+v"(w[i]));
     }
+    // reuse the registers of a float tile for a value derived from it
+    NEON_DEV void put(int j, float v) {
+        static_assert(sizeof(T) == 4, "one word per element only");
+        w[j] = nh_bits_of<float>(v);
+    }
 };
 
 template <typename T, int V> struct nh_out {

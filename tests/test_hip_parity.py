@@ -178,6 +178,32 @@ def test_compound_and_mixed_axes(pair):
     both(pair, lambda be, x, y: (x * y).T + 1.0, [a, b])
 
 
+@pytest.mark.parametrize("axis", [0, 1])
+@pytest.mark.parametrize("shape", [(1000, 4096), (333, 130), (32000, 256), (256, 3000)])
+def test_values_that_take_the_place_of_a_resident_operand(pair, shape, axis):
+    """softmax keeps exp(x - max) in x's registers; variants that read x again
+    afterwards, or two operands of which one is reused, must not be disturbed
+    by that"""
+    rs = np.random.RandomState(shape[0])
+    a = (rs.standard_normal(shape) * 2).astype(np.float32)
+    b = rs.standard_normal(shape).astype(np.float32)
+    cpu, hip = pair
+
+    def softmax(be, x):
+        e = be.exp(x - be.max(x, axis=axis))
+        return e / be.sum(e, axis=axis)
+
+    cases = [("softmax + x", lambda be, x, y: softmax(be, x) + x),
+             ("softmax * y", lambda be, x, y: softmax(be, x) * y),
+             ("softmax(x + y) * y", lambda be, x, y: softmax(be, x + y) * y),
+             ("log-softmax", lambda be, x, y: be.log(softmax(be, x)) * y),
+             ("softmax of softmax", lambda be, x, y: softmax(be, softmax(be, x)))]
+    for what, f in cases:
+        got = call_func(f, hip, [a, b])
+        want = call_func(f, cpu, [a, b])
+        assert_close(got, want, rtol=5 * RTOL32 if shape[axis] > 5000 else RTOL32, atol=1e-7, what=what)
+
+
 @pytest.mark.parametrize("shape", [(32000, 256), (5000, 100), (20000, 1000), (9001, 36)])
 def test_tall_multilevel_axis0(pair, shape):
     """deep axis-0 trees over more rows than one workgroup holds: the

@@ -293,3 +293,43 @@ def test_long_rows_of_two_tensors_keep_one_resident(pb):
     assert spec.family == "row" and spec.params["NCH"] == 13 and spec.params["passing"] == 1
     # x is loaded once, the deltas once per sweep
     assert spec.source.count(".load_stream(") == 3
+
+
+def test_softmax_reuses_the_registers_of_x_for_the_exponentials(pb):
+    """exp(x - max) is needed by the sum and by the quotient; x by nothing after
+    the sum's sweep: the exponentials take x's registers (one exp per element).
+    Not when x is read again later, and not for fp16 storage (two elements per
+    register)."""
+    x, out = pb.empty((1000, 4096)), pb.empty((1000, 4096))
+
+    def softmax(t):
+        e = pb.exp(t - pb.max(t, axis=0))
+        return e / pb.sum(e, axis=0)
+
+    spec = plan_of(pb, lambda: out.__setitem__(slice(None), softmax(x))).spec
+    assert spec.family == "col" and spec.params["over"] == 1
+    assert spec.source.count("expf(") == 1 and ".put(j, " in spec.source
+
+    spec = plan_of(pb, lambda: out.__setitem__(slice(None), softmax(x) + x)).spec
+    assert spec.params["over"] == 0 and ".put(j, " not in spec.source
+
+    xh = pb.empty((1000, 4096), np.float16)
+    spec = plan_of(pb, lambda: out.__setitem__(slice(None), softmax(xh))).spec
+    assert spec.params["over"] == 0 and ".put(j, " not in spec.source
+
+
+def test_row_softmax_reuses_registers_when_the_row_is_resident(pb):
+    x, out = pb.empty((4096, 1000)), pb.empty((4096, 1000))
+
+    def softmax(t):
+        e = pb.exp(t - pb.max(t, axis=1))
+        return e / pb.sum(e, axis=1)
+
+    spec = plan_of(pb, lambda: out.__setitem__(slice(None), softmax(x))).spec
+    assert spec.family == "row" and spec.params["NCH"] > 0 and spec.params["over"] == 1
+    assert spec.source.count("expf(") == 1
+    # a row too long for the registers is streamed in every sweep: nothing to reuse
+    xl, outl = pb.empty((16, 1 << 20)), pb.empty((16, 1 << 20))
+    spec = plan_of(pb, lambda: outl.__setitem__(slice(None), softmax(xl))).spec
+    assert spec.family == "row" and spec.params["NCH"] == 0 and spec.params["over"] == 0
+    assert spec.source.count("expf(") == 2
