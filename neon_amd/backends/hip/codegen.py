@@ -799,7 +799,16 @@ def _emit_col_fold(g, L, n, LX, LY, T, V, src, dst_decl=True):
     row order."""
     op = _RED_OP[n.op]
     ty_ = "nh_pair" if n.is_index else "float"
-    if LX < 64:
+    VK = V            # values a lane contributes to the LDS stage
+    if LX < 64 and T > 64:
+        # the wave's row-lanes are folded with lane exchanges that split the V
+        # values among the lanes; LDS collects the pieces
+        steps = (64 // LX).bit_length() - 1
+        VK = max(1, V >> steps)
+        WY = T // 64
+        wy = "(threadIdx.x >> 6)"
+        writer = "((threadIdx.x & 63) < %d)" % (LX * (V // VK))
+    elif LX < 64:
         stride = LX
         while stride < 64:
             L("#pragma unroll")
@@ -826,30 +835,44 @@ def _emit_col_fold(g, L, n, LX, LY, T, V, src, dst_decl=True):
         else:
             L("for (int j = 0; j < %d; ++j) rv%d[j] = %s[j];" % (V, n.nid, src))
         return
-    L.open("if (%s)" % writer)
-    L("#pragma unroll")
-    L("for (int j = 0; j < %d; ++j) %s[%s][tx * %d + j] = %s[j];" % (V, buf, wy, V, src))
-    L.close()
-    L("__syncthreads();")
-    L("#pragma unroll")
-    L.open("for (int j = 0; j < %d; ++j)" % V)
-    L("%s f = %s[0][tx * %d + j];" % (ty_, buf, V))
-    L("#pragma unroll")
-    L("for (int y = 1; y < %d; ++y) f = %s::f(f, %s[y][tx * %d + j]);" % (WY, op, buf, V))
-    if n.is_index:
-        L("ri%d[j] = f.i; %s[j] = f;" % (n.nid, src))
+    if LX < 64:
+        L.open("")
+        L("const int j0 = nh_col_wave_fold<%s, %d, %d>(%s);" % (op, V, LX, src))
+        L.open("if (%s)" % writer)
+        L("#pragma unroll")
+        L("for (int j = 0; j < %d; ++j) %s[%s][tx * %d + j0 + j] = %s[j];" % (VK, buf, wy, V, src))
+        L.close()
+        L.close()
     else:
-        L("rv%d[j] = f; %s[j] = f;" % (n.nid, src))
+        L.open("if (%s)" % writer)
+        L("#pragma unroll")
+        L("for (int j = 0; j < %d; ++j) %s[%s][tx * %d + j] = %s[j];" % (V, buf, wy, V, src))
+        L.close()
+    L("__syncthreads();")
+    # a lane's V partials of one wave group are adjacent and 16-byte aligned:
+    # walking the groups in the outer loop lets them come in as one LDS read
+    L("#pragma unroll")
+    L("for (int j = 0; j < %d; ++j) %s[j] = %s[0][tx * %d + j];" % (V, src, buf, V))
+    L("#pragma unroll")
+    L.open("for (int y = 1; y < %d; ++y)" % WY)
+    L("#pragma unroll")
+    L("for (int j = 0; j < %d; ++j) %s[j] = %s::f(%s[j], %s[y][tx * %d + j]);" % (V, src, op, src, buf, V))
     L.close()
+    L("#pragma unroll")
+    if n.is_index:
+        L("for (int j = 0; j < %d; ++j) ri%d[j] = %s[j].i;" % (V, n.nid, src))
+    else:
+        L("for (int j = 0; j < %d; ++j) rv%d[j] = %s[j];" % (V, n.nid, src))
     L("__syncthreads();")
 
 
 def _col_lds(L, LX, LY, T, V, any_index):
     WY = (T // 64) if LX < 64 else LY
-    L("__shared__ float s_f[%d][%d];" % (WY, LX * V + 1))
+    pitch = -(-(LX * V) // 4) * 4       # rows stay 16-byte aligned
+    L("__shared__ __attribute__((aligned(16))) float s_f[%d][%d];" % (WY, pitch))
     if any_index:
-        L("__shared__ nh_pair s_p[%d][%d];" % (WY, LX * V + 1))
-    return WY * (LX * V + 1) * (4 + (8 if any_index else 0))
+        L("__shared__ __attribute__((aligned(16))) nh_pair s_p[%d][%d];" % (WY, pitch))
+    return WY * pitch * (4 + (8 if any_index else 0))
 
 
 def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):

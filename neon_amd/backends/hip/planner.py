@@ -402,7 +402,8 @@ def _plan_col(prog, cu_count):
     # ones leave more row-lanes, i.e. fewer rows per lane: take the widest
     # strip for which all rows fit in registers.
     lx_min = max(1, min(64, 128 // (V * isz)))
-    if R * C * isz <= (4 << 20):
+    tiny = R * C * isz <= (4 << 20)
+    if tiny:
         lx_min = 1                       # tiny inputs are latency-bound: favour more workgroups
     lx_pref = max(lx_min, min(64, _pow2floor(max(1, nvec // 32))))
     lx_pref = min(lx_pref, _pow2ceil(nvec))
@@ -412,7 +413,9 @@ def _plan_col(prog, cu_count):
     while fit is None and LX >= lx_min:
         strips = _ceil_div(nvec, LX)
         # few strips: spend more lanes on each so the rows-per-lane count drops
-        for T in ((256, 512, 1024) if strips >= cu_count else (1024, 512, 256)):
+        # (tiny inputs: joining 16 waves costs more than a second row per lane
+        # -- softmax over (1000,128): 1024 lanes 5.3 us, 512 lanes 4.4 us)
+        for T in ((256, 512, 1024) if strips >= cu_count else (512, 1024, 256) if tiny else (1024, 512, 256)):
             LY = T // LX
             NR = _ceil_div(R, LY)
             budget = _COL_BUDGET[T]

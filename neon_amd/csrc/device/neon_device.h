@@ -378,6 +378,38 @@ template <int S> NEON_DEV nh_pair nh_lane_xor(nh_pair p) {
     nh_pair r; r.v = nh_lane_xor<S>(p.v); r.i = nh_lane_xor<S>(p.i); return r;
 }
 
+// Fold, over the lanes of a wave that share (lane % LX), LEN values per lane.
+// While a lane carries more than one value each step halves them: partners
+// (lane ^ S) split the values between them, each sends the half the other
+// keeps.  V values cost V - 1 + (steps - log2 V) exchanges instead of
+// V * steps; afterwards a lane holds a[0 .. V >> halvings) for elements
+// j0, j0 + 1, ... of its column tile, j0 (returned through `j0`) given by the
+// lane's bits at the halving strides.
+template <class OP, int LEN, int S, typename T> NEON_DEV void nh_fold_step(T* a, int lane, int& j0) {
+    if constexpr (S < 64) {
+        if constexpr (LEN > 1) {
+            constexpr int H = LEN / 2;
+            const bool up = (lane & S) != 0;
+#pragma unroll
+            for (int m = 0; m < H; ++m) {
+                const T send = up ? a[m] : a[m + H];
+                const T keep = up ? a[m + H] : a[m];
+                a[m] = OP::f(keep, nh_lane_xor<S>(send));
+            }
+            j0 += up ? H : 0;
+            nh_fold_step<OP, H, S * 2, T>(a, lane, j0);
+        } else {
+            a[0] = OP::f(a[0], nh_lane_xor<S>(a[0]));
+            nh_fold_step<OP, 1, S * 2, T>(a, lane, j0);
+        }
+    }
+}
+template <class OP, int V, int LX, typename T> NEON_DEV int nh_col_wave_fold(T (&a)[V]) {
+    int j0 = 0;
+    nh_fold_step<OP, V, LX, T>(a, (int)(threadIdx.x & 63u), j0);
+    return j0;
+}
+
 // All-reduce over aligned groups of WIDTH lanes (WIDTH in 1,2,4,...,64): every
 // lane of a group ends with the group's result.  Steps 1-2 are quad
 // permutes; steps 4 and 8 use the mirror patterns, valid because the previous
