@@ -762,6 +762,43 @@ class Backend(metaclass=_BackendRegistry):
     def bprop_skipnode(self, error, deltas, alpha, beta):
         deltas[:] = deltas * beta + alpha * error
 
+    # -- layer bookkeeping the reference's containers call on any backend: no
+    #    backend-side state here, the merges just drive their branches with the
+    #    right accumulate flags (reference nervanagpu.py:3179-3231) ---------------
+    def relu_layer(self):
+        return None
+
+    def batchnorm_layer(self, in_shape):
+        return None
+
+    def mergesum_layer(self, layer_num):
+        return None
+
+    def mergebroadcast_layer(self, layer_num):
+        return None
+
+    def fprop_mergesum(self, ngLayer, inputs, inference, layers, outputs, out_shape):
+        """every branch adds into the shared output; the first one overwrites it"""
+        for k, layer in enumerate(layers):
+            layer.fprop(inputs, inference, beta=0 if k == 0 else 1)
+
+    def bprop_mergesum(self, ngLayer, alpha, beta, layers, error, deltas):
+        """branches in reverse; the one that runs first applies the caller's
+        ``beta``, the others accumulate"""
+        last = len(layers) - 1
+        for k in range(last, -1, -1):
+            layers[k].bprop(error, alpha=alpha, beta=beta if k == last else 1)
+
+    def fprop_mergebroadcast(self, ngLayer, inputs, inference, outputs, layers, out_shape):
+        for layer in layers:
+            layer.fprop(inputs, inference)
+
+    def bprop_mergebroadcast(self, ngLayer, layers, error_views, error, delta, out_shape, alpha, beta,
+                             alphas, betas):
+        betas[-1] = beta
+        for k in range(len(layers) - 1, -1, -1):
+            layers[k].bprop(error_views[k], alpha=alphas[k] * alpha, beta=betas[k])
+
     # -- outside the op-tree path ----------------------------------------------
     def compound_dot(self, A, B, C, alpha=1.0, beta=0.0, relu=False, bsum=None):
         raise NotImplementedError("dense contraction is outside the op-tree path")

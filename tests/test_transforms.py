@@ -252,3 +252,41 @@ def test_classification_metrics_hip_match_oracle(pair):
     assert abs(res[1][2] - res[0][2]) < 1e-5
     assert_close(res[1][3], res[0][3], rtol=1e-5, atol=1e-6)
     assert_close(res[1][4], res[0][4], rtol=1e-5, atol=1e-6)
+
+
+# ---- layer-facing helpers of the Backend base ---------------------------------------
+class _Branch(object):
+    """stands in for a layer: y (+)= w * x going forward, deltas (+)= alpha * w * error back"""
+
+    def __init__(self, be, w, out, deltas):
+        self.be, self.w, self.out, self.deltas = be, w, out, deltas
+
+    def fprop(self, inputs, inference, beta=0):
+        self.out[:] = self.out * beta + inputs * self.w
+
+    def bprop(self, error, alpha=1.0, beta=0.0):
+        self.deltas[:] = self.deltas * beta + error * (alpha * self.w)
+
+
+def test_merge_helpers_drive_branches_with_the_right_accumulation(cpu):
+    be = cpu
+    x = be.array(np.arange(6, dtype=np.float32).reshape(2, 3))
+    out, deltas = be.array(np.full((2, 3), 100.0, np.float32)), be.array(np.full((2, 3), 10.0, np.float32))
+    branches = [_Branch(be, w, out, deltas) for w in (1.0, 2.0, 4.0)]
+    assert be.relu_layer() is None and be.batchnorm_layer((3, 4, 4)) is None
+    assert be.mergesum_layer(3) is None and be.mergebroadcast_layer(3) is None
+    be.fprop_mergesum(None, x, False, branches, out, None)
+    assert np.array_equal(out.get(), 7.0 * x.get())             # the stale 100s are overwritten
+    be.bprop_mergesum(None, 0.5, 2.0, branches, x, deltas)
+    assert np.array_equal(deltas.get(), 2.0 * 10.0 + 0.5 * 7.0 * x.get())
+    # broadcast merge: every branch has its own error view and its own (alpha, beta)
+    d = [be.array(np.full((2, 3), 1.0, np.float32)) for _ in range(3)]
+    outs = [be.zeros((2, 3)) for _ in range(3)]
+    bb = [_Branch(be, w, o, dk) for w, o, dk in zip((1.0, 2.0, 4.0), outs, d)]
+    be.fprop_mergebroadcast(None, x, False, None, bb, None)
+    assert all(np.array_equal(o.get(), w * x.get()) for o, w in zip(outs, (1.0, 2.0, 4.0)))
+    betas = [1.0, 0.0, None]
+    be.bprop_mergebroadcast(None, bb, [x, x, x], x, None, None, 2.0, 3.0, [1.0, 0.5, 0.25], betas)
+    assert betas[-1] == 3.0
+    want = [1.0 + 2.0 * x.get(), 0.0 + 2.0 * x.get(), 3.0 + 2.0 * x.get()]
+    assert all(np.array_equal(dk.get(), w) for dk, w in zip(d, want))
