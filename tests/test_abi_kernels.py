@@ -133,7 +133,8 @@ def test_launch_validation(hip):
 
 @pytest.mark.parametrize("nbins,offset", [(64, -48), (100, -60), (256, -130), (7, -3)])
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
-@pytest.mark.parametrize("n,skew", [(1, 0), (4099, 0), (1 << 20, 0), (3 * 1000 * 1000 + 5, 1)])
+@pytest.mark.parametrize("n,skew", [(1, 0), (4099, 0), (1 << 20, 0), (3 * 1000 * 1000 + 5, 1),
+                                    (5 * 1000 * 1000 + 3, 0), (5 * 1000 * 1000 + 3, 1)])
 def test_hist_log2_entry_point(dev, n, skew, dtype, nbins, offset):
     """both counting schemes (private counters up to 64 bins, wave-agreed bins
     beyond), vector body and scalar tail, aligned and unaligned start, against
