@@ -439,6 +439,11 @@ class NervanaCPU(Backend):
             bsum[:] = self.sum(C, 1)
         return C
 
+    def make_binary_mask(self, out, keepthresh=0.5):
+        # ones where a host uniform draw falls below the threshold (reference
+        # nervanacpu.py:1052-1063)
+        out._tensor[:] = (self.rng.uniform(size=out._tensor.shape) < keepthresh).astype(out._tensor.dtype)
+
     def _uniform_like(self, ary):
         # host draws, as in the reference's binarize (nervanacpu.py:1835)
         return self.array(self.rng.uniform(0, 1, size=ary.shape))
