@@ -925,9 +925,13 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
             L("const long long r = (long long)i * %d + ty;" % LY)
         L("const bool ok = col_ok && (r < R);")
 
-    def exchange(reds):
+    def exchange(reds, last_one_folds=False):
         """fold the workgroups of a strip: afterwards acc/rv/ri hold the
-        result over all rows in every lane of every workgroup"""
+        result over all rows in every lane of every workgroup.
+
+        ``last_one_folds``: nothing but one value per column remains to be
+        written, so nobody waits: the workgroup whose arrival completes the
+        count gathers, folds and goes on alone, the others are done."""
         exchanges[0] += 1
         QMAX = -(-chunks // LY)
         for n in reds:
@@ -944,6 +948,18 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
         L.close()
         L.close()
         L("__syncthreads();     // every lane's partial stores have completed")
+        if last_one_folds:
+            L.open("if (threadIdx.x == 0)")
+            L("const unsigned int before = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
+            L("s_abort = before != %du;" % (chunks * exchanges[0] - 1))
+            L.close()
+            L("__syncthreads();")
+            L("if (s_abort) return;     // not the last to arrive: the last one finishes the strip")
+        else:
+            exchange_wait()
+        exchange_gather(reds)
+
+    def exchange_wait():
         L.open("if (threadIdx.x == 0)")
         L("__hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
         L("unsigned int spins = 0; int bad = 0;")
@@ -958,6 +974,9 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
         L("if (threadIdx.x == 0) __hip_atomic_store(ctr + 1, 0xDEADu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
         L("return;              // the other workgroups never showed up: give up rather than hang")
         L.close()
+
+    def exchange_gather(reds):
+        QMAX = -(-chunks // LY)
         for n in reds:
             L("nh_pair q%d[%d][%d];" % (n.nid, QMAX, V))
         L("#pragma unroll")
@@ -1068,6 +1087,7 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
             if n.nid in kept_ids and n.nid not in vals and n.nid not in over:
                 L("float val%d[%d][%d];" % (n.nid, NR, V))
 
+    ticket_finish = False
     for s in range(nsweeps):
         reds = per_level.get(s, [])
         if not reds:
@@ -1099,13 +1119,16 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
             _emit_col_fold(g, L, n, LX, LY, T, V, "acc%d" % n.nid)
             done[n.nid] = n
         if coop:
-            exchange(reds)
+            ticket_finish = not full_out and not any(per_level.get(k) for k in range(s + 1, nsweeps))
+            exchange(reds, last_one_folds=ticket_finish)
 
     if line_out:
         roots = [st.root for st in line_out]
         nodes = _needed(roots, done)
         leaves = g.leaf_nodes(nodes)
-        L.open("if (col_ok && ty == 0%s)" % (" && blockIdx.y == 0" if coop else ""))
+        # (cooperative strips: after a waiting exchange every workgroup has the
+        # values and the first one writes; after a ticket only the last arrival is left)
+        L.open("if (col_ok && ty == 0%s)" % (" && blockIdx.y == 0" if coop and not ticket_finish else ""))
         for n in leaves:
             g.emit_load(n, "0", "c", V, "_l")
         for st in line_out:
@@ -1150,7 +1173,10 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
             L("o%d.%s(%s);" % (st.out.index, g.st, g.addr(st.out, "r", "c")))
         L.close()
         L.close()
-    if coop:
+    if coop and ticket_finish:
+        # everyone has arrived for the last time: re-arm the counter for the next launch
+        L("if (threadIdx.x == 0) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
+    elif coop:
         # the last workgroup of the strip to get here has seen everyone pass
         # the final wait: it re-arms both counters for the next launch
         L.open("if (threadIdx.x == 0)")

@@ -423,6 +423,28 @@ def test_config5_argmax_max_ce(pair):
     assert np.array_equal(res[1][0].ravel(), np.argmax(x, axis=0))
 
 
+@pytest.mark.parametrize("shape", [(32000, 256), (9001, 36), (20000, 1000)])
+def test_tall_trees_with_one_value_per_column_repeat(hip, shape):
+    """deep axis-0 trees whose result is one value per column: after the last
+    sweep no workgroup waits, the last arrival of each strip folds alone.  Run
+    three times on fresh data: the arrival counters must re-arm every time."""
+    be = hip
+    for rep in range(3):
+        rs = np.random.RandomState(rep + shape[1])
+        a = (rs.standard_normal(shape) * 3).astype(np.float32)
+        idx = rs.randint(0, shape[0], size=(1, shape[1])).astype(np.int32)
+        tx, ti = be.array(a), be.array(idx, dtype=np.int32)
+        ce, lse = be.empty((1, shape[1])), be.empty((1, shape[1]))
+        configs.c5c_cross_entropy(be, ce, tx, be.onehot(ti, axis=0))
+        lse[:] = be.log(be.sum(be.exp(tx - be.max(tx, axis=0)), axis=0)) + be.max(tx, axis=0)
+        a64 = a.astype(np.float64)
+        m = a64.max(axis=0)
+        want_lse = np.log(np.exp(a64 - m).sum(axis=0)) + m
+        want_ce = want_lse - a64[idx.ravel(), np.arange(shape[1])]
+        assert_close(lse.get().ravel(), want_lse, rtol=RTOL32, atol=1e-6, what="log-sum-exp, repetition %d" % rep)
+        assert_close(ce.get().ravel(), want_ce, rtol=2e-5, atol=2e-5, what="cross-entropy, repetition %d" % rep)
+
+
 def test_full_size_properties(hip):
     """size-independent checks at the benchmark shapes"""
     be = hip
