@@ -740,7 +740,10 @@ class NervanaHIP(Backend):
             if launches is not None:
                 launch = self.rt.launch_packed
                 for kernel, grid, block, args in launches:
-                    launch(kernel, grid, block, args)
+                    if kernel is None:
+                        grid(*args)             # a recorded call of a prebuilt kernel's entry point
+                    else:
+                        launch(kernel, grid, block, args)
                 if self._recording is not None:
                     self._recording.extend(launches)
                     self._rec_temps.extend(entry.temps)
@@ -784,6 +787,8 @@ class NervanaHIP(Backend):
         self.plan_stats["launches"] += 1
 
     def _run_slow(self, trees):
+        if len(trees) == 1 and not self._originals and self._stage_transposed_views(trees[0]):
+            return
         try:
             prog = Program()
             prog.originals = self._originals
@@ -868,6 +873,62 @@ class NervanaHIP(Backend):
             self.plans[key] = plan
         return plan.launch_timed_sets(progs, reps), plan
 
+    def _record_call(self, fn, args):
+        """call a prebuilt kernel's entry point and keep the call with the
+        launches being recorded, so that the group can be replayed"""
+        fn(*args)
+        if self._recording is not None:
+            self._recording.append((None, fn, None, args))
+            self._rec_single = None
+        self.plan_stats["launches"] += 1
+
+    def _strided_copy(self, dst, src):
+        """dst[i, j] = src[i, j] for two 2-d views of one dtype, whatever their
+        strides, through the tiled transpose kernel (coalesced on both sides)"""
+        dims = [(dst.shape[i], dst.strides[i], src.strides[i]) for i in range(2) if dst.shape[i] != 1]
+        self._record_call(self.rt.copy_transpose,
+                          (dst.gpudata, src.gpudata, src.dtype.itemsize, [d[0] for d in dims],
+                           [d[1] for d in dims], [d[2] for d in dims]))
+
+    def _stage_transposed_views(self, tree):
+        """Large transposed tensor views among the operands of ``tree`` (``x.T``
+        of a row-major tensor: unit stride down the columns) would be read
+        4 bytes per lane with a large stride by an elementwise kernel -- about
+        a sixth of the bandwidth of the tiled transpose.  Each is copied into a
+        dense temporary first (``out[:] = x.T`` goes straight into ``out``).
+        Returns True when the tree was run that way."""
+        out, expr = tree[1], tree[2]
+        if isinstance(expr, HIPTensor):
+            leaves = [expr]
+        elif isinstance(expr, OpTreeNode):
+            leaves = [p for p in expr.traverse(list()) if isinstance(p, HIPTensor)]
+        else:
+            return False
+        views = dict((id(t), t) for t in leaves if _is_large_transposed_view(t))
+        if not views:
+            return False
+        if (expr is leaves[0] and isinstance(expr, HIPTensor) and out.is_contiguous and not out.rounding
+                and out.dtype == expr.dtype and out.shape == expr.shape and out.gpudata != expr.gpudata):
+            self._strided_copy(out, expr)
+            return True
+        temps = []
+        try:
+            dense = {}
+            for key, t in views.items():
+                dense[key] = self._temp(t.shape, t.dtype, temps)
+                self._strided_copy(dense[key], t)
+
+            def swap(node):
+                if isinstance(node, OpTreeNode):
+                    return OpTreeNode(node[0], swap(node[1]), swap(node[2]))
+                return dense.get(id(node), node)
+
+            self._run([OpTreeNode({"op": "assign"}, out, swap(expr))])
+        finally:
+            for t in temps:
+                self._temp_release(t)
+        return True
+
     def _run_split(self, tree):
         """Evaluate a tree that does not fit one kernel stage by stage through
         temporaries: every reduction (innermost first) and every transposed
@@ -930,6 +991,8 @@ class NervanaHIP(Backend):
                 self._temp_release(t)
 
     def _run_leaf(self, tree):
+        if self._stage_transposed_views(tree):
+            return
         prog = Program()
         prog.add_statement(tree)
         prog.finalize()
@@ -1277,6 +1340,15 @@ def _matrix_geometry(rows, cols, sr, sc):
         if cols == 1 or sc >= rows:
             return True, max(sc, rows, 1)
     return None
+
+
+TRANSPOSED_VIEW_STAGING_MIN = 1 << 21     # elements; below this the strided reads stay in cache
+
+
+def _is_large_transposed_view(t):
+    return (len(t.shape) == 2 and t.shape[0] > 1 and t.shape[1] > 1 and not t.take_array
+            and t.strides[0] == 1 and t.strides[1] >= t.shape[0]
+            and t.size >= TRANSPOSED_VIEW_STAGING_MIN)
 
 
 def _splittable(tree):

@@ -151,3 +151,41 @@ def test_compensated_sum_hip_long_run_and_stochastic(hip):
     want = 1.0 + 256 * float(np.float16(1e-3))
     assert abs(got.astype(np.float64).mean() - want) < 2e-3
     assert_close(got, np.full((n, n), want, np.float32), rtol=0, atol=2.0 ** -6)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
+@pytest.mark.parametrize("shape", [(2048, 1500), (1111, 2003)])
+def test_large_transposed_views_are_staged_through_the_tiled_transpose(hip, shape, dtype):
+    """x.T of a large tensor as an operand: copied dense first (or straight
+    into the output); same values as numpy, also on the replayed second run and
+    when the output aliases the operand"""
+    be = hip
+    rs = np.random.RandomState(shape[0])
+    m, n = shape
+    a = rs.standard_normal((m, n)).astype(dtype)
+    b = rs.standard_normal((n, m)).astype(dtype)
+    c = rs.standard_normal((m, n)).astype(dtype)
+    ta, tb, tc = be.array(a, dtype=dtype), be.array(b, dtype=dtype), be.array(c, dtype=dtype)
+    out = be.empty((n, m), dtype=dtype)
+    out32 = be.empty((n, m))
+    a32, b32, c32 = (v.astype(np.float32) for v in (a, b, c))
+    before = be.plan_stats["launches"]
+    for rep in range(2):
+        out[:] = ta.T
+        assert np.array_equal(out.get(), a.T)
+    assert be.plan_stats["launches"] - before == 2          # one tiled copy each, nothing else
+    for rep in range(2):
+        out32[:] = ta.T + tb
+        assert_close(out32.get(), a32.T + b32, rtol=1e-6, atol=1e-6)
+        out32[:] = ta.T * tc.T - tb
+        assert_close(out32.get(), a32.T * c32.T - b32, rtol=1e-6, atol=1e-6)
+        out32[:] = (ta + tc).T
+        assert_close(out32.get(), (a32 + c32).T, rtol=1e-6, atol=1e-6)
+        out32[:] = be.sum(ta.T, axis=0) + tb
+        assert_close(out32.get(), a32.T.sum(axis=0, keepdims=True) + b32, rtol=1e-5, atol=1e-4)
+    if dtype == np.float32:
+        sq = rs.standard_normal((1600, 1600)).astype(np.float32)
+        t = be.array(sq)
+        t[:] = t.T + 1.0                                    # the staging copy makes this well defined
+        assert np.array_equal(t.get(), sq.T + 1.0)
