@@ -194,6 +194,8 @@ def _try_flatten(prog):
         if n.kind == "H":
             return
     N = R * C
+    if N > 0x7FFFFFFF:
+        return                  # extents are 32-bit kernel arguments: stay two-dimensional
     for t in prog.tensors:
         if t.shape != (1, 1):
             t.shape, t.strides = (1, N), (N, 1)

@@ -520,3 +520,33 @@ def test_compound_batchnorm(pair, shape, dtype):
         # forward ran as one row kernel: x read once
         fams = [p.spec.family for p in hip.plans.values() if len(p.spec.source) and "row" == p.spec.family]
         assert fams
+
+
+def test_more_than_2_31_elements(hip):
+    """a tensor of 46341 x 46342 fp16 (2^31 + 83k elements, 4.3 GB): fill,
+    elementwise tree and both reduction axes address it with 64-bit offsets;
+    checked on the first and the last rows, which hold host data"""
+    be = hip
+    R, C = 46341, 46342
+    x = be.empty((R, C), dtype=np.float16)
+    out = be.empty((R, C), dtype=np.float16)
+    x[:] = 1.5
+    rs = np.random.RandomState(11)
+    head = rs.uniform(-2, 2, (3, C)).astype(np.float16)
+    tail = rs.uniform(-2, 2, (5, C)).astype(np.float16)
+    x[0:3, :].set(head)
+    x[R - 5:R, :].set(tail)
+    out[:] = x * 2.0 + 1.0
+    assert np.array_equal(out[0:3, :].get(), (head.astype(np.float32) * 2 + 1).astype(np.float16))
+    assert np.array_equal(out[R - 5:R, :].get(), (tail.astype(np.float32) * 2 + 1).astype(np.float16))
+    assert np.all(out[R // 2:R // 2 + 2, :].get() == 4.0)
+    rows = be.empty((R, 1))
+    rows[:] = be.sum(x, axis=1)
+    got = rows.get().ravel()
+    assert_close(got[R - 5:], tail.astype(np.float64).sum(axis=1), rtol=1e-5, atol=1e-2)
+    assert np.all(got[3:R - 5] == 1.5 * C)
+    cols = be.empty((1, C))
+    cols[:] = be.max(x, axis=0)
+    want = np.maximum(np.maximum(head.max(axis=0), tail.max(axis=0)), np.float16(1.5)).astype(np.float32)
+    assert np.array_equal(cols.get().ravel(), want)
+    del x, out

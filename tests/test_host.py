@@ -333,3 +333,17 @@ def test_row_softmax_reuses_registers_when_the_row_is_resident(pb):
     spec = plan_of(pb, lambda: outl.__setitem__(slice(None), softmax(xl))).spec
     assert spec.family == "row" and spec.params["NCH"] == 0 and spec.params["over"] == 0
     assert spec.source.count("expf(") == 2
+
+
+def test_more_than_2_31_elements_stay_two_dimensional(pb):
+    """extents travel as 32-bit kernel arguments: a contiguous elementwise
+    program is flattened to one long row only while that row fits"""
+    big, small = (60000, 50000), (6000, 5000)
+    x, y, out = (pb.empty(big) for _ in range(3))
+    spec = plan_of(pb, lambda: out.__setitem__(slice(None), x * 0.5 + y)).spec
+    assert spec.family == "ew" and spec.params["LY"] * spec.params["LX"] == 256
+    assert pb.choices[-1].grid[0] * spec.params["LX"] * spec.params["V"] >= big[1]
+    assert pb.choices[-1].grid[0] * spec.params["LX"] * spec.params["V"] < 2 * big[1]      # a row, not the whole tensor
+    x, y, out = (pb.empty(small) for _ in range(3))
+    ch = plan_of(pb, lambda: out.__setitem__(slice(None), x * 0.5 + y))
+    assert ch.grid[0] * 256 * ch.spec.params["V"] >= small[0] * small[1]                    # flattened
