@@ -550,3 +550,25 @@ def test_more_than_2_31_elements(hip):
     want = np.maximum(np.maximum(head.max(axis=0), tail.max(axis=0)), np.float16(1.5)).astype(np.float32)
     assert np.array_equal(cols.get().ravel(), want)
     del x, out
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
+@pytest.mark.parametrize("shape", [(37, 1032), (130, 264), (1000, 4096), (16, 8)])
+def test_row_vectors_fetched_once_per_workgroup(pair, shape, dtype):
+    """(1, C) operands of a two-dimensional elementwise kernel are loaded ahead
+    of the row loop and shared by the rows a lane handles"""
+    R, C = shape
+    rs = np.random.RandomState(R + C)
+    x = rs.standard_normal(shape).astype(dtype)
+    row = rs.standard_normal((1, C)).astype(np.float32)
+    row2 = rs.standard_normal((1, C)).astype(dtype)
+    col = rs.standard_normal((R, 1)).astype(np.float32)
+    cases = [lambda be, a, r, r2, c: a * r,
+             lambda be, a, r, r2, c: a * r + c,
+             lambda be, a, r, r2, c: (a - r2) * r + r2 * c,
+             lambda be, a, r, r2, c: be.maximum(a, r) - be.minimum(r2, c)]
+    cpu, hip = pair
+    for f in cases:
+        got = call_func(f, hip, [x, row, row2, col])
+        want = call_func(f, cpu, [x.astype(np.float32), row, row2.astype(np.float32), col])
+        assert_close(got, want, rtol=RTOL32, atol=1e-6)
