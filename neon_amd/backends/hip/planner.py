@@ -134,9 +134,13 @@ class KernelCache(object):
 # ---------------------------------------------------------------------------------------
 # vector width
 # ---------------------------------------------------------------------------------------
-def _vector_width(prog, single_row_tail_ok):
-    """Largest V (elements per lane access) such that every column-varying
-    operand can be touched with aligned vector instructions."""
+def _vector_width(prog, tail_ok):
+    """V (elements per lane access): 16 bytes of the narrowest column-varying
+    operand, at most 8 elements.  Addresses need no alignment beyond the
+    element's (the device's vector accesses are typed byte-aligned), so views
+    that start mid-row and odd row lengths keep full-width accesses; what V
+    must do is divide the row length, unless the family handles a partial last
+    tile (``tail_ok``: the elementwise family)."""
     R, C = prog.domain
     cols = [t for t in prog.tensors if t.shape[1] > 1]
     used = used_nodes([st.root for st in prog.statements])
@@ -147,20 +151,10 @@ def _vector_width(prog, single_row_tail_ok):
         return 1
     isz_min = min([t.dtype.itemsize for t in cols] + [4 for _ in hot0])
     V = min(8, 16 // isz_min)
-    while V > 1:
-        ok = (C % V == 0) or (single_row_tail_ok and R == 1)
-        for t in cols:
-            align = min(16, V * t.dtype.itemsize)
-            if t.ptr % align:
-                ok = False
-            if t.shape[0] > 1 and (t.strides[0] * t.dtype.itemsize) % align:
-                ok = False
-        for t in hot0:
-            if t.ptr % min(16, V * 4):
-                ok = False
-        if ok:
-            break
+    while V > 1 and C % V and not tail_ok:
         V //= 2
+    if C < V:
+        V = 1 if not tail_ok else max(1, _pow2floor(C))
     return V
 
 
@@ -326,7 +320,7 @@ def make_plan(prog, rt, cache, cu_count):
 def _plan_ew(prog, cu_count):
     _try_flatten(prog)
     R, C = prog.domain
-    V = _vector_width(prog, single_row_tail_ok=True)
+    V = _vector_width(prog, tail_ok=True)
     nvec = _ceil_div(C, V)
     if R == 1:
         LX, LY, UR, UC = 256, 1, 1, 1
@@ -349,7 +343,7 @@ def _plan_ew(prog, cu_count):
 
 def _plan_row(prog, cu_count):
     R, C = prog.domain
-    V = _vector_width(prog, single_row_tail_ok=False)
+    V = _vector_width(prog, tail_ok=False)
     nvec = _ceil_div(C, V)
     words = _words_per_tile(prog, V, 1)
     options = []
@@ -393,7 +387,7 @@ COLSPLIT_THREADS = 256
 
 def _plan_col(prog, cu_count):
     R, C = prog.domain
-    V = _vector_width(prog, single_row_tail_ok=False)
+    V = _vector_width(prog, tail_ok=False)
     nvec = _ceil_div(C, V)
     isz = max([t.dtype.itemsize for t in prog.tensors if t.shape[1] > 1] + [1])
     words = _words_per_tile(prog, V, 0)

@@ -64,35 +64,71 @@ template <typename T, int V> struct __attribute__((aligned(sizeof(T) * V > 16 ? 
     T v[V];
 };
 
+// NW consecutive 32-bit words, 16 bytes per instruction; NT = streaming access
+// (non-temporal: the line is not kept in cache, for data touched once).
+// The access types claim byte alignment only: global memory takes 16-byte
+// instructions at any address (a tensor view that starts mid-row, rows whose
+// length is not a multiple of the vector), at the same speed as aligned ones
+// when the address happens to be aligned -- and 1.7x (fp32) to 2.9x (fp16) the
+// speed of element-wise accesses when it is not.
+typedef nh_u32 nh_u32x2 __attribute__((ext_vector_type(2)));
+typedef nh_u32 nh_u32x4 __attribute__((ext_vector_type(4)));
+typedef nh_u32 nh_u32_any __attribute__((aligned(1)));
+typedef nh_u32x2 nh_u32x2_any __attribute__((aligned(1)));
+typedef nh_u32x4 nh_u32x4_any __attribute__((aligned(1)));
+
+// (elements of a vector value are copied to scalars before any bit cast: a
+// bit cast applied directly to ``t.y`` reads ``t.x`` with this compiler)
 template <typename T, int V> NEON_DEV void nh_load_vec(const T* __restrict__ p, T (&raw)[V]) {
-    const nh_vec<T, V> t = *reinterpret_cast<const nh_vec<T, V>*>(p);
+    static_assert(sizeof(T) == 4, "word vectors only");
+    nh_u32 w[V];
+    if constexpr (V == 1) {
+        w[0] = *reinterpret_cast<const nh_u32_any*>(p);
+    } else if constexpr (V == 2) {
+        const nh_u32x2 t = *reinterpret_cast<const nh_u32x2_any*>(p);
+        w[0] = t.x; w[1] = t.y;
+    } else {
 #pragma unroll
-    for (int j = 0; j < V; ++j) raw[j] = t.v[j];
+        for (int i = 0; i < V; i += 4) {
+            const nh_u32x4 t = *reinterpret_cast<const nh_u32x4_any*>(p + i);
+            w[i] = t.x; w[i + 1] = t.y; w[i + 2] = t.z; w[i + 3] = t.w;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < V; ++j) raw[j] = __builtin_bit_cast(T, w[j]);
 }
 
 template <typename T, int V> NEON_DEV void nh_store_vec(T* p, const T (&raw)[V]) {
-    nh_vec<T, V> t;
+    static_assert(sizeof(T) == 4, "word vectors only");
+    nh_u32 w[V];
 #pragma unroll
-    for (int j = 0; j < V; ++j) t.v[j] = raw[j];
-    *reinterpret_cast<nh_vec<T, V>*>(p) = t;
+    for (int j = 0; j < V; ++j) w[j] = __builtin_bit_cast(nh_u32, raw[j]);
+    if constexpr (V == 1) {
+        *reinterpret_cast<nh_u32_any*>(p) = w[0];
+    } else if constexpr (V == 2) {
+        nh_u32x2 t; t.x = w[0]; t.y = w[1];
+        *reinterpret_cast<nh_u32x2_any*>(p) = t;
+    } else {
+#pragma unroll
+        for (int i = 0; i < V; i += 4) {
+            nh_u32x4 t; t.x = w[i]; t.y = w[i + 1]; t.z = w[i + 2]; t.w = w[i + 3];
+            *reinterpret_cast<nh_u32x4_any*>(p + i) = t;
+        }
+    }
 }
 
-// NW consecutive 32-bit words, 16 bytes per instruction; NT = streaming access
-// (non-temporal: the line is not kept in cache, for data touched once).
-typedef nh_u32 nh_u32x2 __attribute__((ext_vector_type(2)));
-typedef nh_u32 nh_u32x4 __attribute__((ext_vector_type(4)));
 template <int NW, bool NT> NEON_DEV void nh_load_words(const nh_u32* p, nh_u32 (&w)[NW]) {
     if constexpr (!NT) {
         nh_load_vec<nh_u32, NW>(p, w);
     } else if constexpr (NW == 1) {
-        w[0] = __builtin_nontemporal_load(p);
+        w[0] = __builtin_nontemporal_load(reinterpret_cast<const nh_u32_any*>(p));
     } else if constexpr (NW == 2) {
-        const nh_u32x2 t = __builtin_nontemporal_load(reinterpret_cast<const nh_u32x2*>(p));
+        const nh_u32x2 t = __builtin_nontemporal_load(reinterpret_cast<const nh_u32x2_any*>(p));
         w[0] = t.x; w[1] = t.y;
     } else {
 #pragma unroll
         for (int i = 0; i < NW; i += 4) {
-            const nh_u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const nh_u32x4*>(p + i));
+            const nh_u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const nh_u32x4_any*>(p + i));
             w[i] = t.x; w[i + 1] = t.y; w[i + 2] = t.z; w[i + 3] = t.w;
         }
     }
@@ -101,15 +137,15 @@ template <int NW, bool NT> NEON_DEV void nh_store_words(nh_u32* p, const nh_u32 
     if constexpr (!NT) {
         nh_store_vec<nh_u32, NW>(p, w);
     } else if constexpr (NW == 1) {
-        __builtin_nontemporal_store(w[0], p);
+        __builtin_nontemporal_store(w[0], reinterpret_cast<nh_u32_any*>(p));
     } else if constexpr (NW == 2) {
         nh_u32x2 t; t.x = w[0]; t.y = w[1];
-        __builtin_nontemporal_store(t, reinterpret_cast<nh_u32x2*>(p));
+        __builtin_nontemporal_store(t, reinterpret_cast<nh_u32x2_any*>(p));
     } else {
 #pragma unroll
         for (int i = 0; i < NW; i += 4) {
             nh_u32x4 t; t.x = w[i]; t.y = w[i + 1]; t.z = w[i + 2]; t.w = w[i + 3];
-            __builtin_nontemporal_store(t, reinterpret_cast<nh_u32x4*>(p + i));
+            __builtin_nontemporal_store(t, reinterpret_cast<nh_u32x4_any*>(p + i));
         }
     }
 }

@@ -572,3 +572,31 @@ def test_row_vectors_fetched_once_per_workgroup(pair, shape, dtype):
         got = call_func(f, hip, [x, row, row2, col])
         want = call_func(f, cpu, [x.astype(np.float32), row, row2.astype(np.float32), col])
         assert_close(got, want, rtol=RTOL32, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16, np.uint8, np.int32], ids=["f32", "f16", "u8", "i32"])
+@pytest.mark.parametrize("shape,lo,hi", [((67, 1001), 3, 2), ((300, 519), 1, 0), ((5, 40), 7, 9), ((1, 4099), 1, 1)])
+def test_views_that_start_mid_row_and_odd_row_lengths(pair, shape, lo, hi, dtype):
+    """16-byte accesses at addresses that are only element-aligned, with a
+    partial last tile in every row: bit-exact against the oracle"""
+    R, C = shape
+    rs = np.random.RandomState(C)
+    if np.dtype(dtype).kind == "f":
+        x = rs.uniform(-4, 4, shape).astype(dtype)
+        y = rs.uniform(-4, 4, shape).astype(dtype)
+    else:
+        x = rs.randint(0, 100, shape).astype(dtype)
+        y = rs.randint(0, 100, shape).astype(dtype)
+    res = []
+    for be in pair:
+        tx, ty = be.array(x, dtype=dtype), be.array(y, dtype=dtype)
+        out = be.zeros(shape, dtype=dtype)
+        out[:, lo:C - hi] = tx[:, lo:C - hi] * 2 + ty[:, lo:C - hi]
+        whole = be.empty(shape, dtype=np.float32)
+        if be is pair[0] and dtype == np.float16:
+            # the oracle would do this arithmetic in fp16; the device computes in fp32
+            tx, ty = be.array(x.astype(np.float32)), be.array(y.astype(np.float32))
+        whole[:] = tx * 0.5 - ty
+        res.append((out.get(), whole.get()))
+    assert np.array_equal(res[1][0], res[0][0])
+    assert_close(res[1][1], res[0][1], rtol=RTOL32, atol=1e-6)
