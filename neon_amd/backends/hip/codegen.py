@@ -192,7 +192,17 @@ class _Gen(object):
         name = target or self.tile_name(n, sfx)
         if declare:
             self.L("%s %s;" % (self.tile_type(n, V), name))
-        self.L("%s.%s(%s);" % (name, self.ld, self.tile_addr(n, r, c)))
+        self.L("%s.%s(%s);" % (name, self.load_op(n), self.tile_addr(n, r, c)))
+
+    def load_op(self, n):
+        """streaming (non-temporal) loads are for data touched once: operands
+        that are broadcast along an axis are re-read by many workgroups and
+        stay on ordinary loads"""
+        t = self.prog.tensors[n.slot]
+        if self.ld == "load_stream" and n.kind == "T" and (
+                (t.shape[0] == 1 and self.R > 1) or (t.shape[1] == 1 and self.C > 1)):
+            return "load"
+        return self.ld
 
     # -- expressions -----------------------------------------------------------------
     def leaf_value(self, n, tile, r, c, V):

@@ -328,7 +328,11 @@ def _plan_ew(prog, cu_count):
         LX = min(256, _pow2ceil(nvec))
         LY = 256 // LX
         UC = 1
-        UR = max(1, min(4, R // (LY * 8)))
+        # rows per lane: several for cache-resident inputs (fewer workgroups to
+        # start), one when streaming from HBM (bias add over (4096,65536): 357 us
+        # with four rows per lane, 334 us with one -- as for the flat kernels,
+        # more loads in flight per lane only add read/write turnarounds)
+        UR = 1 if _streams(prog) else max(1, min(4, R // (LY * 8)))
     # one pass over far more data than the caches hold: streaming accesses
     stream = _streams(prog)
     tail = (C % V) != 0
