@@ -1230,7 +1230,13 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
                         NRED=len(all_reds), kept=len(kept), over=len(over)))
 
 
+# (more chunks do not help tall narrow matrices: the one workgroup per strip that
+# folds the partials becomes the bottleneck -- (200704,128) fp32 with 384 chunks
+# 28 us, with 128 chunks 24 us)
 COLSPLIT_MAX_CHUNKS = 128
+
+
+COLSPLIT_FOLD_BATCH = 8
 
 
 COLSPLIT_ROWS_IN_FLIGHT = 4
@@ -1337,12 +1343,19 @@ def gen_colsplit(prog, V, LX, LY, stream=False):
     L.close()
     L("__syncthreads();")
     L("if (!s_last) return;")
-    QMAX = -(-COLSPLIT_MAX_CHUNKS // LY)
+    # the last workgroup folds the strip's partials: row-lane ty takes chunks
+    # ty, ty + LY, ..., QB of them in flight at a time
+    QB = COLSPLIT_FOLD_BATCH
     for n in reds:
-        L("nh_pair q%d[%d][%d];" % (n.nid, QMAX, V))
+        op = _RED_OP[n.op]
+        L("#pragma unroll")
+        L("for (int j = 0; j < %d; ++j) acc%d[j] = %s::init();" % (V, n.nid, op))
+    L.open("for (int kb = 0; kb * %d < nchunks; kb += %d)" % (LY, QB))
+    for n in reds:
+        L("nh_pair q%d[%d][%d];" % (n.nid, QB, V))
     L("#pragma unroll")
-    L.open("for (int k = 0; k < %d; ++k)" % QMAX)
-    L("const int q = ty + k * %d;" % LY)
+    L.open("for (int k = 0; k < %d; ++k)" % QB)
+    L("const int q = ty + (kb + k) * %d;" % LY)
     L("const bool live = col_ok && (q < nchunks);")
     L("#pragma unroll")
     L.open("for (int j = 0; j < %d; ++j)" % V)
@@ -1352,12 +1365,8 @@ def gen_colsplit(prog, V, LX, LY, stream=False):
         L("q%d[k][j] = live ? nh_part_load(&part%d[(long long)q * C + c + j]) : %s;" % (n.nid, n.nid, init))
     L.close()
     L.close()
-    for n in reds:
-        op = _RED_OP[n.op]
-        L("#pragma unroll")
-        L("for (int j = 0; j < %d; ++j) acc%d[j] = %s::init();" % (V, n.nid, op))
     L("#pragma unroll")
-    L.open("for (int k = 0; k < %d; ++k)" % QMAX)
+    L.open("for (int k = 0; k < %d; ++k)" % QB)
     L("#pragma unroll")
     L.open("for (int j = 0; j < %d; ++j)" % V)
     for n in reds:
@@ -1366,6 +1375,7 @@ def gen_colsplit(prog, V, LX, LY, stream=False):
             L("acc%d[j] = %s::f(acc%d[j], q%d[k][j]);" % (n.nid, op, n.nid, n.nid))
         else:
             L("acc%d[j] = %s::f(acc%d[j], q%d[k][j].v);" % (n.nid, op, n.nid, n.nid))
+    L.close()
     L.close()
     L.close()
     for n in reds:
