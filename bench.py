@@ -333,20 +333,21 @@ def next_rows(be, rows):
         rt.event_sync(e1)
         add(label, rt.event_elapsed_ms(e0, e1) / reps, nbytes, plan, flops=flops)
 
-    # batch norm over (256 feature maps, 100352 = N*H*W) fp16, as one fused kernel each way
-    K, N = 256, 100352
-    x = _fresh(be, (K, N), dtype=f16, rs=rs, scale=2.0, shift=0.5)
-    y = be.empty((K, N), dtype=f16)
-    vec = lambda fill: _fresh(be, (K, 1), fill=fill)
-    xsum, xvar, gmean, gvar, gamma, beta = vec(0.0), vec(0.0), vec(0.0), vec(1.0), vec(1.0), vec(0.0)
-    trees("BN fprop fused (256,100352) f16", lambda: be.compound_fprop_bn(
-        x, xsum, xvar, gmean, gvar, gamma, beta, y, 1e-5, 0.9, True), 2 * K * N * 2)
-    delta = _fresh(be, (K, N), dtype=f16, rs=rs, scale=0.1)
-    dout = be.empty((K, N), dtype=f16)
-    gg, gb = vec(0.0), vec(0.0)
-    trees("BN bprop fused (256,100352) f16", lambda: be.compound_bprop_bn(
-        dout, gg, gb, delta, x, xsum, xvar, gamma, 1e-5), 3 * K * N * 2)
-    del x, y, delta, dout
+    # batch norm over (256 feature maps, 100352 = N*H*W) fp16, as one fused kernel each way;
+    # then the same bytes as 64 feature maps (an early convolution): four workgroups per row
+    for K, N in ((256, 100352), (64, 401408)):
+        x = _fresh(be, (K, N), dtype=f16, rs=rs, scale=2.0, shift=0.5)
+        y = be.empty((K, N), dtype=f16)
+        vec = lambda fill: _fresh(be, (K, 1), fill=fill)
+        xsum, xvar, gmean, gvar, gamma, beta = vec(0.0), vec(0.0), vec(0.0), vec(1.0), vec(1.0), vec(0.0)
+        trees("BN fprop fused (%d,%d) f16" % (K, N), lambda: be.compound_fprop_bn(
+            x, xsum, xvar, gmean, gvar, gamma, beta, y, 1e-5, 0.9, True), 2 * K * N * 2)
+        delta = _fresh(be, (K, N), dtype=f16, rs=rs, scale=0.1)
+        dout = be.empty((K, N), dtype=f16)
+        gg, gb = vec(0.0), vec(0.0)
+        trees("BN bprop fused (%d,%d) f16" % (K, N), lambda: be.compound_bprop_bn(
+            dout, gg, gb, delta, x, xsum, xvar, gamma, 1e-5), 3 * K * N * 2)
+        del x, y, delta, dout
 
     # random numbers and rounding on the Adam shape
     shape = (5000, 5000)

@@ -559,7 +559,7 @@ class _RedGen(_Gen):
 # =====================================================================================
 # family: row  (axis 1)
 # =====================================================================================
-def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None):
+def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1):
     """Axis-1 reductions.  A team of LX lanes (a power of two up to 64, or the
     whole workgroup) owns one row; the workgroup holds LY rows.  A lane visits
     column tiles tx, tx+LX, ...; with ``NCH`` > 0 that loop has a fixed trip
@@ -570,15 +570,28 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None):
     resident tiles may take: operands are made resident in order of first use
     while they fit, the others are fetched again, a few tiles at a time, in
     every sweep that reads them (batch-norm backward keeps ``x`` and re-reads
-    the deltas: four passes over HBM instead of five)."""
+    the deltas: four passes over HBM instead of five).
+
+    ``chunks`` > 1 (family ``rowcoop``; whole-workgroup rows with ``NCH`` > 0
+    only): few, very long rows.  grid = (rows, chunks); workgroup (r, q) owns
+    tiles q*NCH ... q*NCH+NCH-1 of row r, and the ``chunks`` workgroups of a row
+    -- all resident at once, the planner keeps the grid within one workgroup
+    per compute unit -- exchange their partial results after every sweep
+    through device-coherent memory: publish, count arrivals on the row's
+    counter, wait (bounded), gather and fold.  Extra parameters: workspace
+    pointer and the byte offset of the counters (two per row: arrivals,
+    departures; zero before the first launch, reset by the last workgroup to
+    leave)."""
     g = _RedGen(prog, V, stream, "row")
     L = g.L
     T = LX * LY
     assert LX <= 64 or LY == 1
     resident = NCH > 0
+    coop = chunks > 1
+    assert not coop or (resident and LY == 1 and T % 64 == 0 and chunks <= T)
     words_left = [keep_words]       # None: everything is kept
     transient = set()               # nids of row operands that are not kept
-    params, fmt = g.param_list([])
+    params, fmt = g.param_list([("char* ws", "P"), ("long long ctr_offset", "q")] if coop else [])
     head = ('extern "C" __global__ __launch_bounds__(%d) void @NAME@(%s)\n' % (T, params))
     per_level = _levels(prog)
     nsweeps = prog.nlevels
@@ -597,13 +610,62 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None):
     L("const long long rr = row_ok ? r : 0;")   # address clamp for idle teams
     if not resident:
         L("const int nch = (C + %d - 1) / %d;" % (LX * V, LX * V))
+    all_reds = [n for lv in sorted(per_level) for n in per_level[lv]]
+    red_slot = dict((n.nid, k) for k, n in enumerate(all_reds))
+    exchanges = [0]
+    if coop:
+        L("__shared__ int s_abort;")
+        L("unsigned int* ctr = reinterpret_cast<unsigned int*>(ws + ctr_offset) + 2 * blockIdx.x;")
+        L("nh_pair* part = reinterpret_cast<nh_pair*>(ws) + (long long)blockIdx.x * %d;" % (len(all_reds) * chunks))
 
     SU = 4      # column tiles in flight per lane when the row is streamed
     NCHP = -(-NCH // SU) * SU
 
     def chunk_position(k):
-        L("const long long c = ((long long)(%s) * %d + tx) * %d;" % (k, LX, V))
-        L("const bool ok = row_ok && (c < C);")
+        if coop:
+            # (batch loops may run k past NCH: those tiles belong to the next workgroup)
+            L("const long long c = (((long long)blockIdx.y * %d + (%s)) * %d + tx) * %d;" % (NCH, k, LX, V))
+            L("const bool ok = row_ok && (c < C) && ((%s) < %d);" % (k, NCH))
+        else:
+            L("const long long c = ((long long)(%s) * %d + tx) * %d;" % (k, LX, V))
+            L("const bool ok = row_ok && (c < C);")
+
+    def exchange(reds):
+        """join the workgroups of a row: red<id> of every reduction of this
+        sweep becomes the result over the whole row, in every lane of every
+        workgroup"""
+        exchanges[0] += 1
+        L.open("if (threadIdx.x == 0)")
+        for n in reds:
+            val = ("red%d" % n.nid) if n.is_index else ("nh_pair{red%d, 0}" % n.nid)
+            L("nh_part_store(&part[%d + blockIdx.y], %s);" % (red_slot[n.nid] * chunks, val))
+        L.close()
+        L("__syncthreads();     // the partial stores have completed")
+        L.open("if (threadIdx.x == 0)")
+        L("__hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
+        L("unsigned int spins = 0; int bad = 0;")
+        L.open("while (__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < %du)" % (chunks * exchanges[0]))
+        L("__builtin_amdgcn_s_sleep(4);")
+        L("if (++spins > NH_SPIN_LIMIT) { bad = 1; break; }")
+        L.close()
+        L("s_abort = bad;")
+        L.close()
+        L("__syncthreads();")
+        L.open("if (s_abort)")
+        L("if (threadIdx.x == 0) __hip_atomic_store(ctr + 1, 0xDEADu, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
+        L("return;              // the other workgroups never showed up: give up rather than hang")
+        L.close()
+        for n in reds:
+            op = _RED_OP[n.op]
+            init = ("%s::init()" % op) if n.is_index else ("nh_pair{%s::init(), 0}" % op)
+            L("const nh_pair g%d = (threadIdx.x < %d) ? nh_part_load(&part[%d + threadIdx.x]) : %s;"
+              % (n.nid, chunks, red_slot[n.nid] * chunks, init))
+        for n in reds:
+            op = _RED_OP[n.op]
+            if n.is_index:
+                L("red%d = nh_block_allreduce<%s, %d, nh_pair>(g%d, s_p);" % (n.nid, op, T // 64, n.nid))
+            else:
+                L("red%d = nh_block_allreduce<%s, %d, float>(g%d.v, s_f);" % (n.nid, op, T // 64, n.nid))
 
     def sweep(leaves, emit_body):
         """Loop over the lane's column tiles.  All loads of a batch of tiles
@@ -761,11 +823,15 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None):
         for n in reds:
             op = _RED_OP[n.op]
             ty_ = "nh_pair" if n.is_index else "float"
+            const = "" if coop else "const "
             if LX <= 64:
-                L("const %s red%d = nh_wave_allreduce<%s, %d, %s>(acc%d);" % (ty_, n.nid, op, LX, ty_, n.nid))
+                L("%s%s red%d = nh_wave_allreduce<%s, %d, %s>(acc%d);" % (const, ty_, n.nid, op, LX, ty_, n.nid))
             else:
-                L("const %s red%d = nh_block_allreduce<%s, %d, %s>(acc%d, %s);"
-                  % (ty_, n.nid, op, T // 64, ty_, n.nid, "s_p" if n.is_index else "s_f"))
+                L("%s%s red%d = nh_block_allreduce<%s, %d, %s>(acc%d, %s);"
+                  % (const, ty_, n.nid, op, T // 64, ty_, n.nid, "s_p" if n.is_index else "s_f"))
+        if coop:
+            exchange(reds)
+        for n in reds:
             if n.is_index:
                 L("const int ri%d = red%d.i;" % (n.nid, n.nid))
             else:
@@ -777,7 +843,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None):
         roots = [st.root for st in line_out]
         nodes = _needed(roots, done)
         leaves = g.leaf_nodes(nodes)
-        L.open("if (row_ok && tx == 0)")
+        L.open("if (row_ok && tx == 0%s)" % (" && blockIdx.y == 0" if coop else ""))
         for n in leaves:
             g.emit_load(n, "r", "0", 1, "_l")
         L.open("")
@@ -821,9 +887,20 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None):
             L.close()
 
         sweep(leaves, store_body)
+    if coop:
+        # the last workgroup of the row to get here has seen everyone pass the
+        # final wait: it re-arms both counters for the next launch
+        L.open("if (threadIdx.x == 0)")
+        L("const unsigned int t = __hip_atomic_fetch_add(ctr + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
+        L.open("if (t == %du)" % (chunks - 1))
+        L("__hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
+        L("__hip_atomic_store(ctr + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
+        L.close()
+        L.close()
     L.close()
-    return _finish("row", g, head, fmt, T, 0, dict(V=V, LX=LX, LY=LY, NCH=NCH, stream=bool(stream),
-                                                   passing=len(transient), over=len(vals)))
+    return _finish("rowcoop" if coop else "row", g, head, fmt, T, 0,
+                   dict(V=V, LX=LX, LY=LY, NCH=NCH, stream=bool(stream), passing=len(transient),
+                        over=len(vals), chunks=chunks, NRED=len(all_reds)))
 
 
 # =====================================================================================

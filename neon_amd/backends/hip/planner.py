@@ -373,6 +373,24 @@ def _plan_row(prog, cu_count):
                         for t in prog.tensors if t.read and t.shape[1] > 1] or [1 << 30])
         if nch <= 16 and nch * smallest <= 64:
             LX, T, NCH, keep_words = 1024, 1024, nch, 64
+    # Few, very long rows (batch norm over the 64 feature maps of an early
+    # convolution): one workgroup per row would leave most compute units idle
+    # and the row may not fit its registers.  Spread every row over several
+    # workgroups that exchange their partial results; all of them must be
+    # resident at once, so rows x chunks stays within the compute units.
+    tiles = _ceil_div(nvec, 1024)
+    if R * 2 <= cu_count and tiles >= 8 and prog.nlevels >= 1:
+        chunks = min(cu_count // R, tiles // 4, 64)
+        per = _ceil_div(tiles, chunks)
+        chunks = _ceil_div(tiles, per)
+        smallest = min([max(1, (V * t.dtype.itemsize + 3) // 4)
+                        for t in prog.tensors if t.read and t.shape[1] > 1] or [1 << 30])
+        if chunks >= 2 and per <= 16 and per * smallest <= 64:
+            kw = None if per * words <= 64 else 64
+            spec = codegen.gen_row(prog, V, 1024, 1, per, _streams(prog), keep_words=kw, chunks=chunks)
+            part_bytes = R * spec.params["NRED"] * chunks * 8
+            ctr_off = _ceil_div(part_bytes, 256) * 256
+            return Choice(spec, (R, chunks, 1), workspace=(ctr_off + R * 8, ctr_off, 2 * R))
     LY = T // LX
     spec = codegen.gen_row(prog, V, LX, LY, NCH, _streams(prog), keep_words=keep_words)
     gx = _ceil_div(R, LY)

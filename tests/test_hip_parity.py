@@ -600,3 +600,31 @@ def test_views_that_start_mid_row_and_odd_row_lengths(pair, shape, lo, hi, dtype
         res.append((out.get(), whole.get()))
     assert np.array_equal(res[1][0], res[0][0])
     assert_close(res[1][1], res[0][1], rtol=RTOL32, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
+@pytest.mark.parametrize("shape", [(8, 70000), (3, 200003 * 8), (64, 131072), (1, 1 << 20)])
+def test_few_very_long_rows(pair, shape, dtype):
+    """axis-1 trees over few, very long rows: each row is spread over several
+    workgroups that exchange partials after every sweep.  Twice each: the
+    arrival counters must re-arm."""
+    R, C = shape
+    rs = np.random.RandomState(R)
+    x = (rs.standard_normal(shape) * 2 + 0.5).astype(dtype)
+    x32 = x.astype(np.float32)
+    cpu, hip = pair
+    x64 = x.astype(np.float64)
+    e64 = np.exp(x64 - x64.max(axis=1, keepdims=True))
+    cases = [("x - mean", lambda be, a: a - be.mean(a, axis=1), x64 - x64.mean(axis=1, keepdims=True), 2e-5),
+             ("softmax", lambda be, a: be.fprop_softmax(a, 1), e64 / e64.sum(axis=1, keepdims=True), 2e-5),
+             ("std", lambda be, a: be.sqrt(be.var(a, axis=1)), x64.std(axis=1, keepdims=True), 2e-5),
+             ("sum", lambda be, a: be.sum(a, axis=1), x64.sum(axis=1, keepdims=True), 1e-5)]
+    for what, f, truth, rtol in cases:
+        for rep in range(2):
+            got = call_func(f, hip, [x])
+            scale = np.abs(truth).max()
+            assert np.abs(got - truth).max() <= rtol * scale + 1e-6 * np.sqrt(C), (what, rep)
+    got = call_func(lambda be, a: be.argmax(a, axis=1), hip, [x], out_dtype=np.int32)
+    assert np.array_equal(got.ravel(), np.argmax(x32, axis=1))
+    got = call_func(lambda be, a: be.max(a, axis=1) - be.min(a, axis=1), hip, [x])
+    assert np.array_equal(got.ravel(), x32.max(axis=1) - x32.min(axis=1))

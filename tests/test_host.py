@@ -328,8 +328,14 @@ def test_row_softmax_reuses_registers_when_the_row_is_resident(pb):
     spec = plan_of(pb, lambda: out.__setitem__(slice(None), softmax(x))).spec
     assert spec.family == "row" and spec.params["NCH"] > 0 and spec.params["over"] == 1
     assert spec.source.count("expf(") == 1
-    # a row too long for the registers is streamed in every sweep: nothing to reuse
+    # few rows too long for one workgroup's registers are spread over several
+    # workgroups and stay resident
     xl, outl = pb.empty((16, 1 << 20)), pb.empty((16, 1 << 20))
+    ch = plan_of(pb, lambda: outl.__setitem__(slice(None), softmax(xl)))
+    assert ch.spec.family == "rowcoop" and ch.grid == (16, 16, 1) and ch.spec.params["over"] == 1
+    assert ch.spec.source.count("expf(") == 1
+    # many such rows are streamed in every sweep: nothing to reuse
+    xl, outl = pb.empty((512, 1 << 20)), pb.empty((512, 1 << 20))
     spec = plan_of(pb, lambda: outl.__setitem__(slice(None), softmax(xl))).spec
     assert spec.family == "row" and spec.params["NCH"] == 0 and spec.params["over"] == 0
     assert spec.source.count("expf(") == 2
