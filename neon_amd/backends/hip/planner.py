@@ -488,15 +488,24 @@ def _plan_col(prog, cu_count):
 
     # (b) one level, one value per column, many rows: split rows over workgroups
     if single_level and line_only:
-        LX = max(lx_min, min(16, _pow2ceil(nvec)))
-        LY = COLSPLIT_THREADS // LX
-        strips = _ceil_div(nvec, LX)
         # Workgroups are cheap to run but not free to start: give each one at
         # least ~128 KiB to stream, one per compute unit for small inputs and
         # up to eight for large ones.
         bytes_total = R * C * isz
         per_cu = max(1, min(8, bytes_total // (cu_count * (128 << 10))))
         target = per_cu * cu_count
+        # 16 column-lanes per strip; 8 when the chunk limit would leave fewer than
+        # two workgroups per compute unit, or when the input is small enough that
+        # the last workgroup's fold of the partials shows (fewer, longer chunks).
+        # Measured: (200704,128) fp32 23 -> 21 us, fp16 26 -> 18 us, (32000,256)
+        # fp32 10.1 -> 9.3 us; (200704,256) fp32 already has 512 workgroups with
+        # 16 lanes and loses with 8 (36 us against 44 us).
+        LX = max(lx_min, min(16, _pow2ceil(nvec)))
+        if LX == 16 and (per_cu == 1 or
+                         _ceil_div(nvec, LX) * codegen.COLSPLIT_MAX_CHUNKS < min(target, 2 * cu_count)):
+            LX = max(lx_min, 8)
+        LY = COLSPLIT_THREADS // LX
+        strips = _ceil_div(nvec, LX)
         chunks = max(1, min(codegen.COLSPLIT_MAX_CHUNKS, target // strips))
         rpc = max(codegen.COLSPLIT_ROWS_IN_FLIGHT * LY, _ceil_div(R, chunks))
         rpc = _ceil_div(rpc, LY) * LY
