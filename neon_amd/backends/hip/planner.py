@@ -506,7 +506,13 @@ def _plan_col(prog, cu_count):
             LX = max(lx_min, 8)
         LY = COLSPLIT_THREADS // LX
         strips = _ceil_div(nvec, LX)
-        chunks = max(1, min(codegen.COLSPLIT_MAX_CHUNKS, target // strips))
+        # (the limit bounds what the last workgroup of a strip has to fold; strips
+        # under 64 columns may take more chunks, as far as it takes to get two
+        # workgroups per compute unit: (802816,32) fp32 34 -> 23 us)
+        cap = codegen.COLSPLIT_MAX_CHUNKS
+        wide_cap = cap * max(1, 64 // (LX * V))
+        cap = max(cap, min(wide_cap, _ceil_div(2 * cu_count, strips)))
+        chunks = max(1, min(cap, target // strips))
         rpc = max(codegen.COLSPLIT_ROWS_IN_FLIGHT * LY, _ceil_div(R, chunks))
         rpc = _ceil_div(rpc, LY) * LY
         chunks = _ceil_div(R, rpc)
