@@ -1,0 +1,101 @@
+"""Random op-trees on the hip backend against the numpy oracle (GPU box).
+
+Seeded, so every run sees the same trees: shapes from a list that mixes
+vector-friendly and odd extents, operands that are full, row, column or 1x1
+tensors (a third of the full ones views into larger tensors, offset in both
+directions), fp32 and fp16 storage, up to three levels of unary / binary
+operators with reductions along one axis nested up to three deep.  A second set
+uses extents up to 150000 so that the cooperative and split families run."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+SMALL = [1, 2, 3, 7, 16, 33, 64, 100, 257, 1000, 1031, 4099]
+LARGE = [1, 2, 5, 16, 40, 128, 256, 1000, 8192, 20000, 40003, 150000]
+
+
+def _case(rs, dims, limit):
+    R, C = int(rs.choice(dims)), int(rs.choice(dims))
+    if R * C > limit:
+        if rs.rand() < 0.5:
+            C = max(1, limit // R)
+        else:
+            R = max(1, limit // C)
+    dtype = rs.choice([np.float32, np.float32, np.float32, np.float16])
+    leaves = []
+    for k in range(rs.randint(1, 4)):
+        kind = "full" if k == 0 else rs.choice(["full", "full", "col", "row", "one"])
+        shp = {"full": (R, C), "col": (R, 1), "row": (1, C), "one": (1, 1)}[kind]
+        leaves.append(rs.uniform(-2, 2, shp).astype(dtype if shp == (R, C) else np.float32))
+    axis = int(rs.randint(0, 2))
+
+    def expr(be, ts, depth, allow_red):
+        r = rs.rand()
+        if depth == 0 or r < 0.25:
+            if rs.rand() < 0.15:
+                return float(np.round(rs.uniform(-2, 2), 3))
+            return ts[rs.randint(len(ts))]
+        if r < 0.5:
+            a = expr(be, ts, depth - 1, allow_red)
+            op = rs.choice(["neg", "abs", "sqrtabs", "tanh", "sig", "square", "expclip"])
+            if isinstance(a, float):
+                a = ts[0] * a
+            return {"neg": lambda: -a, "abs": lambda: be.absolute(a), "sqrtabs": lambda: be.sqrt(be.absolute(a)),
+                    "tanh": lambda: be.tanh(a), "sig": lambda: be.sig(a), "square": lambda: be.square(a),
+                    "expclip": lambda: be.exp(be.minimum(a, 3.0))}[op]()
+        if r < 0.85 or not allow_red:
+            a, b = expr(be, ts, depth - 1, allow_red), expr(be, ts, depth - 1, allow_red)
+            if isinstance(a, float) and isinstance(b, float):
+                a = ts[0]
+            op = rs.choice(["add", "sub", "mul", "max", "min", "div", "gt", "le"])
+            if op == "div":
+                return a / ((be.absolute(b) if not isinstance(b, float) else abs(b)) + 1.0)
+            return {"add": lambda: a + b, "sub": lambda: a - b, "mul": lambda: a * b,
+                    "max": lambda: be.maximum(a, b), "min": lambda: be.minimum(a, b),
+                    "gt": lambda: be.greater(a, b) * 1.0, "le": lambda: be.less_equal(a, b) * 1.0}[op]()
+        a = expr(be, ts, depth - 1, True)
+        if isinstance(a, float):
+            a = ts[0] * a
+        return getattr(be, rs.choice(["sum", "max", "min", "mean"]))(a, axis=axis)
+    return R, C, leaves, axis, expr
+
+
+def _run(be, seed, dims, limit, oracle):
+    rs = np.random.RandomState(seed)
+    R, C, leaves, axis, expr = _case(rs, dims, limit)
+    ts = []
+    for leaf in leaves:
+        host = leaf.astype(np.float32) if oracle else leaf          # the oracle computes in fp32 on exact copies
+        if leaf.shape == (R, C) and rs.rand() < 0.3 and R > 1 and C > 1:
+            pr, pc = int(rs.randint(0, 3)), int(rs.randint(0, 4))
+            big = np.zeros((R + pr + 1, C + pc + 2), host.dtype)
+            big[pr:pr + R, pc:pc + C] = host
+            ts.append(be.array(big, dtype=big.dtype)[pr:pr + R, pc:pc + C])
+        else:
+            ts.append(be.array(host, dtype=host.dtype))
+    tree = expr(be, ts, 3, True)
+    if isinstance(tree, float):
+        tree = ts[0] + tree
+    out = be.empty(tree.shape, dtype=np.float32)
+    out[:] = tree
+    return (R, C, axis), out.get()
+
+
+@pytest.mark.parametrize("first,count,dims,limit", [(1000, 120, SMALL, 2000000), (5000, 40, LARGE, 30000000)],
+                         ids=["small", "large"])
+def test_random_trees_match_the_oracle(pair, first, count, dims, limit):
+    cpu, hip = pair
+    for seed in range(first, first + count):
+        (R, C, axis), want = _run(cpu, seed, dims, limit, True)
+        _, got = _run(hip, seed, dims, limit, False)
+        assert got.shape == want.shape, seed
+        w64 = want.astype(np.float64)
+        finite = np.isfinite(w64)
+        assert np.array_equal(finite, np.isfinite(got)), seed
+        scale = max(1.0, np.abs(w64[finite]).max() if finite.any() else 1.0)
+        err = np.abs(got.astype(np.float64) - w64)
+        err[~finite] = 0
+        # the reductions add up to R or C terms in a different order on the device
+        tol = 3e-6 * max(8, R if axis == 0 else C)
+        assert err.max() / scale <= tol, (seed, R, C, axis, err.max() / scale)
