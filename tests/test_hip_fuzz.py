@@ -99,3 +99,42 @@ def test_random_trees_match_the_oracle(pair, first, count, dims, limit):
         # the reductions add up to R or C terms in a different order on the device
         tol = 3e-6 * max(8, R if axis == 0 else C)
         assert err.max() / scale <= tol, (seed, R, C, axis, err.max() / scale)
+
+
+def _flat_expr(be, rs, ts, depth):
+    r = rs.rand()
+    if depth == 0 or r < 0.3:
+        return ts[rs.randint(len(ts))] if rs.rand() < 0.85 else float(np.round(rs.uniform(-1, 1), 2))
+    a, b = _flat_expr(be, rs, ts, depth - 1), _flat_expr(be, rs, ts, depth - 1)
+    if isinstance(a, float) and isinstance(b, float):
+        a = ts[0]
+    op = rs.choice(["add", "sub", "mul", "max", "root", "div"])
+    if op == "root":
+        return be.sqrt(be.absolute(b if isinstance(a, float) else a))
+    if op == "div":
+        return a / ((be.absolute(b) if not isinstance(b, float) else abs(b)) + 1.0)
+    return {"add": lambda: a + b, "sub": lambda: a - b, "mul": lambda: a * b,
+            "max": lambda: be.maximum(a, b)}[op]()
+
+
+def test_random_fused_statement_groups_match_the_oracle(pair):
+    """two to four assigns into four tensors between begin / end: one kernel on
+    the device, statement after statement on the oracle; later statements read
+    what earlier ones wrote"""
+    from neon_amd.backends.backend import Block
+    cpu, hip = pair
+    for seed in range(100):
+        res = []
+        for be in (cpu, hip):
+            rs = np.random.RandomState(seed)
+            shape = [(64, 100), (1000, 33), (1, 5000), (257, 257), (4096, 128)][rs.randint(5)]
+            ts = [be.array(rs.uniform(-2, 2, shape).astype(np.float32)) for _ in range(4)]
+            be.begin(Block.update, 0)
+            for _ in range(rs.randint(2, 5)):
+                target = ts[rs.randint(len(ts))]
+                e = _flat_expr(be, rs, ts, 2)
+                target[:] = ts[0] * e if isinstance(e, float) else e
+            be.end(Block.update, 0)
+            res.append([t.get() for t in ts])
+        for want, got in zip(*res):
+            assert np.allclose(got, want, rtol=2e-5, atol=2e-5), seed
