@@ -762,6 +762,37 @@ class Backend(metaclass=_BackendRegistry):
     def bprop_skipnode(self, error, deltas, alpha, beta):
         deltas[:] = deltas * beta + alpha * error
 
+    # -- small aliases and hooks of the reference's base class (backend.py:627-650,
+    #    808-823, 907-921, 1539-1557) ---------------------------------------------
+    def true_divide(self, a, b, out=None):
+        return OpTreeNode.build("div", a, b, out=out)
+
+    def fabs(self, a, out=None):
+        return OpTreeNode.build("abs", a, None, out=out)
+
+    def update_fc_bias(self, err, out):
+        """bias gradient of a fully connected layer: row sums of the error"""
+        self.sum(err, axis=1, out=out)
+
+    def add_fc_bias(self, inputs, bias):
+        """add one bias value per row, in place"""
+        self.add(inputs, bias, out=inputs)
+
+    def is_mkl(self):
+        return False
+
+    def convert_data(self, tensor, layer_mkl):
+        return None
+
+    def clean_data(self, tensor, layer_mkl):
+        return None
+
+    def allocate_new_deltas(self, delta, in_shape, parallelism):
+        return delta
+
+    def allocate_new_outputs(self, layer, share_output):
+        layer.allocate(shared_outputs=share_output)
+
     # -- layer bookkeeping the reference's containers call on any backend: no
     #    backend-side state here, the merges just drive their branches with the
     #    right accumulate flags (reference nervanagpu.py:3179-3231) ---------------

@@ -290,3 +290,21 @@ def test_merge_helpers_drive_branches_with_the_right_accumulation(cpu):
     assert betas[-1] == 3.0
     want = [1.0 + 2.0 * x.get(), 0.0 + 2.0 * x.get(), 3.0 + 2.0 * x.get()]
     assert all(np.array_equal(dk.get(), w) for dk, w in zip(d, want))
+
+
+def test_small_aliases_of_the_backend_base(cpu):
+    be = cpu
+    x = be.array(np.array([[1.0, -2.0, 4.0], [-8.0, 16.0, -32.0]], np.float32))
+    out = be.empty((2, 3))
+    be.fabs(x, out=out)
+    assert np.array_equal(out.get(), np.abs(x.get()))
+    be.true_divide(x, 2.0, out=out)
+    assert np.array_equal(out.get(), x.get() / 2)
+    bias = be.array(np.array([[10.0], [20.0]], np.float32))
+    grad = be.empty((2, 1))
+    be.update_fc_bias(x, grad)
+    assert np.array_equal(grad.get(), x.get().sum(axis=1, keepdims=True))
+    be.add_fc_bias(x, bias)
+    assert np.array_equal(x.get(), np.array([[11.0, 8.0, 14.0], [12.0, 36.0, -12.0]], np.float32))
+    assert be.is_mkl() is False and be.convert_data(x, False) is None and be.clean_data(x, False) is None
+    assert be.allocate_new_deltas(x, (2, 3), "Data") is x
