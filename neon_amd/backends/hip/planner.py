@@ -155,6 +155,10 @@ def _vector_width(prog, tail_ok):
         V //= 2
     if C < V:
         V = 1 if not tail_ok else max(1, _pow2floor(C))
+    # a lane's tile is held in whole 32-bit words: narrower vectors of 1- and
+    # 2-byte elements do not exist
+    while V > 1 and any((V * t.dtype.itemsize) % 4 for t in cols):
+        V //= 2
     return V
 
 

@@ -628,3 +628,22 @@ def test_few_very_long_rows(pair, shape, dtype):
     assert np.array_equal(got.ravel(), np.argmax(x32, axis=1))
     got = call_func(lambda be, a: be.max(a, axis=1) - be.min(a, axis=1), hip, [x])
     assert np.array_equal(got.ravel(), x32.max(axis=1) - x32.min(axis=1))
+
+
+@pytest.mark.parametrize("dtype", [np.uint8, np.int8, np.float16, np.int16], ids=["u8", "i8", "f16", "i16"])
+@pytest.mark.parametrize("shape", [(5, 6), (9, 2), (4, 3), (33, 10), (7, 12)])
+def test_narrow_elements_with_short_rows(pair, shape, dtype):
+    """row lengths that leave no whole 32-bit word of 1- or 2-byte elements per
+    lane: element-wise tiles, in every family"""
+    rs = np.random.RandomState(shape[1])
+    x = rs.randint(0, 50, shape).astype(dtype)
+    res = []
+    for be in pair:
+        t = be.array(x if be is pair[1] else x.astype(np.float32), dtype=(dtype if be is pair[1] else np.float32))
+        e, c, r = be.empty(shape), be.empty((1, shape[1])), be.empty((shape[0], 1))
+        e[:] = t * 2 + 1
+        c[:] = be.sum(t, axis=0)
+        r[:] = be.max(t, axis=1) - be.min(t, axis=1)
+        res.append((e.get(), c.get(), r.get()))
+    for want, got in zip(*res):
+        assert np.array_equal(got, want)
