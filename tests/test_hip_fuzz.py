@@ -138,3 +138,39 @@ def test_random_fused_statement_groups_match_the_oracle(pair):
             res.append([t.get() for t in ts])
         for want, got in zip(*res):
             assert np.allclose(got, want, rtol=2e-5, atol=2e-5), seed
+
+
+def test_random_storage_types_and_small_extents(pair):
+    """every storage type on either operand, extents from 1 to 5000 (many of
+    them shorter than a vector): elementwise, both reduction axes, float and
+    int32 results"""
+    cpu, hip = pair
+    types = [np.uint8, np.int8, np.int16, np.uint16, np.int32, np.uint32, np.float16, np.float32]
+    dims = [1, 2, 3, 4, 5, 6, 7, 8, 9, 12, 15, 16, 17, 31, 33, 64, 100, 129, 1000, 1031, 5000]
+    for seed in range(160):
+        rs = np.random.RandomState(seed)
+        R, C = int(rs.choice(dims)), int(rs.choice(dims))
+        da, db = types[rs.randint(len(types))], types[rs.randint(len(types))]
+        a = rs.randint(0, 100, (R, C)).astype(da)
+        b = rs.randint(1, 50, (R, C)).astype(db)
+        kind = rs.randint(6)
+        res = []
+        for be in (cpu, hip):
+            if be is cpu:       # exact fp32 copies: numpy would do integer arithmetic on integer arrays
+                ta, tb = be.array(a.astype(np.float32)), be.array(b.astype(np.float32))
+            else:
+                ta, tb = be.array(a, dtype=da), be.array(b, dtype=db)
+            tree = [lambda: ta * 2 + tb, lambda: be.sum(ta * tb, axis=0), lambda: be.max(ta - tb, axis=1),
+                    lambda: ta - be.mean(ta, axis=1) + tb, lambda: be.maximum(ta, tb) - be.min(tb, axis=0),
+                    lambda: be.sum(ta, axis=1) + be.sum(tb, axis=1)][kind]()
+            out = be.empty(tree.shape)
+            out[:] = tree
+            ints = None
+            if kind != 3:       # integer-valued results also go into an int32 tensor
+                oi = be.empty(tree.shape, dtype=np.int32)
+                oi[:] = tree
+                ints = oi.get()
+            res.append((out.get(), ints))
+        (want, want_i), (got, got_i) = res
+        assert np.allclose(got, want, rtol=1e-5, atol=1e-3), (seed, R, C, da, db, kind)
+        assert want_i is None or np.array_equal(got_i, want_i), (seed, R, C, da, db, kind)
