@@ -559,7 +559,7 @@ class _RedGen(_Gen):
 # =====================================================================================
 # family: row  (axis 1)
 # =====================================================================================
-def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1):
+def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=False):
     """Axis-1 reductions.  A team of LX lanes (a power of two up to 64, or the
     whole workgroup) owns one row; the workgroup holds LY rows.  A lane visits
     column tiles tx, tx+LX, ...; with ``NCH`` > 0 that loop has a fixed trip
@@ -581,7 +581,11 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1):
     counter, wait (bounded), gather and fold.  Extra parameters: workspace
     pointer and the byte offset of the counters (two per row: arrivals,
     departures; zero before the first launch, reset by the last workgroup to
-    leave)."""
+    leave).
+
+    ``tail``: the row length is not a multiple of V; the last tile of a row is
+    loaded and stored element by element and only its valid elements enter
+    the reductions."""
     g = _RedGen(prog, V, stream, "row")
     L = g.L
     T = LX * LY
@@ -629,6 +633,16 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1):
         else:
             L("const long long c = ((long long)(%s) * %d + tx) * %d;" % (k, LX, V))
             L("const bool ok = row_ok && (c < C);")
+        if tail:
+            L("const bool full = c + %d <= C;" % V)
+            L("const int lim = full ? %d : (int)(C - c);" % V)
+
+    def tile_load(name, n):
+        addr = g.tile_addr(n, "rr", "c")
+        if tail and g.tile_width(n, V) > 1:
+            return ("if (ok && full) %s.%s(%s); else if (ok) %s.load_partial(%s, lim); else %s.zero();"
+                    % (name, g.ld, addr, name, addr, name))
+        return "if (ok) %s.%s(%s); else %s.zero();" % (name, g.ld, addr, name)
 
     def exchange(reds):
         """join the workgroups of a row: red<id> of every reduction of this
@@ -684,8 +698,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1):
                 chunk_position("k")
                 for n in fresh:
                     cached[n.nid] = "keep%d" % n.nid
-                    L("if (ok) keep%d[k].%s(%s); else keep%d[k].zero();"
-                      % (n.nid, g.ld, g.tile_addr(n, "rr", "c"), n.nid))
+                    L(tile_load("keep%d[k]" % n.nid, n))
                 L.close()
             passing = [n for n in moving if n.nid in transient]
             for n in moving:
@@ -709,8 +722,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1):
             L("const int k = kb + u;")
             chunk_position("k")         # k beyond the row: c >= C, so ok is false
             for n in passing:
-                L("if (ok) %s[u].%s(%s); else %s[u].zero();"
-                  % (g.tile_name(n, "_s"), g.ld, g.tile_addr(n, "rr", "c"), g.tile_name(n, "_s")))
+                L(tile_load("%s[u]" % g.tile_name(n, "_s"), n))
             L.close()
             L("#pragma unroll")
             L.open("for (int u = 0; u < %d; ++u)" % SU)
@@ -728,8 +740,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1):
         L.open("for (int u = 0; u < %d; ++u)" % SU)
         chunk_position("kb + u")
         for n in moving:
-            L("if (ok) %s[u].%s(%s); else %s[u].zero();"
-              % (g.tile_name(n, "_s"), g.ld, g.tile_addr(n, "rr", "c"), g.tile_name(n, "_s")))
+            L(tile_load("%s[u]" % g.tile_name(n, "_s"), n))
         L.close()
         L("#pragma unroll")
         L.open("for (int u = 0; u < %d; ++u)" % SU)
@@ -808,12 +819,16 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1):
             if V > 1:
                 L("#pragma unroll")
             L.open("for (int j = 0; j < %d; ++j)" % V)
+            if tail:
+                L.open("if (j < lim)")
             ref = g.make_ref("_s", "rr", "c", V, tiles, vals)
             g.emit_exprs(nodes, ref, stops())
             for n in reds:
                 g.accumulate(n, ref(n.args[0]), "c + j")
             for n in fresh:
                 L("keep%d[k].put(j, t%d);" % (over[n.nid].nid, n.nid))
+            if tail:
+                L.close()
             L.close()
             L.close()
 
@@ -883,7 +898,11 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1):
                     L("o%d.set(j, %s);" % (st.out.index, ref(st.root)))
             L.close()
             for st in full_out:
-                L("o%d.%s(%s);" % (st.out.index, g.st, g.addr(st.out, "r", "c")))
+                if tail:
+                    L("if (full) o%d.%s(%s); else o%d.store_partial(%s, lim);"
+                      % (st.out.index, g.st, g.addr(st.out, "r", "c"), st.out.index, g.addr(st.out, "r", "c")))
+                else:
+                    L("o%d.%s(%s);" % (st.out.index, g.st, g.addr(st.out, "r", "c")))
             L.close()
 
         sweep(leaves, store_body)
@@ -900,7 +919,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1):
     L.close()
     return _finish("rowcoop" if coop else "row", g, head, fmt, T, 0,
                    dict(V=V, LX=LX, LY=LY, NCH=NCH, stream=bool(stream), passing=len(transient),
-                        over=len(vals), chunks=chunks, NRED=len(all_reds)))
+                        over=len(vals), chunks=chunks, NRED=len(all_reds), tail=bool(tail)))
 
 
 # =====================================================================================

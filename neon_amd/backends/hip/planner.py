@@ -351,7 +351,8 @@ def _plan_ew(prog, cu_count):
 
 def _plan_row(prog, cu_count):
     R, C = prog.domain
-    V = _vector_width(prog, tail_ok=False)
+    V = _vector_width(prog, tail_ok=True)
+    tail = (C % V) != 0
     nvec = _ceil_div(C, V)
     words = _words_per_tile(prog, V, 1)
     options = []
@@ -391,12 +392,12 @@ def _plan_row(prog, cu_count):
                         for t in prog.tensors if t.read and t.shape[1] > 1] or [1 << 30])
         if chunks >= 2 and per <= 16 and per * smallest <= 64:
             kw = None if per * words <= 64 else 64
-            spec = codegen.gen_row(prog, V, 1024, 1, per, _streams(prog), keep_words=kw, chunks=chunks)
+            spec = codegen.gen_row(prog, V, 1024, 1, per, _streams(prog), keep_words=kw, chunks=chunks, tail=tail)
             part_bytes = R * spec.params["NRED"] * chunks * 8
             ctr_off = _ceil_div(part_bytes, 256) * 256
             return Choice(spec, (R, chunks, 1), workspace=(ctr_off + R * 8, ctr_off, 2 * R))
     LY = T // LX
-    spec = codegen.gen_row(prog, V, LX, LY, NCH, _streams(prog), keep_words=keep_words)
+    spec = codegen.gen_row(prog, V, LX, LY, NCH, _streams(prog), keep_words=keep_words, tail=tail)
     gx = _ceil_div(R, LY)
     return Choice(spec, (gx, 1, 1))
 

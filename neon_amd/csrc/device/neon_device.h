@@ -228,6 +228,18 @@ template <typename T, int V> struct nh_raw {
 #pragma unroll
         for (int i = 0; i < NW; ++i) asm volatile("" : "+v"(w[i]));
     }
+    // the first n (< V) elements, one at a time; the rest of the tile is zero
+    NEON_DEV void load_partial(const T* p, int n) {
+        zero();
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            if (j < n) {
+                const nh_u32 bits = nh_bits_of<T>(p[j]);
+                if constexpr (sizeof(T) == 4) w[PACKED ? j : 0] = bits;
+                else w[PACKED ? j / PER : 0] |= bits << (8 * (int)sizeof(T) * (PACKED ? j % PER : 0));
+            }
+        }
+    }
     // reuse the registers of a float tile for a value derived from it
     NEON_DEV void put(int j, float v) {
         static_assert(sizeof(T) == 4, "one word per element only");
@@ -259,6 +271,17 @@ template <typename T, int V> struct nh_out {
     NEON_DEV void store_stream(T* p) const {
         if constexpr (PACKED) nh_store_words<NW, true>(reinterpret_cast<nh_u32*>(p), w);
         else __builtin_nontemporal_store(nh_from_bits<T>(w[0]), p);
+    }
+    // the first n (< V) elements, one at a time
+    NEON_DEV void store_partial(T* p, int n) const {
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            if (j < n) {
+                const nh_u32 word = w[PACKED ? j / PER : 0];
+                const nh_u32 bits = (sizeof(T) == 4) ? word : (word >> (8 * (int)sizeof(T) * (PACKED ? j % PER : 0)));
+                p[j] = nh_from_bits<T>(bits);
+            }
+        }
     }
 };
 

@@ -204,7 +204,9 @@ def test_shape_class_selection(pb):
         pb.empty((4000000, 256)).__setitem__(slice(None), pb.fprop_softmax(huge, 0))
     odd = pb.empty((64, 327))
     ch = plan_of(pb, lambda: pb.empty((64, 1)).__setitem__(slice(None), pb.sum(odd, axis=1)))
-    assert ch.spec.family == "row" and ch.spec.params["V"] == 1           # 327 columns: no vector access
+    # 327 columns: vector accesses, the last tile of a row element by element
+    assert ch.spec.family == "row" and ch.spec.params["V"] == 4 and ch.spec.params["tail"]
+    assert "load_partial" in ch.spec.source
     xt = pb.empty((128, 4096)).T
     ch = plan_of(pb, lambda: o.__setitem__(slice(None), xt + 1.0))
     assert ch.spec.params["V"] == 1                                          # strided operand
