@@ -188,11 +188,25 @@ class _Gen(object):
         # the axis that is *not* hot
         return "a%d + (long long)(%s)" % (slot.index, c if n.axis == 0 else r)
 
+    col_tail = False     # column families: the last column tile is partial (`cfull`, `clim` in scope)
+
     def emit_load(self, n, r, c, V, sfx, declare=True, target=None):
         name = target or self.tile_name(n, sfx)
         if declare:
             self.L("%s %s;" % (self.tile_type(n, V), name))
-        self.L("%s.%s(%s);" % (name, self.load_op(n), self.tile_addr(n, r, c)))
+        self.L(self.load_stmt(name, n, r, c, V))
+
+    def load_stmt(self, name, n, r, c, V, op=None):
+        addr = self.tile_addr(n, r, c)
+        op = op or self.load_op(n)
+        if self.col_tail and self.tile_width(n, V) > 1:
+            return "if (cfull) %s.%s(%s); else %s.load_partial(%s, clim);" % (name, op, addr, name, addr)
+        return "%s.%s(%s);" % (name, op, addr)
+
+    def store_stmt(self, name, op, addr, width):
+        if self.col_tail and width > 1:
+            return "if (cfull) %s.%s(%s); else %s.store_partial(%s, clim);" % (name, op, addr, name, addr)
+        return "%s.%s(%s);" % (name, op, addr)
 
     def load_op(self, n):
         """streaming (non-temporal) loads are for data touched once: operands
@@ -1009,7 +1023,7 @@ def _col_lds(L, LX, LY, T, V, any_index):
     return WY * pitch * (4 + (8 if any_index else 0))
 
 
-def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
+def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False):
     """Axis-0 reductions with the rows resident in registers (LX column-lanes x
     LY row-lanes per workgroup, NR rows per lane).
 
@@ -1026,6 +1040,8 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
     before the first launch, reset by the last workgroup to leave)."""
     coop = chunks > 1
     g = _RedGen(prog, V, stream, "col")
+    g.col_tail = bool(tail)     # C is not a multiple of V: the last column tile is loaded and stored
+    #                             element by element; its surplus columns compute on zeros and are dropped
     L = g.L
     T = LX * LY
     params, fmt = g.param_list([("char* ws", "P"), ("long long ctr_offset", "q")] if coop else [])
@@ -1043,6 +1059,9 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
     L("const long long c = ((long long)blockIdx.x * %d + tx) * %d;" % (LX, V))
     L("const bool col_ok = c < C;")
     L("const long long cc = col_ok ? c : 0;")
+    if tail:
+        L("const bool cfull = c + %d <= C;" % V)
+        L("const int clim = cfull ? %d : (col_ok ? (int)(C - c) : 0);" % V)
     if coop:
         L("__shared__ int s_abort;")
         L("unsigned int* ctr = reinterpret_cast<unsigned int*>(ws + ctr_offset) + 2 * blockIdx.x;")
@@ -1074,11 +1093,15 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
         L.open("if (col_ok && ty == 0)")
         L("#pragma unroll")
         L.open("for (int j = 0; j < %d; ++j)" % V)
+        if tail:
+            L.open("if (j < clim)")
         for n in reds:
             if n.is_index:
                 L("nh_part_store(&part%d[(long long)blockIdx.y * C + c + j], acc%d[j]);" % (n.nid, n.nid))
             else:
                 L("nh_part_store(&part%d[(long long)blockIdx.y * C + c + j], nh_pair{rv%d[j], 0});" % (n.nid, n.nid))
+        if tail:
+            L.close()
         L.close()
         L.close()
         L("__syncthreads();     // every lane's partial stores have completed")
@@ -1122,7 +1145,8 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
         for n in reds:
             op = _RED_OP[n.op]
             init = ("%s::init()" % op) if n.is_index else ("nh_pair{%s::init(), 0}" % op)
-            L("q%d[k][j] = live ? nh_part_load(&part%d[(long long)q * C + c + j]) : %s;" % (n.nid, n.nid, init))
+            L("q%d[k][j] = (live%s) ? nh_part_load(&part%d[(long long)q * C + c + j]) : %s;"
+              % (n.nid, " && j < clim" if tail else "", n.nid, init))
         L.close()
         L.close()
         for n in reds:
@@ -1166,7 +1190,7 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
             row_loop_open()
             for n in fresh:
                 cached[n.nid] = "keep%d" % n.nid
-                L("if (ok) keep%d[i].%s(%s); else keep%d[i].zero();" % (n.nid, g.ld, g.tile_addr(n, "r", "cc"), n.nid))
+                L("if (ok) { %s } else keep%d[i].zero();" % (g.load_stmt("keep%d[i]" % n.nid, n, "r", "cc", V, op=g.ld), n.nid))
             L.close()
         for n in leaves:
             tiles[n.nid] = ("keep%d[i]" % n.nid) if varies_in_loop(n) else line_tiles[n.nid]
@@ -1180,7 +1204,7 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
                     name = "line%d" % n.nid
                     line_tiles[n.nid] = name
                     L("%s %s;" % (g.tile_type(n, V), name))
-                    L("%s.load(%s);" % (name, g.tile_addr(n, "0", "cc")))
+                    L(g.load_stmt(name, n, "0", "cc", V, op="load"))
             elif n.nid not in cached:
                 L("%s keep%d[%d];" % (g.tile_type(n, V), n.nid, NR))
 
@@ -1279,7 +1303,7 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
                 L("o%d.set(j, %s);" % (st.out.index, ref(st.root)))
         L.close()
         for st in line_out:
-            L("o%d.store(%s);" % (st.out.index, g.addr(st.out, "0", "c")))
+            L(g.store_stmt("o%d" % st.out.index, "store", g.addr(st.out, "0", "c"), V))
         L.close()
 
     if full_out:
@@ -1304,7 +1328,7 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
                 L("o%d.set(j, %s);" % (st.out.index, ref(st.root)))
         L.close()
         for st in full_out:
-            L("o%d.%s(%s);" % (st.out.index, g.st, g.addr(st.out, "r", "c")))
+            L(g.store_stmt("o%d" % st.out.index, g.st, g.addr(st.out, "r", "c"), V if st.out.shape[1] > 1 else 1))
         L.close()
         L.close()
     if coop and ticket_finish:
@@ -1323,7 +1347,7 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0):
     L.close()
     return _finish("colcoop" if coop else "col", g, head, fmt, T, lds,
                    dict(V=V, LX=LX, LY=LY, NR=NR, stream=bool(stream), chunks=chunks,
-                        NRED=len(all_reds), kept=len(kept), over=len(over)))
+                        NRED=len(all_reds), kept=len(kept), over=len(over), tail=bool(tail)))
 
 
 # (more chunks do not help tall narrow matrices: the one workgroup per strip that
@@ -1338,7 +1362,7 @@ COLSPLIT_FOLD_BATCH = 8
 COLSPLIT_ROWS_IN_FLIGHT = 4
 
 
-def gen_colsplit(prog, V, LX, LY, stream=False):
+def gen_colsplit(prog, V, LX, LY, stream=False, tail=False):
     """One level of axis-0 reductions over a tall matrix.  grid = (column
     strips, row chunks).  Each workgroup reduces its chunk, leaves one partial
     per column in the workspace and takes a ticket; the workgroup that draws
@@ -1350,6 +1374,7 @@ def gen_colsplit(prog, V, LX, LY, stream=False):
     tickets after ``ticket_offset`` bytes)."""
     assert prog.nlevels == 1
     g = _RedGen(prog, V, stream, "colsplit")
+    g.col_tail = bool(tail)     # partial last column tile, as in gen_col
     L = g.L
     T = LX * LY
     params, fmt = g.param_list([("int rows_per_chunk", "i"), ("char* ws", "P"),
@@ -1368,6 +1393,9 @@ def gen_colsplit(prog, V, LX, LY, stream=False):
     L("const long long c = ((long long)blockIdx.x * %d + tx) * %d;" % (LX, V))
     L("const bool col_ok = c < C;")
     L("const long long cc = col_ok ? c : 0;")
+    if tail:
+        L("const bool cfull = c + %d <= C;" % V)
+        L("const int clim = cfull ? %d : (col_ok ? (int)(C - c) : 0);" % V)
     L("const long long r0 = (long long)blockIdx.y * rows_per_chunk;")
     L("const long long r1 = (r0 + rows_per_chunk < R) ? (r0 + rows_per_chunk) : (long long)R;")
     L("const int nchunks = gridDim.y;")
@@ -1418,7 +1446,7 @@ def gen_colsplit(prog, V, LX, LY, stream=False):
     L("unsigned int* tickets = reinterpret_cast<unsigned int*>(ws + ticket_offset);")
     L.open("if (col_ok && ty == 0)")
     L("#pragma unroll")
-    L.open("for (int j = 0; j < %d; ++j)" % V)
+    L.open("for (int j = 0; j < %s; ++j)" % ("clim" if tail else str(V)))
     for n in reds:
         L("nh_pair p%d; p%d.v = %s; p%d.i = %s;" % (n.nid, n.nid,
                                                      ("acc%d[j].v" % n.nid) if n.is_index else ("rv%d[j]" % n.nid),
@@ -1458,7 +1486,8 @@ def gen_colsplit(prog, V, LX, LY, stream=False):
     for n in reds:
         op = _RED_OP[n.op]
         init = ("%s::init()" % op) if n.is_index else ("nh_pair{%s::init(), 0}" % op)
-        L("q%d[k][j] = live ? nh_part_load(&part%d[(long long)q * C + c + j]) : %s;" % (n.nid, n.nid, init))
+        L("q%d[k][j] = (live%s) ? nh_part_load(&part%d[(long long)q * C + c + j]) : %s;"
+          % (n.nid, " && j < clim" if tail else "", n.nid, init))
     L.close()
     L.close()
     L("#pragma unroll")
@@ -1501,7 +1530,8 @@ def gen_colsplit(prog, V, LX, LY, stream=False):
             L("o%d.set(j, %s);" % (st.out.index, ref(st.root)))
     L.close()
     for st in prog.statements:
-        L("o%d.store(%s);" % (st.out.index, g.addr(st.out, "0", "c")))
+        L(g.store_stmt("o%d" % st.out.index, "store", g.addr(st.out, "0", "c"), V))
     L.close()
     L.close()
-    return _finish("colsplit", g, head, fmt, T, lds, dict(V=V, LX=LX, LY=LY, NRED=len(reds), stream=bool(stream)))
+    return _finish("colsplit", g, head, fmt, T, lds,
+                   dict(V=V, LX=LX, LY=LY, NRED=len(reds), stream=bool(stream), tail=bool(tail)))

@@ -414,7 +414,8 @@ COLSPLIT_THREADS = 256
 
 def _plan_col(prog, cu_count):
     R, C = prog.domain
-    V = _vector_width(prog, tail_ok=False)
+    V = _vector_width(prog, tail_ok=True)
+    tail = (C % V) != 0
     nvec = _ceil_div(C, V)
     isz = max([t.dtype.itemsize for t in prog.tensors if t.shape[1] > 1] + [1])
     words = _words_per_tile(prog, V, 0)
@@ -455,7 +456,7 @@ def _plan_col(prog, cu_count):
         T, LY, NR = fit
         budget = _COL_BUDGET[T]
         spare = max(0, (budget - NR * words) // (NR * V))
-        spec = codegen.gen_col(prog, V, LX, LY, NR, _streams(prog), max_vals=min(2, spare))
+        spec = codegen.gen_col(prog, V, LX, LY, NR, _streams(prog), max_vals=min(2, spare), tail=tail)
         return Choice(spec, (_ceil_div(nvec, LX), 1, 1))
 
     # (c) deeper trees (or full-shape results) over many rows: the workgroups of a
@@ -485,7 +486,7 @@ def _plan_col(prog, cu_count):
                         break
                     spare = max(0, (budget - NR * words) // (NR * V))
                     spec = codegen.gen_col(prog, V, lxc, LY, NR, _streams(prog), chunks=chunks,
-                                           max_vals=min(2, spare))
+                                           max_vals=min(2, spare), tail=tail)
                     part_bytes = spec.params["NRED"] * chunks * C * 8
                     ctr_off = _ceil_div(part_bytes, 256) * 256
                     return Choice(spec, (strips_c, chunks, 1),
@@ -523,7 +524,7 @@ def _plan_col(prog, cu_count):
         chunks = _ceil_div(R, rpc)
         if chunks > 65535:
             raise ValueError("tensor too large for one launch")
-        spec = codegen.gen_colsplit(prog, V, LX, LY, _streams(prog))
+        spec = codegen.gen_colsplit(prog, V, LX, LY, _streams(prog), tail=tail)
         nred = spec.params["NRED"]
         part_bytes = nred * chunks * C * 8
         ticket_off = _ceil_div(part_bytes, 256) * 256
