@@ -946,7 +946,6 @@ def _emit_col_fold(g, L, n, LX, LY, T, V, src, dst_decl=True):
     folded with lane-xor exchanges first; LDS then joins the wave groups in
     row order."""
     op = _RED_OP[n.op]
-    ty_ = "nh_pair" if n.is_index else "float"
     VK = V            # values a lane contributes to the LDS stage
     if LX < 64 and T > 64:
         # the wave's row-lanes are folded with lane exchanges that split the V
@@ -1086,7 +1085,6 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False)
         written, so nobody waits: the workgroup whose arrival completes the
         count gathers, folds and goes on alone, the others are done."""
         exchanges[0] += 1
-        QMAX = -(-chunks // LY)
         for n in reds:
             L("nh_pair* part%d = reinterpret_cast<nh_pair*>(ws) + (long long)%d * C;"
               % (n.nid, red_slot[n.nid] * chunks))

@@ -140,8 +140,8 @@ def _vector_width(prog, tail_ok):
     element's (the device's vector accesses are typed byte-aligned), so views
     that start mid-row and odd row lengths keep full-width accesses; what V
     must do is divide the row length, unless the family handles a partial last
-    tile (``tail_ok``: the elementwise family)."""
-    R, C = prog.domain
+    tile (``tail_ok``)."""
+    C = prog.domain[1]
     cols = [t for t in prog.tensors if t.shape[1] > 1]
     used = used_nodes([st.root for st in prog.statements])
     hot0 = [prog.tensors[n.slot] for n in used if n.kind == "H" and n.axis == 0]
