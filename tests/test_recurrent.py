@@ -10,10 +10,11 @@ import pytest
 
 from neon_amd import NervanaObject
 from neon_amd.initializers import Array
-from neon_amd.layers import LSTM, Recurrent, RecurrentLast, RecurrentMean, RecurrentSum, Sequential
+from neon_amd.layers import GRU, LSTM, Recurrent, RecurrentLast, RecurrentMean, RecurrentSum, Sequential
 from neon_amd.transforms import Logistic, Tanh
 
 NIN, NOUT, STEPS, BSZ = 5, 6, 4, 3
+NGATES = {"rnn": 1, "lstm": 4, "gru": 3}
 
 
 @contextlib.contextmanager
@@ -33,7 +34,7 @@ def _sig(z):
 def _forward64(kind, W, x, proj):
     """loss = sum(proj * outputs) of the layer with packed parameters W
     ((nin + nout + 1, ngates * nout), the layer's own layout) in float64"""
-    ng = 4 if kind == "lstm" else 1
+    ng = NGATES[kind]
     g_nout = ng * NOUT
     W_in = W[:NIN].reshape(g_nout, NIN)
     W_rec = W[NIN:-1].reshape(g_nout, NOUT)
@@ -42,6 +43,14 @@ def _forward64(kind, W, x, proj):
     outs = []
     for s in range(STEPS):
         xs = x[:, s * BSZ:(s + 1) * BSZ]
+        if kind == "gru":
+            zx = W_in @ xs + b
+            rz = _sig(zx[:2 * NOUT] + W_rec[:2 * NOUT] @ h)
+            r, u = rz[:NOUT], rz[NOUT:]
+            cand = np.tanh(zx[2 * NOUT:] + W_rec[2 * NOUT:] @ (r * h))
+            h = (1 - u) * h + u * cand
+            outs.append(h)
+            continue
         z = W_in @ xs + W_rec @ h + b
         if kind == "rnn":
             h = np.tanh(z)
@@ -71,11 +80,11 @@ def _numeric_grad(f, a, eps=1e-6):
 
 def _make(be, kind, W):
     nrows = NIN + NOUT + 1
-    ng = 4 if kind == "lstm" else 1
+    ng = NGATES[kind]
     init = Array(np.zeros((NOUT, NIN), np.float32))         # placeholder: the packed W is set below
-    if kind == "lstm":
-        layer = LSTM(NOUT, init, init_inner=Array(np.zeros((NOUT, NOUT), np.float32)),
-                     activation=Tanh(), gate_activation=Logistic())
+    if kind in ("lstm", "gru"):
+        layer = (LSTM if kind == "lstm" else GRU)(NOUT, init, init_inner=Array(np.zeros((NOUT, NOUT), np.float32)),
+                                                  activation=Tanh(), gate_activation=Logistic())
     else:
         layer = Recurrent(NOUT, init, init_inner=Array(np.zeros((NOUT, NOUT), np.float32)), activation=Tanh())
     layer.configure((NIN, STEPS))
@@ -93,8 +102,8 @@ def _make(be, kind, W):
 
 def _check_layer(be, kind, rtol):
     with using(be, BSZ):
-        rs = np.random.RandomState(5 if kind == "lstm" else 6)
-        ng = 4 if kind == "lstm" else 1
+        rs = np.random.RandomState(5 + NGATES[kind])
+        ng = NGATES[kind]
         W = rs.uniform(-0.6, 0.6, (NIN + NOUT + 1, ng * NOUT))
         x = rs.uniform(-1, 1, (NIN, STEPS * BSZ))
         proj = rs.uniform(-1, 1, (NOUT, STEPS * BSZ))
@@ -115,7 +124,7 @@ def _check_layer(be, kind, rtol):
         return out.get(), layer.dW.get(), deltas.get()
 
 
-@pytest.mark.parametrize("kind", ["rnn", "lstm"])
+@pytest.mark.parametrize("kind", ["rnn", "lstm", "gru"])
 def test_recurrent_layers_against_float64_and_finite_differences(cpu, kind):
     _check_layer(cpu, kind, 2e-4)
 
@@ -145,7 +154,7 @@ def test_recurrent_output_layers(cpu):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("kind", ["rnn", "lstm"])
+@pytest.mark.parametrize("kind", ["rnn", "lstm", "gru"])
 def test_recurrent_layers_on_hip(pair, kind):
     cpu, hip = pair
     want = _check_layer(cpu, kind, 2e-4)
