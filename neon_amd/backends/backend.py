@@ -778,6 +778,34 @@ class Backend(metaclass=_BackendRegistry):
         """add one bias value per row, in place"""
         self.add(inputs, bias, out=inputs)
 
+    def compound_rnn_unroll_fprop(self, W_recur, h_prev_s, h_ff_s, h_s, bias, nout, num_steps,
+                                  num_used_steps, activation, reverse=False):
+        """The time loop of a plain recurrent layer (reference
+        backend.py:1559-1601): h[t] = activation(W_recur h[t-1] + h_ff[t] +
+        bias) over lists of per-step views; ``h_ff_s`` may be ``h_s`` itself
+        when the input projection was written into the outputs."""
+        used = num_steps if num_used_steps is None else min(num_used_steps, num_steps)
+        order = range(used - 1, -1, -1) if reverse else range(used)
+        for t in order:
+            h, h_prev, h_ff = h_s[t], h_prev_s[t], h_ff_s[t]
+            if h_ff is h:
+                self.compound_dot(W_recur, h_prev, h, beta=1.0)
+                h[:] = activation(h + bias)
+            else:
+                self.compound_dot(W_recur, h_prev, h)
+                h[:] = activation(h + h_ff + bias)
+
+    def compound_rnn_unroll_bprop(self, W_recur, delta_prev_s, delta_s, h_s, nout, num_steps,
+                                  num_used_steps, activation, reverse=True):
+        """The time loop of a plain recurrent layer's backward pass (reference
+        backend.py:1603-1638); ``W_recur`` arrives already transposed."""
+        used = num_steps if num_used_steps is None else min(num_used_steps, num_steps)
+        n = min(used, len(delta_s), len(delta_prev_s))
+        order = range(n - 1, -1, -1) if reverse else range(n)
+        for t in order:
+            delta_s[t][:] = activation.bprop(h_s[t]) * delta_s[t]
+            self.compound_dot(W_recur, delta_s[t], delta_prev_s[t], beta=1.0)
+
     def is_mkl(self):
         return False
 

@@ -153,6 +153,69 @@ def test_recurrent_output_layers(cpu):
             assert np.allclose(deltas.get(), np.concatenate(back, axis=1), atol=1e-6), cls.__name__
 
 
+def _check_unroll(be, reverse):
+    """compound_rnn_unroll_fprop / bprop against a float64 loop: forward over
+    the steps (or backward, for the reverse direction of a bidirectional
+    layer), and the back-propagated deltas of the same loop"""
+    rs = np.random.RandomState(11 + reverse)
+    Wr = rs.uniform(-0.6, 0.6, (NOUT, NOUT)).astype(np.float32)
+    b = rs.uniform(-0.5, 0.5, (NOUT, 1)).astype(np.float32)
+    ff = rs.uniform(-1, 1, (NOUT, STEPS * BSZ)).astype(np.float32)
+    err = rs.uniform(-1, 1, (NOUT, STEPS * BSZ)).astype(np.float32)
+    used = STEPS - 1
+    order = list(range(used))[::-1] if reverse else list(range(used))
+    sl = [slice(t * BSZ, (t + 1) * BSZ) for t in range(STEPS)]
+    h64 = np.zeros((NOUT, STEPS * BSZ))
+    prev = np.zeros((NOUT, BSZ))
+    for t in order:
+        h64[:, sl[t]] = np.tanh(Wr.astype(np.float64) @ prev + ff[:, sl[t]] + b)
+        prev = h64[:, sl[t]]
+    d64 = err.astype(np.float64).copy()
+    for t in order[::-1]:
+        d64[:, sl[t]] *= 1 - h64[:, sl[t]] ** 2
+        src = order[order.index(t) - 1] if order.index(t) > 0 else None
+        if src is not None:
+            d64[:, sl[src]] += Wr.T.astype(np.float64) @ d64[:, sl[t]]
+    with using(be, BSZ):
+        act = Tanh()
+        W_d, b_d = be.array(Wr), be.array(b)
+        zero = be.zeros((NOUT, BSZ))
+        for shared in (False, True):
+            h_buf = be.array(ff) if shared else be.zeros((NOUT, STEPS * BSZ))
+            ff_buf = h_buf if shared else be.array(ff)
+            h_s = [h_buf[:, s] for s in sl]
+            ff_s = h_s if shared else [ff_buf[:, s] for s in sl]
+            prev_s = (h_s[1:used] + [zero] * (STEPS - used + 1)) if reverse else ([zero] + h_s[:-1])
+            be.compound_rnn_unroll_fprop(W_d, prev_s, ff_s, h_s, b_d, NOUT, STEPS, used, act, reverse)
+            got = h_buf.get()
+            for t in order:
+                assert np.allclose(got[:, sl[t]], h64[:, sl[t]], rtol=1e-5, atol=1e-6), (shared, t)
+            if not shared:
+                assert not got[:, sl[STEPS - 1]].any()       # the unused step stays untouched
+        d_buf = be.array(err)
+        d_s = [d_buf[:, s] for s in sl][:used]
+        sink = be.zeros((NOUT, BSZ))
+        dprev_s = (d_s[1:] + [sink]) if reverse else ([sink] + d_s[:-1])   # d_s holds the used steps only
+        be.compound_rnn_unroll_bprop(W_d.T, dprev_s, d_s, h_s, NOUT, STEPS, used, act, not reverse)
+        got = d_buf.get()
+        for t in order:
+            assert np.allclose(got[:, sl[t]], d64[:, sl[t]], rtol=1e-5, atol=1e-6), t
+        return h_buf.get(), got
+
+
+@pytest.mark.parametrize("reverse", [False, True])
+def test_rnn_unroll_helpers(cpu, reverse):
+    _check_unroll(cpu, reverse)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("reverse", [False, True])
+def test_rnn_unroll_helpers_on_hip(pair, reverse):
+    cpu, hip = pair
+    for g, w in zip(_check_unroll(hip, reverse), _check_unroll(cpu, reverse)):
+        assert np.allclose(g, w, rtol=2e-5, atol=2e-6)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("kind", ["rnn", "lstm", "gru"])
 def test_recurrent_layers_on_hip(pair, kind):
