@@ -97,6 +97,26 @@ class Softmax(Transform):
         return 1
 
 
+class PixelwiseSoftmax(Transform):
+    """Softmax over ``c`` channels for every pixel: the input (c * pixels,
+    batch) is viewed as (c, pixels * batch) and normalised down each column, in
+    place (reference activation.py:241-258)"""
+
+    def __init__(self, c, name=None, epsilon=2 ** -23):
+        super(PixelwiseSoftmax, self).__init__(name)
+        self.epsilon = epsilon
+        self.c = c
+
+    def __call__(self, x):
+        y = x.reshape((self.c, -1))
+        shifted = self.be.exp(y - self.be.max(y, axis=0))
+        y[:] = self.be.reciprocal(self.be.sum(shifted, axis=0)) * shifted
+        return x
+
+    def bprop(self, x):
+        return 1
+
+
 class Tanh(Transform):
     """tanh(x); derivative 1 - y^2 from the output y"""
 

@@ -8,9 +8,9 @@ import numpy as np
 import pytest
 
 from neon_amd import NervanaObject
-from neon_amd.transforms import (Accuracy, CrossEntropyBinary, CrossEntropyMulti, Explin, Identity,
-                                 LogLoss, Logistic, MeanSquared, Misclassification, Normalizer,
-                                 PrecisionRecall, Rectlin, Rectlinclip, SmoothL1Loss, Softmax,
+from neon_amd.transforms import (Accuracy, CrossEntropyBinary, CrossEntropyMulti, Explin, GANCost, Identity,
+                                 LogLoss, Logistic, MeanSquared, Misclassification, MultiMetric, Normalizer,
+                                 PixelwiseSoftmax, PrecisionRecall, Rectlin, Rectlinclip, SmoothL1Loss, Softmax,
                                  SquareHingeLoss, SumSquared, Tanh, TopKMisclassification)
 from utils import assert_close
 
@@ -89,6 +89,127 @@ def test_activation_known_answers(cpu, name, make, inputs, expected, deriv, tol)
     want = np.asarray(expected, dtype=np.float64)
     assert got.shape == want.shape or want.shape == (1, 1)
     assert np.all(np.abs(got - want) <= tol + 1e-12), (got, want)
+
+
+def _pixelwise(be, c, x):
+    with using(be):
+        t = be.array(x)
+        act = PixelwiseSoftmax(c=c)
+        assert act(t) is t and act.bprop(t) == 1
+        return t.get()
+
+
+def test_pixelwise_softmax_known_answer(cpu):
+    """reference tests/test_activations.py:187-201: two channels, three pixels, one image"""
+    inputs = np.array([0, 1, 3, 1, 2, -2], dtype=np.float64).reshape((2, 3))
+    e = np.exp(inputs - inputs.max(axis=0))
+    got = _pixelwise(cpu, 2, inputs.reshape((1, -1)).astype(np.float32))
+    assert np.all(np.abs(got - (e / e.sum(axis=0)).reshape((1, -1))) <= 1e-6)
+
+
+def _pixelwise_case():
+    rs = np.random.RandomState(31)
+    c, pixels, batch = 21, 36 * 36, 8
+    x = (rs.standard_normal((c * pixels, batch)) * 4).astype(np.float32)
+    x64 = x.astype(np.float64).reshape(c, -1)
+    e = np.exp(x64 - x64.max(axis=0))
+    return c, x, (e / e.sum(axis=0)).reshape(x.shape)
+
+
+def test_pixelwise_softmax_over_many_pixels(cpu):
+    c, x, want = _pixelwise_case()
+    assert_close(_pixelwise(cpu, c, x), want, rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.gpu
+def test_pixelwise_softmax_hip(pair):
+    c, x, want = _pixelwise_case()
+    got = [_pixelwise(be, c, x) for be in pair]
+    assert_close(got[1], want, rtol=1e-5, atol=1e-7)
+    assert_close(got[1], got[0], rtol=1e-5, atol=1e-7)
+
+
+def _gan(be, func, y_data, y_noise):
+    with using(be, bsz=y_data.shape[1]):
+        cost = GANCost(func=func)
+        yd, yn = be.array(y_data), be.array(y_noise)
+        res = {}
+        for kind in ("dis", "dis_data", "dis_noise", "gen"):
+            out = be.iobuf(1)
+            out[:] = cost(yd, yn, cost_type=kind)
+            res[kind] = out.get()
+        for name, fn, arg in (("d_data", cost.bprop_data, yd), ("d_noise", cost.bprop_noise, yn),
+                              ("d_gen", cost.bprop_generator, yn)):
+            delta = be.iobuf(y_data.shape[0])
+            delta[:] = fn(arg)
+            res[name] = delta.get()
+        assert cost(yd, yn, cost_type="other") is None
+        return res
+
+
+def _gan_expected(func, yd, yn):
+    """closed forms; each derivative is the derivative of the matching cost term
+    (for 'modified' the reference keeps -1/y for the generator, the gradient
+    of the 'original' generator cost: the usual non-saturating trick)"""
+    yd, yn = yd.astype(np.float64), yn.astype(np.float64)
+    slog = lambda v: np.log(np.maximum(v, np.exp(-50)))
+    m = lambda v: v.mean(axis=0, keepdims=True)
+    one = np.ones_like(yd)
+    if func == "wasserstein":
+        return {"dis": m(yd - yn), "dis_data": m(yd), "dis_noise": m(-yn), "gen": m(yn),
+                "d_data": one, "d_noise": -one, "d_gen": one}
+    gen = -slog(yn) if func == "original" else slog(1 - yn)
+    return {"dis": m(-slog(yd) - slog(1 - yn)), "dis_data": m(-slog(yd)), "dis_noise": m(-slog(1 - yn)),
+            "gen": m(gen), "d_data": -1 / yd, "d_noise": 1 / (1 - yn),
+            "d_gen": 1 / (yn - 1) if func == "original" else -1 / yn}
+
+
+def _gan_inputs(rows=5, batch=7):
+    rs = np.random.RandomState(41)
+    return (rs.uniform(0.05, 0.95, (rows, batch)).astype(np.float32),
+            rs.uniform(0.05, 0.95, (rows, batch)).astype(np.float32))
+
+
+@pytest.mark.parametrize("func", ["original", "modified", "wasserstein"])
+def test_gan_cost_closed_forms(cpu, func):
+    yd, yn = _gan_inputs()
+    got, want = _gan(cpu, func, yd, yn), _gan_expected(func, yd, yn)
+    for k in want:
+        assert_close(got[k], want[k], rtol=2e-6, atol=1e-6, what=k)
+    # the reference's own case (tests/test_gan.py:49-76): y_data = 1, y_noise = 2, where 1 - y_noise is clamped
+    ones, twos = np.ones((5, 7), np.float32), np.full((5, 7), 2, np.float32)
+    got = _gan(cpu, func, ones, twos)
+    if func == "modified":
+        assert np.all(got["dis"] == 50.0) and np.all(got["d_data"] == -1) and np.all(got["d_noise"] == -1)
+        assert np.all(got["d_gen"] == -0.5)
+    if func == "wasserstein":
+        assert np.all(got["dis"] == -1.0) and np.all(got["d_gen"] == 1)
+    with using(cpu, bsz=4):
+        with pytest.raises(AssertionError):
+            GANCost(func="other")
+        with pytest.raises(AssertionError):
+            GANCost(cost_type="both")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("func", ["original", "modified", "wasserstein"])
+def test_gan_cost_hip(pair, func):
+    yd, yn = _gan_inputs(rows=300, batch=512)
+    res = [_gan(be, func, yd, yn) for be in pair]
+    want = _gan_expected(func, yd, yn)
+    for k in want:
+        assert_close(res[1][k], want[k], rtol=2e-5, atol=1e-6, what=k)
+        assert_close(res[1][k], res[0][k], rtol=2e-5, atol=1e-6, what=k)
+
+
+def test_multi_metric_picks_one_output(cpu):
+    rs = np.random.RandomState(3)
+    with using(cpu, bsz=6):
+        outs = tuple(cpu.array(rs.uniform(0.1, 1, (4, 6)).astype(np.float32)) for _ in range(3))
+        mm = MultiMetric(LogLoss(), 1)
+        assert mm.metric_names == ['LogLoss']                      # attributes come from the wrapped metric
+        y = outs[1].get().astype(np.float64)
+        assert abs(float(mm(outs, None)) - np.mean(-np.log((y * y).sum(axis=0)))) < 1e-6
 
 
 def test_softmax_big_inputs(cpu):
