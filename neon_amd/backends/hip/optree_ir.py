@@ -393,7 +393,10 @@ class Program(object):
                 self.key_parts.append(("fold2", op))
                 stack.append(Num(_fold_binary(op, a.value, b.value), ("2", op, a.expr, b.expr)))
                 return
-            self.key_parts.append(op)
+            # a number becomes a node (and a key part) only here, after the
+            # operator's own part: say on which side it stands, or ``x - 1``
+            # and ``1 - x`` would share a key and therefore a kernel
+            self.key_parts.append((op, isinstance(a, Node), isinstance(b, Node)))
             a, b = self._as_node(a), self._as_node(b)
             stack.append(self._intern(("E", op, a.nid, b.nid), lambda: Node("E", op=op, args=(a, b))))
         elif op in REDUCE:

@@ -63,6 +63,26 @@ def test_binary_ops_and_broadcast(pair, shapes):
         both(pair, f, [a, b], what=name)
 
 
+def test_numbers_on_either_side_of_an_operator(pair):
+    """the same backend evaluates each form right after its mirror image: they
+    differ only in the side the number stands on, and must not share a kernel"""
+    rs = np.random.RandomState(21)
+    a = gen_inputs(rs, (300, 512)) * 0.4 + 0.5
+    forms = {
+        "x-c": lambda be, x: x - 1.0, "c-x": lambda be, x: 1.0 - x,
+        "x/c": lambda be, x: x / 2.0, "c/x": lambda be, x: 2.0 / x,
+        "x>c": lambda be, x: x > 0.5, "c>x": lambda be, x: 0.5 > x,
+        "x<=c": lambda be, x: x <= 0.5, "c<=x": lambda be, x: 0.5 <= x,
+        "x**c": lambda be, x: be.power(be.absolute(x), 2.5), "c**x": lambda be, x: be.power(2.5, x),
+        "c/(x-c)": lambda be, x: 1.0 / (x - 3.0), "c/(c-x)": lambda be, x: 1.0 / (3.0 - x),
+        "sum(x-c)": lambda be, x: be.sum(x - 1.0, axis=0) + 0 * x, "sum(c-x)": lambda be, x: be.sum(1.0 - x, axis=0) + 0 * x,
+        "max(x/c)": lambda be, x: be.max(x / 3.0, axis=1) + 0 * x, "max(c/x)": lambda be, x: be.max(3.0 / x, axis=1) + 0 * x,
+    }
+    for _ in range(2):              # the second pass runs from the launch cache
+        for name, f in forms.items():
+            both(pair, f, [a], what=name, atol=1e-5)
+
+
 def test_inplace_and_views(pair):
     rs = np.random.RandomState(3)
     a = gen_inputs(rs, (50, 128))

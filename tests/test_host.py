@@ -139,6 +139,22 @@ def test_constant_folding_and_key(pb):
     assert len(p3.consts) == 1 and len(p4.consts) == 2 and p3.key() != p4.key()
 
 
+def test_key_tells_which_side_a_number_stands_on(pb):
+    """a number turns into a node only when its operator is applied, after the
+    tensor beside it: ``x - 1`` and ``1 - x`` must still get different keys
+    (equal keys share one compiled kernel)"""
+    x, out = pb.empty((8, 8)), pb.empty((8, 8))
+    forms = [lambda: x - 1.0, lambda: 1.0 - x, lambda: x / 2.0, lambda: 2.0 / x, lambda: x > 0.5, lambda: 0.5 > x,
+             lambda: pb.power(x, 2.0), lambda: pb.power(2.0, x), lambda: 1.0 / (x - 1.0), lambda: 1.0 / (1.0 - x),
+             lambda: (x - 1.0) - x, lambda: x - (1.0 - x), lambda: pb.sqrt(4.0) - x, lambda: x - pb.sqrt(4.0)]
+    progs = [_prog(pb, lambda f=f: out.__setitem__(slice(None), f())) for f in forms]
+    keys = [p.key() for p in progs]
+    assert len(set(keys)) == len(keys)
+    # the same form with another number keeps its key (the number is an argument)
+    again = _prog(pb, lambda: out.__setitem__(slice(None), 3.0 - x))
+    assert again.key() == keys[1] and again.consts != progs[1].consts
+
+
 def test_identity_reduction_of_broadcast_operand(pb):
     row, out = pb.empty((1, 16)), pb.empty((1, 16))
     p = _prog(pb, lambda: out.__setitem__(slice(None), pb.sum(row, axis=0) + pb.argmax(row, axis=0)))
