@@ -155,6 +155,51 @@ def test_key_tells_which_side_a_number_stands_on(pb):
     assert again.key() == keys[1] and again.consts != progs[1].consts
 
 
+def test_equal_keys_mean_equal_programs(pb):
+    """random small statement groups over a fixed set of tensors: whenever two
+    of them get the same key they must be the same DAG up to the values of the
+    numbers, since the key decides which compiled kernel runs"""
+    R, C = 8, 16
+    x, y, out, out2 = pb.empty((R, C)), pb.empty((R, C)), pb.empty((R, C)), pb.empty((R, C))
+    leaves = [x, y, pb.empty((R, 1)), pb.empty((1, C))]
+    idx = pb.empty((1, C), dtype=np.int32)
+    rs = np.random.RandomState(0)
+    unary = {"neg": pb.negative, "sqrt": pb.sqrt, "exp": pb.exp}
+    binary = {"add": pb.add, "sub": pb.subtract, "mul": pb.multiply, "div": pb.divide, "gt": pb.greater,
+              "pow": pb.power, "max": pb.maximum}
+
+    def expr(depth, axis):
+        r = rs.rand()
+        if depth == 0 or r < 0.3:
+            return float(rs.choice([0.5, 1.0, 2.0])) if rs.rand() < 0.35 else leaves[rs.randint(len(leaves))]
+        if r < 0.45:
+            return unary[rs.choice(sorted(unary))](expr(depth - 1, axis))
+        if r < 0.9:
+            return binary[rs.choice(sorted(binary))](expr(depth - 1, axis), expr(depth - 1, axis))
+        if rs.rand() < 0.2:
+            return pb.onehot(idx, axis=0)
+        a = expr(depth - 1, axis)
+        return getattr(pb, rs.choice(["sum", "max"]))(x * a if isinstance(a, float) else a, axis=axis)
+
+    def group():
+        axis = int(rs.randint(0, 2))
+        for k in range(1 if rs.rand() < 0.7 else 2):
+            t = expr(int(rs.randint(1, 4)), axis)
+            (out if k == 0 else (out2 if rs.rand() < 0.5 else x))[:] = (x + t if isinstance(t, float) else t)
+
+    seen, built = {}, 0
+    for _ in range(6000):
+        try:
+            p = _prog(pb, group)
+        except (TypeError, ValueError, NotImplementedError, planner.NeedsSplit, MixedAxes):
+            continue            # mixed axes and the like: never reach a kernel as one program
+        built += 1
+        dag = (tuple((n.kind, n.op, tuple(a.nid for a in n.args), n.slot, n.axis) for n in p.nodes),
+               tuple((st.out.index, st.root.nid) for st in p.statements))
+        assert seen.setdefault(p.key(), dag) == dag, p.key()[0]
+    assert built > 3000 and len(seen) > 1000
+
+
 def test_identity_reduction_of_broadcast_operand(pb):
     row, out = pb.empty((1, 16)), pb.empty((1, 16))
     p = _prog(pb, lambda: out.__setitem__(slice(None), pb.sum(row, axis=0) + pb.argmax(row, axis=0)))
