@@ -140,6 +140,75 @@ def test_random_fused_statement_groups_match_the_oracle(pair):
             assert np.allclose(got, want, rtol=2e-5, atol=2e-5), seed
 
 
+def _near_twin(be, rs, ts, idx, depth, axis):
+    """small trees from a small vocabulary (five numbers, four tensors): many
+    of them differ from an earlier one only in a number, in the side a number
+    stands on or in one operator"""
+    r = rs.rand()
+    if depth == 0 or r < 0.3:
+        return float(rs.choice([0.5, 1.0, 2.0, -1.5, 3.0])) if rs.rand() < 0.35 else ts[rs.randint(len(ts))]
+    if r < 0.45:
+        a = _near_twin(be, rs, ts, idx, depth - 1, axis)
+        op = rs.choice(["neg", "sqrtabs", "expclip", "tanh", "sq"])
+        return {"neg": lambda: -a, "sqrtabs": lambda: be.sqrt(be.absolute(a)),
+                "expclip": lambda: be.exp(be.minimum(a, 3.0)), "tanh": lambda: be.tanh(a),
+                "sq": lambda: be.square(a)}[op]()
+    if r < 0.9:
+        a, b = _near_twin(be, rs, ts, idx, depth - 1, axis), _near_twin(be, rs, ts, idx, depth - 1, axis)
+        op = rs.choice(["add", "sub", "mul", "div", "gt", "le", "max", "min", "pow"])
+        if op == "div":
+            return be.divide(a, be.absolute(b) + 1.0)
+        if op == "pow":
+            return be.power(be.absolute(a) + 0.5, be.minimum(be.maximum(b, -2.0), 2.0))
+        if op in ("gt", "le"):          # as numbers: numpy would add two boolean arrays as a logical or
+            return {"gt": be.greater, "le": be.less_equal}[op](a, b) * 1.0
+        return {"add": be.add, "sub": be.subtract, "mul": be.multiply, "max": be.maximum, "min": be.minimum}[op](a, b)
+    if rs.rand() < 0.2:
+        return be.onehot(idx, axis=0)
+    a = _near_twin(be, rs, ts, idx, depth - 1, axis)
+    return getattr(be, rs.choice(["sum", "max", "min", "mean"]))(ts[0] * a if isinstance(a, float) else a, axis=axis)
+
+
+def test_many_near_twin_trees_on_the_same_tensors(pair):
+    """one backend instance, one set of tensors, several hundred small trees in
+    a row: plans are found again by key, recorded launches are replayed and
+    re-bound to other numbers -- every result still has to be the tree's own"""
+    from neon_amd.backends.backend import Block
+    cpu, hip = pair
+    R, C = 64, 96
+    rs0 = np.random.RandomState(7)
+    host = [rs0.uniform(-2, 2, shp).astype(np.float32) for shp in ((R, C), (R, C), (R, 1), (1, C))]
+    hidx = rs0.randint(0, R, (1, C)).astype(np.int32)
+    env = {be: ([be.array(h) for h in host], be.array(hidx, dtype=np.int32), be.empty((R, C)), be.empty((R, C)))
+           for be in pair}
+    before = dict(hip.plan_stats)
+    for seed in range(500):
+        res = []
+        for be in (cpu, hip):
+            ts, idx, out, out2 = env[be]
+            rs = np.random.RandomState(seed)
+            axis = int(rs.randint(0, 2))
+            targets = [out] if rs.rand() < 0.7 else [out, out2]
+            fuse = be is hip and len(targets) == 2 and seed % 2 == 0
+            if fuse:
+                be.begin(Block.update, 0)
+            for target in targets:
+                t = _near_twin(be, rs, ts, idx, int(rs.randint(1, 4)), axis)
+                target[:] = ts[0] + t if isinstance(t, float) else t
+            if fuse:
+                be.end(Block.update, 0)
+            res.append([t.get() for t in targets])
+        for want, got in zip(*res):
+            w64 = want.astype(np.float64)
+            finite = np.isfinite(w64)
+            assert np.array_equal(finite, np.isfinite(got)), seed
+            scale = max(1.0, np.abs(w64[finite]).max() if finite.any() else 1.0)
+            err = np.abs(got.astype(np.float64) - w64)
+            err[~finite] = 0
+            assert err.max() / scale <= 3e-6 * C, (seed, err.max() / scale)
+    assert hip.plan_stats["replayed"] > before["replayed"] + 100 and hip.plan_stats["hit"] > before["hit"] + 10
+
+
 def test_random_storage_types_and_small_extents(pair):
     """every storage type on either operand, extents from 1 to 5000 (many of
     them shorter than a vector): elementwise, both reduction axes, float and
