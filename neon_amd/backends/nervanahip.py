@@ -1034,7 +1034,7 @@ class NervanaHIP(Backend):
                 return t, geom[0], geom[1]
         tmp = self._temp(t.shape, t.dtype, temps)
         self._run([OpTreeNode({"op": "assign"}, tmp, t)])
-        return tmp, False, max(cols, 1)
+        return tmp, False, max(t.shape[1], 1)
 
     def _gemm(self, A, B, C, alpha, beta, temps):
         """C = alpha * A.B + beta * C for dense 2-D C (unit column stride)"""

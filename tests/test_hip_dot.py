@@ -95,11 +95,34 @@ def test_compound_dot_views_hip(pair):
         A, B, C = be.array(a), be.array(b), be.array(c)
         # row/column windows of the operands, a column window of the output
         be.compound_dot(A[8:72, 16:64], B[16:64, 4:44], C[8:72, 30:70], alpha=1.0, beta=0.5)
-        # every second row of A is neither dense nor transposed: staged through a copy
+        # every second row of A: read in place with a doubled leading dimension
         be.compound_dot(A[0:64:2, :], B, C[0:32, 0:72])
         res.append(C.get())
     assert_close(res[1], res[0], rtol=1e-5, atol=1e-5 * 80)
     assert np.array_equal(res[1][72:, :], c[72:, :])
+
+
+@pytest.mark.gpu
+def test_compound_dot_operands_staged_through_a_copy(pair):
+    """operands the GEMM cannot read in place: a view strided along both
+    dimensions and a gather view (rows picked by an index tensor)"""
+    cpu, hip = pair
+    rs = np.random.RandomState(6)
+    a, b = _rand(rs, (96, 80)), _rand(rs, (80, 72))
+    rows = rs.randint(0, 96, size=(1, 40)).astype(np.int32)
+    res = []
+    for be in pair:
+        A, B = be.array(a), be.array(b)
+        C1, C2, C3 = be.zeros((48, 72)), be.zeros((40, 72)), be.zeros((96, 36))
+        be.compound_dot(A[0:96:2, 0:80:2], B[0:40, :], C1)
+        be.compound_dot(A.take(be.array(rows, dtype=np.int32), axis=0), B, C2)
+        be.compound_dot(A, B[:, 0:72:2], C3)
+        res.append((C1.get(), C2.get(), C3.get()))
+    want = (a[0:96:2, 0:80:2].astype(np.float64) @ b[0:40], a[rows[0]].astype(np.float64) @ b,
+            a.astype(np.float64) @ b[:, 0:72:2])
+    for got, oracle, w in zip(res[1], res[0], want):
+        assert_close(got, w, rtol=1e-5, atol=1e-5 * 80)
+        assert_close(got, oracle, rtol=1e-5, atol=1e-5 * 80)
 
 
 @pytest.mark.gpu
