@@ -947,7 +947,8 @@ def _emit_col_fold(g, L, n, LX, LY, T, V, src, dst_decl=True):
     row order."""
     op = _RED_OP[n.op]
     VK = V            # values a lane contributes to the LDS stage
-    if LX < 64 and T > 64:
+    assert T > 64, "workgroups of the column families span several waves"
+    if LX < 64:
         # the wave's row-lanes are folded with lane exchanges that split the V
         # values among the lanes; LDS collects the pieces
         steps = (64 // LX).bit_length() - 1
@@ -955,16 +956,6 @@ def _emit_col_fold(g, L, n, LX, LY, T, V, src, dst_decl=True):
         WY = T // 64
         wy = "(threadIdx.x >> 6)"
         writer = "((threadIdx.x & 63) < %d)" % (LX * (V // VK))
-    elif LX < 64:
-        stride = LX
-        while stride < 64:
-            L("#pragma unroll")
-            L("for (int j = 0; j < %d; ++j) %s[j] = %s::f(%s[j], nh_lane_xor<%d>(%s[j]));"
-              % (V, src, op, src, stride, src))
-            stride *= 2
-        WY = T // 64
-        wy = "(threadIdx.x >> 6)"
-        writer = "((threadIdx.x & 63) < %d)" % LX
     else:
         WY = LY
         wy = "ty"

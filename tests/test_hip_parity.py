@@ -83,6 +83,86 @@ def test_numbers_on_either_side_of_an_operator(pair):
             both(pair, f, [a], what=name, atol=1e-5)
 
 
+def test_onehot_along_rows_in_vector_tiles(pair):
+    """onehot(idx, axis=1): one hot column per row, on tiles several elements wide"""
+    rs = np.random.RandomState(22)
+    R, C = 512, 1024
+    x = gen_inputs(rs, (R, C))
+    idx = rs.randint(0, C, size=(R, 1)).astype(np.int32)
+    res = []
+    for be in pair:
+        t, out, picked = be.array(x), be.empty((R, C)), be.empty((R, 1))
+        hot = be.onehot(be.array(idx, dtype=np.int32), axis=1)
+        out[:] = hot * t + 0.5 * t
+        picked[:] = be.sum(hot * t, axis=1)
+        res.append((out.get(), picked.get()))
+    want = x * 0.5
+    want[np.arange(R), idx[:, 0]] += x[np.arange(R), idx[:, 0]]
+    assert_close(res[1][0], want, what="onehot axis 1")
+    assert np.array_equal(res[1][1][:, 0], x[np.arange(R), idx[:, 0]])
+    assert_close(res[1][0], res[0][0])
+    assert_close(res[1][1], res[0][1])
+
+
+@pytest.mark.parametrize("shape,axis", [((300, 4096), 1), ((16, 300000), 1), ((2000, 384), 0), ((40000, 64), 0),
+                                        ((200000, 16), 0), ((64, 96), 0), ((64, 96), 1)])
+def test_index_reductions_broadcast_into_full_tensors(pair, shape, axis):
+    """argmax / argmin stored straight into a tensor of the operand's shape
+    (every row or column repeats the index), float and int32"""
+    rs = np.random.RandomState(23)
+    x = gen_inputs(rs, shape)
+    res = []
+    for be in pair:
+        t = be.array(x)
+        fo, io = be.empty(shape), be.empty(shape, dtype=np.int32)
+        fo[:] = be.argmax(t, axis=axis)
+        io[:] = be.argmin(t, axis=axis)
+        res.append((fo.get(), io.get()))
+    assert np.array_equal(res[1][0], np.broadcast_to(x.argmax(axis=axis, keepdims=True), shape).astype(np.float32))
+    assert np.array_equal(res[1][1], np.broadcast_to(x.argmin(axis=axis, keepdims=True), shape).astype(np.int32))
+    assert np.array_equal(res[1][0], res[0][0]) and np.array_equal(res[1][1], res[0][1])
+
+
+def test_reductions_of_operands_that_do_not_vary_along_the_axis(pair):
+    """a (1,C) operand reduced down the rows, a (R,1) operand reduced along the
+    columns: value reductions return the operand (times the extent for sum),
+    index reductions return zero"""
+    rs = np.random.RandomState(24)
+    R, C = 300, 2000
+    x, row, col = gen_inputs(rs, (R, C)), gen_inputs(rs, (1, C)), gen_inputs(rs, (R, 1))
+    fns = {
+        "argmax row": lambda be, a, r, c: a + be.argmax(r * 2.0, axis=0),
+        "argmin col": lambda be, a, r, c: a - be.argmin(c + 1.0, axis=1),
+        "max row": lambda be, a, r, c: a * be.max(r, axis=0),
+        "min col": lambda be, a, r, c: a * be.min(c, axis=1),
+        "argmax alone": lambda be, a, r, c: be.argmax(r, axis=0) + 0 * r,
+    }
+    for name, f in fns.items():
+        both(pair, f, [x, row, col], what=name)
+
+
+def test_group_with_a_column_shaped_and_a_full_output(pair):
+    """one statement of the group writes a (R,1) tensor, the other a (R,C) one:
+    the narrow store happens once per row"""
+    from neon_amd.backends.backend import Block
+    rs = np.random.RandomState(25)
+    R, C = 257, 1000
+    x, col = gen_inputs(rs, (R, C)), gen_inputs(rs, (R, 1))
+    res = []
+    for be in pair:
+        t, c = be.array(x), be.array(col)
+        narrow, full = be.empty((R, 1)), be.empty((R, C))
+        be.begin(Block.update, 0)
+        narrow[:] = c * 2.0 + 1.0
+        full[:] = t + c
+        be.end(Block.update, 0)
+        res.append((narrow.get(), full.get()))
+    assert_close(res[1][0], col * 2.0 + 1.0)
+    assert_close(res[1][1], x + col)
+    assert_close(res[1][0], res[0][0])
+    assert_close(res[1][1], res[0][1])
+
+
 def test_inplace_and_views(pair):
     rs = np.random.RandomState(3)
     a = gen_inputs(rs, (50, 128))
