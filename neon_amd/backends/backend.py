@@ -42,10 +42,6 @@ class Block(object):
     epoch, minibatch, fprop, bprop, update = list(range(5))
 
 
-def _operand_ok(x):
-    return x is None or isinstance(x, (int, float, Tensor, OpTreeNode))
-
-
 _NO_OPERAND, _SCALAR_SHAPE = (0, 0), (1, 1)
 
 
@@ -70,15 +66,6 @@ def _shape_of_operand(x):
     if len(shp) == 1:
         return (shp[0], 1)
     return shp if type(shp) is tuple else tuple(shp)
-
-
-def _operand_shape(x):
-    if isinstance(x, (Tensor, OpTreeNode)):
-        shp = tuple(x.shape)
-        return shp + (1,) if len(shp) == 1 else shp
-    if isinstance(x, (int, float)):
-        return (1, 1)
-    return (0, 0)
 
 
 class _LazyOperators(object):

@@ -367,3 +367,67 @@ def test_configs_against_float64_truth(cpu):
     configs.c5a_argmax(be, am, be.array(x5))
     assert np.array_equal(am.get().ravel(), x5.argmax(axis=0))
     assert am.get().min() >= 0 and am.get().max() < 2000
+
+
+def test_optree_node_utilities(cpu):
+    """reflected power, !=, infix printing, list round trip, astensor /
+    asnumpyarray, transpose of a node (reference backend.py:1893-2013)"""
+    a = np.array([[1.0, 2.0], [3.0, 0.5]], dtype=np.float32)
+    x = cpu.array(a, name="x")
+    assert np.allclose((2.0 ** x).asnumpyarray(), 2.0 ** a)
+    assert np.array_equal((x != 2.0).asnumpyarray(), (a != 2.0))
+    tree = -(x * 2.0 + x ** 2.0)
+    assert tree.pp() == "(neg ((x * (2.0)) + (x ** (2.0))))"
+    assert str(x + 1.0) == "({'op': 'add', 'shape': (2, 2)}, x, 1.0)"
+    lst = OpTreeNode.optree_to_list(tree)
+    assert isinstance(lst, list) and lst[0]["op"] == "neg" and lst[2] is None and lst[1][1][1] is x
+    back = OpTreeNode.list_to_optree(lst)
+    assert isinstance(back, OpTreeNode) and np.array_equal(back.asnumpyarray(), tree.asnumpyarray())
+    t = tree.astensor()
+    assert t.shape == (2, 2) and np.allclose(t.get(), -(a * 2 + a ** 2))
+    assert np.allclose((x * 2.0).transpose().asnumpyarray(), (a * 2).T)
+    out = cpu.empty((2, 2))
+    (x * 2.0).transpose(out=out)
+    assert np.allclose(out.get(), (a * 2).T)
+    with pytest.raises(ValueError):
+        OpTreeNode.build("add", 1.0, 2.0).astensor()                # no tensor to take a backend from
+    with pytest.raises(TypeError):
+        x + "text"
+
+
+def test_backend_base_helpers(cpu):
+    """window arithmetic (reference backend.py:506-532 with the values its
+    layers rely on), iobuf shapes, skip-node accumulation, compat mode"""
+    from neon_amd.backends.backend import Backend
+    assert cpu.output_dim(224, 7, 3, 2) == 112                      # (224 - 7 + 6) // 2 + 1
+    assert cpu.output_dim(32, 3, 0, 1) == 30 and cpu.output_dim(32, 3, 1, 1) == 32
+    assert cpu.output_dim(28, 3, 0, 1, dilation=2) == 24            # window widened to 5
+    assert cpu.output_dim(13, 3, 0, 2, pooling=True) == 6
+    with pytest.raises(ValueError):
+        cpu.output_dim(13, 3, 3, 2, pooling=True)
+    caffe = Backend.allocate_backend("cpu", rng_seed=0, compat_mode="caffe")
+    assert caffe.check_caffe_compat() and not cpu.check_caffe_compat()
+    assert caffe.output_dim(14, 3, 0, 2, pooling=True) == 7         # ceil((14 - 3) / 2) + 1; plain floor gives 6
+    assert caffe.output_dim(14, 3, 0, 2) == 6                       # convolutions keep the floor
+    assert caffe.output_dim(8, 3, 1, 2, pooling=True) == 5 and caffe.output_dim(7, 2, 1, 2, pooling=True) == 4
+    with pytest.raises(ValueError):
+        Backend.allocate_backend("cpu", rng_seed=0, compat_mode="other")
+    bsz = cpu.bsz
+    assert cpu.iobuf(10).shape == (10, bsz) and cpu.iobuf((10, 4)).shape == (10, 4 * bsz)
+    assert cpu.iobuf((3, 4, 5)).shape == (60, bsz)
+    given = cpu.empty((2, 2))
+    assert cpu.iobuf(10, x=given) is given
+    pool = cpu.zeros((20, bsz))
+    shared = cpu.iobuf(10, shared=pool)
+    assert shared.shape == (10, bsz) and not shared.get().any()
+    x, y = cpu.array(np.full((3, 2), 2.0, np.float32)), cpu.array(np.full((3, 2), 5.0, np.float32))
+    cpu.fprop_skipnode(x, y, beta=0.5)
+    assert np.array_equal(y.get(), np.full((3, 2), 4.5))
+    d = cpu.array(np.full((3, 2), 1.0, np.float32))
+    cpu.bprop_skipnode(x, d, alpha=3.0, beta=2.0)
+    assert np.array_equal(d.get(), np.full((3, 2), 8.0))
+    state = cpu.rng_get_state()
+    first = cpu.rng.uniform(size=3)
+    cpu.rng_set_state(state)
+    assert np.array_equal(cpu.rng.uniform(size=3), first)
+    cpu.rng_reset()
