@@ -466,10 +466,9 @@ def _plan_col(prog, cu_count):
     if not (single_level and line_only):
         # narrow strips keep the partials each workgroup has to gather small
         # (measured on (32000,256): 8 column-lanes 37 us, 16 lanes 43 us, 4 lanes
-        # 41 us); 16 lanes only when 8 would need more strips than compute units
+        # 41 us).  More strips than half the compute units leave no second
+        # workgroup per strip: such widths go to the families below
         lxc = max(1, min(8, _pow2ceil(nvec)))
-        if _ceil_div(nvec, lxc) > cu_count:
-            lxc = max(1, min(16, _pow2ceil(nvec)))
         strips_c = _ceil_div(nvec, lxc)
         if strips_c <= cu_count:
             chunks = max(1, min(128, cu_count // strips_c))
