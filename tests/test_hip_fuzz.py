@@ -209,6 +209,53 @@ def test_many_near_twin_trees_on_the_same_tensors(pair):
     assert hip.plan_stats["replayed"] > before["replayed"] + 100 and hip.plan_stats["hit"] > before["hit"] + 10
 
 
+def test_near_twin_trees_over_operands_in_many_layouts(pair):
+    """operands: dense, window of a larger tensor, transposed view, fp16, column,
+    row, 1x1 and a one-column window; results into a dense tensor, a window, a
+    transposed view or an fp16 tensor -- 300 trees in a row on one instance"""
+    cpu, hip = pair
+    R, C = 40, 56
+    rs0 = np.random.RandomState(11)
+    u = lambda *shp: rs0.uniform(-2, 2, shp).astype(np.float32)
+    host = dict(x=u(R, C), big=u(R + 3, C + 5), zt=u(C, R), h=u(R, C).astype(np.float16), col=u(R, 1), row=u(1, C),
+                one=u(1, 1), bigcol=u(R + 2, 3))
+    hidx = rs0.randint(0, R, (1, C)).astype(np.int32)
+    env = {}
+    for be in pair:
+        # the oracle computes in fp32 on exact copies of the fp16 operand
+        put = (lambda a: be.array(a.astype(np.float32))) if be is cpu else (lambda a: be.array(a, dtype=a.dtype))
+        t = {k: put(v) for k, v in host.items()}
+        leaves = [t["x"], t["big"][1:R + 1, 2:C + 2], t["zt"].T, t["h"], t["col"], t["row"], t["one"],
+                  t["bigcol"][1:R + 1, 1:2]]
+        outs = dict(dense=be.empty((R, C)), big=be.zeros((R + 2, C + 4)), t=be.zeros((C, R)),
+                    half=be.empty((R, C), dtype=np.float32 if be is cpu else np.float16))
+        env[be] = (leaves, be.array(hidx, dtype=np.int32), outs)
+    for seed in range(300):
+        res = []
+        for be in pair:
+            leaves, idx, outs = env[be]
+            rs = np.random.RandomState(seed)
+            axis = int(rs.randint(0, 2))
+            tree = _near_twin(be, rs, leaves, idx, int(rs.randint(1, 4)), axis)
+            tree = (leaves[0] + tree if isinstance(tree, float) else tree) + 0.0 * leaves[0]       # full shape
+            kind = rs.choice(["dense", "big", "t", "half"])
+            if kind == "big":
+                outs["big"][1:R + 1, 3:C + 3] = tree
+            elif kind == "t":
+                outs["t"].T[:] = tree
+            else:
+                outs[kind][:] = tree
+            res.append(outs[kind].get().astype(np.float32))
+        want, got = res
+        w64 = want.astype(np.float64)
+        finite = np.isfinite(w64)
+        assert np.array_equal(finite, np.isfinite(got)), (seed, kind)
+        scale = max(1.0, np.abs(w64[finite]).max() if finite.any() else 1.0)
+        err = np.abs(got.astype(np.float64) - w64)
+        err[~finite] = 0
+        assert err.max() / scale <= (1.5e-3 if kind == "half" else 3e-6 * C), (seed, kind, err.max() / scale)
+
+
 def test_random_storage_types_and_small_extents(pair):
     """every storage type on either operand, extents from 1 to 5000 (many of
     them shorter than a vector): elementwise, both reduction axes, float and
