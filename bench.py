@@ -178,22 +178,6 @@ def gpu_leg(steps, warmup, detail=True):
             reps=20)
     measure("C3 Adam as 3 assigns, 3 kernels (5000,5000) f32",
             lambda: configs.c3_adam_step(be, p, g, m, v, t + 2), configs.bytes_c3(fused=False), n3, reps=20)
-    # the same update through the optimizer class (what a model's training loop calls)
-    from neon_amd.optimizers import Adam
-
-    class _Params(object):
-        def __init__(self, plist):
-            self.plist = plist
-
-        def get_params(self):
-            return self.plist
-
-    adam = Adam(learning_rate=configs.ADAM["lr"], beta_1=configs.ADAM["beta1"], beta_2=configs.ADAM["beta2"],
-                epsilon=configs.ADAM["eps"])
-    adam.be = be
-    layer = _Params([((p, g), [m, v])])
-    measure("C3 Adam.optimize (optimizer class), 1 kernel (5000,5000) f32", lambda: adam.optimize([layer], 0),
-            configs.bytes_c3(fused=True), n3, reps=20)
     # C4
     x4h, gh, bh = configs.inputs_c4()
     x4, o4 = be.array(x4h, dtype=np.float16), be.empty(configs.C4_SHAPE, dtype=np.float16)

@@ -8,58 +8,41 @@ import os
 import numpy as np
 import pytest
 
-from neon_amd import NervanaObject
 from neon_amd.backends.autodiff import Autodiff
-from neon_amd.optimizers import Adam
-from neon_amd.transforms import (CrossEntropyBinary, CrossEntropyMulti, Logistic, MeanSquared,
-                                 Misclassification, PrecisionRecall, Rectlin, Softmax, SumSquared, Tanh)
+import clients
 
 with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "known_answers.json")) as _f:
     CASES = json.load(_f)["cases"]
 
 
 @contextlib.contextmanager
-def _using(be, bsz):
-    old, old_bsz = NervanaObject.be, be.bsz
-    NervanaObject.be, be.bsz = be, bsz
+def _batch(be, bsz):
+    old = be.bsz
+    be.bsz = bsz
     try:
         yield
     finally:
-        NervanaObject.be, be.bsz = old, old_bsz
-
-
-class _Layer(object):
-    def __init__(self, plist):
-        self.plist = plist
-
-    def get_params(self):
-        return self.plist
+        be.bsz = old
 
 
 def _evaluate(be, case):
     kind = case["kind"]
     arrays = [np.asarray(a, dtype=np.float32) for a in case["inputs"]]
     tensors = [be.array(a) for a in arrays]
-    batch = arrays[0].shape[1]
-    with _using(be, batch):
-        act = {"softmax_axis0": lambda: Softmax(), "tanh": lambda: Tanh(), "sig": lambda: Logistic(),
-               "relu": lambda: Rectlin(slope=case.get("slope", 0))}
-        cost = {"ce_binary": CrossEntropyBinary, "ce_multi": CrossEntropyMulti, "sum_squared": SumSquared,
-                "mean_squared": MeanSquared}
-        if kind in act:
-            tree = act[kind]()(tensors[0])
-            out = be.empty(tree.shape)
-            out[:] = tree
-            return out.get()
-        if kind in cost:
-            tree = cost[kind]()(*tensors)
+    trees = {"softmax_axis0": clients.softmax, "tanh": clients.tanh, "sig": clients.logistic,
+             "relu": lambda be_, x: clients.rectlin(be_, x, case.get("slope", 0)),
+             "ce_binary": clients.cross_entropy_binary, "ce_multi": clients.cross_entropy_multi,
+             "sum_squared": clients.sum_squared, "mean_squared": clients.mean_squared}
+    with _batch(be, arrays[0].shape[1]):
+        if kind in trees:
+            tree = trees[kind](be, *tensors)
             out = be.empty(tree.shape)
             out[:] = tree
             return out.get()
         if kind == "misclassification":
-            return np.array([[Misclassification()(*tensors)]])
+            return np.array([[clients.misclassification(be, *tensors)]])
         if kind == "precision_recall":
-            return PrecisionRecall(arrays[0].shape[0])(*tensors)
+            return clients.precision_recall(be, *tensors)
         if kind == "autodiff_poly":
             x0, x1, x2, x3 = tensors
             f = x0 * x0 - x1 * x0 + x0 * x2 - x2 * x1 * x0 + x3 * x3 * x3
@@ -71,9 +54,8 @@ def _evaluate(be, case):
             prm = case["params"]
             be.bsz = prm["bsz"]
             p, g, m, v = tensors
-            opt = Adam(learning_rate=prm["lr"], beta_1=prm["beta_1"], beta_2=prm["beta_2"], epsilon=prm["epsilon"])
-            opt.be = be
-            opt.optimize([_Layer([((p, g), [m, v])])], epoch=0)
+            clients.adam_update(be, p, g, m, v, 1, lr=prm["lr"], b1=prm["beta_1"], b2=prm["beta_2"],
+                                eps=prm["epsilon"])
             return p.get()
     raise AssertionError("unknown case kind %s" % kind)
 

@@ -1,0 +1,121 @@
+"""Parameter-update statement groups (the bodies of the reference's optimizers,
+neon/optimizers/optimizer.py, written from their formulas in tests/clients.py)
+between ``be.begin(Block.update)`` / ``be.end(Block.update)``: each rule against
+a float64 numpy restatement on the oracle (the idiom of the reference's
+tests/test_optimizer.py:280-299), and on the GPU against the oracle, where the
+whole group must run as ONE fused kernel."""
+import numpy as np
+import pytest
+
+import clients
+from utils import assert_close
+
+SHAPE = (37, 53)
+
+
+def _np_adam(p, g, m, v, t, bsz, lr=1e-3, b1=0.9, b2=0.999, eps=1e-8):
+    g = g / bsz
+    m = m * b1 + (1 - b1) * g
+    v = v * b2 + (1 - b2) * g * g
+    p = p - (lr * np.sqrt(1 - b2 ** t) / (1 - b1 ** t)) * m / (np.sqrt(v) + eps)
+    return p, m, v
+
+
+def _np_momentum(p, g, vel, bsz, lr=0.1, mom=0.9, wd=0.0005):
+    vel = mom * vel - lr * (g / bsz + wd * p)
+    return p + vel, vel
+
+
+def _np_rmsprop(p, g, s, bsz, lr=2e-3, decay=0.95, eps=1e-6):
+    g = g / bsz
+    s = decay * s + g * g * (1 - decay)
+    return p - g * lr / (np.sqrt(s + eps) + eps), s
+
+
+def _np_adadelta(p, g, gsq, dsq, bsz, decay=0.95, eps=1e-6):
+    g = g / bsz
+    gsq = gsq * decay + (1 - decay) * g * g
+    d = np.sqrt((dsq + eps) / (gsq + eps)) * g
+    dsq = dsq * decay + (1 - decay) * d * d
+    return p - d, gsq, dsq, d
+
+
+def _draw(nstates, seed=0, shape=SHAPE):
+    rs = np.random.RandomState(seed)
+    p = rs.standard_normal(shape).astype(np.float32)
+    g = (rs.standard_normal(shape) * 0.1).astype(np.float32)
+    states = [np.abs(rs.standard_normal(shape) * 0.01).astype(np.float32) for _ in range(nstates)]
+    return p, g, states
+
+
+def _apply(be, rule, steps=3, seed=0, shape=SHAPE, dtype=np.float32, quantise=None):
+    nstates = {"adam": 2, "momentum": 1, "rmsprop": 1, "adadelta": 3}[rule]
+    p, g, st = _draw(nstates, seed, shape)
+    if quantise is not None:
+        p, g, st = p.astype(quantise), g.astype(quantise), [s.astype(quantise) for s in st]
+    P, G = be.array(p, dtype=dtype), be.array(g, dtype=dtype)
+    S = [be.array(s, dtype=dtype) for s in st]
+    for t in range(1, steps + 1):
+        if rule == "adam":
+            clients.adam_update(be, P, G, S[0], S[1], t)
+        elif rule == "momentum":
+            clients.momentum_update(be, P, G, S[0])
+        elif rule == "rmsprop":
+            clients.rmsprop_update(be, P, G, S[0])
+        else:
+            clients.adadelta_update(be, P, G, S[0], S[1], S[2])
+    return [P.get()] + [s.get() for s in S]
+
+
+def _expected(rule, steps=3, seed=0, bsz=128):
+    nstates = {"adam": 2, "momentum": 1, "rmsprop": 1, "adadelta": 3}[rule]
+    p, g, st = _draw(nstates, seed)
+    p, g = p.astype(np.float64), g.astype(np.float64)
+    st = [s.astype(np.float64) for s in st]
+    for t in range(1, steps + 1):
+        if rule == "adam":
+            p, st[0], st[1] = _np_adam(p, g, st[0], st[1], t, bsz)
+        elif rule == "momentum":
+            p, st[0] = _np_momentum(p, g, st[0], bsz)
+        elif rule == "rmsprop":
+            p, st[0] = _np_rmsprop(p, g, st[0], bsz)
+        else:
+            p, st[0], st[1], st[2] = _np_adadelta(p, g, st[0], st[1], bsz)
+    return [p] + st
+
+
+RULES = ["adam", "momentum", "rmsprop", "adadelta"]
+
+
+@pytest.mark.parametrize("rule", RULES)
+def test_rule_matches_float64_numpy_on_the_oracle(cpu, rule):
+    for got, want in zip(_apply(cpu, rule), _expected(rule)):
+        assert_close(got, want.astype(np.float32), rtol=2e-5, atol=1e-7, what=rule)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rule", RULES)
+def test_rule_hip_matches_oracle_as_one_kernel(pair, rule):
+    cpu, hip = pair
+    want = _apply(cpu, rule, shape=(300, 257), seed=3)
+    before = hip.plan_stats["launches"]
+    got = _apply(hip, rule, shape=(300, 257), seed=3)
+    assert hip.plan_stats["launches"] - before == 3, "each update group must be a single launch"
+    for g, w in zip(got, want):
+        assert_close(g, w, rtol=1e-5, atol=1e-7, what=rule)
+
+
+@pytest.mark.gpu
+def test_adam_fp16_parameters_hip_matches_oracle(pair):
+    """fp16 storage, fp32 arithmetic: the oracle evaluates the step in fp32 on
+    the fp16-quantised inputs (numpy would compute fp16 operands in fp16) and
+    its results are rounded to fp16 once, like the device's stores"""
+    cpu, hip = pair
+    want = _apply(cpu, "adam", steps=1, shape=(64, 520), seed=5, quantise=np.float16)
+    got = _apply(hip, "adam", steps=1, shape=(64, 520), seed=5, dtype=np.float16)
+    for g, w in zip(got, want):
+        assert g.dtype == np.float16
+        # the parameter is computed from m and v after THEIR rounding to fp16 on the
+        # device (a later statement reads what an earlier one stored): 1e-3 relative
+        assert_close(g.astype(np.float32), w.astype(np.float16).astype(np.float32), rtol=1e-3, atol=1e-6,
+                     what="adam f16")
