@@ -12,7 +12,11 @@ import numpy as np
 
 from neon_amd import NervanaObject
 from neon_amd.backends.backend import Backend, Block, OpTreeNode, OpCollection, Tensor  # noqa: F401
-from neon_amd.backends import nervanahip  # noqa: F401  (registers 'hip')
+from neon_amd.backends import nervanahip
+
+# registers 'hip' in this package's own registry; a host package (neon) binds the
+# backend to ITS classes instead -- see nervanahip.bind
+NervanaHIP, HIPTensor = nervanahip.bind(Backend, OpTreeNode, Tensor, Block)
 
 _atexit_registered = False
 

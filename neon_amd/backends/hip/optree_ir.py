@@ -30,7 +30,6 @@ import math
 
 import numpy as np
 
-from neon_amd.backends.backend import OpCollection, Tensor
 
 UNARY = {"neg", "abs", "sgn", "sqrt", "sqr", "exp", "log", "exp2", "log2", "sig",
          "sig2", "tanh", "tanh2", "safelog", "rint", "finite"}
@@ -136,6 +135,12 @@ def eval_const(expr, raw):
     if tag == "1":
         return _fold_unary(expr[1], eval_const(expr[2], raw))
     return _fold_binary(expr[1], eval_const(expr[2], raw), eval_const(expr[3], raw))
+
+
+def is_tensor(x):
+    """a tensor operand, of whatever package's ``Tensor`` class the backend was
+    bound to: anything that carries a device address and element strides"""
+    return hasattr(x, "ptr") and hasattr(x, "strides")
 
 
 class MixedAxes(ValueError):
@@ -314,21 +319,21 @@ class Program(object):
         """Append ``assign(out, expr)`` given as an OpTreeNode."""
         assert optree[0]["op"] == "assign"
         out_t, value = optree[1], optree[2]
-        if not isinstance(out_t, Tensor):
+        if not is_tensor(out_t):
             raise TypeError("assignment target must be a tensor")
         out_slot = self.tensor_slot(out_t)
         stack = []
         postfix = []
         if isinstance(value, (int, float)):
             postfix = [value]
-        elif isinstance(value, Tensor):
+        elif is_tensor(value):
             postfix = [value]
         else:
             value.traverse(postfix)
         for p in postfix:
             if isinstance(p, dict):
                 self._apply(p, stack)
-            elif isinstance(p, Tensor):
+            elif is_tensor(p):
                 stack.append(self._read_tensor(p))
             elif isinstance(p, (int, float)):
                 stack.append(Num(float(p), ("r", self.raw_count)))      # folded lazily

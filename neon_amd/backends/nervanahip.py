@@ -17,7 +17,7 @@ import struct
 
 import numpy as np
 
-from neon_amd.backends.backend import Backend, OpTreeNode, Tensor
+from neon_amd.backends import backend as _own
 from neon_amd.backends.hip import runtime as hiprt
 from neon_amd.backends.hip.optree_ir import MixedAxes, Program, REDUCE, eval_const
 from neon_amd.backends.hip.planner import KernelCache, NeedsSplit, make_plan
@@ -57,15 +57,22 @@ def _reshape_strides(strides, shape, new_shape):
     return tuple(strides[:matched]) + _contiguous_strides(new_shape[matched:])
 
 
-class HIPTensor(Tensor):
+class HIPTensorBase(object):
     """Device tensor: a pointer into an allocation plus shape and element
     strides; indexing produces views (reference GPUTensor,
-    nervanagpu.py:48-659)."""
+    nervanagpu.py:48-659).
+
+    This is the implementation half of the tensor class: ``bind`` combines it
+    with the ``Tensor`` base of the package that hosts the backend (this one,
+    or neon itself), which supplies the lazy operators.  ``_api`` names the
+    classes of that package."""
+    _api = None
+    _min_dims = 2
 
     def __init__(self, backend, shape=None, dtype=np.float32, name=None,
                  persist_values=True, base=None, gpudata=None, strides=None,
                  take_array=None, is_trans=False, rounding=0):
-        super(HIPTensor, self).__init__(backend, shape, dtype, name, persist_values)
+        super(HIPTensorBase, self).__init__(backend, shape, dtype, name, persist_values)
         dtype = np.dtype(dtype)
         assert dtype.type in _DTYPES, "unsupported dtype %s" % dtype
         if not isinstance(shape, (tuple, list)):
@@ -156,7 +163,7 @@ class HIPTensor(Tensor):
                 offset += self.strides[aa] * start * self.dtype.itemsize
                 ia += 1
                 aa += 1
-            elif isinstance(entry, (HIPTensor, np.ndarray, list, tuple)):
+            elif isinstance(entry, (HIPTensorBase, np.ndarray, list, tuple)):
                 if isinstance(entry, (list, tuple)):
                     entry = np.array(entry, dtype=np.int32)
                 if isinstance(entry, np.ndarray):
@@ -220,16 +227,16 @@ class HIPTensor(Tensor):
                         {1: np.uint8, 2: np.uint16, 4: np.uint32}[self.dtype.itemsize])[0]
                     be.rt.memset(self.gpudata, int(bits), self.size, self.dtype.itemsize)
             else:
-                OpTreeNode.build("assign", self, value)
-        elif isinstance(value, HIPTensor):
+                self._api.OpTreeNode.build("assign", self, value)
+        elif isinstance(value, HIPTensorBase):
             if (self.is_contiguous and value.is_contiguous and self.dtype == value.dtype and
                     self.shape == value.shape and not be._fusing):
                 if self.nbytes:
                     be.rt.memcpy_d2d(self.gpudata, value.gpudata, self.nbytes)
             else:
-                OpTreeNode.build("assign", self, value)
-        elif isinstance(value, OpTreeNode):
-            OpTreeNode.build("assign", self, value)
+                self._api.OpTreeNode.build("assign", self, value)
+        elif isinstance(value, self._api.OpTreeNode):
+            self._api.OpTreeNode.build("assign", self, value)
         elif isinstance(value, np.ndarray):
             self.set(value)
         else:
@@ -330,7 +337,7 @@ class HIPTensor(Tensor):
 
     def transpose(self, out=None):
         if out:
-            return OpTreeNode.build("assign", out, self.T)
+            return self._api.OpTreeNode.build("assign", out, self.T)
         return self.T
 
     def hist(self, tag):
@@ -431,16 +438,16 @@ class _CaptureScope(object):
         return False
 
 
-class NervanaHIP(Backend):
-    """MI355X backend for the op-tree path.
+class NervanaHIPBase(object):
+    """MI355X backend for the op-tree path (implementation half; ``bind``
+    derives the registered backend class from it and from the ``Backend`` base
+    of the hosting package, whose op builders it then inherits).
 
     Arguments mirror ``gen_backend``'s keyword set (reference
     neon/backends/__init__.py:107-114).  ``stochastic_round`` must be False,
     as the reference insists: stochastic rounding is requested per tensor
     through its ``rounding`` attribute (mantissa bits, or True for 10).
     """
-    backend_name = "hip"
-
     def __init__(self, rng_seed=None, default_dtype=np.float32, stochastic_round=False,
                  deterministic=None, device_id=0, bench=False, scratch_size=0,
                  hist_bins=64, hist_offset=-48, compat_mode=None, num_devices=None,
@@ -454,8 +461,8 @@ class NervanaHIP(Backend):
         self.rt = hiprt.Runtime(device_id or 0)       # raises if library or device is missing
         if not self.rt.arch.startswith("gfx950"):
             logger.warning("hip backend is written for gfx950; found %s", self.rt.arch)
-        super(NervanaHIP, self).__init__(rng_seed, default_dtype, compat_mode=compat_mode)
-        self.tensor_cls = HIPTensor
+        super(NervanaHIPBase, self).__init__(rng_seed, default_dtype, compat_mode=compat_mode)
+        self._min_dims = 2
         self.device_type = 1
         self.device_id = device_id or 0
         self.round_mode = None
@@ -547,7 +554,7 @@ class NervanaHIP(Backend):
 
     def rand(self, out=None):
         """uniform [0, 1) as an op-tree leaf"""
-        return OpTreeNode.build("rand", None, None, out=out)
+        return self._api.OpTreeNode.build("rand", None, None, out=out)
 
     def _uniform_like(self, ary):
         return self.rand()          # drawn inside the kernel that consumes it
@@ -571,7 +578,7 @@ class NervanaHIP(Backend):
     def empty(self, shape, dtype=None, name=None, persist_values=True,
               parallel=False, distributed=False, allocator=None):
         dtype = self.default_dtype if dtype is None else dtype
-        return HIPTensor(self, shape, dtype=dtype, name=name, persist_values=persist_values)
+        return self.tensor_cls(self, shape, dtype=dtype, name=name, persist_values=persist_values)
 
     def array(self, ary, dtype=None, name=None, persist_values=True,
               parallel=False, distributed=False, allocator=None):
@@ -581,7 +588,7 @@ class NervanaHIP(Backend):
             ary = ary.reshape(ary.size, 1)
         if ary.dtype != np.dtype(dtype):
             ary = ary.astype(dtype)
-        return HIPTensor(self, ary.shape, dtype=dtype, name=name,
+        return self.tensor_cls(self, ary.shape, dtype=dtype, name=name,
                          persist_values=persist_values).set(ary)
 
     def zeros(self, shape, dtype=None, name=None, persist_values=True,
@@ -593,7 +600,7 @@ class NervanaHIP(Backend):
         return self.empty(shape, dtype, name, persist_values)._assign(1)
 
     def empty_like(self, other_ary, name=None, persist_values=True):
-        return HIPTensor(self, other_ary.shape, dtype=other_ary.dtype, name=name,
+        return self.tensor_cls(self, other_ary.shape, dtype=other_ary.dtype, name=name,
                          persist_values=persist_values)
 
     def zeros_like(self, other_ary, name=None, persist_values=True):
@@ -626,14 +633,12 @@ class NervanaHIP(Backend):
     def begin(self, block, identifier):
         """``Block.update`` opens a fusion group (the reference documents
         begin/end as optimisation hints, backend.py:671-709)."""
-        from neon_amd.backends.backend import Block
-        if block == Block.update:
+        if block == self._api.Block.update:
             self._fuse_depth += 1
             self._fusing = True
 
     def end(self, block, identifier):
-        from neon_amd.backends.backend import Block
-        if block == Block.update and self._fuse_depth > 0:
+        if block == self._api.Block.update and self._fuse_depth > 0:
             self._fuse_depth -= 1
             if self._fuse_depth == 0:
                 self._fusing = False
@@ -660,12 +665,13 @@ class NervanaHIP(Backend):
         if self._pending and self._pending[0][1].shape != shape:
             return False
         not_fusable = self._NOT_FUSABLE
+        tensor_cls = self.tensor_cls
         for p in post:
             tp = type(p)
             if tp is dict:
                 if p["op"] in not_fusable:
                     return False
-            elif tp is HIPTensor:
+            elif tp is tensor_cls:
                 if p.size == 1 and p.is_contiguous:
                     ptr = p.gpudata
                     if ptr == out.gpudata or any(ptr == q[1].gpudata for q in self._pending):
@@ -698,6 +704,7 @@ class NervanaHIP(Backend):
         arguments."""
         parts, raw = [], []
         add = parts.append
+        tensor_cls = self.tensor_cls
         for k, tree in enumerate(trees):
             if tree[1].rounding:
                 raise TypeError("stochastically rounded stores are never replayed")
@@ -712,7 +719,7 @@ class NervanaHIP(Backend):
                             add((p["op"], p["axis"]))
                     else:
                         add(p["op"])
-                elif type(p) is HIPTensor:
+                elif type(p) is tensor_cls:
                     add(p._geom)
                 else:
                     add(None)
@@ -812,15 +819,15 @@ class NervanaHIP(Backend):
                     self._run([t])
                 return
             out, expr = trees[0][1], trees[0][2]
-            if out.rounding and isinstance(expr, OpTreeNode):
+            if out.rounding and isinstance(expr, self._api.OpTreeNode):
                 # a stochastically rounded store needs one value per element of
                 # the kernel's domain: evaluate into a float32 temporary of the
                 # output's shape first, then round while copying
                 temps = []
                 try:
                     tmp = self._temp(out.shape, np.float32, temps)
-                    self._run([OpTreeNode({"op": "assign"}, tmp, expr)])
-                    self._run([OpTreeNode({"op": "assign"}, out, tmp)])
+                    self._run([self._api.OpTreeNode({"op": "assign"}, tmp, expr)])
+                    self._run([self._api.OpTreeNode({"op": "assign"}, out, tmp)])
                 finally:
                     for t in temps:
                         self._temp_release(t)
@@ -898,16 +905,16 @@ class NervanaHIP(Backend):
         dense temporary first (``out[:] = x.T`` goes straight into ``out``).
         Returns True when the tree was run that way."""
         out, expr = tree[1], tree[2]
-        if isinstance(expr, HIPTensor):
+        if isinstance(expr, HIPTensorBase):
             leaves = [expr]
-        elif isinstance(expr, OpTreeNode):
-            leaves = [p for p in expr.traverse(list()) if isinstance(p, HIPTensor)]
+        elif isinstance(expr, self._api.OpTreeNode):
+            leaves = [p for p in expr.traverse(list()) if isinstance(p, HIPTensorBase)]
         else:
             return False
         views = dict((id(t), t) for t in leaves if _is_large_transposed_view(t))
         if not views:
             return False
-        if (expr is leaves[0] and isinstance(expr, HIPTensor) and out.is_contiguous and not out.rounding
+        if (expr is leaves[0] and isinstance(expr, HIPTensorBase) and out.is_contiguous and not out.rounding
                 and out.dtype == expr.dtype and out.shape == expr.shape and out.gpudata != expr.gpudata):
             self._strided_copy(out, expr)
             return True
@@ -919,11 +926,11 @@ class NervanaHIP(Backend):
                 self._strided_copy(dense[key], t)
 
             def swap(node):
-                if isinstance(node, OpTreeNode):
-                    return OpTreeNode(node[0], swap(node[1]), swap(node[2]))
+                if isinstance(node, self._api.OpTreeNode):
+                    return self._api.OpTreeNode(node[0], swap(node[1]), swap(node[2]))
                 return dense.get(id(node), node)
 
-            self._run([OpTreeNode({"op": "assign"}, out, swap(expr))])
+            self._run([self._api.OpTreeNode({"op": "assign"}, out, swap(expr))])
         finally:
             for t in temps:
                 self._temp_release(t)
@@ -940,7 +947,7 @@ class NervanaHIP(Backend):
         memo = {}
 
         def lower(node, top=False):
-            if not isinstance(node, OpTreeNode):
+            if not isinstance(node, self._api.OpTreeNode):
                 return node
             op = node[0]["op"]
             left = lower(node[1])
@@ -950,27 +957,27 @@ class NervanaHIP(Backend):
                 # temporaries, the product goes through the GEMM hand-off
                 ops = []
                 for side in (left, right):
-                    if isinstance(side, OpTreeNode):
+                    if isinstance(side, self._api.OpTreeNode):
                         tmp = self._temp(side.shape, np.float32, temps)
-                        self._run([OpTreeNode({"op": "assign"}, tmp, side)])
+                        self._run([self._api.OpTreeNode({"op": "assign"}, tmp, side)])
                         side = tmp
                     ops.append(side)
                 if ops[0].dtype != ops[1].dtype:
                     for i, side in enumerate(ops):
                         if side.dtype != np.float32:
                             tmp = self._temp(side.shape, np.float32, temps)
-                            self._run([OpTreeNode({"op": "assign"}, tmp, side)])
+                            self._run([self._api.OpTreeNode({"op": "assign"}, tmp, side)])
                             ops[i] = tmp
                 tmp = self._temp(node[0]["shape"], ops[0].dtype, temps)
                 self._gemm(ops[0], ops[1], tmp, 1.0, 0.0, temps)
                 return tmp
             if op == "transpose":
-                if isinstance(left, HIPTensor):
+                if isinstance(left, HIPTensorBase):
                     return left.T
                 tmp = self._temp(left.shape, np.float32, temps)
-                self._run([OpTreeNode({"op": "assign"}, tmp, left)])
+                self._run([self._api.OpTreeNode({"op": "assign"}, tmp, left)])
                 return tmp.T
-            rebuilt = OpTreeNode(node[0], left, right)
+            rebuilt = self._api.OpTreeNode(node[0], left, right)
             if op in REDUCE:
                 if top:
                     return rebuilt
@@ -978,14 +985,14 @@ class NervanaHIP(Backend):
                 if k in memo:
                     return memo[k]
                 tmp = self._temp(node[0]["shape"], np.float32, temps)
-                self._run([OpTreeNode({"op": "assign"}, tmp, rebuilt)])
+                self._run([self._api.OpTreeNode({"op": "assign"}, tmp, rebuilt)])
                 memo[k] = tmp
                 return tmp
             return rebuilt
 
         try:
             lowered = lower(expr, top=True)
-            self._run_leaf(OpTreeNode({"op": "assign"}, out, lowered))
+            self._run_leaf(self._api.OpTreeNode({"op": "assign"}, out, lowered))
         finally:
             for t in temps:
                 self._temp_release(t)
@@ -1012,7 +1019,7 @@ class NervanaHIP(Backend):
     def _temp(self, shape, dtype, temps):
         key = (tuple(shape), np.dtype(dtype))
         pool = self._temp_pool.setdefault(key, [])
-        t = pool.pop() if pool else HIPTensor(self, shape, dtype=dtype)
+        t = pool.pop() if pool else self.tensor_cls(self, shape, dtype=dtype)
         temps.append(t)
         if self._rec_temps is not None:
             self._rec_temps.append(t)      # recorded launches point into it: keep it allocated
@@ -1033,7 +1040,7 @@ class NervanaHIP(Backend):
             if geom is not None:
                 return t, geom[0], geom[1]
         tmp = self._temp(t.shape, t.dtype, temps)
-        self._run([OpTreeNode({"op": "assign"}, tmp, t)])
+        self._run([self._api.OpTreeNode({"op": "assign"}, tmp, t)])
         return tmp, False, max(t.shape[1], 1)
 
     def _gemm(self, A, B, C, alpha, beta, temps):
@@ -1053,7 +1060,7 @@ class NervanaHIP(Backend):
         CPU statement order nervanacpu.py:906-960).  The product is the library
         GEMM's, the ReLU / beta / row-sum epilogues are op-tree kernels."""
         for t in (A, B, C):
-            assert isinstance(t, HIPTensor) and len(t.shape) == 2, "compound_dot takes 2-D tensors"
+            assert isinstance(t, HIPTensorBase) and len(t.shape) == 2, "compound_dot takes 2-D tensors"
         assert A.dtype == B.dtype == C.dtype
         assert C.dtype.type in (np.float32, np.float16), "compound_dot takes float32 or float16 tensors"
         assert A.shape[0] == C.shape[0]
@@ -1140,7 +1147,7 @@ class NervanaHIP(Backend):
         (nervanacpu.py:1762-1782, which like this ignores alpha / beta); done
         as the reference's deterministic path does it (nervanagpu.py:2591-2660):
         transpose the error, sort the positions by word id, sum every run."""
-        assert isinstance(inputs, HIPTensor) and inputs.dtype == np.int32, "word ids must be an int32 tensor"
+        assert isinstance(inputs, HIPTensorBase) and inputs.dtype == np.int32, "word ids must be an int32 tensor"
         assert error.dtype == error_t.dtype == dW.dtype and dW.dtype.type in (np.float32, np.float16)
         count = inputs.size
         embed, vocab = dW.shape[1], dW.shape[0]
@@ -1218,7 +1225,7 @@ class NervanaHIP(Backend):
         # second handles on the same memory: reads through them see the values
         # from before the update even after `sum_tensor` has been assigned
         def alias(t):
-            return HIPTensor(backend=self, shape=t.shape, dtype=t.dtype, base=t, gpudata=t.gpudata,
+            return self.tensor_cls(backend=self, shape=t.shape, dtype=t.dtype, base=t, gpudata=t.gpudata,
                              strides=t.strides, name=t.name)
         old_sum, old_cmp = alias(sum_tensor), alias(cmp_tensor)
         y = add_tensor * add_scale - old_cmp * cmp_scale
@@ -1229,10 +1236,9 @@ class NervanaHIP(Backend):
             self._originals = frozenset()
 
     # -- batch normalisation as fused statement groups -------------------------------------------
-    @staticmethod
-    def _stmt(out, value):
+    def _stmt(self, out, value):
         """an assign tree that has not been executed"""
-        return OpTreeNode({"op": "assign"}, out, value)
+        return self._api.OpTreeNode({"op": "assign"}, out, value)
 
     def _run_group(self, trees):
         """run statements as one kernel when the families allow it, otherwise
@@ -1306,7 +1312,7 @@ class NervanaHIP(Backend):
             self.hist_map = dict()
             self.hist_idx = 0
             self.hist_max = 4 * 4096
-            self.hist_base = HIPTensor(self, (self.hist_max, self.hist_bins), dtype=np.int32)
+            self.hist_base = self.tensor_cls(self, (self.hist_max, self.hist_bins), dtype=np.int32)
             self.hist_base._assign(0)
 
     def _hist_tensor(self, tag):
@@ -1328,6 +1334,90 @@ class NervanaHIP(Backend):
         self.hist_map = dict()
         self.hist_idx = 0
         return data, hist_map
+
+
+    # -- layer kernels outside the op-tree path (abstract in the reference's base class,
+    #    backend.py:1640-1680 and abstract_backend.py; here they refuse) -----------------
+    def _outside(self, *args, **kwargs):
+        raise NotImplementedError("convolution and pooling kernels are outside the op-tree path of the hip backend")
+
+    conv_layer = fprop_conv = bprop_conv = update_conv = deconv_layer = _outside
+    pool_layer = fprop_pool = bprop_pool = _outside
+
+
+# Helpers that the reference's concrete backends define themselves rather than
+# inherit (nervanacpu.py:1810-1959, nervanagpu.py:3120-3231): all of them are
+# compositions of op builders, written once in this package's base class and
+# given to the backend class whatever base it is bound to.
+_COMPOSED_HELPERS = ("fprop_softmax", "fprop_relu", "bprop_relu", "fprop_transform", "bprop_transform",
+                     "fprop_skipnode", "bprop_skipnode", "relu_layer", "batchnorm_layer", "mergesum_layer",
+                     "mergebroadcast_layer", "fprop_mergesum", "bprop_mergesum", "fprop_mergebroadcast",
+                     "bprop_mergebroadcast", "binarize", "shift", "update_fc_bias", "add_fc_bias",
+                     "compound_rnn_unroll_fprop", "compound_rnn_unroll_bprop")
+for _name in _COMPOSED_HELPERS:
+    setattr(NervanaHIPBase, _name, getattr(_own.Backend, _name))
+del _name
+
+
+class _Api(object):
+    """the classes of the package a backend class is bound to"""
+    __slots__ = ("Backend", "OpTreeNode", "Tensor", "Block")
+
+    def __init__(self, Backend, OpTreeNode, Tensor, Block):
+        self.Backend, self.OpTreeNode, self.Tensor, self.Block = Backend, OpTreeNode, Tensor, Block
+
+
+_bound = {}
+
+
+def bind(Backend=None, OpTreeNode=None, Tensor=None, Block=None):
+    """Build the backend class on a host package's API classes and return
+    ``(NervanaHIP, HIPTensor)``.
+
+    neon finds its backends through the metaclass of ``Backend``
+    (abstract_backend.py:23-36: every named subclass lands in
+    ``Backend.backends``, which ``gen_backend`` / ``-b`` consult,
+    backend.py:465-472) and its layers hand ``execute`` nodes of ITS
+    ``OpTreeNode`` holding ITS ``Tensor`` objects (backend.py:1852-1866).  So
+    the class that serves ``-b hip`` has to derive from those very classes:
+
+        from neon.backends.backend import Backend, OpTreeNode, Tensor, Block
+        NervanaHIP, HIPTensor = bind(Backend, OpTreeNode, Tensor, Block)
+
+    creates ``NervanaHIP(NervanaHIPBase, Backend)`` with ``Backend``'s
+    metaclass -- which registers it as ``'hip'`` -- and
+    ``HIPTensor(HIPTensorBase, Tensor)``.  Without arguments the classes are
+    built on this package's own API (``neon_amd.backends.backend``).  One class
+    pair per API triple; calling again returns the same pair.  ``Block`` (the
+    enumeration behind ``be.begin / be.end``) defaults to the one defined next
+    to ``Backend``."""
+    if Backend is None:
+        Backend, OpTreeNode, Tensor, Block = _own.Backend, _own.OpTreeNode, _own.Tensor, _own.Block
+    if OpTreeNode is None or Tensor is None:
+        raise TypeError("bind needs the Backend, OpTreeNode and Tensor classes of one package")
+    key = (Backend, OpTreeNode, Tensor)
+    if key in _bound:
+        return _bound[key]
+    if Block is None:
+        import sys
+        Block = getattr(sys.modules.get(Backend.__module__), "Block", _own.Block)
+    api = _Api(Backend, OpTreeNode, Tensor, Block)
+    tensor_cls = type(Tensor)("HIPTensor", (HIPTensorBase, Tensor),
+                              {"_api": api, "__module__": __name__, "__doc__": HIPTensorBase.__doc__})
+    backend_cls = type(Backend)("NervanaHIP", (NervanaHIPBase, Backend),
+                                {"_api": api, "tensor_cls": tensor_cls, "backend_name": "hip",
+                                 "__module__": __name__, "__doc__": NervanaHIPBase.__doc__})
+    _bound[key] = (backend_cls, tensor_cls)
+    return _bound[key]
+
+
+def __getattr__(name):
+    """``NervanaHIP`` / ``HIPTensor`` as module attributes: the pair bound to
+    this package's own API, built on first use"""
+    if name in ("NervanaHIP", "HIPTensor"):
+        pair = bind()
+        return pair[0] if name == "NervanaHIP" else pair[1]
+    raise AttributeError("module %r has no attribute %r" % (__name__, name))
 
 
 def _matrix_geometry(rows, cols, sr, sc):
