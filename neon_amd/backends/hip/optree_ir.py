@@ -27,6 +27,7 @@ reduction axis outside {0,1} or two different axes -> ValueError; operand
 shapes that do not broadcast -> TypeError; unknown op or operand -> TypeError.
 """
 import math
+import os
 
 import numpy as np
 
@@ -143,6 +144,10 @@ def is_tensor(x):
     return hasattr(x, "ptr") and hasattr(x, "strides")
 
 
+ONLINE_LSE = os.environ.get("NEON_HIP_ONLINE_LSE", "1") != "0"
+ONEHOT_GATHER = os.environ.get("NEON_HIP_ONEHOT_GATHER", "1") != "0"
+
+
 class MixedAxes(ValueError):
     """Reductions along both axes in one tree: needs more than one kernel."""
 
@@ -166,9 +171,11 @@ def stochastic_bits(tensor):
 
 class Node(object):
     """DAG node.  kind: 'T' tensor leaf, 'C' constant slot, 'E' elementwise op,
-    'R' reduction, 'H' one-hot of an index tensor."""
+    'R' reduction, 'H' one-hot of an index tensor, 'G' an expression evaluated
+    at the hot row of a one-hot (``args = (expression, one-hot)``; what
+    ``sum(onehot * expression, axis=0)`` is rewritten to)."""
     __slots__ = ("kind", "op", "args", "slot", "axis", "vr", "vc", "level",
-                 "nid", "is_index", "shape")
+                 "nid", "is_index", "shape", "lse_max", "lse_sum")
 
     def __init__(self, kind, op=None, args=(), slot=None, axis=None):
         self.kind = kind
@@ -181,6 +188,8 @@ class Node(object):
         self.nid = -1
         self.is_index = False
         self.shape = (1, 1)
+        self.lse_max = None     # on sum(exp(x - max(x))): the max node it shares a sweep with
+        self.lse_sum = None     # on that max node: the sum
 
     def __repr__(self):
         return "N%d<%s %s %s>" % (self.nid, self.kind, self.op or "", self.slot if self.slot is not None else "")
@@ -189,11 +198,12 @@ class Node(object):
 class TensorSlot(object):
     """One kernel pointer argument: a distinct (memory, geometry, dtype)."""
     __slots__ = ("index", "tensor", "dtype", "shape", "strides", "ptr", "written",
-                 "read", "geom", "take_axis", "take_slot")
+                 "read", "geom", "take_axis", "take_slot", "take_extent")
 
     def __init__(self, index, tensor, shape, strides):
         self.take_axis = None      # gather / scatter view: indexed axis ...
-        self.take_slot = None      # ... and the slot of its int32 index vector
+        self.take_slot = None      # ... the slot of its int32 index vector ...
+        self.take_extent = None    # ... and the extent of the indexed axis in the underlying tensor
         self.index = index
         self.tensor = tensor
         self.dtype = np.dtype(tensor.dtype)
@@ -276,8 +286,9 @@ class Program(object):
             take_slot = self.tensor_slot(idx)
             self.index_slots.add(take_slot.index)
         shape, strides = view_2d(t)
+        take_extent = getattr(t, "take_extent", None) if take else None
         geom = (t.ptr, shape, strides, np.dtype(t.dtype),
-                take_axis, take_slot.index if take_slot else None)
+                take_axis, take_slot.index if take_slot else None, take_extent)
         slot = self._tensor_by_geom.get(geom)
         if slot is None:
             if np.dtype(t.dtype) not in DTYPE_CODE:
@@ -285,6 +296,7 @@ class Program(object):
             slot = TensorSlot(len(self.tensors), t, shape, strides)
             slot.take_axis = take_axis
             slot.take_slot = take_slot.index if take_slot else None
+            slot.take_extent = take_extent
             slot.geom = geom
             self.tensors.append(slot)
             self._tensor_by_geom[geom] = slot
@@ -458,6 +470,25 @@ class Program(object):
         for t in shaped:
             if t.shape[0] not in (1, R) or t.shape[1] not in (1, C):
                 raise TypeError("Input shape:%s not compatible with %s" % (t.shape, (R, C)))
+        self._analyse()
+        self.lse_pairs = 0
+        self.gathers = 0
+        if self.axis == 0:
+            if ONLINE_LSE:
+                self._pair_max_with_sum_of_exp()
+            if ONEHOT_GATHER:
+                self._gather_at_hot_rows()
+            if self.lse_pairs or self.gathers:
+                self._analyse()
+        for st in self.statements:
+            rs, os_ = st.root.shape, st.out.shape
+            if (rs[0] not in (1, os_[0])) or (rs[1] not in (1, os_[1])):
+                raise TypeError("Input shape:%s not compatible with %s" % (rs, os_))
+        return self
+
+    def _analyse(self):
+        """per node: along which axes it varies, its reduction level, its shape"""
+        R, C = self.domain
         for n in self.nodes:
             if n.kind == "T":
                 shp = self.tensors[n.slot].shape
@@ -480,6 +511,9 @@ class Program(object):
                 n.vr = any(a.vr for a in n.args)
                 n.vc = any(a.vc for a in n.args)
                 n.level = max(a.level for a in n.args)
+            elif n.kind == "G":
+                # one value per column, computable once the reductions inside the expression are
+                n.vr, n.vc, n.level = False, C > 1, n.args[0].level
             elif n.kind == "R":
                 a = n.args[0]
                 varies = a.vr if n.axis == 0 else a.vc
@@ -494,20 +528,104 @@ class Program(object):
                     n.vr = a.vr and n.axis != 0
                     n.vc = a.vc and n.axis != 1
                     n.level = a.level + 1
+                    if n.lse_max is not None:
+                        n.level = n.lse_max.level        # accumulated in the sweep that finds the maximum
             n.shape = (R if n.vr else 1, C if n.vc else 1)
         if not any(n.kind == "R" for n in self.nodes):
             self.axis = None
         self.nlevels = max([n.level for n in self.nodes] + [0])
-        for st in self.statements:
-            rs, os_ = st.root.shape, st.out.shape
-            if (rs[0] not in (1, os_[0])) or (rs[1] not in (1, os_[1])):
-                raise TypeError("Input shape:%s not compatible with %s" % (rs, os_))
-        return self
+
+    def _pair_max_with_sum_of_exp(self):
+        """``sum(exp(x - max(x, 0)), 0)``: the sum joins the sweep that finds the
+        maximum, as a running (max, sum) pair that is rescaled whenever the
+        maximum grows -- softmax and cross-entropy trees need one pass (and, when
+        the rows are spread over several workgroups, one exchange) less.  The
+        sum's terms are added in another order and rescaled by exp(m - M)
+        factors: equal to the two-sweep result within a few units in the last
+        place, not bit for bit (``NEON_HIP_ONLINE_LSE=0`` keeps two sweeps)."""
+        for sm in self.nodes:
+            if sm.kind != "R" or sm.op != "sum":
+                continue
+            e = sm.args[0]
+            if e.kind != "E" or e.op != "exp":
+                continue
+            d = e.args[0]
+            if d.kind != "E" or d.op != "sub":
+                continue
+            x, mx = d.args
+            if (mx.kind == "R" and mx.op == "max" and mx.axis == sm.axis and mx.args[0] is x
+                    and mx.lse_sum is None):
+                mx.lse_sum, sm.lse_max = sm, mx
+                self.lse_pairs += 1
+
+    def unpair_lse(self):
+        """back to one sweep for the maximum and one for the sum"""
+        for n in self.nodes:
+            n.lse_max = n.lse_sum = None
+        self.lse_pairs = 0
+        self._analyse()
+
+    def _gather_at_hot_rows(self):
+        """``sum(onehot(idx, 0) * expr, 0)`` adds one term of ``expr`` per column
+        and zeros: it becomes ``expr`` evaluated at row ``idx[c]`` only (0 when
+        the index is out of range) -- for a cross-entropy tree the second pass
+        over the matrix disappears.  Exact as long as ``expr`` is finite in the
+        other rows (0 * inf would be NaN in the sum).  Applied when the value is
+        only used for one-value-per-column results (``NEON_HIP_ONEHOT_GATHER=0``
+        keeps the sum)."""
+        roots = [st.root for st in self.statements]
+        live = used_nodes(roots)
+        users = {}
+        for n in live:
+            for a in n.args:
+                users.setdefault(a.nid, []).append(n)
+        line_roots = set(st.root.nid for st in self.statements if st.out.shape[0] == 1)
+        other_roots = set(st.root.nid for st in self.statements) - line_roots
+
+        def only_feeds_column_values(n):
+            todo, seen = [n], set()
+            while todo:
+                m = todo.pop()
+                if m.nid in seen:
+                    continue
+                seen.add(m.nid)
+                if m.nid in other_roots:
+                    return False
+                for u in users.get(m.nid, ()):
+                    if u.kind != "E" or u.vr or u.op.startswith("sround:"):
+                        return False
+                    todo.append(u)
+            return True
+
+        def plain(expr):
+            for m in used_nodes([expr]):
+                if m.kind == "G" or (m.kind == "H" and m.axis != 0):
+                    return False
+                if m.kind == "E" and (not m.args or m.op.startswith("sround:")):
+                    return False
+                if m.kind == "T" and self.tensors[m.slot].take_axis is not None:
+                    return False
+            return True
+
+        for n in live:
+            if n.kind != "R" or n.op != "sum" or n.axis != 0:
+                continue
+            p = n.args[0]
+            if p.kind != "E" or p.op != "mul":
+                continue
+            a, b = p.args
+            hot, expr = (a, b) if a.kind == "H" else (b, a)
+            if hot.kind != "H" or hot.axis != 0 or expr.kind == "H":
+                continue
+            if not plain(expr) or not only_feeds_column_values(n):
+                continue
+            n.kind, n.op, n.args = "G", "gather0", (expr, hot)
+            self.gathers += 1
 
     def key(self):
         """Hashable identity of the program's structure and operand geometry."""
         geo = tuple((DTYPE_CODE[t.dtype], t.shape, t.strides, t.ptr % 16 == 0, t.written,
-                     t.take_axis, t.take_slot) for t in self.tensors)
+                     t.take_axis, t.take_slot, t.take_extent) for t in self.tensors)
         return (tuple(self.key_parts), geo, self._alias_signature())
 
     def _alias_signature(self):

@@ -207,14 +207,19 @@ class Plan(object):
     """A compiled kernel + grid; ``launch(prog)`` binds the argument values of
     any program with the same key."""
 
-    def __init__(self, rt, kernel, spec, grid, extras_fn=None, workspace=None):
+    def __init__(self, rt, kernel, spec, grid, extras_fn=None, workspace=None, status_ptr=None, counters=None):
         self.rt = rt
+        # cooperative families: device address of the word an aborting workgroup
+        # marks, and (address, count) of the arrival counters -- for the host's check
+        self.status_ptr = status_ptr
+        self.counters = counters
         self.kernel = kernel
         self.spec = spec
         self.grid = grid
         self.block = (spec.block, 1, 1)
         self.extras_fn = extras_fn
         self.workspace = workspace     # device allocation owned by the plan
+        self.key = None                # program key the backend filed the plan under
         self.domain = None             # set by make_plan: the (R, C) the kernel iterates
 
     def _values(self, prog):
@@ -285,15 +290,19 @@ class Choice(object):
     """Outcome of shape-class selection: generated kernel, grid and what the
     extra kernel parameters are.  Needs no device."""
 
-    def __init__(self, spec, grid, extras=(), workspace=None):
+    def __init__(self, spec, grid, extras=(), workspace=None, status_offset=None):
         self.spec = spec
         self.grid = grid
         self.extras = tuple(extras)          # literal values appended after R, C
         self.workspace = workspace           # None or (bytes, ticket_offset, n_tickets)
+        self.status_offset = status_offset   # cooperative families: byte offset of the status word
 
 
-def choose(prog, cu_count=256):
-    """Pick family + tiling for a finalized program and generate its source."""
+def choose(prog, cu_count=256, coop=True):
+    """Pick family + tiling for a finalized program and generate its source.
+    ``coop=False`` keeps to the families whose workgroups never wait for one
+    another (what the backend falls back to once a cooperative plan's bounded
+    wait has expired, e.g. on a device it does not have to itself)."""
     R, C = prog.domain
     if R > 0x7FFFFFFF or C > 0x7FFFFFFF:
         raise ValueError("tensor dimension too large")
@@ -301,22 +310,24 @@ def choose(prog, cu_count=256):
     if prog.axis is None:
         return _plan_ew(prog, cu_count)
     if prog.axis == 1:
-        return _plan_row(prog, cu_count)
-    return _plan_col(prog, cu_count)
+        return _plan_row(prog, cu_count, coop)
+    return _plan_col(prog, cu_count, coop)
 
 
-def make_plan(prog, rt, cache, cu_count):
-    ch = choose(prog, cu_count)
+def make_plan(prog, rt, cache, cu_count, coop=True):
+    ch = choose(prog, cu_count, coop)
     kernel = cache.kernel(rt, ch.spec)
     extras = ch.extras
-    ws = None
+    ws = status = counters = None
     if ch.workspace is not None:
         ws_bytes, ticket_off, n_tickets = ch.workspace
         ws = rt.malloc(ws_bytes)
         rt.memset(ws + ticket_off, 0, n_tickets, 4)   # tickets start at zero and reset themselves
         extras = extras + (ws, ticket_off)
+        if ch.status_offset is not None:
+            status, counters = ws + ch.status_offset, (ws + ticket_off, n_tickets)
     plan = Plan(rt, kernel, ch.spec, ch.grid, extras_fn=(lambda e=extras: e) if extras else None,
-                workspace=ws)
+                workspace=ws, status_ptr=status, counters=counters)
     plan.domain = tuple(prog.domain)
     return plan
 
@@ -349,7 +360,7 @@ def _plan_ew(prog, cu_count):
     return Choice(spec, (gx, gy, 1), extras=(row_tiles,))
 
 
-def _plan_row(prog, cu_count):
+def _plan_row(prog, cu_count, coop=True):
     R, C = prog.domain
     V = _vector_width(prog, tail_ok=True)
     tail = (C % V) != 0
@@ -384,7 +395,7 @@ def _plan_row(prog, cu_count):
     # workgroups that exchange their partial results; all of them must be
     # resident at once, so rows x chunks stays within the compute units.
     tiles = _ceil_div(nvec, 1024)
-    if R * 2 <= cu_count and tiles >= 8 and prog.nlevels >= 1:
+    if coop and R * 2 <= cu_count and tiles >= 8 and prog.nlevels >= 1:
         chunks = min(cu_count // R, tiles // 4, 64)
         per = _ceil_div(tiles, chunks)
         chunks = _ceil_div(tiles, per)
@@ -395,7 +406,8 @@ def _plan_row(prog, cu_count):
             spec = codegen.gen_row(prog, V, 1024, 1, per, _streams(prog), keep_words=kw, chunks=chunks, tail=tail)
             part_bytes = R * spec.params["NRED"] * chunks * 8
             ctr_off = _ceil_div(part_bytes, 256) * 256
-            return Choice(spec, (R, chunks, 1), workspace=(ctr_off + R * 8, ctr_off, 2 * R))
+            return Choice(spec, (R, chunks, 1), workspace=(ctr_off + R * 8 + 4, ctr_off, 2 * R + 1),
+                          status_offset=ctr_off + R * 8)
     LY = T // LX
     spec = codegen.gen_row(prog, V, LX, LY, NCH, _streams(prog), keep_words=keep_words, tail=tail)
     gx = _ceil_div(R, LY)
@@ -409,10 +421,12 @@ def _plan_row(prog, cu_count):
 _COL_BUDGET = {1024: 40, 512: 120, 256: 300}
 
 
-COLSPLIT_THREADS = 256
+COLSPLIT_THREADS = int(os.environ.get("NEON_HIP_CS_T", "256"))
+
+ONLINE_LSE_IN_ONE_WORKGROUP = os.environ.get("NEON_HIP_ONLINE_LSE_COL", "0") != "0"
 
 
-def _plan_col(prog, cu_count):
+def _plan_col(prog, cu_count, coop=True):
     R, C = prog.domain
     V = _vector_width(prog, tail_ok=True)
     tail = (C % V) != 0
@@ -454,6 +468,10 @@ def _plan_col(prog, cu_count):
     big = R * C >= (1 << 18)
     if fit and not (single_level and line_only and big and R >= 512):
         T, LY, NR = fit
+        if prog.lse_pairs and not ONLINE_LSE_IN_ONE_WORKGROUP:
+            # no exchange between workgroups to save here, and the running pair
+            # costs two more exponentials per element than a sweep of its own
+            prog.unpair_lse()
         budget = _COL_BUDGET[T]
         spare = max(0, (budget - NR * words) // (NR * V))
         spec = codegen.gen_col(prog, V, LX, LY, NR, _streams(prog), max_vals=min(2, spare), tail=tail)
@@ -463,7 +481,7 @@ def _plan_col(prog, cu_count):
     # strip keep their rows in registers and exchange partials between sweeps.
     # Everything must be resident at once, so the grid stays within one
     # workgroup per compute unit.
-    if not (single_level and line_only):
+    if coop and not (single_level and line_only):
         # narrow strips keep the partials each workgroup has to gather small
         # (measured on (32000,256): 8 column-lanes 37 us, 16 lanes 43 us, 4 lanes
         # 41 us).  More strips than half the compute units leave no second
@@ -489,7 +507,8 @@ def _plan_col(prog, cu_count):
                     part_bytes = spec.params["NRED"] * chunks * C * 8
                     ctr_off = _ceil_div(part_bytes, 256) * 256
                     return Choice(spec, (strips_c, chunks, 1),
-                                  workspace=(ctr_off + strips_c * 8, ctr_off, 2 * strips_c))
+                                  workspace=(ctr_off + strips_c * 8 + 4, ctr_off, 2 * strips_c + 1),
+                                  status_offset=ctr_off + strips_c * 8)
 
     # (b) one level, one value per column, many rows: split rows over workgroups
     if single_level and line_only:
@@ -509,7 +528,11 @@ def _plan_col(prog, cu_count):
         if LX == 16 and (per_cu == 1 or
                          _ceil_div(nvec, LX) * codegen.COLSPLIT_MAX_CHUNKS < min(target, 2 * cu_count)):
             LX = max(lx_min, 8)
-        LY = COLSPLIT_THREADS // LX
+        # one workgroup per compute unit (small inputs): twice the lanes, so that a SIMD has a
+        # second wave to run while the first waits for its rows ((32000,256): argmax 11.0 ->
+        # 10.7 us, max 8.1 -> 7.3 us); larger inputs already get several workgroups per unit
+        threads = COLSPLIT_THREADS * 2 if (per_cu == 1 and COLSPLIT_THREADS == 256) else COLSPLIT_THREADS
+        LY = threads // LX
         strips = _ceil_div(nvec, LX)
         # (the limit bounds what the last workgroup of a strip has to fold; strips
         # under 64 columns may take more chunks, as far as it takes to get two
@@ -523,7 +546,10 @@ def _plan_col(prog, cu_count):
         chunks = _ceil_div(R, rpc)
         if chunks > 65535:
             raise ValueError("tensor too large for one launch")
-        spec = codegen.gen_colsplit(prog, V, LX, LY, _streams(prog), tail=tail)
+        # partials a lane of the last workgroup has in flight: P = lanes per column there
+        lanes_per_column = min(threads // (LX * V), 64)
+        fold_batch = max(1, min(codegen.COLSPLIT_FOLD_BATCH, _ceil_div(chunks, lanes_per_column)))
+        spec = codegen.gen_colsplit(prog, V, LX, LY, _streams(prog), tail=tail, fold_batch=fold_batch)
         nred = spec.params["NRED"]
         part_bytes = nred * chunks * C * 8
         ticket_off = _ceil_div(part_bytes, 256) * 256

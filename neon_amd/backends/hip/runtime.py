@@ -21,6 +21,7 @@ DEVICE_HEADER = os.path.join(_PKG, "csrc", "device", "neon_device.h")
 NH_RTC_ERROR_BASE = 10000
 NH_EINVAL = 20001
 NH_ENOTINIT = 20002
+NH_ECOOP = 20003        # raised by the backend, never returned by the library: a cooperative kernel gave up
 
 # Options every device compilation uses, prebuilt or run-time: no contraction of
 # a*b+c into fma (results then follow the expression as written, like numpy's

@@ -71,7 +71,7 @@ class HIPTensorBase(object):
 
     def __init__(self, backend, shape=None, dtype=np.float32, name=None,
                  persist_values=True, base=None, gpudata=None, strides=None,
-                 take_array=None, is_trans=False, rounding=0):
+                 take_array=None, is_trans=False, rounding=0, take_extent=None):
         super(HIPTensorBase, self).__init__(backend, shape, dtype, name, persist_values)
         dtype = np.dtype(dtype)
         assert dtype.type in _DTYPES, "unsupported dtype %s" % dtype
@@ -93,6 +93,8 @@ class HIPTensorBase(object):
         self.strides = _contiguous_strides(self.shape) if strides is None else tuple(int(s) for s in strides)
         self.base = base
         self.take_array = take_array
+        # gather view: rows (columns) of the tensor it indexes -- kernels clamp indices into that range
+        self.take_extent = take_extent
         self.is_trans = is_trans
         self.rounding = rounding
         self.kahan_count = 0
@@ -108,7 +110,7 @@ class HIPTensorBase(object):
                               self.strides == _contiguous_strides(self.shape))
         # identity for the launch cache: same memory + same layout = same kernel arguments
         self._geom = (self.gpudata, self.shape, self.strides, dtype.char,
-                      (take_array[0]._geom, take_array[1]) if take_array else 0)
+                      (take_array[0]._geom, take_array[1], take_extent) if take_array else 0)
 
     def __del__(self):
         if getattr(self, "_owns", False) and self.gpudata:
@@ -123,6 +125,13 @@ class HIPTensorBase(object):
     @property
     def ptr(self):
         return self.gpudata
+
+    def get_original_base(self):
+        """the tensor that owns the memory this view looks into"""
+        t = self
+        while t.base is not None:
+            t = t.base
+        return t
 
     def __int__(self):
         return int(self.gpudata)
@@ -149,7 +158,7 @@ class HIPTensorBase(object):
                 return self
             index = (index,)
         new_shape, new_strides, offset = [], [], 0
-        take = None
+        take = take_extent = None
         seen_ellipsis = False
         ia = aa = 0
         while ia < len(index):
@@ -176,6 +185,7 @@ class HIPTensorBase(object):
                 if entry.dtype.type is not np.int32:
                     raise IndexError("Fancy indexing only currently supported with int32 types.")
                 take = (entry, aa)
+                take_extent = self.shape[aa]
                 new_shape.append(size)
                 new_strides.append(self.strides[aa])
                 ia += 1
@@ -213,7 +223,7 @@ class HIPTensorBase(object):
             aa += 1
         return self.__class__(backend=self.backend, shape=tuple(new_shape), dtype=self.dtype,
                               base=self, gpudata=self.gpudata + offset, strides=new_strides,
-                              take_array=take, name=self.name, rounding=self.rounding)
+                              take_array=take, name=self.name, rounding=self.rounding, take_extent=take_extent)
 
     def _assign(self, value):
         """Constant fill and same-layout copy use the device's fill / copy
@@ -272,6 +282,7 @@ class HIPTensorBase(object):
             tmp.copy(self)
             be._flush()
             be.rt.memcpy_d2h(out, tmp.gpudata)
+        be._check_cooperative_plans()       # the copy waited for the stream: results are final
         return out
 
     def raw(self):
@@ -390,9 +401,10 @@ class _FuseScope(object):
 
 class _Recorded(object):
     """Launches recorded for one statement group."""
-    __slots__ = ("launches", "temps", "raw", "patch")
+    __slots__ = ("launches", "temps", "raw", "patch", "coop")
 
-    def __init__(self, launches, temps, raw, patch):
+    def __init__(self, launches, temps, raw, patch, coop=()):
+        self.coop = coop             # cooperative plans among the launches (checked at the next synchronisation)
         self.launches = launches
         self.temps = temps           # temporaries the recorded arguments point into
         self.raw = raw               # the numbers of the trees when recorded
@@ -477,18 +489,24 @@ class NervanaHIPBase(object):
         self.plan_stats = {"hit": 0, "miss": 0, "split": 0, "launches": 0, "replayed": 0}
         self._pending = []
         self._pending_post = []       # postfix walks of the pending statements
+        self._pending_sig = None      # what kind of group the pending statements form
         self._fusing = False
         self._fuse_depth = 0
         self._captured = None
         self._launch_cache = {}      # statement-group identity -> recorded launches
         self._recording = None
         self._rec_temps = None
+        self._rec_coop = None
         self._rec_foreign = False     # the group being recorded made a call that is not a kernel launch
         self._lut_ws = None           # (pointer, bytes) scratch of compound_bprop_lut
         self._originals = frozenset() # ids of handles whose reads mean "before the running group" (compensated_sum)
         self._rec_single = None
         self._temp_pool = {}
         self._live_allocs = 0
+        # cooperative plans (workgroups that wait for one another) launched since the
+        # last look at their status words, and the program keys whose plan gave up
+        self._coop_pending = {}
+        self._coop_failed = set()
 
     # -- memory ---------------------------------------------------------------------
     def _mem_alloc(self, nbytes):
@@ -521,6 +539,35 @@ class NervanaHIPBase(object):
     def synchronize(self):
         self._flush()
         self.rt.synchronize()
+        self._check_cooperative_plans()
+
+    def _check_cooperative_plans(self):
+        """Call with the stream idle.  The cooperative families (``rowcoop``,
+        ``colcoop``) need all workgroups of a strip resident at once; where they
+        are not (a device shared with other work, masked compute units) a
+        workgroup's bounded wait expires, it marks the plan's status word and
+        returns WITHOUT results.  That must not pass silently: raise, reset the
+        plan's counters, and from now on evaluate that program with the
+        families that never wait (stage by stage where one kernel cannot)."""
+        if not self._coop_pending:
+            return
+        pending, self._coop_pending = self._coop_pending, {}
+        failed = []
+        word = np.zeros(1, np.uint32)
+        for key, plan in pending.items():
+            self.rt.memcpy_d2h(word, plan.status_ptr)
+            if int(word[0]) != 0:
+                failed.append(key)
+                ptr, count = plan.counters
+                self.rt.memset(ptr, 0, count, 4)     # (a holder of the old plan object finds it re-armed)
+                self._coop_failed.add(key)
+                self.plans.pop(key, None)
+        if failed:
+            self._launch_cache.clear()       # recorded launches of the abandoned plans must not be replayed
+            self.rt.synchronize()
+            raise hiprt.HipError(hiprt.NH_ECOOP, "a cooperative kernel gave up waiting for its other workgroups "
+                                 "(%d plan(s)): results since the last synchronisation are invalid; these "
+                                 "op-trees now run without inter-workgroup waits" % len(failed))
 
     # -- random numbers (reference nervanagpu.py:901-1049, 1825-1861) ---------------------
     def gen_rng(self, seed=None):
@@ -654,31 +701,79 @@ class NervanaHIPBase(object):
                 self._run(trees, posts)
 
     _NOT_FUSABLE = frozenset(REDUCE) | {"dot", "transpose", "onehot"}
+    _NEVER_FUSABLE = frozenset({"dot", "transpose", "rand"})
 
     def _can_join(self, tree, post):
-        """A statement joins the pending group when it is purely elementwise,
-        every tensor in it has the group's shape and is contiguous (or is
-        1x1), so each lane only ever touches its own elements.  ``post`` is
-        the statement's postfix walk."""
+        """Whether a statement may join the pending group.  Two kinds of group:
+
+        * elementwise: every tensor has the group's shape and is contiguous (or
+          is 1x1), so each lane only ever touches its own elements;
+        * reductions of one operand shape along one axis into one-value-per-line
+          tensors (``argmax`` and ``max`` of the same logits): one kernel reads
+          the operands once for all of them.
+
+        ``post`` is the statement's postfix walk."""
+        sig = self._group_signature(tree, post)
+        if sig is None:
+            return False
+        if not self._pending:
+            self._pending_sig = sig
+            return True
+        if sig != self._pending_sig:
+            return False
+        if sig[0] == "red":
+            # results are written while operands are still being read by other
+            # workgroups: a result that lives inside an operand would be a race
+            outs = [q[1] for q in self._pending] + [tree[1]]
+            bases = set(id(o.get_original_base()) for o in outs)
+            for grp_post in self._pending_post + [post]:
+                for p in grp_post:
+                    if isinstance(p, HIPTensorBase) and p.size > 1 and id(p.get_original_base()) in bases \
+                            and not any(p is o for o in outs):
+                        return False
+        return True
+
+    def _group_signature(self, tree, post):
         out = tree[1]
         shape = out.shape
-        if self._pending and self._pending[0][1].shape != shape:
-            return False
-        not_fusable = self._NOT_FUSABLE
         tensor_cls = self.tensor_cls
+        axis = None
+        full = None
         for p in post:
             tp = type(p)
             if tp is dict:
-                if p["op"] in not_fusable:
-                    return False
+                op = p["op"]
+                if op in self._NEVER_FUSABLE:
+                    return None
+                if op in REDUCE or op == "onehot":
+                    a = p.get("axis")
+                    if a not in (0, 1) or (op in REDUCE and axis not in (None, a)):
+                        return None
+                    if op in REDUCE:
+                        axis = a
             elif tp is tensor_cls:
                 if p.size == 1 and p.is_contiguous:
                     ptr = p.gpudata
                     if ptr == out.gpudata or any(ptr == q[1].gpudata for q in self._pending):
-                        return False        # a scalar that is also written: order matters
-                elif p.shape != shape or not p.is_contiguous:
-                    return False
-        return True
+                        return None         # a scalar that is also written: order matters
+                elif not p.is_contiguous or len(p.shape) != 2:
+                    return None
+                elif p.shape != shape:
+                    if full is None:
+                        full = p.shape
+                    elif p.shape != full and p.shape != shape:
+                        return None
+        if axis is None:
+            # purely elementwise: no one-hot either (its index vector has another shape)
+            if full is not None or any(type(p) is dict and p["op"] == "onehot" for p in post):
+                return None
+            return ("ew", shape)
+        if full is None or len(shape) != 2 or out.rounding or not out.is_contiguous:
+            return None
+        line = (1, full[1]) if axis == 0 else (full[0], 1)
+        if shape != line or full[axis] == 1:
+            return None
+        return ("red", axis, full, shape)
 
     # -- execution -----------------------------------------------------------------------
     def execute(self, optree):
@@ -751,16 +846,19 @@ class NervanaHIPBase(object):
                         grid(*args)             # a recorded call of a prebuilt kernel's entry point
                     else:
                         launch(kernel, grid, block, args)
+                for plan in entry.coop:
+                    self._coop_pending[plan.key] = plan
                 if self._recording is not None:
                     self._recording.extend(launches)
                     self._rec_temps.extend(entry.temps)
+                    self._rec_coop.extend(entry.coop)
                     self._rec_single = None
                 self.plan_stats["replayed"] += 1
                 self.plan_stats["launches"] += len(launches)
                 return
         outer = self._recording is None
         if outer:
-            self._recording, self._rec_temps, self._rec_single = [], [], None
+            self._recording, self._rec_temps, self._rec_single, self._rec_coop = [], [], None, []
             self._rec_foreign = False
         ok = False
         try:
@@ -768,14 +866,14 @@ class NervanaHIPBase(object):
             ok = True
         finally:
             if outer:
-                rec, temps, single = self._recording, self._rec_temps, self._rec_single
-                self._recording, self._rec_temps, self._rec_single = None, None, None
+                rec, temps, single, coop = self._recording, self._rec_temps, self._rec_single, self._rec_coop
+                self._recording, self._rec_temps, self._rec_single, self._rec_coop = None, None, None, None
                 if ok and key is not None and not self._rec_foreign:
                     if len(self._launch_cache) >= 8192:
                         self._launch_cache.clear()
                     if len(rec) != 1:
                         single = None
-                    self._launch_cache[key] = _Recorded(rec, temps, raw, single)
+                    self._launch_cache[key] = _Recorded(rec, temps, raw, single, tuple(coop))
 
     def _launch_plan(self, plan, prog):
         if prog.rand_count:
@@ -786,6 +884,10 @@ class NervanaHIPBase(object):
             self._rng_dev_counter += n
         args = plan.pack(prog)
         self.rt.launch_packed(plan.kernel, plan.grid, plan.block, args)
+        if plan.status_ptr is not None:
+            self._coop_pending[plan.key] = plan
+            if self._rec_coop is not None:
+                self._rec_coop.append(plan)
         if self._recording is not None:
             self._recording.append((plan.kernel, plan.grid, plan.block, args))
             # a group that is exactly one launch of one program can be re-bound
@@ -806,7 +908,8 @@ class NervanaHIPBase(object):
             plan = self.plans.get(key)
             if plan is None:
                 self.plan_stats["miss"] += 1
-                plan = make_plan(prog, self.rt, self.kernels, self.cu_count)
+                plan = make_plan(prog, self.rt, self.kernels, self.cu_count, coop=key not in self._coop_failed)
+                plan.key = key
                 self.plans[key] = plan
             else:
                 self.plan_stats["hit"] += 1
@@ -856,7 +959,8 @@ class NervanaHIPBase(object):
         key = prog.key()
         plan = self.plans.get(key)
         if plan is None:
-            plan = make_plan(prog, self.rt, self.kernels, self.cu_count)
+            plan = make_plan(prog, self.rt, self.kernels, self.cu_count, coop=key not in self._coop_failed)
+            plan.key = key
             self.plans[key] = plan
         return plan.launch_timed(prog, reps), plan
 
@@ -876,7 +980,8 @@ class NervanaHIPBase(object):
         assert all(prog.key() == key for prog in progs), "groups differ in more than their tensors"
         plan = self.plans.get(key)
         if plan is None:
-            plan = make_plan(progs[0], self.rt, self.kernels, self.cu_count)
+            plan = make_plan(progs[0], self.rt, self.kernels, self.cu_count, coop=key not in self._coop_failed)
+            plan.key = key
             self.plans[key] = plan
         return plan.launch_timed_sets(progs, reps), plan
 
@@ -1008,9 +1113,10 @@ class NervanaHIPBase(object):
         if plan is None:
             self.plan_stats["miss"] += 1
             try:
-                plan = make_plan(prog, self.rt, self.kernels, self.cu_count)
+                plan = make_plan(prog, self.rt, self.kernels, self.cu_count, coop=key not in self._coop_failed)
             except NeedsSplit:
                 raise ValueError("op-tree cannot be mapped to the available kernel families")
+            plan.key = key
             self.plans[key] = plan
         else:
             self.plan_stats["hit"] += 1

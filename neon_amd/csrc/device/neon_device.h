@@ -30,6 +30,10 @@ typedef unsigned int nh_u32;
 // Upper bound on the polls of a bounded wait for other workgroups (each poll
 // is a device-scope load plus a short sleep, roughly a microsecond).
 #define NH_SPIN_LIMIT (1u << 22)
+// Left in a cooperative plan's status word by a workgroup whose bounded wait
+// expired (it returns without results); the host looks for it at the next
+// synchronisation.
+#define NH_COOP_ABORTED 0xDEADu
 
 #define NH_INF __builtin_inff()
 #define NH_FLT_MAX 3.402823466e+38f
@@ -52,6 +56,9 @@ template <> struct nh_store_cvt<nh_i16>  { static NEON_DEV nh_i16  f(float x) { 
 template <> struct nh_store_cvt<nh_u16>  { static NEON_DEV nh_u16  f(float x) { return (nh_u16)(nh_i32)x; } };
 template <> struct nh_store_cvt<nh_i8>   { static NEON_DEV nh_i8   f(float x) { return (nh_i8)(nh_i32)x; } };
 template <> struct nh_store_cvt<nh_u8>   { static NEON_DEV nh_u8   f(float x) { return (nh_u8)(nh_i32)x; } };
+
+// Index of a gather / scatter view, kept inside the indexed tensor.
+NEON_DEV int nh_clamp_index(int i, int extent) { return i < 0 ? 0 : (i >= extent ? extent - 1 : i); }
 
 // An index produced by argmax/argmin goes to an integer target unchanged and
 // to a floating target as its value.
@@ -305,6 +312,19 @@ NEON_DEV float nh_sig(float x) { return 1.0f / (1.0f + expf(-x)); }
 NEON_DEV float nh_sig2(float x) { return 1.0f / (1.0f + exp2f(-x)); }
 NEON_DEV float nh_tanh2(float x) { const float e = exp2f(2.0f * x); return (e - 1.0f) / (e + 1.0f); }
 NEON_DEV float nh_finite(float x) { return (__builtin_fabsf(x) <= NH_FLT_MAX) ? 1.0f : 0.0f; }
+// x / d for a divisor that is constant along the loop the quotient varies in (a
+// row's standard deviation, a column's softmax sum): the reciprocal and the
+// test are loop invariants, leaving a multiply per element instead of an IEEE
+// division (about ten instructions); at most 1.5 units in the last place from
+// the quotient.  Where 1/d is not a normal number (d zero, denormal, huge,
+// infinite or NaN) the quotient is computed as written.
+NEON_DEV float nh_div_by_line(float x, float d) {
+    const float r = 1.0f / d;
+    const float ar = __builtin_fabsf(r);
+    float q = x * r;
+    if (__builtin_expect(!(ar <= NH_FLT_MAX) || ar < 1.17549435e-38f, 0)) q = x / d;
+    return q;
+}
 
 // Counter-based random numbers.  Word `w` of the stream `seed` is one half of
 // splitmix64(w >> 1): stateless, so a tensor filled twice from the same
@@ -389,27 +409,107 @@ struct nh_op_max { static NEON_DEV float init() { return -NH_INF; }   static NEO
 struct nh_op_min { static NEON_DEV float init() { return NH_INF; }    static NEON_DEV float f(float a, float b) { return nh_min(a, b); } };
 
 struct __attribute__((aligned(8))) nh_pair { float v; int i; };
+// NaN follows numpy (np.argmax / np.argmin return the position of the first
+// NaN when there is one, as np.max / np.min return NaN): a NaN beats every
+// number and an earlier NaN beats a later one.
 struct nh_op_argmax {
     static NEON_DEV nh_pair init() { nh_pair p; p.v = -NH_INF; p.i = 0; return p; }
     static NEON_DEV nh_pair f(nh_pair a, nh_pair b) {
-        const bool take_b = (b.v > a.v) || (b.v == a.v && b.i < a.i);
+        const bool an = a.v != a.v, bn = b.v != b.v;
+        const bool take_b = bn ? (!an || b.i < a.i) : (!an && ((b.v > a.v) || (b.v == a.v && b.i < a.i)));
         nh_pair r; r.v = take_b ? b.v : a.v; r.i = take_b ? b.i : a.i; return r;
     }
-    // sequential update with strictly increasing indices keeps the first hit
-    static NEON_DEV void step(nh_pair& a, float v, int i) { if (v > a.v) { a.v = v; a.i = i; } }
+    // sequential update with strictly increasing indices keeps the first hit:
+    // !(v <= a.v) holds for a larger value and for a NaN on either side; a NaN
+    // already held (a.v != a.v) stays
+    static NEON_DEV void step(nh_pair& a, float v, int i) { if (!(v <= a.v) && (a.v == a.v)) { a.v = v; a.i = i; } }
 };
 struct nh_op_argmin {
     static NEON_DEV nh_pair init() { nh_pair p; p.v = NH_INF; p.i = 0; return p; }
     static NEON_DEV nh_pair f(nh_pair a, nh_pair b) {
-        const bool take_b = (b.v < a.v) || (b.v == a.v && b.i < a.i);
+        const bool an = a.v != a.v, bn = b.v != b.v;
+        const bool take_b = bn ? (!an || b.i < a.i) : (!an && ((b.v < a.v) || (b.v == a.v && b.i < a.i)));
         nh_pair r; r.v = take_b ? b.v : a.v; r.i = take_b ? b.i : a.i; return r;
     }
-    static NEON_DEV void step(nh_pair& a, float v, int i) { if (v < a.v) { a.v = v; a.i = i; } }
+    static NEON_DEV void step(nh_pair& a, float v, int i) { if (!(v >= a.v) && (a.v == a.v)) { a.v = v; a.i = i; } }
 };
 
-// Partial results handed from one workgroup to another (possibly on another
-// XCD, behind another L2): stored through to device-coherent memory and loaded
-// past the local L2, as single 8-byte relaxed device-scope atomics.
+// Running log-sum-exp state of a column: v = maximum so far, i = the bits of
+// s = sum of exp(x - v) over the elements seen.  Carried as an nh_pair so that
+// it travels through the same lane exchanges, LDS slots and partial buffers
+// as an arg-reduction.  Merging two states rescales both sums to the larger
+// maximum: (m, s) + (m', s') = (M, s e^(m-M) + s' e^(m'-M)), M = max(m, m').
+// A state that has seen nothing (or only -inf) has v = -inf: its sum is then
+// taken as 0 instead of evaluating exp(-inf + inf).  NaN and +inf propagate
+// as in the two-sweep form (the sum becomes NaN).
+NEON_DEV float nh_lse_sum(nh_pair p) { return __builtin_bit_cast(float, p.i); }
+// exp(d) for d <= 0 (a term of a sum whose largest term is 1): the product
+// d * log2(e) is carried in two pieces so that the result is good to about a
+// unit in the last place, like expf, at half its instruction count; what
+// expf spends on results below the normal range is left out -- such terms
+// vanish next to the 1.  NaN comes back as NaN, -inf as 0.
+NEON_DEV float nh_exp_nonpos(float d) {
+    d = nh_max(d, -150.0f);
+    const float t = d * 1.44269502e+00f;
+    float e = __builtin_fmaf(d, 1.44269502e+00f, -t);
+    e = __builtin_fmaf(d, 1.92596299e-08f, e);
+    const float r = __builtin_amdgcn_exp2f(t);
+    return __builtin_fmaf(r, e * 6.93147182e-01f, r);
+}
+struct nh_op_lse {
+    static NEON_DEV nh_pair init() { nh_pair p; p.v = -NH_INF; p.i = 0; return p; }    // bits of +0.0f
+    static NEON_DEV nh_pair f(nh_pair a, nh_pair b) {
+        const float m = nh_max(a.v, b.v);
+        const float mz = (m == -NH_INF) ? 0.0f : m;
+        const float s = nh_lse_sum(a) * nh_exp_nonpos(a.v - mz) + nh_lse_sum(b) * nh_exp_nonpos(b.v - mz);
+        nh_pair r; r.v = m; r.i = __builtin_bit_cast(int, s); return r;
+    }
+    static NEON_DEV void step(nh_pair& a, float x) {
+        const float m = nh_max(a.v, x);
+        const float mz = (m == -NH_INF) ? 0.0f : m;
+        const float s = nh_lse_sum(a) * nh_exp_nonpos(a.v - mz) + nh_exp_nonpos(x - mz);
+        a.v = m; a.i = __builtin_bit_cast(int, s);
+    }
+    // N elements at once: one rescaling of the running sum for all of them
+    template <int N> static NEON_DEV void stepn(nh_pair& a, const float (&x)[N]) {
+        float m = a.v;
+#pragma unroll
+        for (int k = 0; k < N; ++k) m = nh_max(m, x[k]);
+        const float mz = (m == -NH_INF) ? 0.0f : m;
+        float s = nh_lse_sum(a) * nh_exp_nonpos(a.v - mz);
+#pragma unroll
+        for (int k = 0; k < N; ++k) s += nh_exp_nonpos(x[k] - mz);
+        a.v = m; a.i = __builtin_bit_cast(int, s);
+    }
+};
+
+// ---------------------------------------------------------------------------
+// Hand-off of partial results between workgroups (possibly on another XCD,
+// behind another L2).
+//
+// Producer: nh_part_store (8-byte relaxed device-scope atomic store: written
+// through to device-coherent memory), then nh_publish_barrier, then one lane
+// bumps the strip's counter with nh_ticket_take / nh_arrive.
+// Consumer: reads the counter (its own nh_ticket_take result, or nh_arrivals in
+// a bounded wait), a workgroup barrier, then nh_part_load (relaxed device-scope
+// atomic load: served from device-coherent memory, never from a stale line).
+//
+// Ordering.  The partial stores must be performed at device scope before the
+// counter update is.  Default build: every storing lane waits for its own
+// outstanding vector-memory operations (s_waitcnt vmcnt(0): on this part a
+// device-scope write-through store is acknowledged only once performed at
+// device scope), then the workgroup barrier, then the counter atomic -- so the
+// counter cannot be seen ahead of a partial.  This leans on that hardware
+// behaviour rather than on the language's memory model, which would want a
+// device-scope release before the counter update and an acquire after reading
+// it; those compile to a write-back and an invalidate of the whole L2, and
+// cost more than the kernels they sit in.  Defining NH_FORMAL_FENCES builds
+// exactly that variant (for comparison and for parts where the assumption
+// does not hold).
+// ---------------------------------------------------------------------------
+#ifndef NH_FORMAL_FENCES
+#define NH_FORMAL_FENCES 0
+#endif
 NEON_DEV void nh_part_store(nh_pair* p, nh_pair v) {
     __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), __builtin_bit_cast(unsigned long long, v),
                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -417,6 +517,33 @@ NEON_DEV void nh_part_store(nh_pair* p, nh_pair v) {
 NEON_DEV nh_pair nh_part_load(const nh_pair* p) {
     return __builtin_bit_cast(nh_pair, __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p),
                                                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+// All threads of the workgroup call it, after the last nh_part_store.
+NEON_DEV void nh_publish_barrier() {
+#if NH_FORMAL_FENCES
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+#else
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
+    __syncthreads();
+}
+// Counter update after nh_publish_barrier; returns the count before.
+NEON_DEV nh_u32 nh_ticket_take(nh_u32* ctr) {
+#if NH_FORMAL_FENCES
+    return __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+#else
+    return __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#endif
+}
+NEON_DEV nh_u32 nh_arrivals(const nh_u32* ctr) {
+#if NH_FORMAL_FENCES
+    return __hip_atomic_load(ctr, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+#else
+    return __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#endif
+}
+NEON_DEV void nh_ticket_reset(nh_u32* ctr) {
+    __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 template <int CTRL> NEON_DEV nh_pair nh_dpp(nh_pair p) { nh_pair r; r.v = nh_dpp<CTRL>(p.v); r.i = nh_dpp<CTRL>(p.i); return r; }

@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <string>
 
 #include "neonhip.h"
 #include "device/neon_device.h"
@@ -232,56 +233,73 @@ void launch_rownorm(uint16_t* out, const uint16_t* x, const float* gamma, const 
 
 // ---------------------------------------------------------------------------
 // Column (axis-0) max / argmax.  Lanes run across columns so every load is
-// coalesced; a workgroup is CR_LX column-lanes x CR_LY row-lanes and owns a
-// (rows_per_chunk x CR_LX*V) tile.  Tiles of one column strip leave (value,
-// index) partials in the workspace; the last workgroup of the strip to finish
-// (ticket counter) folds them into the result.  No workgroup ever waits for
-// another.  Partials cross XCDs as write-through stores / L2-bypassing loads,
-// so no device-wide fence (a whole-L2 write-back) is needed.
+// coalesced; a workgroup is LX column-lanes x (CR_T / LX) row-lanes and owns a
+// (rows_per_chunk x LX*V) tile: 8 lanes x 16 bytes = one 128-byte segment per
+// row, 32 rows per step and four steps in flight per lane.  The row-lanes of a
+// wave fold with lane exchanges that split the V values between the partners
+// (nh_col_wave_fold), LDS joins the four waves.  Tiles of one column strip
+// leave (value, index) partials in the scratch area; the last workgroup of the
+// strip to finish (ticket counter) folds them and writes the result.  No
+// workgroup ever waits for another.
+// Partials cross XCDs as write-through stores / L2-bypassing loads; each lane
+// waits for its own stores before the barrier that precedes the ticket.
 // ---------------------------------------------------------------------------
-constexpr int CR_LX = 16;
-constexpr int CR_LY = 16;
-constexpr int CR_T = CR_LX * CR_LY;
-constexpr int CR_WY = CR_T / 64;          // wave groups to join through LDS
+constexpr int CR_T = 256;
+constexpr int CR_WAVES = CR_T / 64;
+constexpr int CR_U = 4;                   // rows in flight per lane
+constexpr int CR_FOLD_BATCH = 4;          // partials in flight per lane in the final fold
 constexpr int CR_MAX_STRIPS = 4096;
 constexpr int CR_MAX_CHUNKS = 128;
-constexpr int CR_QMAX = CR_MAX_CHUNKS / CR_LY;
 
 __device__ unsigned int g_cr_tickets[CR_MAX_STRIPS];  // zero at load; each strip's last workgroup resets its ticket
 
-template <int V>
-__device__ __forceinline__ void cr_fold_rows(nh_pair (&acc)[V], nh_pair (*sp)[CR_LX * V + 1], int tx) {
-    // lanes of a wave that share a column tile differ in lane bits 4 and 5
-#pragma unroll
-    for (int j = 0; j < V; ++j) acc[j] = nh_op_argmax::f(acc[j], nh_lane_xor<16>(acc[j]));
-#pragma unroll
-    for (int j = 0; j < V; ++j) acc[j] = nh_op_argmax::f(acc[j], nh_lane_xor<32>(acc[j]));
+// Join the row-lanes of the workgroup: the row-lanes of a wave fold with lane
+// exchanges, the waves leave their pieces in LDS and ONE lane per column
+// (threads 0 .. LX*V-1) joins them.  The steps after the sweep are a chain of
+// dependent operations on a few values, so that chain is kept short rather
+// than wide.
+template <int V, int LX>
+__device__ __forceinline__ nh_pair cr_join_rows(nh_pair (&acc)[V], nh_pair (*sp)[LX * V]) {
+    constexpr int S = LX * V;
+    const int tx = threadIdx.x % LX;
     const int wave = threadIdx.x >> 6;
-    if ((threadIdx.x & 63) < CR_LX) {
+    if constexpr (LX < 64) {
+        constexpr int STEPS = __builtin_ctz(64 / LX);
+        constexpr int VK = (V >> STEPS) > 0 ? (V >> STEPS) : 1;     // values a lane still holds after the wave fold
+        const int j0 = nh_col_wave_fold<nh_op_argmax, V, LX>(acc);
+        if ((int)(threadIdx.x & 63) < LX * (V / VK)) {
+#pragma unroll
+            for (int j = 0; j < VK; ++j) sp[wave][tx * V + j0 + j] = acc[j];
+        }
+    } else {
 #pragma unroll
         for (int j = 0; j < V; ++j) sp[wave][tx * V + j] = acc[j];
     }
     __syncthreads();
+    nh_pair one = nh_op_argmax::init();
+    if ((int)threadIdx.x < S) {
+        one = sp[0][threadIdx.x];
 #pragma unroll
-    for (int j = 0; j < V; ++j) {
-        nh_pair r = sp[0][tx * V + j];
-#pragma unroll
-        for (int y = 1; y < CR_WY; ++y) r = nh_op_argmax::f(r, sp[y][tx * V + j]);
-        acc[j] = r;
+        for (int y = 1; y < CR_WAVES; ++y) one = nh_op_argmax::f(one, sp[y][threadIdx.x]);
     }
-    __syncthreads();
+    return one;
 }
 
-template <int V>
+template <int V, int LX>
 __global__ __launch_bounds__(CR_T) void colmax_kernel(const float* __restrict__ x, uint32_t rows, uint32_t cols,
                                                       size_t ld, uint32_t rows_per_chunk, nh_pair* part,
                                                       float* __restrict__ outv, int* __restrict__ outi,
                                                       unsigned int* tickets) {
-    __shared__ nh_pair sp[CR_WY][CR_LX * V + 1];
+    constexpr int LY = CR_T / LX;
+    constexpr int S = LX * V;                       // columns of a strip
+    constexpr int P = CR_T / S;                     // lanes per column in the last workgroup's fold
+    static_assert(S <= CR_T && P <= 64, "strip geometry");
+    __shared__ __attribute__((aligned(16))) nh_pair sp[CR_WAVES][S];
     __shared__ int s_last;
     const int tid = threadIdx.x;
-    const int tx = tid % CR_LX, ty = tid / CR_LX;
-    const uint32_t c = (blockIdx.x * CR_LX + tx) * V;
+    const int tx = tid % LX, ty = tid / LX;
+    const uint32_t c0 = blockIdx.x * S;
+    const uint32_t c = c0 + tx * V;
     const uint32_t r0 = blockIdx.y * rows_per_chunk;
     const uint32_t r1 = (r0 + rows_per_chunk < rows) ? r0 + rows_per_chunk : rows;
     const bool live = c < cols;  // cols % V == 0 is checked on the host
@@ -292,68 +310,60 @@ __global__ __launch_bounds__(CR_T) void colmax_kernel(const float* __restrict__ 
     if (live) {
         const float* xp = x + c;
         uint32_t r = r0 + ty;
-        // four independent rows in flight per lane
-        for (; r + 3 * CR_LY < r1; r += 4 * CR_LY) {
-            float a0[V], a1[V], a2[V], a3[V];
-            nh_load_vec<float, V>(xp + (size_t)r * ld, a0);
-            nh_load_vec<float, V>(xp + (size_t)(r + CR_LY) * ld, a1);
-            nh_load_vec<float, V>(xp + (size_t)(r + 2 * CR_LY) * ld, a2);
-            nh_load_vec<float, V>(xp + (size_t)(r + 3 * CR_LY) * ld, a3);
+        for (; r + (CR_U - 1) * LY < r1; r += CR_U * LY) {
+            float a[CR_U][V];
 #pragma unroll
-            for (int j = 0; j < V; ++j) {
-                nh_op_argmax::step(acc[j], a0[j], (int)r);
-                nh_op_argmax::step(acc[j], a1[j], (int)(r + CR_LY));
-                nh_op_argmax::step(acc[j], a2[j], (int)(r + 2 * CR_LY));
-                nh_op_argmax::step(acc[j], a3[j], (int)(r + 3 * CR_LY));
-            }
+            for (int u = 0; u < CR_U; ++u) nh_load_vec<float, V>(xp + (size_t)(r + u * LY) * ld, a[u]);
+#pragma unroll
+            for (int u = 0; u < CR_U; ++u)
+#pragma unroll
+                for (int j = 0; j < V; ++j) nh_op_argmax::step(acc[j], a[u][j], (int)(r + u * LY));
         }
-        for (; r < r1; r += CR_LY) {
+        for (; r < r1; r += LY) {
             float a0[V];
             nh_load_vec<float, V>(xp + (size_t)r * ld, a0);
 #pragma unroll
             for (int j = 0; j < V; ++j) nh_op_argmax::step(acc[j], a0[j], (int)r);
         }
     }
-    cr_fold_rows<V>(acc, sp, tx);
+    nh_pair one = cr_join_rows<V, LX>(acc, sp);     // threads 0 .. S-1: the strip's column c0 + tid
 
     const uint32_t nchunks = gridDim.y;
+    uint32_t col = tid;
+    bool writer = tid < S && c0 + tid < cols;
     if (nchunks > 1) {
-        if (ty == 0 && live) {
-#pragma unroll
-            for (int j = 0; j < V; ++j) nh_part_store(&part[(size_t)blockIdx.y * cols + c + j], acc[j]);
-        }
-        __syncthreads();  // every lane's partial stores have completed before the ticket is taken
+        if (writer) nh_part_store(&part[(size_t)blockIdx.y * cols + c0 + tid], one);
+        nh_publish_barrier();     // every lane's partial stores have been performed before the ticket is taken
         if (tid == 0) {
-            const unsigned int t = atomicAdd(&tickets[blockIdx.x], 1u);
+            const unsigned int t = nh_ticket_take(&tickets[blockIdx.x]);
             s_last = (t == nchunks - 1);
         }
         __syncthreads();
         if (!s_last) return;
 
-        nh_pair q[CR_QMAX][V];
+        // P adjacent lanes share a column; lane k0 of them takes chunks k0, k0 + P, ...
+        col = tid / P;
+        const uint32_t k0 = tid % P;
+        const bool fold_ok = c0 + col < cols;
+        one = nh_op_argmax::init();
+        for (uint32_t kb = k0; kb < nchunks; kb += P * CR_FOLD_BATCH) {
+            nh_pair q[CR_FOLD_BATCH];
 #pragma unroll
-        for (int k = 0; k < CR_QMAX; ++k) {
-            const uint32_t chunk = ty + k * CR_LY;
-#pragma unroll
-            for (int j = 0; j < V; ++j)
-                q[k][j] = (live && chunk < nchunks) ? nh_part_load(&part[(size_t)chunk * cols + c + j])
+            for (int k = 0; k < CR_FOLD_BATCH; ++k) {
+                const uint32_t chunk = kb + k * P;
+                q[k] = (fold_ok && chunk < nchunks) ? nh_part_load(&part[(size_t)chunk * cols + c0 + col])
                                                     : nh_op_argmax::init();
+            }
+#pragma unroll
+            for (int k = 0; k < CR_FOLD_BATCH; ++k) one = nh_op_argmax::f(one, q[k]);
         }
-#pragma unroll
-        for (int j = 0; j < V; ++j) acc[j] = nh_op_argmax::init();
-#pragma unroll
-        for (int k = 0; k < CR_QMAX; ++k)
-#pragma unroll
-            for (int j = 0; j < V; ++j) acc[j] = nh_op_argmax::f(acc[j], q[k][j]);
-        cr_fold_rows<V>(acc, sp, tx);
-        if (tid == 0) tickets[blockIdx.x] = 0;  // ready for the next launch on this stream
+        one = nh_wave_allreduce<nh_op_argmax, P, nh_pair>(one);
+        if (tid == 0) nh_ticket_reset(&tickets[blockIdx.x]);  // ready for the next launch on this stream
+        writer = k0 == 0 && fold_ok;
     }
-    if (ty == 0 && live) {
-#pragma unroll
-        for (int j = 0; j < V; ++j) {
-            if (outv) outv[c + j] = acc[j].v;
-            if (outi) outi[c + j] = acc[j].i;
-        }
+    if (writer) {
+        if (outv) outv[c0 + col] = one.v;
+        if (outi) outi[c0 + col] = one.i;
     }
 }
 
@@ -478,12 +488,16 @@ __global__ __launch_bounds__(HIST_T) void hist_log2_kernel(const T* __restrict__
     }
 }
 
-struct CrPlan { uint32_t strips, chunks, rows_per_chunk; int v; };
+struct CrPlan { uint32_t strips, chunks, rows_per_chunk; int v, lx; };
 
 CrPlan cr_plan(uint32_t rows, uint32_t cols, bool vec) {
     CrPlan p;
+    // 16-byte accesses, 8 column-lanes (128 bytes per row segment); matrices
+    // whose row length is not a multiple of four: one element per lane, 64 lanes
     p.v = vec ? 4 : 1;
-    const uint32_t strip_cols = CR_LX * p.v;
+    p.lx = vec ? 8 : 64;
+    const uint32_t ly = CR_T / p.lx;
+    const uint32_t strip_cols = p.lx * p.v;
     p.strips = (cols + strip_cols - 1) / strip_cols;
     // one workgroup per compute unit for small inputs, up to eight for large
     // ones, each with at least ~128 KiB to stream
@@ -496,9 +510,9 @@ CrPlan cr_plan(uint32_t rows, uint32_t cols, bool vec) {
     if (chunks < 1) chunks = 1;
     if (chunks > CR_MAX_CHUNKS) chunks = CR_MAX_CHUNKS;
     uint32_t rpc = (rows + chunks - 1) / chunks;
-    const uint32_t min_rpc = 4 * CR_LY;
+    const uint32_t min_rpc = CR_U * ly;
     if (rpc < min_rpc) rpc = min_rpc;
-    rpc = (rpc + CR_LY - 1) / CR_LY * CR_LY;
+    rpc = (rpc + ly - 1) / ly * ly;
     p.rows_per_chunk = rpc;
     p.chunks = (rows + rpc - 1) / rpc;
     if (p.chunks < 1) p.chunks = 1;
@@ -811,33 +825,45 @@ size_t nh_colreduce_workspace_bytes(uint32_t rows, uint32_t cols) {
     return (size_t)CR_MAX_CHUNKS * (size_t)cols * sizeof(nh_pair) + 256;
 }
 
+static int colmax_launch(const char* who, float* maxval, int32_t* argmax, const float* x, uint32_t rows, uint32_t cols,
+                         size_t ld, const CrPlan& p, nh_pair* part, unsigned int* tickets, hipStream_t s) {
+    dim3 grid(p.strips, p.chunks);
+    if (p.v == 4)
+        hipLaunchKernelGGL((colmax_kernel<4, 8>), grid, dim3(CR_T), 0, s, x, rows, cols, ld, p.rows_per_chunk, part,
+                           maxval, (int*)argmax, tickets);
+    else
+        hipLaunchKernelGGL((colmax_kernel<1, 64>), grid, dim3(CR_T), 0, s, x, rows, cols, ld, p.rows_per_chunk, part,
+                           maxval, (int*)argmax, tickets);
+    return launch_status(who);
+}
+
+static int colmax_check(const char* who, const float* maxval, const int32_t* argmax, const float* x, uint32_t rows,
+                        uint32_t cols, size_t ld, CrPlan* plan) {
+    if (!x || (!maxval && !argmax)) return nh_internal_fail(NH_EINVAL, (std::string(who) + ": null pointer").c_str());
+    if (ld < cols) return nh_internal_fail(NH_EINVAL, (std::string(who) + ": ld < cols").c_str());
+    if (rows > 0x7FFFFFFFu)
+        return nh_internal_fail(NH_EINVAL, (std::string(who) + ": too many rows for an int32 index").c_str());
+    const bool vec = (cols % 4 == 0) && (ld % 4 == 0);
+    *plan = cr_plan(rows, cols, vec);
+    if (plan->strips > CR_MAX_STRIPS) return nh_internal_fail(NH_EINVAL, (std::string(who) + ": too many columns").c_str());
+    if (plan->chunks > 65535u) return nh_internal_fail(NH_EINVAL, (std::string(who) + ": grid too large").c_str());
+    return 0;
+}
+
 int nh_colmax_argmax_f32(float* maxval, int32_t* argmax, const float* x, uint32_t rows, uint32_t cols, size_t ld,
                          void* workspace, void* stream) {
     if (!nh_internal_ready()) return nh_internal_fail(NH_ENOTINIT, "nh_init has not been called");
     if (rows == 0 || cols == 0) return 0;
-    if (!x || (!maxval && !argmax)) return nh_internal_fail(NH_EINVAL, "nh_colmax_argmax_f32: null pointer");
-    if (ld < cols) return nh_internal_fail(NH_EINVAL, "nh_colmax_argmax_f32: ld < cols");
-    if (rows > 0x7FFFFFFFu) return nh_internal_fail(NH_EINVAL, "nh_colmax_argmax_f32: too many rows for an int32 index");
-    const bool vec = (cols % 4 == 0) && (ld % 4 == 0) && aligned16(x);
-    const CrPlan p = cr_plan(rows, cols, vec);
-    if (p.strips > CR_MAX_STRIPS) return nh_internal_fail(NH_EINVAL, "nh_colmax_argmax_f32: too many columns");
+    CrPlan p;
+    if (int rc = colmax_check("nh_colmax_argmax_f32", maxval, argmax, x, rows, cols, ld, &p)) return rc;
     if (p.chunks > 1 && !workspace) return nh_internal_fail(NH_EINVAL, "nh_colmax_argmax_f32: workspace required");
-    if (p.chunks > 65535u) return nh_internal_fail(NH_EINVAL, "nh_colmax_argmax_f32: grid too large");
     if (p.chunks > 1 && (reinterpret_cast<uintptr_t>(workspace) & 7u))
         return nh_internal_fail(NH_EINVAL, "nh_colmax_argmax_f32: workspace must be 8-byte aligned");
-    nh_pair* part = (nh_pair*)workspace;
     unsigned int* tickets = nullptr;
     hipError_t e = hipGetSymbolAddress((void**)&tickets, HIP_SYMBOL(g_cr_tickets));
     if (e != hipSuccess) return nh_internal_fail((int)e, "nh_colmax_argmax_f32: ticket symbol lookup failed");
-    hipStream_t s = (hipStream_t)stream;
-    dim3 grid(p.strips, p.chunks);
-    if (vec)
-        hipLaunchKernelGGL((colmax_kernel<4>), grid, dim3(CR_T), 0, s, x, rows, cols, ld, p.rows_per_chunk, part,
-                           maxval, (int*)argmax, tickets);
-    else
-        hipLaunchKernelGGL((colmax_kernel<1>), grid, dim3(CR_T), 0, s, x, rows, cols, ld, p.rows_per_chunk, part,
-                           maxval, (int*)argmax, tickets);
-    return launch_status("nh_colmax_argmax_f32");
+    return colmax_launch("nh_colmax_argmax_f32", maxval, argmax, x, rows, cols, ld, p, (nh_pair*)workspace, tickets,
+                         (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -747,3 +747,70 @@ def test_narrow_elements_with_short_rows(pair, shape, dtype):
         res.append((e.get(), c.get(), r.get()))
     for want, got in zip(*res):
         assert np.array_equal(got, want)
+
+
+# ---- several reductions of one operand in one launch -----------------------------------------
+@pytest.mark.gpu
+def test_argmax_and_max_of_one_operand_fuse_into_one_launch(pair):
+    cpu, hip = pair
+    rs = np.random.RandomState(31)
+    x = (rs.standard_normal((5000, 200)) * 4).astype(np.float32)
+    x[17, 3] = x[900, 3] = x[:, 3].max() + 1.0          # a tie: the first row wins
+    X = hip.array(x)
+    am, mx, sm = hip.empty((1, 200), dtype=np.int32), hip.empty((1, 200)), hip.empty((1, 200))
+    before = hip.plan_stats["launches"]
+    with hip.fused():
+        am[:] = hip.argmax(X, axis=0)
+        mx[:] = hip.max(X, axis=0)
+        sm[:] = hip.sum(X, axis=0)
+    assert hip.plan_stats["launches"] - before == 1
+    assert np.array_equal(am.get(), x.argmax(axis=0).reshape(1, -1).astype(np.int32)) and am.get()[0, 3] == 17
+    assert np.array_equal(mx.get(), x.max(axis=0, keepdims=True))
+    assert_close(sm.get(), x.astype(np.float64).sum(axis=0, keepdims=True), rtol=1e-5, atol=1e-3)
+    # along the other axis, and a result that lives inside the operand stays out of the group
+    rm, rmin = hip.empty((5000, 1)), hip.empty((5000, 1))
+    before = hip.plan_stats["launches"]
+    with hip.fused():
+        rm[:] = hip.max(X, axis=1)
+        rmin[:] = hip.min(X, axis=1)
+    assert hip.plan_stats["launches"] - before == 1
+    assert np.array_equal(rm.get(), x.max(axis=1, keepdims=True)) and np.array_equal(rmin.get(), x.min(axis=1, keepdims=True))
+    before = hip.plan_stats["launches"]
+    with hip.fused():
+        mx[:] = hip.max(X, axis=0)
+        X[0:1, :] = hip.min(X, axis=0)
+    assert hip.plan_stats["launches"] - before == 2
+    want = x.copy()
+    want[0, :] = x.min(axis=0)
+    assert np.array_equal(X.get(), want) and np.array_equal(mx.get(), x.max(axis=0, keepdims=True))
+
+
+@pytest.mark.gpu
+def test_argmax_argmin_follow_numpy_on_nan(pair):
+    """np.argmax / np.argmin return the position of the first NaN
+    (reference nervanacpu.py:453-473 calls them directly)"""
+    cpu, hip = pair
+    rs = np.random.RandomState(32)
+    for shape in ((300, 40), (6000, 64), (40000, 16)):
+        x = rs.standard_normal(shape).astype(np.float32)
+        x[shape[0] // 2, 1] = np.nan
+        x[5, 2] = x[shape[0] - 3, 2] = np.nan
+        x[0, 3] = np.nan
+        x[shape[0] - 1, 4] = np.nan
+        x[:, 5] = -np.inf
+        x[7, 6] = np.inf
+        for name in ("argmax", "argmin"):
+            for axis in (0, 1):
+                def f(be):
+                    out = be.empty((1, shape[1]) if axis == 0 else (shape[0], 1), dtype=np.int32)
+                    out[:] = getattr(be, name)(be.array(x), axis=axis)
+                    return out.get()
+                want = getattr(np, name)(x, axis=axis).reshape(f(cpu).shape).astype(np.int32)
+                assert np.array_equal(f(cpu), want)
+                assert np.array_equal(f(hip), want), (name, axis, shape)
+    # and the values: max / min give NaN for those lines
+    x = rs.standard_normal((6000, 64)).astype(np.float32)
+    x[100, 1] = np.nan
+    mx = hip.empty((1, 64))
+    mx[:] = hip.max(hip.array(x), axis=0)
+    assert np.array_equal(mx.get(), x.max(axis=0, keepdims=True), equal_nan=True)

@@ -1,0 +1,87 @@
+"""The inter-workgroup hand-off of the split and cooperative kernel families
+(``colsplit`` ticket, ``colcoop`` / ``rowcoop`` waiting exchanges): a long
+alternating run on fresh data against numpy, and the host's handling of a
+cooperative kernel that gave up waiting."""
+import numpy as np
+import pytest
+
+from neon_amd.backends.hip import runtime as hiprt
+from utils import assert_close
+
+
+def _families(hip):
+    return set(p.spec.family for p in hip.plans.values())
+
+
+@pytest.mark.gpu
+def test_soak_alternating_split_and_cooperative_launches(hip):
+    """2100 launches, three families in turn, new random data every round
+    (drawn on the device); max / argmax bit-exact against numpy, sums against
+    float64; stops at the first mismatch"""
+    xs = hip.empty((2048, 128))          # colsplit: one level, one value per column
+    xc = hip.empty((20000, 64))          # colcoop: two levels over more rows than a workgroup holds
+    xr = hip.empty((8, 40000))           # rowcoop: few very long rows
+    am, mx = hip.empty((1, 128), dtype=np.int32), hip.empty((1, 128))
+    lse = hip.empty((1, 64))
+    rs_, dev = hip.empty((8, 1)), hip.empty((8, 40000))
+    for rnd in range(700):
+        for t in (xs, xc, xr):
+            t[:] = hip.rand() * 8.0 - 4.0
+        am[:] = hip.argmax(xs, axis=0)
+        mx[:] = hip.max(xs, axis=0)
+        lse[:] = hip.sum(hip.exp(xc - hip.max(xc, axis=0)), axis=0)
+        rs_[:] = hip.sum(xr, axis=1)
+        dev[:] = xr - hip.mean(xr, axis=1)
+        hs, hc, hr = xs.get(), xc.get().astype(np.float64), xr.get().astype(np.float64)
+        assert np.array_equal(am.get(), hs.argmax(axis=0).reshape(1, -1).astype(np.int32)), "argmax, round %d" % rnd
+        assert np.array_equal(mx.get(), hs.max(axis=0, keepdims=True)), "max, round %d" % rnd
+        want = np.exp(hc - hc.max(axis=0, keepdims=True)).sum(axis=0, keepdims=True)
+        assert_close(lse.get(), want, rtol=1e-5, atol=0, what="sum exp, round %d" % rnd)
+        assert_close(rs_.get(), hr.sum(axis=1, keepdims=True), rtol=1e-5, atol=1e-3, what="row sum, round %d" % rnd)
+        assert_close(dev.get(), hr - hr.mean(axis=1, keepdims=True), rtol=1e-5, atol=1e-5,
+                     what="row deviation, round %d" % rnd)
+    assert {"colsplit", "colcoop", "rowcoop"} <= _families(hip)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("family", ["colcoop", "rowcoop"])
+def test_a_cooperative_kernel_that_gave_up_is_reported_and_replaced(pair, family):
+    """Nothing is made to hang: the word an aborting workgroup would leave is
+    written into the plan's workspace from the host.  The next synchronisation
+    raises, and from then on the tree runs without inter-workgroup waits."""
+    cpu, hip = pair
+    rs = np.random.RandomState(9)
+    if family == "colcoop":
+        x = (rs.standard_normal((20000, 48)) * 2).astype(np.float32)
+
+        def run(be):
+            X, out = be.array(x), be.empty(x.shape)
+            out[:] = be.exp(X - be.max(X, axis=0)) / be.sum(be.exp(X - be.max(X, axis=0)), axis=0)
+            return out
+    else:
+        x = (rs.standard_normal((6, 50000)) * 2).astype(np.float32)
+
+        def run(be):
+            X, out = be.array(x), be.empty(x.shape)
+            out[:] = (X - be.mean(X, axis=1)) / be.sqrt(be.var(X, axis=1) + 1e-5)
+            return out
+    want = run(cpu).get()
+    hip.synchronize()
+    before = set(hip.plans)
+    assert_close(run(hip).get(), want, rtol=1e-5, atol=1e-6, what=family)
+    fresh = [hip.plans[k] for k in hip.plans if k not in before and hip.plans[k].spec.family == family]
+    assert len(fresh) == 1, "the tree should have run as one %s kernel" % family
+    plan = fresh[0]
+    hip.rt.memset(plan.status_ptr, 0xDEAD, 1, 4)
+    out = run(hip)                                   # runs normally, but the plan carries the mark
+    with pytest.raises(hiprt.HipError) as err:
+        hip.synchronize()
+    assert err.value.code == hiprt.NH_ECOOP
+    assert plan.key in hip._coop_failed and plan.key not in hip.plans
+    hip.synchronize()                                # reported once
+    again = run(hip)
+    got = again.get()
+    assert_close(got, want, rtol=1e-5, atol=1e-6, what=family + " after the fallback")
+    assert all(p.status_ptr is None for k, p in hip.plans.items() if k not in before), \
+        "the replacement must not wait between workgroups"
+    del out

@@ -120,8 +120,36 @@ def test_cse_and_levels(pb):
                                           pb.sum(pb.exp(x - pb.max(x, axis=0)), axis=0)))
     ops = [n.op for n in p.nodes if n.kind in ("E", "R")]
     assert ops.count("max") == 1 and ops.count("exp") == 1 and ops.count("sub") == 1   # duplicates merged
-    assert p.axis == 0 and p.nlevels == 2 and p.domain == (1000, 128)
+    assert p.axis == 0 and p.domain == (1000, 128)
     assert len(p.tensors) == 2 and p.tensors[0].written and p.tensors[1].read
+    # sum(exp(x - max)) shares the sweep that finds the maximum (running pair): one level;
+    # taking the pairing back restores one sweep each
+    assert p.lse_pairs == 1 and p.nlevels == 1
+    sm = [n for n in p.nodes if n.kind == "R" and n.op == "sum"][0]
+    assert sm.lse_max.op == "max" and sm.lse_max.lse_sum is sm and sm.level == sm.lse_max.level == 1
+    p.unpair_lse()
+    assert p.lse_pairs == 0 and p.nlevels == 2 and sm.lse_max is None and sm.level == 2
+
+
+def test_sum_over_a_one_hot_becomes_a_gather(pb):
+    x, ce = pb.empty((4000, 256)), pb.empty((1, 256))
+    idx = pb.empty((1, 256), dtype=np.int32)
+    full = pb.empty((4000, 256))
+
+    def cross_entropy():
+        sm = pb.exp(x - pb.max(x, axis=0)) / pb.sum(pb.exp(x - pb.max(x, axis=0)), axis=0)
+        ce[:] = -pb.sum(pb.onehot(idx, axis=0) * pb.log(sm), axis=0)
+    p = _prog(pb, cross_entropy)
+    assert p.gathers == 1 and p.lse_pairs == 1 and p.nlevels == 1
+    g = [n for n in p.nodes if n.kind == "G"][0]
+    assert g.args[1].kind == "H" and g.args[0].op == "log" and not g.vr and g.vc and g.level == 1
+    # a column-sum that is broadcast back over the rows stays a sum
+    p2 = _prog(pb, lambda: full.__setitem__(slice(None), x - pb.sum(pb.onehot(idx, axis=0) * x, axis=0)))
+    assert p2.gathers == 0 and p2.nlevels == 1
+    # ... as does one along the other axis of the one-hot
+    rows = pb.empty((4000, 1))
+    p3 = _prog(pb, lambda: rows.__setitem__(slice(None), pb.sum(pb.onehot(idx, axis=0) * x, axis=1)))
+    assert p3.gathers == 0
 
 
 def test_constant_folding_and_key(pb):
@@ -256,10 +284,17 @@ def test_shape_class_selection(pb):
     ch = plan_of(pb, lambda: pb.empty((1, 256), np.int32).__setitem__(slice(None), pb.argmax(x5, axis=0)))
     assert ch.spec.family == "colsplit" and ch.workspace is not None
     assert ch.grid[0] * ch.grid[1] <= 2 * 256 and ch.grid[1] <= codegen.COLSPLIT_MAX_CHUNKS
-    # three sweeps over 32000 rows do not fit one workgroup: the workgroups of a strip cooperate
+    # several sweeps over 32000 rows do not fit one workgroup: the workgroups of a strip cooperate;
+    # maximum and sum of exponentials travel together, so they meet once, not twice
     ch = plan_of(pb, lambda: pb.empty((32000, 256)).__setitem__(slice(None), pb.fprop_softmax(x5, 0)))
     assert ch.spec.family == "colcoop" and ch.grid[0] * ch.grid[1] <= 256 and ch.workspace is not None
-    assert ch.spec.source.count("nh_part_store") == 2 and "NH_SPIN_LIMIT" in ch.spec.source
+    assert ch.spec.source.count("nh_part_store") == 1 and "NH_SPIN_LIMIT" in ch.spec.source
+    assert "nh_op_lse" in ch.spec.source and ch.status_offset is not None
+    # cross-entropy with the one-hot made in the kernel: one pass, no waiting at all
+    i5 = pb.empty((1, 256), np.int32)
+    ch = plan_of(pb, lambda: pb.empty((1, 256)).__setitem__(slice(None), -pb.sum(
+        pb.onehot(i5, axis=0) * pb.log(pb.fprop_softmax(x5, 0)), axis=0)))
+    assert ch.spec.family == "colsplit" and "NH_SPIN_LIMIT" not in ch.spec.source and "nh_op_lse" in ch.spec.source
     huge = pb.empty((4000000, 256))
     with pytest.raises(planner.NeedsSplit):        # too many rows to keep on chip: evaluated stage by stage
         pb.empty((4000000, 256)).__setitem__(slice(None), pb.fprop_softmax(huge, 0))
