@@ -176,6 +176,25 @@ int nh_colmax_argmax_f32(float* maxval, int32_t* argmax, const float* x,
                          uint32_t rows, uint32_t cols, size_t ld,
                          void* workspace, void* stream);
 
+/* The same reduction for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): no workspace argument and no allocation of any kind -- the
+ * partials and tickets live in a static device array of
+ * NH_STATIC_SCRATCH_BYTES that every device holds from library load until the
+ * process ends.  There is no counterpart in the reference (PyCUDA allocates
+ * freely; neon/backends/nervanagpu.py:87,147).  Shapes whose partials do not
+ * fit (16 KiB of tickets + row chunks * cols * 8 bytes; the launch geometry
+ * keeps that within the array for every matrix whose row length is a multiple
+ * of four, and for other row lengths up to about 8000 columns) are refused
+ * with NH_EINVAL before anything is launched.  All calls on one device
+ * share the array: calls that overlap in time on one device (different
+ * streams or threads) race; calls on one stream are safe back to back (the
+ * tickets are cleared by a small kernel ahead of the reduction, so the call
+ * can be recorded into a graph).                                             */
+#define NH_STATIC_SCRATCH_BYTES (1u << 20)
+int nh_colmax_argmax_f32_static(float* maxval, int32_t* argmax, const float* x,
+                                uint32_t rows, uint32_t cols, size_t ld, void* stream);
+
 /* 64-bin (nbins <= 256) histogram of rint(log2|x|) over n contiguous fp32
  * (itemsize 4) or fp16 (itemsize 2) elements into hist[nbins] (cleared
  * first): bin 0 reaches down to -inf, bin k >= 1 holds offset+k, the last bin

@@ -104,6 +104,8 @@ SIGNATURES = {
     "nh_colreduce_workspace_bytes": (c_size_t, [c_uint32, c_uint32]),
     "nh_colmax_argmax_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_uint32, c_uint32,
                                      c_size_t, c_void_p, c_void_p]),
+    "nh_colmax_argmax_f32_static": (c_int, [c_void_p, c_void_p, c_void_p, c_uint32, c_uint32,
+                                            c_size_t, c_void_p]),
 }
 
 _lib = None

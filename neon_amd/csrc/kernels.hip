@@ -13,6 +13,7 @@
 bool nh_internal_ready();
 int nh_internal_fail(int code, const char* msg);
 int nh_internal_cu_count();
+int nh_internal_device();
 
 namespace {
 
@@ -253,6 +254,12 @@ constexpr int CR_MAX_CHUNKS = 128;
 
 __device__ unsigned int g_cr_tickets[CR_MAX_STRIPS];  // zero at load; each strip's last workgroup resets its ticket
 
+// Scratch of the entry point that allocates nothing: tickets first, partials
+// after them.  One copy per device, alive until the process ends; host code
+// reaches it through the address hipGetSymbolAddress returns for the device.
+constexpr size_t CR_STATIC_TICKET_BYTES = (size_t)CR_MAX_STRIPS * sizeof(unsigned int);
+static __device__ __align__(256) unsigned char scratch[NH_STATIC_SCRATCH_BYTES];
+
 // Join the row-lanes of the workgroup: the row-lanes of a wave fold with lane
 // exchanges, the waves leave their pieces in LDS and ONE lane per column
 // (threads 0 .. LX*V-1) joins them.  The steps after the sweep are a chain of
@@ -365,6 +372,13 @@ __global__ __launch_bounds__(CR_T) void colmax_kernel(const float* __restrict__ 
         if (outv) outv[c0 + col] = one.v;
         if (outi) outi[c0 + col] = one.i;
     }
+}
+
+// clears the tickets of the static scratch area (a kernel rather than a
+// memset so that the call can be recorded into a graph)
+__global__ void cr_clear_tickets_kernel(unsigned int* tickets, uint32_t n) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) tickets[i] = 0u;
 }
 
 // ---------------------------------------------------------------------------
@@ -519,6 +533,11 @@ CrPlan cr_plan(uint32_t rows, uint32_t cols, bool vec) {
     return p;
 }
 
+// per device: address of this file's `scratch` array on that device (the
+// array's name is only a host-side handle), looked up once by nh_init
+constexpr int CR_MAX_DEVICES = 64;
+void* g_scratch_ptr[CR_MAX_DEVICES];
+
 // ---------------------------------------------------------------------------
 // Dimension shuffle (numpy.transpose into a destination tensor).  Dimensions
 // are given in OUTPUT order, each with its output and its input stride.  A
@@ -672,6 +691,21 @@ void launch_transpose(void* out, const void* in, const TrGeom& g, bool swap, uns
 
 
 }  // namespace
+
+// Called by nh_init with `device` current: every device holds its own copy of
+// `scratch` at its own address.
+int nh_internal_scratch_setup(int device) {
+    if (device < 0 || device >= CR_MAX_DEVICES) return 0;      // such a device simply has no static entry point
+    if (g_scratch_ptr[device]) return 0;
+    void* ptr = nullptr;
+    hipError_t e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return nh_internal_fail((int)e, "nh_init: address lookup of the static scratch area failed");
+    }
+    g_scratch_ptr[device] = ptr;
+    return 0;
+}
 
 extern "C" {
 
@@ -864,6 +898,33 @@ int nh_colmax_argmax_f32(float* maxval, int32_t* argmax, const float* x, uint32_
     if (e != hipSuccess) return nh_internal_fail((int)e, "nh_colmax_argmax_f32: ticket symbol lookup failed");
     return colmax_launch("nh_colmax_argmax_f32", maxval, argmax, x, rows, cols, ld, p, (nh_pair*)workspace, tickets,
                          (hipStream_t)stream);
+}
+
+int nh_colmax_argmax_f32_static(float* maxval, int32_t* argmax, const float* x, uint32_t rows, uint32_t cols,
+                                size_t ld, void* stream) {
+    if (!nh_internal_ready()) return nh_internal_fail(NH_ENOTINIT, "nh_init has not been called");
+    if (rows == 0 || cols == 0) return 0;
+    CrPlan p;
+    if (int rc = colmax_check("nh_colmax_argmax_f32_static", maxval, argmax, x, rows, cols, ld, &p)) return rc;
+    const int dev = nh_internal_device();
+    if (dev < 0 || dev >= CR_MAX_DEVICES || !g_scratch_ptr[dev])
+        return nh_internal_fail(NH_ENOTINIT, "nh_colmax_argmax_f32_static: no scratch area for this device");
+    const size_t need = CR_STATIC_TICKET_BYTES + (p.chunks > 1 ? (size_t)p.chunks * cols * sizeof(nh_pair) : 0);
+    if (need > (size_t)NH_STATIC_SCRATCH_BYTES)
+        return nh_internal_fail(NH_EINVAL,
+                                ("nh_colmax_argmax_f32_static: needs " + std::to_string(need) +
+                                 " bytes of scratch, the static area holds " + std::to_string((size_t)NH_STATIC_SCRATCH_BYTES) +
+                                 " (use nh_colmax_argmax_f32 with a workspace)").c_str());
+    unsigned char* base = (unsigned char*)g_scratch_ptr[dev];
+    unsigned int* tickets = (unsigned int*)base;
+    nh_pair* part = (nh_pair*)(base + CR_STATIC_TICKET_BYTES);
+    hipStream_t s = (hipStream_t)stream;
+    if (p.chunks > 1) {
+        // the area keeps whatever the last call left: tickets have to start at zero
+        hipLaunchKernelGGL(cr_clear_tickets_kernel, dim3((p.strips + 255) / 256), dim3(256), 0, s, tickets, p.strips);
+        if (int rc = launch_status("nh_colmax_argmax_f32_static: clearing the tickets")) return rc;
+    }
+    return colmax_launch("nh_colmax_argmax_f32_static", maxval, argmax, x, rows, cols, ld, p, part, tickets, s);
 }
 
 }  // extern "C"

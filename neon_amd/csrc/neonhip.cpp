@@ -15,6 +15,7 @@
 #include <vector>
 
 void nh_internal_blas_release();      // gemm.cpp: drops the rocBLAS handle, if one was created
+int nh_internal_scratch_setup(int device);   // kernels.hip: per-device address of the static scratch area
 
 namespace {
 
@@ -77,6 +78,10 @@ int nh_init(int device, nh_props* props) {
     NH_HIP(hipFree(nullptr));  // force context creation now, not inside a timed region
     g_device = device;
     g_init = true;
+    if (int rc = nh_internal_scratch_setup(device)) {
+        g_init = false;
+        return rc;
+    }
     if (props) {
         std::memset(props, 0, sizeof(*props));
         std::snprintf(props->arch, sizeof(props->arch), "%s", g_prop.gcnArchName);
@@ -416,3 +421,4 @@ int nh_launch_timed(void* function, const uint32_t grid[3], const uint32_t block
 bool nh_internal_ready() { return g_init; }
 int nh_internal_fail(int code, const char* msg) { return fail(code, msg); }
 int nh_internal_cu_count() { return g_init ? g_prop.multiProcessorCount : 0; }
+int nh_internal_device() { return g_init ? g_device : -1; }
