@@ -112,6 +112,16 @@ class _Gen(object):
         self.ld = "load_stream" if stream else "load"
         self.st = "store_stream" if (stream and STREAM_STORES[family]) else "store"
         self.prefetched = set()    # gather nodes whose operands were fetched ahead of the sweep
+        self.one_declared = False  # the kernel holds ``nh_one`` (see declare_one)
+
+    def is_half_leaf(self, n):
+        return n.kind == "T" and DTYPE_CODE[self.prog.tensors[n.slot].dtype] == "f2"
+
+    def declare_one(self):
+        """kernels that read fp16 tensors keep an opaque 1.0f for mixed-precision fma forms"""
+        if any(t.read and DTYPE_CODE[t.dtype] == "f2" for t in self.prog.tensors):
+            self.L("const float nh_one = nh_opaque_one();")
+            self.one_declared = True
 
     # -- parameters -----------------------------------------------------------------
     def slot_ctype(self, slot):
@@ -258,6 +268,12 @@ class _Gen(object):
             return "nh_sround(%s, %s, %s)" % (a[0], n.op.split(":")[1], word)
         if len(a) == 1:
             return _UN[n.op].format(*a)
+        if n.op in ("add", "sub") and self.one_declared and any(self.is_half_leaf(x) for x in n.args):
+            # widening of the fp16 operand and the addition in one instruction
+            # (v_fma_mix_f32); bit-identical to the plain sum / difference
+            if self.is_half_leaf(n.args[0]):
+                return "__builtin_fmaf({0}, nh_one, {2}{1})".format(a[0], a[1], "-" if n.op == "sub" else "")
+            return "__builtin_fmaf({1}, {2}nh_one, {0})".format(a[0], a[1], "-" if n.op == "sub" else "")
         if n.op == "div" and in_loop and RECIPROCAL_OF_BROADCAST and _broadcast_under(n.args[1], n.args[0]):
             # the divisor is constant along an axis the dividend varies on
             return "nh_div_by_line({0}, {1})".format(*a)
@@ -356,11 +372,53 @@ class _Gen(object):
 
 
 RECIPROCAL_OF_BROADCAST = os.environ.get("NEON_HIP_RCP", "1") != "0"
+FMA_IN_SUMS = os.environ.get("NEON_HIP_FMA_SUMS", "1") != "0"
+# results stored as 16-bit floats: a chain of multiplications / divisions by
+# per-line values and a final per-line addend collapse into one multiply-add
+AFFINE_16BIT_OUTPUTS = os.environ.get("NEON_HIP_AFFINE16", "1") != "0"
 
 
 def _broadcast_under(b, a):
     """b is constant along at least one axis on which a varies, and varies on none that a does not"""
     return (b.vr <= a.vr and b.vc <= a.vc) and (b.vr < a.vr or b.vc < a.vc)
+
+
+def _affine_in_line(root, constant):
+    """``root`` as ``atom * A + B``: walks down from ``root`` through additions of
+    and multiplications / divisions by values that are constant along the line
+    (``constant(node)``), never distributing a product over a sum -- the
+    subtraction that centres the data stays as written inside ``atom``.
+    Returns (atom, [('mul'|'div', node)...], [('add'|'sub', node)...]) with the
+    factors in evaluation order, or None when nothing can be peeled off.
+    Addends are only taken from the outside (before any factor), so that
+    ``root == atom * prod(factors) + sum(addends)`` holds term for term."""
+    addends, mults = [], []
+    n = root
+    # outer additive terms
+    while n.kind == "E" and n.op in ("add", "sub") and len(n.args) == 2:
+        a, b = n.args
+        if constant(b) and not constant(a):
+            addends.append(("add" if n.op == "add" else "sub", b))
+            n = a
+        elif constant(a) and not constant(b) and n.op == "add":
+            addends.append(("add", a))
+            n = b
+        else:
+            break
+    # multiplicative chain below them
+    while n.kind == "E" and n.op in ("mul", "div") and len(n.args) == 2:
+        a, b = n.args
+        if constant(b) and not constant(a):
+            mults.append((n.op, b))
+            n = a
+        elif constant(a) and not constant(b) and n.op == "mul":
+            mults.append(("mul", a))
+            n = b
+        else:
+            break
+    if constant(n) or n is root:
+        return None
+    return n, mults, addends
 
 
 def _needed(targets, available):
@@ -463,6 +521,7 @@ def gen_ew(prog, V, LX, LY, UC, UR, tail, stream=False):
             L("o%d%s.%s(%s);" % (st.out.index, sfx, g.st, g.addr(st.out, r, c)))
 
     L.open("")
+    g.declare_one()
     L("const int tx = threadIdx.x %% %d, ty = threadIdx.x / %d;" % (LX, LX))
     if hoisted:
         for uc in range(UC):
@@ -667,10 +726,19 @@ class _RedGen(_Gen):
         else:
             L("%s acc%d = %s::init();" % ("nh_pair" if n.is_index else "float", n.nid, op))
 
-    def accumulate(self, n, val, index):
+    def accumulate(self, n, val, index, ref=None):
         """fold one element into the lane's accumulator (inside the j loop)"""
         op = self.red_op(n)
         acc = ("acc%d[j]" % n.nid) if self.col_axis else ("acc%d" % n.nid)
+        arg = n.args[0]
+        if (ref is not None and n.op == "sum" and not self.fused_sum(n) and arg.kind == "E"
+                and arg.op in ("sqr", "mul") and FMA_IN_SUMS):
+            # sum of products: multiply-add with one rounding per term (the
+            # sum's order already differs from the CPU's; this only makes each
+            # term a little more accurate)
+            a, b = (arg.args[0], arg.args[0]) if arg.op == "sqr" else arg.args
+            self.L("%s = __builtin_fmaf(%s, %s, %s);" % (acc, ref(a), ref(b), acc))
+            return
         if self.fused_max(n):
             self.L("%s::step(%s, %s);" % (op, acc, val))
         elif n.is_index:
@@ -732,6 +800,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
         L("__shared__ float s_f[%d];" % (T // 64))
         L("__shared__ nh_pair s_p[%d];" % (T // 64))
     L("const int tx = threadIdx.x %% %d, ty = threadIdx.x / %d;" % (LX, LX))
+    g.declare_one()
     L("const long long r = (long long)blockIdx.x * %d + ty;" % LY)
     L("const bool row_ok = r < R;")
     L("const long long rr = row_ok ? r : 0;")   # address clamp for idle teams
@@ -941,6 +1010,16 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
 
         def reduce_body(tiles, nodes=nodes, reds=reds, fresh=fresh):
             L.open("if (ok)")
+            # plain sums of a packed fp16 operand: two elements per instruction, straight
+            # from the tile (a partial last tile is zero-filled, so it needs no guard)
+            pairwise = [n for n in reds if n.op == "sum" and g.is_half_leaf(n.args[0]) and V % 2 == 0
+                        and n.args[0].nid not in vals and g.tile_width(n.args[0], V) == V]
+            for n in pairwise:
+                L("acc%d = %s.sum_into(acc%d);" % (n.nid, tiles[n.args[0].nid], n.nid))
+            reds = [n for n in reds if n not in pairwise]
+            if not reds and not fresh:
+                L.close()
+                return
             if V > 1:
                 L("#pragma unroll")
             L.open("for (int j = 0; j < %d; ++j)" % V)
@@ -949,7 +1028,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
             ref = g.make_ref("_s", "rr", "c", V, tiles, vals)
             g.emit_exprs(nodes, ref, stops())
             for n in reds:
-                g.accumulate(n, ref(n.args[0]), "c + j")
+                g.accumulate(n, ref(n.args[0]), "c + j", ref)
             for n in fresh:
                 L("keep%d[k].put(j, t%d);" % (over[n.nid].nid, n.nid))
             if tail:
@@ -1007,6 +1086,36 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
         leaves = g.leaf_nodes(nodes)
         declare_tiles(leaves)
 
+        # Results stored as 16-bit floats: root = atom * A + B with A, B constant along the row
+        # (a chain of multiplications / divisions by per-row values and a last per-row addend)
+        # is evaluated as ONE multiply-add per element, A and B once per row.
+        collapsed = {}
+        if AFFINE_16BIT_OUTPUTS:
+            line_ref = g.make_ref("_s", "rr", "0", 1, dict((nid, name) for nid, name in line_tiles.items()), vals)
+            for st in full_out:
+                if DTYPE_CODE[st.out.dtype] != "f2" or st.root.kind != "E":
+                    continue
+                aff = _affine_in_line(st.root, lambda m: not m.vc)
+                if aff is None:
+                    continue
+                atom, mults, addends = aff
+                if not mults and not addends:
+                    continue
+                consts = _needed([m for _, m in mults] + [m for _, m in addends], stops())
+                L("float fa%d = 1.0f, fb%d = 0.0f;" % (st.out.index, st.out.index))
+                L.open("")
+                L("const int j = 0; (void)j;")
+                g.emit_exprs(consts, line_ref, stops())
+                for kind, m in mults:
+                    L("fa%d = fa%d %s %s;" % (st.out.index, st.out.index, "*" if kind == "mul" else "/", line_ref(m)))
+                for kind, m in addends:
+                    L("fb%d = fb%d %s %s;" % (st.out.index, st.out.index, "+" if kind == "add" else "-", line_ref(m)))
+                L.close()
+                collapsed[st.out.index] = atom
+            if collapsed:
+                nodes = _needed([collapsed.get(st.out.index, st.root) for st in full_out], stops())
+                leaves = g.leaf_nodes(nodes)
+
         def store_body(tiles):
             L.open("if (ok)")
             for st in full_out:
@@ -1019,6 +1128,9 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
             for st in full_out:
                 if st.root.kind == "R" and st.root.is_index:
                     L("o%d.seti(j, ri%d);" % (st.out.index, st.root.nid))
+                elif st.out.index in collapsed:
+                    L("o%d.set(j, __builtin_fmaf(%s, fa%d, fb%d));"
+                      % (st.out.index, ref(collapsed[st.out.index]), st.out.index, st.out.index))
                 else:
                     L("o%d.set(j, %s);" % (st.out.index, ref(st.root)))
             L.close()
@@ -1162,6 +1274,7 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False)
 
     L.open("")
     lds = _col_lds(L, LX, LY, T, V, any_index or coop)
+    g.declare_one()
     L("const int tx = threadIdx.x %% %d, ty = threadIdx.x / %d;" % (LX, LX))
     L("const long long c = ((long long)blockIdx.x * %d + tx) * %d;" % (LX, V))
     L("const bool col_ok = c < C;")
@@ -1403,7 +1516,7 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False)
             if n in local:
                 L("ls%d[j] += nh_exp_nonpos(%s - lz%d[j]);" % (n.nid, ref(n.args[0]), n.nid))
             else:
-                g.accumulate(n, ref(n.args[0]), "r")
+                g.accumulate(n, ref(n.args[0]), "r", ref)
         fresh = stash_new_values(nodes)
         L.close()
         L.close()
@@ -1549,6 +1662,7 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1):
         L("__shared__ __attribute__((aligned(16))) %s s_r%d[%d];" % (ty_, n.nid, S))
         lds += (WY + 1) * S * (8 if g.is_pair(n) else 4)
     L("__shared__ int s_last;")
+    g.declare_one()
     L("const int tx = threadIdx.x %% %d, ty = threadIdx.x / %d;" % (LX, LX))
     L("const long long c0 = (long long)blockIdx.x * %d;" % S)
     L("const long long c = c0 + tx * %d;" % V)
@@ -1593,7 +1707,7 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1):
                 if n in batched:
                     L("lv%d[%d] = %s;" % (n.nid, u, ref(n.args[0])))
                 else:
-                    g.accumulate(n, ref(n.args[0]), "r + %d" % (u * LY))
+                    g.accumulate(n, ref(n.args[0]), "r + %d" % (u * LY), ref)
             L.close()
         for n in batched:
             L("nh_op_lse::stepn<%d>(acc%d[j], lv%d);" % (U, n.nid, n.nid))
@@ -1606,7 +1720,7 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1):
             ref = g.make_ref("_%d" % u, "r + %d" % (u * LY), "c", V)
             g.emit_exprs(nodes, ref, {})
             for n in reds:
-                g.accumulate(n, ref(n.args[0]), "r + %d" % (u * LY))
+                g.accumulate(n, ref(n.args[0]), "r + %d" % (u * LY), ref)
             L.close()
     L.close()
     L.open("for (; r < r1; r += %d)" % LY)
@@ -1618,7 +1732,7 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1):
     ref = g.make_ref("_t", "r", "c", V)
     g.emit_exprs(nodes, ref, {})
     for n in reds:
-        g.accumulate(n, ref(n.args[0]), "r")
+        g.accumulate(n, ref(n.args[0]), "r", ref)
     L.close()
     L.close()
     L.close()

@@ -165,6 +165,17 @@ NEON_DEV nh_u32 nh_f16_pack(float lo, float hi) {
     nh_f16x2 h; h.x = (nh_f16)lo; h.y = (nh_f16)hi;
     return __builtin_bit_cast(nh_u32, h);
 }
+// acc + lo + hi of a packed fp16 pair in one instruction (v_dot2c_f32_f16 with
+// a pair of ones; fp32 accumulation)
+NEON_DEV float nh_sum2_f16(nh_u32 w, float acc) {
+    nh_f16x2 ones; ones.x = (nh_f16)1.0f; ones.y = (nh_f16)1.0f;
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(nh_f16x2, w), ones, acc, false);
+}
+// 1.0f the compiler cannot see through.  fma(x, one, y) with x widened from
+// fp16 selects v_fma_mix_f32 -- widening and the addition in ONE instruction,
+// same result as (float)x + y -- where a plain x + y would be folded back into
+// a conversion followed by an add.
+NEON_DEV float nh_opaque_one() { float one; asm volatile("v_mov_b32 %0, 1.0" : "=v"(one)); return one; }
 NEON_DEV float nh_bf16_lo(nh_u32 w) { return __builtin_bit_cast(float, w << 16); }
 NEON_DEV float nh_bf16_hi(nh_u32 w) { return __builtin_bit_cast(float, w & 0xFFFF0000u); }
 // Compiler barrier on register-resident data: the values are unchanged but
@@ -235,6 +246,13 @@ template <typename T, int V> struct nh_raw {
 #pragma unroll
         for (int i = 0; i < NW; ++i) asm volatile("" : "+v"(w[i]));
     }
+    // acc + all V elements of a packed fp16 tile, two elements per instruction
+    NEON_DEV float sum_into(float acc) const {
+        static_assert(sizeof(T) == 2 && PACKED, "packed 16-bit tiles only");
+#pragma unroll
+        for (int i = 0; i < NW; ++i) acc = nh_sum2_f16(w[i], acc);
+        return acc;
+    }
     // the first n (< V) elements, one at a time; the rest of the tile is zero
     NEON_DEV void load_partial(const T* p, int n) {
         zero();
@@ -269,7 +287,18 @@ template <typename T, int V> struct nh_out {
         if constexpr (sizeof(T) == 4) w[PACKED ? j : 0] = bits;
         else w[PACKED ? j / PER : 0] |= bits << (8 * (int)sizeof(T) * (PACKED ? j % PER : 0));
     }
-    NEON_DEV void set(int j, float x) { put_bits(j, nh_bits_of<T>(nh_store_cvt<T>::f(x))); }
+    NEON_DEV void set(int j, float x) {
+        if constexpr (sizeof(T) == 2 && PACKED && nh_is_float<T>::value) {
+            // element insert into the pair (with a compile-time j, a conversion that
+            // writes its half of the register directly)
+            typedef T pair_t __attribute__((ext_vector_type(2)));
+            pair_t v = __builtin_bit_cast(pair_t, w[j / 2]);
+            if (j & 1) v.y = nh_store_cvt<T>::f(x); else v.x = nh_store_cvt<T>::f(x);
+            w[j / 2] = __builtin_bit_cast(nh_u32, v);
+        } else {
+            put_bits(j, nh_bits_of<T>(nh_store_cvt<T>::f(x)));
+        }
+    }
     NEON_DEV void seti(int j, int i) { put_bits(j, nh_bits_of<T>(nh_store_index<T>(i))); }
     NEON_DEV void store(T* p) const {
         if constexpr (PACKED) nh_store_vec<nh_u32, NW>(reinterpret_cast<nh_u32*>(p), w);
