@@ -111,6 +111,24 @@ int nh_module_get_function(void* module, const char* name, void** function);
 int nh_launch(void* function, const uint32_t grid[3], const uint32_t block[3],
               uint32_t lds_bytes, void* stream, const void* args, size_t arg_bytes);
 
+/* The same launch from a record filled in once: a statement that is issued
+ * again and again (an optimizer step, a layer's forward pass) re-uses its
+ * record, and the call crosses the boundary with a single pointer.  The fields
+ * are validated like nh_launch's arguments on every call (a handful of integer
+ * compares).  `args` must stay valid and unchanged until the call returns.
+ * replaces: kernel.prepare(signature) once + kernel.prepared_async_call(...)
+ *           per launch (float_ew.py:612-615, 929-931).                          */
+typedef struct nh_launch_rec {
+    void* function;
+    uint32_t grid[3];
+    uint32_t block[3];
+    uint32_t lds_bytes;
+    uint32_t arg_bytes;
+    void* stream;
+    const void* args;
+} nh_launch_rec;
+int nh_launch_prepared(const nh_launch_rec* rec);
+
 /* Launch the same kernel `reps` times back to back between two events on
  * `stream`, wait, and return the mean time per launch in milliseconds.
  * replaces: the event bracket of the reference's bench mode

@@ -45,6 +45,12 @@ class Props(ctypes.Structure):
                 ("hbm_bytes", c_uint64)]
 
 
+class LaunchRec(ctypes.Structure):
+    """nh_launch_rec: one prepared launch"""
+    _fields_ = [("function", c_void_p), ("grid", c_uint32 * 3), ("block", c_uint32 * 3),
+                ("lds_bytes", c_uint32), ("arg_bytes", c_uint32), ("stream", c_void_p), ("args", c_void_p)]
+
+
 # name -> (restype, argtypes); must list every symbol include/neonhip.h declares
 SIGNATURES = {
     "nh_abi_version": (c_int, []),
@@ -80,6 +86,7 @@ SIGNATURES = {
     "nh_module_get_function": (c_int, [c_void_p, c_char_p, POINTER(c_void_p)]),
     "nh_launch": (c_int, [c_void_p, POINTER(c_uint32), POINTER(c_uint32), c_uint32,
                           c_void_p, c_void_p, c_size_t]),
+    "nh_launch_prepared": (c_int, [c_void_p]),
     "nh_launch_timed": (c_int, [c_void_p, POINTER(c_uint32), POINTER(c_uint32), c_uint32,
                                 c_void_p, c_void_p, c_size_t, c_uint32, POINTER(c_float)]),
     "nh_launch_timed_sets": (c_int, [c_void_p, POINTER(c_uint32), POINTER(c_uint32), c_uint32,
@@ -168,6 +175,7 @@ class Runtime(object):
         self.stream = c_void_p(None)      # null stream
         self._grid = (c_uint32 * 3)()
         self._block = (c_uint32 * 3)()
+        self._launch_prepared = self.lib.nh_launch_prepared
 
     # -- memory ------------------------------------------------------------------
     def malloc(self, nbytes):
@@ -251,6 +259,25 @@ class Runtime(object):
         g[0], g[1], g[2] = grid
         b[0], b[1], b[2] = block
         rc = self.lib.nh_launch(kernel.function, g, b, 0, self.stream, args, kernel.arg_bytes)
+        if rc:
+            _check(rc)
+
+    def prepare(self, kernel, grid, block, args):
+        """a launch record for ``launch_prepared``: (pointer to the record, the
+        record, the argument buffer -- a mutable copy that may be patched in
+        place between launches)"""
+        buf = ctypes.create_string_buffer(bytes(args), len(args))
+        rec = LaunchRec()
+        rec.function = kernel.function
+        rec.grid[0], rec.grid[1], rec.grid[2] = grid
+        rec.block[0], rec.block[1], rec.block[2] = block
+        rec.lds_bytes, rec.arg_bytes = 0, kernel.arg_bytes
+        rec.stream = self.stream
+        rec.args = ctypes.addressof(buf)
+        return (c_void_p(ctypes.addressof(rec)), rec, buf)
+
+    def launch_prepared(self, prepared):
+        rc = self._launch_prepared(prepared[0])
         if rc:
             _check(rc)
 

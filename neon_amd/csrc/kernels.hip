@@ -173,14 +173,12 @@ __global__ __launch_bounds__(RN_T) void rownorm_f16_kernel(nh_f16* out, const nh
     const float g = gamma[row];
     const float b = beta[row];
 
+    const float one = nh_opaque_one();
     float s = 0.0f;
 #pragma unroll
     for (int k = 0; k < NCH; ++k)
 #pragma unroll
-        for (int j = 0; j < RN_V / 2; ++j) {  // padding chunks hold zeros
-            s += nh_f16_lo(raw[k][j]);
-            s += nh_f16_hi(raw[k][j]);
-        }
+        for (int j = 0; j < RN_V / 2; ++j) s = nh_sum2_f16(raw[k][j], s);  // padding chunks hold zeros
     const float mean = nh_block_allreduce<nh_op_sum, RN_T / 64>(s, slots) * inv_n;
 
 #pragma unroll
@@ -192,16 +190,20 @@ __global__ __launch_bounds__(RN_T) void rownorm_f16_kernel(nh_f16* out, const nh
         if (c < cols) {
 #pragma unroll
             for (int j = 0; j < RN_V / 2; ++j) {
-                q += nh_sqr(nh_f16_lo(raw[k][j]) - mean);
-                q += nh_sqr(nh_f16_hi(raw[k][j]) - mean);
+                // widening and subtraction in one v_fma_mix_f32 each; the squares are
+                // accumulated with one rounding per term
+                const float d0 = __builtin_fmaf(nh_f16_lo(raw[k][j]), one, -mean);
+                const float d1 = __builtin_fmaf(nh_f16_hi(raw[k][j]), one, -mean);
+                q = __builtin_fmaf(d0, d0, q);
+                q = __builtin_fmaf(d1, d1, q);
             }
         }
     }
     const float var = nh_block_allreduce<nh_op_sum, RN_T / 64>(q, slots) * inv_n;
-    // one reciprocal per row, a multiply per element: the kernel is bound by
-    // instruction issue (8 fp16 elements per 16 bytes), and an IEEE division
-    // costs about ten instructions
-    const float inv_denom = 1.0f / sqrtf(var + eps);
+    // gamma * (x - mean) / sqrt(var + eps) + beta as (x - mean) * A + beta with A once
+    // per row: the output is rounded to fp16 anyway, and the kernel is bound by
+    // instruction issue (8 fp16 elements per 16 bytes)
+    const float scale = g / sqrtf(var + eps);
 
 #pragma unroll
     for (int k = 0; k < NCH; ++k) nh_keep_packed(raw[k]);
@@ -211,9 +213,11 @@ __global__ __launch_bounds__(RN_T) void rownorm_f16_kernel(nh_f16* out, const nh
         if (c < cols) {
             nh_u32 o[RN_V / 2];
 #pragma unroll
-            for (int j = 0; j < RN_V / 2; ++j)
-                o[j] = nh_f16_pack((g * (nh_f16_lo(raw[k][j]) - mean)) * inv_denom + b,
-                                   (g * (nh_f16_hi(raw[k][j]) - mean)) * inv_denom + b);
+            for (int j = 0; j < RN_V / 2; ++j) {
+                const float d0 = __builtin_fmaf(nh_f16_lo(raw[k][j]), one, -mean);
+                const float d1 = __builtin_fmaf(nh_f16_hi(raw[k][j]), one, -mean);
+                o[j] = nh_f16_pack(__builtin_fmaf(d0, scale, b), __builtin_fmaf(d1, scale, b));
+            }
             nh_store_words<RN_V / 2, NT>(reinterpret_cast<nh_u32*>(orow + c), o);
         }
     }

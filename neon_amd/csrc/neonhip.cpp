@@ -376,6 +376,11 @@ int nh_launch(void* function, const uint32_t grid[3], const uint32_t block[3],
     return 0;
 }
 
+int nh_launch_prepared(const nh_launch_rec* rec) {
+    if (!rec) return fail(NH_EINVAL, "nh_launch_prepared: null record");
+    return nh_launch(rec->function, rec->grid, rec->block, rec->lds_bytes, rec->stream, rec->args, rec->arg_bytes);
+}
+
 int nh_launch_timed_sets(void* function, const uint32_t grid[3], const uint32_t block[3],
                          uint32_t lds_bytes, void* stream, const void* const* arg_sets, size_t arg_bytes,
                          uint32_t nsets, uint32_t reps, float* mean_ms) {
