@@ -13,6 +13,7 @@ import numpy as np
 from neon_amd import NervanaObject
 from neon_amd.backends.backend import Backend, Block, OpTreeNode, OpCollection, Tensor  # noqa: F401
 from neon_amd.backends import nervanahip
+from neon_amd.backends.hip.bf16 import bfloat16  # noqa: F401  (storage dtype for be.empty / be.array)
 
 # registers 'hip' in this package's own registry; a host package (neon) binds the
 # backend to ITS classes instead -- see nervanahip.bind

@@ -33,7 +33,7 @@ import os
 
 from neon_amd.backends.hip.optree_ir import DTYPE_CODE, used_nodes
 
-CTYPE = {"f4": "float", "f2": "nh_f16", "i4": "nh_i32", "u4": "nh_u32",
+CTYPE = {"f4": "float", "f2": "nh_f16", "b2": "nh_bf16", "i4": "nh_i32", "u4": "nh_u32",
          "i2": "nh_i16", "u2": "nh_u16", "i1": "nh_i8", "u1": "nh_u8"}
 
 _BIN = {"add": "({0} + {1})", "sub": "({0} - {1})", "mul": "({0} * {1})",
@@ -1093,7 +1093,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
         if AFFINE_16BIT_OUTPUTS:
             line_ref = g.make_ref("_s", "rr", "0", 1, dict((nid, name) for nid, name in line_tiles.items()), vals)
             for st in full_out:
-                if DTYPE_CODE[st.out.dtype] != "f2" or st.root.kind != "E":
+                if DTYPE_CODE[st.out.dtype] not in ("f2", "b2") or st.root.kind != "E":
                     continue
                 aff = _affine_in_line(st.root, lambda m: not m.vc)
                 if aff is None:

@@ -31,6 +31,8 @@ import os
 
 import numpy as np
 
+from neon_amd.backends.hip.bf16 import bfloat16
+
 
 UNARY = {"neg", "abs", "sgn", "sqrt", "sqr", "exp", "log", "exp2", "log2", "sig",
          "sig2", "tanh", "tanh2", "safelog", "rint", "finite"}
@@ -42,7 +44,8 @@ REDUCE = {"sum", "max", "min", "argmax", "argmin"}
 DTYPE_CODE = {np.dtype(np.float32): "f4", np.dtype(np.float16): "f2",
               np.dtype(np.int32): "i4", np.dtype(np.uint32): "u4",
               np.dtype(np.int16): "i2", np.dtype(np.uint16): "u2",
-              np.dtype(np.int8): "i1", np.dtype(np.uint8): "u1"}
+              np.dtype(np.int8): "i1", np.dtype(np.uint8): "u1",
+              bfloat16: "b2"}
 
 
 def _fold_unary(op, x):
@@ -164,6 +167,8 @@ def stochastic_bits(tensor):
         cap = 15
     elif dtype == np.float16:
         cap = 10
+    elif dtype == bfloat16:
+        cap = 7
     else:
         raise NotImplementedError("stochastic rounding into %s tensors" % dtype)
     return 10 if rounding is True else max(1, min(int(rounding), cap))

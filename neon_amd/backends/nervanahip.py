@@ -19,6 +19,7 @@ import struct
 import numpy as np
 
 from neon_amd.backends import backend as _own
+from neon_amd.backends.hip import bf16
 from neon_amd.backends.hip import runtime as hiprt
 from neon_amd.backends.hip.optree_ir import MixedAxes, Program, REDUCE, eval_const
 from neon_amd.backends.hip.planner import KernelCache, NeedsSplit, make_plan
@@ -75,7 +76,7 @@ class HIPTensorBase(object):
                  take_array=None, is_trans=False, rounding=0, take_extent=None):
         super(HIPTensorBase, self).__init__(backend, shape, dtype, name, persist_values)
         dtype = np.dtype(dtype)
-        assert dtype.type in _DTYPES, "unsupported dtype %s" % dtype
+        assert dtype.type in _DTYPES or dtype == bf16.bfloat16, "unsupported dtype %s" % dtype
         if not isinstance(shape, (tuple, list)):
             assert isinstance(shape, (int, np.integer))
             shape = (int(shape),)
@@ -234,8 +235,11 @@ class HIPTensorBase(object):
         if isinstance(value, (int, float)):
             if self.is_contiguous and not be._fusing:
                 if self.size:
-                    bits = np.array([value]).astype(self.dtype).view(
-                        {1: np.uint8, 2: np.uint16, 4: np.uint32}[self.dtype.itemsize])[0]
+                    if self.dtype == bf16.bfloat16:
+                        bits = bf16.to_bits(np.array([value]))[0]
+                    else:
+                        bits = np.array([value]).astype(self.dtype).view(
+                            {1: np.uint8, 2: np.uint16, 4: np.uint32}[self.dtype.itemsize])[0]
                     be.rt.memset(self.gpudata, int(bits), self.size, self.dtype.itemsize)
             else:
                 self._api.OpTreeNode.build("assign", self, value)
@@ -261,7 +265,10 @@ class HIPTensorBase(object):
         if ary.size != self.size:
             raise TypeError("ary.size {} != self.size {}".format(ary.size, self.size))
         assert self.is_contiguous, "Array in set() must be contiguous"
-        if ary.dtype != self.dtype:
+        if self.dtype == bf16.bfloat16:
+            if ary.dtype != bf16.bfloat16:
+                ary = bf16.to_bits(ary)          # values: rounded to nearest even
+        elif ary.dtype != self.dtype:
             ary = ary.astype(self.dtype)
         ary = np.ascontiguousarray(ary)
         self.backend._flush()
@@ -285,6 +292,8 @@ class HIPTensorBase(object):
             be._flush()
             be.rt.memcpy_d2h(out, tmp.gpudata)
         be._check_cooperative_plans()       # the copy waited for the stream: results are final
+        if self.dtype == bf16.bfloat16:
+            return bf16.from_bits(out).reshape(self.shape)       # numpy has no bfloat16: values, as float32
         return out
 
     def raw(self):
@@ -650,7 +659,7 @@ class NervanaHIPBase(object):
         ary = np.asarray(ary)
         if ary.ndim < self._min_dims:
             ary = ary.reshape(ary.size, 1)
-        if ary.dtype != np.dtype(dtype):
+        if ary.dtype != np.dtype(dtype) and np.dtype(dtype) != bf16.bfloat16:
             ary = ary.astype(dtype)
         return self.tensor_cls(self, ary.shape, dtype=dtype, name=name,
                          persist_values=persist_values).set(ary)

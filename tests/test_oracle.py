@@ -431,3 +431,53 @@ def test_backend_base_helpers(cpu):
     cpu.rng_set_state(state)
     assert np.array_equal(cpu.rng.uniform(size=3), first)
     cpu.rng_reset()
+
+
+# ---- bfloat16 rounding (oracle/bf16.py) -------------------------------------------------------
+def test_bf16_rounding_is_pinned_bit_for_bit():
+    """exhaustive over the bf16 values and their neighbourhoods, exact rational
+    arithmetic on a sample, and agreement with the product's bit trick"""
+    from fractions import Fraction
+    from oracle.bf16 import round_to_bf16
+    from neon_amd.backends.hip import bf16 as product
+    # every bf16 value is a fixed point; so is its float32 image
+    all_bf16 = (np.arange(65536, dtype=np.uint32) << 16).view(np.float32)
+    finite = np.isfinite(all_bf16)
+    assert np.array_equal(round_to_bf16(all_bf16[finite]).view(np.uint32), all_bf16[finite].view(np.uint32))
+    # halfway points: ties go to the even neighbour; one float32 step either side goes to the nearer one
+    base = (np.arange(0x0080, 0x7F7F, dtype=np.uint32) << 16)                  # positive normal bf16 values
+    for sign in (0, 0x80000000):
+        b = base | np.uint32(sign)
+        tie = (b | np.uint32(0x8000)).view(np.float32)
+        lower_even = ((b >> 16) & 1) == 0
+        want = np.where(lower_even, b, b + np.uint32(0x10000))
+        assert np.array_equal(round_to_bf16(tie).view(np.uint32), want)
+        assert np.array_equal(round_to_bf16((b | np.uint32(0x7FFF)).view(np.float32)).view(np.uint32), b)
+        assert np.array_equal(round_to_bf16((b | np.uint32(0x8001)).view(np.float32)).view(np.uint32),
+                              b + np.uint32(0x10000))
+    # overflow, infinities, NaN, zeros, denormals
+    top = np.array([0x7F7F8000, 0x7F7F7FFF, 0x7F7FFFFF], dtype=np.uint32).view(np.float32)
+    assert np.array_equal(round_to_bf16(top).view(np.uint32), np.array([0x7F800000, 0x7F7F0000, 0x7F800000], np.uint32))
+    special = np.array([np.inf, -np.inf, 0.0, -0.0, 1e-40, -3e-41], dtype=np.float32)
+    got = round_to_bf16(special)
+    assert np.array_equal(got[:4].view(np.uint32), special[:4].view(np.uint32))
+    assert np.isnan(round_to_bf16(np.array([np.nan], np.float32)))[0]
+    # exact rational check of "nearest, ties to even" on random float32 values
+    rs = np.random.RandomState(5)
+    sample = (rs.standard_normal(400) * np.exp(rs.uniform(-60, 60, 400))).astype(np.float32)
+    sample = np.concatenate([sample, special[4:]])
+    for x, r in zip(sample, round_to_bf16(sample)):
+        fx, fr = Fraction(float(x)), Fraction(float(r))
+        b = int(np.array([r], np.float32).view(np.uint32)[0])
+        assert b & 0xFFFF == 0                                              # a bf16 value
+        for nb in (b - 0x10000, b + 0x10000):                               # no neighbour is nearer
+            if 0 <= (nb & 0x7FFFFFFF) < 0x7F800000 and (nb ^ b) >> 31 == 0:
+                other = Fraction(float(np.array([nb], np.uint32).view(np.float32)[0]))
+                assert abs(fx - fr) <= abs(fx - other)
+                if abs(fx - fr) == abs(fx - other):
+                    assert (b >> 16) & 1 == 0
+    # the product's host conversion (add-and-shift) agrees bit for bit, and so do the widening helpers
+    big = (rs.standard_normal(200000) * np.exp(rs.uniform(-80, 80, 200000))).astype(np.float32)
+    big = np.concatenate([big, all_bf16[finite], top, special])
+    assert np.array_equal(product.quantise(big).view(np.uint32), round_to_bf16(big).view(np.uint32))
+    assert np.array_equal(product.from_bits(product.to_bits(big)), product.quantise(big))
