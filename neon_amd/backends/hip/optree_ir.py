@@ -271,6 +271,9 @@ class Program(object):
         self.axis = None           # the one reduction axis, if any
         self.domain = None
         self.nlevels = 0
+        # rewrites applied by finalize (module switches, read when the program is made)
+        self.online_lse = ONLINE_LSE
+        self.onehot_gather = ONEHOT_GATHER
 
     # -- slots -----------------------------------------------------------------
     def tensor_slot(self, t):
@@ -479,9 +482,9 @@ class Program(object):
         self.lse_pairs = 0
         self.gathers = 0
         if self.axis == 0:
-            if ONLINE_LSE:
+            if self.online_lse:
                 self._pair_max_with_sum_of_exp()
-            if ONEHOT_GATHER:
+            if self.onehot_gather:
                 self._gather_at_hot_rows()
             if self.lse_pairs or self.gathers:
                 self._analyse()
@@ -631,7 +634,7 @@ class Program(object):
         """Hashable identity of the program's structure and operand geometry."""
         geo = tuple((DTYPE_CODE[t.dtype], t.shape, t.strides, t.ptr % 16 == 0, t.written,
                      t.take_axis, t.take_slot, t.take_extent) for t in self.tensors)
-        return (tuple(self.key_parts), geo, self._alias_signature())
+        return (tuple(self.key_parts), geo, self._alias_signature(), self.online_lse, self.onehot_gather)
 
     def _alias_signature(self):
         """Which slots overlap in memory (matters for what may be declared

@@ -1,0 +1,142 @@
+"""The benchmark configurations at their FULL shapes against the CPU oracle
+(same seeded inputs, same op-trees: neon_amd/configs.py), plus the rewritten and
+the as-written forms of the softmax / cross-entropy trees side by side.
+
+Tolerances: integer results bit-exact; fp32 1e-5 relative; fp16 storage 1e-3 of
+max(|want|, 1e-3 max|want|) (values near a row's mean are tiny, one fp16 step of
+the store would dominate otherwise).  The sum of 32000 exponentials is added
+in another order than numpy's (and, in the one-sweep form, rescaled by
+exp(m - M) factors): it is compared to 1e-5 as well, and against float64."""
+import contextlib
+
+import numpy as np
+import pytest
+
+from neon_amd import configs
+from neon_amd.backends.backend import Block
+from neon_amd.backends.hip import optree_ir
+from utils import assert_close, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+@contextlib.contextmanager
+def rewrites(hip, online_lse, onehot_gather):
+    """run a block with the tree rewrites switched as given (they are part of a
+    program's key, so both forms get their own kernels)"""
+    old = optree_ir.ONLINE_LSE, optree_ir.ONEHOT_GATHER
+    optree_ir.ONLINE_LSE, optree_ir.ONEHOT_GATHER = online_lse, onehot_gather
+    hip.synchronize()
+    hip._launch_cache.clear()
+    try:
+        yield
+    finally:
+        optree_ir.ONLINE_LSE, optree_ir.ONEHOT_GATHER = old
+        hip.synchronize()
+        hip._launch_cache.clear()
+
+
+def test_c1_and_c2_full_size(pair):
+    cpu, hip = pair
+    x, y = configs.inputs_c1()
+    res = []
+    for be in pair:
+        X, Y, out, fused = be.array(x), be.array(y), be.empty(x.shape), be.empty(x.shape)
+        configs.c1a(be, out, X, Y)
+        configs.c1b(be, out)
+        configs.c1_fused(be, fused, X, Y)
+        res.append((out.get(), fused.get()))
+    for g, w in zip(res[1], res[0]):
+        assert_close(g, w, rtol=1e-5, atol=1e-7)
+    (x2,) = configs.inputs_c2()
+    want = cpu.empty(x2.shape)
+    configs.c2_softmax(cpu, want, cpu.array(x2))
+    for lse in (True, False):
+        with rewrites(hip, lse, True):
+            got = hip.empty(x2.shape)
+            configs.c2_softmax(hip, got, hip.array(x2))
+            assert_close(got.get(), want.get(), rtol=1e-5, atol=1e-9, what="softmax, one-sweep pair %s" % lse)
+            assert np.allclose(got.get().sum(axis=0), 1.0, atol=2e-6)
+
+
+def test_c3_ten_fused_adam_steps_full_size(pair):
+    cpu, hip = pair
+    grad, param = configs.inputs_c3()
+    res = []
+    for be in pair:
+        bsz, be.bsz = be.bsz, 1
+        g, p = be.array(grad), be.array(param)
+        m, v = be.zeros(configs.C3_SHAPE), be.zeros(configs.C3_SHAPE)
+        first = None
+        for t in range(1, 11):
+            be.begin(Block.update, t)
+            configs.c3_adam_step(be, p, g, m, v, t)
+            be.end(Block.update, t)
+            if t == 1:
+                first = (p.get(), m.get(), v.get())
+        res.append((first, (p.get(), m.get(), v.get())))
+        be.bsz = bsz
+        del g, p, m, v
+    for step in (0, 1):
+        for k, name in enumerate(("param", "m", "v")):
+            assert_close(res[1][step][k], res[0][step][k], rtol=1e-5, atol=1e-12,
+                         what="%s after step %d" % (name, (1, 10)[step]))
+
+
+def test_c4_row_normalisation_full_size(pair):
+    cpu, hip = pair
+    x, gamma, beta = configs.inputs_c4()
+    o_cpu = cpu.empty(configs.C4_SHAPE, dtype=np.float16)
+    # oracle: the fp16 values held in fp32 (numpy would evaluate fp16 operands in fp16), fp32 arithmetic, fp16 store
+    configs.c4_rownorm(cpu, o_cpu, cpu.array(x.astype(np.float32)), cpu.array(gamma), cpu.array(beta))
+    o_hip = hip.empty(configs.C4_SHAPE, dtype=np.float16)
+    configs.c4_rownorm(hip, o_hip, hip.array(x, dtype=np.float16), hip.array(gamma), hip.array(beta))
+    want, got = o_cpu.get().astype(np.float64), o_hip.get().astype(np.float64)
+    assert rel_err(got, want, floor_frac=1e-3) <= 1e-3
+    # ... and the fraction of results that differ from the oracle's at all stays small
+    # (two correct fp32 evaluations can round to neighbouring fp16 values)
+    assert (got != want).mean() < 0.02
+
+
+def test_c5_full_size_all_forms(pair):
+    cpu, hip = pair
+    x, idx = configs.inputs_c5()
+    cx, ci = cpu.array(x), cpu.array(idx, dtype=np.int32)
+    cam, cmx, cce = cpu.empty((1, 256), dtype=np.int32), cpu.empty((1, 256)), cpu.empty((1, 256))
+    configs.c5a_argmax(cpu, cam, cx)
+    configs.c5b_max(cpu, cmx, cx)
+    t = cpu.empty(x.shape)
+    t[:] = cpu.onehot(ci, axis=0)
+    configs.c5c_cross_entropy(cpu, cce, cx, t)
+    x64 = x.astype(np.float64)
+    m64 = x64.max(axis=0)
+    ce64 = np.log(np.exp(x64 - m64).sum(axis=0)) + m64 - x64[idx.ravel(), np.arange(256)]
+    assert_close(cce.get().ravel(), ce64, rtol=1e-5, atol=1e-5, what="oracle against float64")
+
+    hx, hi = hip.array(x), hip.array(idx, dtype=np.int32)
+    am, mx = hip.empty((1, 256), dtype=np.int32), hip.empty((1, 256))
+    configs.c5a_argmax(hip, am, hx)
+    configs.c5b_max(hip, mx, hx)
+    assert np.array_equal(am.get(), cam.get()) and np.array_equal(mx.get(), cmx.get())
+    with hip.fused():                                    # both from one pass over the logits
+        configs.c5a_argmax(hip, am, hx)
+        configs.c5b_max(hip, mx, hx)
+    assert np.array_equal(am.get(), cam.get()) and np.array_equal(mx.get(), cmx.get())
+
+    families = {}
+    for lse, gather in ((True, True), (True, False), (False, True), (False, False)):
+        with rewrites(hip, lse, gather):
+            before = set(hip.plans)
+            ce = hip.empty((1, 256))
+            configs.c5c_cross_entropy(hip, ce, hx, hip.onehot(hi, axis=0))
+            got = ce.get()
+            families[(lse, gather)] = sorted(hip.plans[k].spec.family for k in hip.plans if k not in before)
+            assert_close(got, cce.get(), rtol=1e-5, atol=1e-6, what="cross-entropy, pair %s gather %s" % (lse, gather))
+            assert_close(got.ravel(), ce64, rtol=1e-5, atol=1e-5, what="cross-entropy against float64")
+            # the dense one-hot form (what neon's cost layer is handed): same tree, t from memory
+            dense = hip.empty(x.shape)
+            dense[:] = hip.onehot(hi, axis=0)
+            configs.c5c_cross_entropy(hip, ce, hx, dense)
+            assert_close(ce.get(), cce.get(), rtol=1e-5, atol=1e-6, what="dense one-hot, pair %s" % lse)
+    assert families[(True, True)] == ["colsplit"]        # one pass, nobody waits
+    assert families[(False, False)] == ["colcoop"]       # three sweeps over resident rows, as written

@@ -814,3 +814,78 @@ def test_argmax_argmin_follow_numpy_on_nan(pair):
     mx = hip.empty((1, 64))
     mx[:] = hip.max(hip.array(x), axis=0)
     assert np.array_equal(mx.get(), x.max(axis=0, keepdims=True), equal_nan=True)
+
+
+@pytest.mark.gpu
+def test_derived_builders_against_numpy_directly(hip):
+    """mean / var / std / clip / reciprocal / fprop_softmax / whole-tensor
+    reductions are compositions made by the API's base class, which the oracle
+    backend shares: here the hip results are compared with numpy itself
+    (float64), not with the oracle (formulas: reference backend.py:860, 1311,
+    1331-1334, 1446-1502; nervanacpu.py:1916-1919)"""
+    rs = np.random.RandomState(41)
+    x = (rs.standard_normal((700, 260)) * 2 + 0.3).astype(np.float32)
+    x64 = x.astype(np.float64)
+    X = hip.array(x)
+
+    def ev(tree, shape):
+        out = hip.empty(shape)
+        out[:] = tree
+        return out.get()
+
+    for axis in (0, 1):
+        line = (1, 260) if axis == 0 else (700, 1)
+        assert_close(ev(hip.mean(X, axis=axis), line), x64.mean(axis=axis, keepdims=True), rtol=1e-5, atol=1e-6)
+        assert_close(ev(hip.var(X, axis=axis), line), x64.var(axis=axis, keepdims=True), rtol=1e-5, atol=1e-6)
+        assert_close(ev(hip.std(X, axis=axis), line), x64.std(axis=axis, keepdims=True), rtol=1e-5, atol=1e-6)
+        e = np.exp(x64 - x64.max(axis=axis, keepdims=True))
+        assert_close(ev(hip.fprop_softmax(X, axis), x.shape), e / e.sum(axis=axis, keepdims=True), rtol=1e-5, atol=1e-9)
+    assert_close(ev(hip.mean(X), (1, 1)), x64.mean().reshape(1, 1), rtol=1e-5, atol=1e-6)
+    assert_close(ev(hip.var(X), (1, 1)), x64.var().reshape(1, 1), rtol=1e-5, atol=1e-6)
+    assert_close(ev(hip.sum(X), (1, 1)), x64.sum().reshape(1, 1), rtol=1e-5, atol=1e-3)
+    assert np.array_equal(ev(hip.max(X), (1, 1)), x.max().reshape(1, 1))
+    assert np.array_equal(ev(hip.min(X), (1, 1)), x.min().reshape(1, 1))
+    assert np.array_equal(ev(hip.clip(X, -1.0, 0.5), x.shape), np.clip(x, -1.0, 0.5))
+    assert_close(ev(hip.reciprocal(X), x.shape), 1.0 / x64, rtol=1e-6, atol=0)
+    assert_close(ev(hip.absolute(X) ** 1.5, x.shape), np.abs(x64) ** 1.5, rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.gpu
+def test_division_by_a_line_value_with_extreme_divisors(pair):
+    """x / d with d constant along the row is computed as x * (1/d) only while
+    1/d is a normal number; zero, denormal, huge, infinite and NaN divisors
+    give the quotient as written"""
+    cpu, hip = pair
+    rs = np.random.RandomState(43)
+    x = rs.standard_normal((9, 300)).astype(np.float32)
+    x[:, 0] = 0.0
+    x[:, 1] = np.float32(1e-38)
+    d = np.array([[0.0], [1e-42], [3e38], [np.inf], [np.nan], [2.5], [-1e-39], [1.0e-30], [-0.0]], dtype=np.float32)
+    res = []
+    for be in pair:
+        out = be.empty(x.shape)
+        with np.errstate(all="ignore"):
+            out[:] = be.array(x) / be.array(d)
+        res.append(out.get())
+    assert np.array_equal(np.isnan(res[1]), np.isnan(res[0]))
+    ok = ~np.isnan(res[0])
+    assert np.array_equal(np.isinf(res[1][ok]), np.isinf(res[0][ok]))
+    fin = ok & np.isfinite(res[0])
+    assert_close(res[1][fin], res[0][fin], rtol=1e-6, atol=0)
+    assert np.array_equal(np.sign(res[1][ok]), np.sign(res[0][ok]))
+
+
+@pytest.mark.gpu
+def test_gather_views_clamp_indices_outside_the_table(hip):
+    """numpy raises IndexError for an index outside the tensor; a kernel cannot,
+    so gather / scatter views keep every access inside the indexed tensor"""
+    table = np.arange(40 * 6, dtype=np.float32).reshape(40, 6)
+    T = hip.array(table)
+    idx = np.array([[3], [39], [40], [1000000], [-1], [-7]], dtype=np.int32)
+    rows = hip.empty((6, 6))
+    rows[:] = T[hip.array(idx, dtype=np.int32)]
+    want = table[np.clip(idx.ravel(), 0, 39)]
+    assert np.array_equal(rows.get(), want)
+    cols = hip.empty((40, 3))
+    cols[:] = T.take(hip.array(np.array([[5], [6], [-2]], dtype=np.int32), dtype=np.int32), 1)
+    assert np.array_equal(cols.get(), table[:, [5, 5, 0]])
