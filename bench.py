@@ -31,12 +31,24 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the fused Adam kernel from rocprofv3 counters
-# (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a
-# plain copy kernel of known size); summary and commands under
-# profiles/hbm_traffic_adam_rownorm_colreduce_pmc.txt.  Counters cannot be read
-# from inside this process, so the figure is carried here.
-ADAM_FUSED_TRAFFIC_BYTES = 699.9e6
+# HBM bytes per launch from rocprofv3 counters (FETCH_SIZE and WRITE_SIZE, each scaled by what the same
+# counter reads for a plain copy kernel of known size) cannot be read from inside this process: they are
+# collected by two `rocprofv3 --pmc` runs of `bench.py --counter-pass` and kept, with the commands, in the
+# summary below, whose last line is machine-readable.
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "hbm_traffic_all_configs_pmc.txt")
+
+
+def measured_traffic(label):
+    """HBM bytes per launch of the kernel behind ``label`` from the committed
+    counter summary, or None when there is none"""
+    try:
+        with open(TRAFFIC_SUMMARY) as f:
+            lines = [l for l in f if l.startswith("json: ")]
+        return json.loads(lines[-1][6:])[label]["traffic_bytes"]
+    except (IOError, OSError, IndexError, KeyError, ValueError):
+        return None
+
+
 COLD_BYTES = 768 << 20         # tensor sets rotated through by the cold-cache rows
 
 
@@ -99,7 +111,7 @@ def gpu_leg(steps, warmup, detail=True):
     ms, plan = be.time_group(groups[0], reps=max(steps, 5))
     out["roofline"] = {"bound": "hbm", "achieved": step_bytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
                        "unit": "GB/s", "frac": step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                       "traffic": ADAM_FUSED_TRAFFIC_BYTES, "kernel": plan.spec.name, "kernel_ms": ms,
+                       "traffic": measured_traffic("C3 fused Adam"), "kernel": plan.spec.name, "kernel_ms": ms,
                        "algorithmic_bytes": step_bytes}
     if not detail:
         return out, be
@@ -197,6 +209,28 @@ def gpu_leg(steps, warmup, detail=True):
     measure("C5b max axis0 (32000,256) f32", lambda: configs.c5b_max(be, mx, x5), configs.bytes_c5_reduce(), n5)
     measure("C5c cross-entropy axis0 (32000,256) f32, in-kernel one-hot",
             lambda: configs.c5c_cross_entropy(be, ce, x5, be.onehot(i5, axis=0)), configs.bytes_c5c(), n5)
+
+    def c5ab():
+        with be.fused():
+            configs.c5a_argmax(be, am, x5)
+            configs.c5b_max(be, mx, x5)
+    measure("C5a+b argmax and max in one launch (32000,256) f32", c5ab, configs.bytes_c5_reduce() + 4 * configs.C5_SHAPE[1], n5)
+    # C4 on bfloat16 storage
+    from neon_amd.backends import bfloat16
+    x4b, o4b = be.empty(configs.C4_SHAPE, dtype=bfloat16), be.empty(configs.C4_SHAPE, dtype=bfloat16)
+    x4b[:] = x4
+    measure("C4 rownorm (256,100352) bf16", lambda: configs.c4_rownorm(be, o4b, x4b, g4, b4), configs.bytes_c4(),
+            configs.C4_SHAPE[0] * configs.C4_SHAPE[1], reps=30)
+    del x4b, o4b
+    # floors of the latency-bound rows: the same kernel structures on next to no data -- what a
+    # launch, one trip to memory and back, and (for the split column reductions) the
+    # publish / ticket / fold hand-off cost when there is nothing to stream
+    tiny_x, tiny_o = be.zeros((1, 1024)), be.empty((1, 1024))
+    measure("floor: elementwise kernel on 4 KB", lambda: tiny_o.__setitem__(slice(None), tiny_x * 2.0), 8192, 1024)
+    small = be.zeros((8192, 32))
+    small_o = be.empty((1, 32))
+    measure("floor: split column max on 1 MB (8192,32)", lambda: small_o.__setitem__(slice(None), be.max(small, axis=0)),
+            4 * 8192 * 32, 8192 * 32)
     # ---- the same trees with cold caches: each launch works on another set of tensors, enough
     #      sets (>= 768 MB in total) that neither the L2s nor the 256 MB memory-side cache hold them
     def measure_cold(label, make_set, issue, nbytes, elements):
@@ -418,43 +452,73 @@ def cpu_leg(max_seconds=25.0):
 def counter_pass():
     """A short, untimed run for hardware-counter collection
     (``rocprofv3 --pmc FETCH_SIZE -- python3 bench.py --counter-pass``, then the
-    same with WRITE_SIZE): three launches each of a plain copy kernel of known
-    size (the calibration: 100 MB read, 100 MB written) and of the main
-    benchmark kernels."""
+    same with WRITE_SIZE, or with SQ_* counters): three launches each of a
+    plain copy kernel of known size (the calibration: 100 MB read, 100 MB
+    written) and of the kernel behind every benchmark configuration and the
+    batch-norm pair.  Prints which kernel belongs to which configuration and
+    its algorithmic bytes."""
     from neon_amd import configs
     from neon_amd.backends import gen_backend
     from neon_amd.backends.backend import Block
     be = gen_backend("hip", rng_seed=0)
     be.bsz = 1
     rs = np.random.RandomState(3)
+    f16, i32 = np.float16, np.int32
+    table = []
+
+    def run(label, nbytes, issue, reps=3):
+        with be.capture() as grp:
+            issue()
+        assert len(grp) == 1, label
+        _, plan = be.time_group(grp[0], reps=1)
+        for _ in range(reps):
+            issue()
+            be.synchronize()
+        table.append({"label": label, "kernel": plan.spec.name, "family": plan.spec.family,
+                      "algorithmic_bytes": nbytes})
+
     g = _fresh(be, configs.C3_SHAPE, rs=rs, scale=1e-2)
     p = _fresh(be, configs.C3_SHAPE, rs=rs, scale=0.05)
     m, v = be.zeros(configs.C3_SHAPE), be.zeros(configs.C3_SHAPE)
-    x4 = _fresh(be, configs.C4_SHAPE, dtype=np.float16, rs=rs, scale=2.0, shift=0.5)
-    o4 = be.empty(configs.C4_SHAPE, dtype=np.float16)
-    g4, b4 = be.ones((configs.C4_SHAPE[0], 1)), be.zeros((configs.C4_SHAPE[0], 1))
-    x5 = _fresh(be, configs.C5_SHAPE, rs=rs, scale=4.0)
-    am = be.empty((1, configs.C5_SHAPE[1]), dtype=np.int32)
-    mx = be.empty((1, configs.C5_SHAPE[1]))
-    be.synchronize()
-    for t in range(1, 4):
-        m[:] = g * 1.0                     # copy kernel: 100 MB in, 100 MB out
-        be.synchronize()
+    run("copy (calibration)", 200000000, lambda: m.__setitem__(slice(None), g * 1.0))
     v[:] = 0
     m[:] = 0
-    for t in range(1, 4):
-        be.begin(Block.update, t)
-        configs.c3_adam_step(be, p, g, m, v, t)
-        be.end(Block.update, t)
-        be.synchronize()
-    for _ in range(3):
-        configs.c4_rownorm(be, o4, x4, g4, b4)
-        be.synchronize()
-    for _ in range(3):
-        configs.c5a_argmax(be, am, x5)
-        configs.c5b_max(be, mx, x5)
-        be.synchronize()
-    print(json.dumps({"counter_pass": "done"}))
+    step = [0]
+
+    def adam():
+        step[0] += 1
+        be.begin(Block.update, step[0])
+        configs.c3_adam_step(be, p, g, m, v, step[0])
+        be.end(Block.update, step[0])
+    run("C3 fused Adam", configs.bytes_c3(fused=True), adam)
+    del g, p, m, v
+    x1, y1 = (be.array(a) for a in configs.inputs_c1())
+    o1 = be.empty(configs.C1_SHAPE)
+    run("C1 fused sig(0.5x+2y)", configs.bytes_c1a(), lambda: configs.c1_fused(be, o1, x1, y1))
+    x2, o2 = be.array(configs.inputs_c2()[0]), be.empty(configs.C2_SHAPE)
+    run("C2 softmax", configs.bytes_c2(), lambda: configs.c2_softmax(be, o2, x2))
+    x4 = _fresh(be, configs.C4_SHAPE, dtype=f16, rs=rs, scale=2.0, shift=0.5)
+    o4 = be.empty(configs.C4_SHAPE, dtype=f16)
+    g4, b4 = be.ones((configs.C4_SHAPE[0], 1)), be.zeros((configs.C4_SHAPE[0], 1))
+    run("C4 rownorm f16", configs.bytes_c4(), lambda: configs.c4_rownorm(be, o4, x4, g4, b4))
+    K, N = configs.C4_SHAPE
+    vec = lambda fill: _fresh(be, (K, 1), fill=fill)
+    xsum, xvar, gmean, gvar, gamma, beta = vec(0.0), vec(0.0), vec(0.0), vec(1.0), vec(1.0), vec(0.0)
+    run("BN fprop f16", 2 * K * N * 2, lambda: be.compound_fprop_bn(x4, xsum, xvar, gmean, gvar, gamma, beta, o4,
+                                                                    1e-5, 0.9, True))
+    delta = _fresh(be, (K, N), dtype=f16, rs=rs, scale=0.1)
+    gg, gb = vec(0.0), vec(0.0)
+    run("BN bprop f16", 3 * K * N * 2, lambda: be.compound_bprop_bn(o4, gg, gb, delta, x4, xsum, xvar, gamma, 1e-5))
+    del x4, o4, delta
+    x5 = _fresh(be, configs.C5_SHAPE, rs=rs, scale=4.0)
+    i5 = be.array(rs.randint(0, configs.C5_SHAPE[0], size=(1, configs.C5_SHAPE[1])).astype(i32), dtype=i32)
+    am = be.empty((1, configs.C5_SHAPE[1]), dtype=i32)
+    mx, ce = be.empty((1, configs.C5_SHAPE[1])), be.empty((1, configs.C5_SHAPE[1]))
+    run("C5a argmax", configs.bytes_c5_reduce(), lambda: configs.c5a_argmax(be, am, x5))
+    run("C5b max", configs.bytes_c5_reduce(), lambda: configs.c5b_max(be, mx, x5))
+    run("C5c cross-entropy", configs.bytes_c5c(),
+        lambda: configs.c5c_cross_entropy(be, ce, x5, be.onehot(i5, axis=0)))
+    print(json.dumps({"counter_pass": table}))
 
 
 def main():
@@ -496,7 +560,17 @@ def main():
     if cpu:
         line["gpu_over_cpu"] = gpu["value_gbs"] / cpu["value"]
     if "per_config" in gpu:
-        line["per_config"] = gpu["per_config"]
+        # the readable table goes to stderr; the JSON line keeps short rows
+        print("%-72s %9s %9s %7s  %s" % ("config", "kernel us", "API us", "of peak", "plan"), file=sys.stderr)
+        for r in gpu["per_config"]:
+            print("%-72s %9.2f %9s %7.3f  %s" % (r["config"][:72], r["ms"] * 1e3,
+                                                 ("%.2f" % (r["api_ms"] * 1e3)) if r.get("api_ms") else "-",
+                                                 r["frac_of_hbm_peak"], r["plan"]), file=sys.stderr)
+        line["per_config"] = [{"config": r["config"], "us": round(r["ms"] * 1e3, 3),
+                               "api_us": round(r["api_ms"] * 1e3, 3) if r.get("api_ms") else None,
+                               "bytes": r["bytes"], "gbs": round(r["gbs"], 1), "frac": round(r["frac_of_hbm_peak"], 4),
+                               "kernels": r["kernels"], "plan": r["plan"].split("[")[0] if "+" not in r["plan"] else r["plan"]}
+                              for r in gpu["per_config"]]
     print(json.dumps(line))
 
 

@@ -1220,6 +1220,32 @@ def _emit_col_fold(g, L, n, LX, LY, T, V, src, dst_decl=True):
         L("for (int j = 0; j < %d; ++j) %s[%s][tx * %d + j] = %s[j];" % (V, buf, wy, V, src))
         L.close()
     L("__syncthreads();")
+    S = LX * V
+    if pair and S <= T:
+        # (value, index) and (max, sum) pairs cost ten to twenty instructions to combine:
+        # instead of every lane joining all V columns of its tile over all wave groups, P
+        # adjacent lanes share ONE column, each takes every P-th group, a DPP all-reduce
+        # over the P lanes finishes, and the results go round through LDS
+        P = 1
+        while P * 2 <= min(T // S, 64) and P < WY:
+            P *= 2
+        L.open("")
+        L("const int fcol = threadIdx.x / %d, fk = threadIdx.x %% %d;" % (P, P))
+        L("nh_pair one = %s::init();" % op)
+        L.open("if (fcol < %d)" % S)
+        L("for (int y = fk; y < %d; y += %d) one = %s::f(one, %s[y][fcol]);" % (WY, P, op, buf))
+        L.close()
+        if P > 1:
+            L("one = nh_wave_allreduce<%s, %d, nh_pair>(one);" % (op, P))
+        L("__syncthreads();     // every piece has been read: the first row of the buffer takes the results")
+        L("if (fk == 0 && fcol < %d) %s[0][fcol] = one;" % (S, buf))
+        L.close()
+        L("__syncthreads();")
+        L("#pragma unroll")
+        L("for (int j = 0; j < %d; ++j) %s[j] = %s[0][tx * %d + j];" % (V, src, buf, V))
+        unpack()
+        L("__syncthreads();")
+        return
     # a lane's V partials of one wave group are adjacent and 16-byte aligned:
     # walking the groups in the outer loop lets them come in as one LDS read
     L("#pragma unroll")

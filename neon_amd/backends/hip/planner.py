@@ -66,6 +66,10 @@ class KernelCache(object):
         self.arch = arch
         with open(hiprt.DEVICE_HEADER) as f:
             self.header = f.read()
+        if os.environ.get("NEON_HIP_FORMAL_FENCES", "0") != "0":
+            # device-scope release / acquire around the inter-workgroup hand-offs instead of
+            # the store-wait the default build relies on (see neon_device.h)
+            self.header = "#define NH_FORMAL_FENCES 1\n" + self.header
         if cache_dir is None:
             cache_dir = os.environ.get("NEON_HIP_CACHE_DIR")
         if cache_dir is None and os.environ.get("NEON_CACHE_DIR"):

@@ -249,8 +249,8 @@ void launch_rownorm(uint16_t* out, const uint16_t* x, const float* gamma, const 
 // Partials cross XCDs as write-through stores / L2-bypassing loads; each lane
 // waits for its own stores before the barrier that precedes the ticket.
 // ---------------------------------------------------------------------------
-constexpr int CR_T = 256;
-constexpr int CR_WAVES = CR_T / 64;
+constexpr int CR_T = 256;                 // lanes per workgroup; twice that for small inputs (one workgroup per
+                                          // compute unit), where a second wave per SIMD hides the first one's waits
 constexpr int CR_U = 4;                   // rows in flight per lane
 constexpr int CR_FOLD_BATCH = 4;          // partials in flight per lane in the final fold
 constexpr int CR_MAX_STRIPS = 4096;
@@ -269,9 +269,10 @@ static __device__ __align__(256) unsigned char scratch[NH_STATIC_SCRATCH_BYTES];
 // (threads 0 .. LX*V-1) joins them.  The steps after the sweep are a chain of
 // dependent operations on a few values, so that chain is kept short rather
 // than wide.
-template <int V, int LX>
+template <int V, int LX, int T>
 __device__ __forceinline__ nh_pair cr_join_rows(nh_pair (&acc)[V], nh_pair (*sp)[LX * V]) {
     constexpr int S = LX * V;
+    constexpr int CR_WAVES = T / 64;
     const int tx = threadIdx.x % LX;
     const int wave = threadIdx.x >> 6;
     if constexpr (LX < 64) {
@@ -296,15 +297,16 @@ __device__ __forceinline__ nh_pair cr_join_rows(nh_pair (&acc)[V], nh_pair (*sp)
     return one;
 }
 
-template <int V, int LX>
-__global__ __launch_bounds__(CR_T) void colmax_kernel(const float* __restrict__ x, uint32_t rows, uint32_t cols,
-                                                      size_t ld, uint32_t rows_per_chunk, nh_pair* part,
-                                                      float* __restrict__ outv, int* __restrict__ outi,
-                                                      unsigned int* tickets) {
-    constexpr int LY = CR_T / LX;
+template <int V, int LX, int T>
+__global__ __launch_bounds__(T) void colmax_kernel(const float* __restrict__ x, uint32_t rows, uint32_t cols,
+                                                   size_t ld, uint32_t rows_per_chunk, nh_pair* part,
+                                                   float* __restrict__ outv, int* __restrict__ outi,
+                                                   unsigned int* tickets) {
+    constexpr int CR_WAVES = T / 64;
+    constexpr int LY = T / LX;
     constexpr int S = LX * V;                       // columns of a strip
-    constexpr int P = CR_T / S;                     // lanes per column in the last workgroup's fold
-    static_assert(S <= CR_T && P <= 64, "strip geometry");
+    constexpr int P = T / S;                        // lanes per column in the last workgroup's fold
+    static_assert(S <= T && P <= 64, "strip geometry");
     __shared__ __attribute__((aligned(16))) nh_pair sp[CR_WAVES][S];
     __shared__ int s_last;
     const int tid = threadIdx.x;
@@ -337,7 +339,7 @@ __global__ __launch_bounds__(CR_T) void colmax_kernel(const float* __restrict__ 
             for (int j = 0; j < V; ++j) nh_op_argmax::step(acc[j], a0[j], (int)r);
         }
     }
-    nh_pair one = cr_join_rows<V, LX>(acc, sp);     // threads 0 .. S-1: the strip's column c0 + tid
+    nh_pair one = cr_join_rows<V, LX, T>(acc, sp);     // threads 0 .. S-1: the strip's column c0 + tid
 
     const uint32_t nchunks = gridDim.y;
     uint32_t col = tid;
@@ -506,7 +508,7 @@ __global__ __launch_bounds__(HIST_T) void hist_log2_kernel(const T* __restrict__
     }
 }
 
-struct CrPlan { uint32_t strips, chunks, rows_per_chunk; int v, lx; };
+struct CrPlan { uint32_t strips, chunks, rows_per_chunk; int v, lx, threads; };
 
 CrPlan cr_plan(uint32_t rows, uint32_t cols, bool vec) {
     CrPlan p;
@@ -514,7 +516,9 @@ CrPlan cr_plan(uint32_t rows, uint32_t cols, bool vec) {
     // whose row length is not a multiple of four: one element per lane, 64 lanes
     p.v = vec ? 4 : 1;
     p.lx = vec ? 8 : 64;
-    const uint32_t ly = CR_T / p.lx;
+    const uint64_t small = (uint64_t)(nh_internal_cu_count() > 0 ? nh_internal_cu_count() : 256) * (256u << 10);
+    p.threads = (vec && (uint64_t)rows * cols * sizeof(float) < small) ? 2 * CR_T : CR_T;
+    const uint32_t ly = p.threads / p.lx;
     const uint32_t strip_cols = p.lx * p.v;
     p.strips = (cols + strip_cols - 1) / strip_cols;
     // one workgroup per compute unit for small inputs, up to eight for large
@@ -866,12 +870,15 @@ size_t nh_colreduce_workspace_bytes(uint32_t rows, uint32_t cols) {
 static int colmax_launch(const char* who, float* maxval, int32_t* argmax, const float* x, uint32_t rows, uint32_t cols,
                          size_t ld, const CrPlan& p, nh_pair* part, unsigned int* tickets, hipStream_t s) {
     dim3 grid(p.strips, p.chunks);
-    if (p.v == 4)
-        hipLaunchKernelGGL((colmax_kernel<4, 8>), grid, dim3(CR_T), 0, s, x, rows, cols, ld, p.rows_per_chunk, part,
+    if (p.v == 4 && p.threads == 2 * CR_T)
+        hipLaunchKernelGGL((colmax_kernel<4, 8, 2 * CR_T>), grid, dim3(2 * CR_T), 0, s, x, rows, cols, ld,
+                           p.rows_per_chunk, part, maxval, (int*)argmax, tickets);
+    else if (p.v == 4)
+        hipLaunchKernelGGL((colmax_kernel<4, 8, CR_T>), grid, dim3(CR_T), 0, s, x, rows, cols, ld, p.rows_per_chunk, part,
                            maxval, (int*)argmax, tickets);
     else
-        hipLaunchKernelGGL((colmax_kernel<1, 64>), grid, dim3(CR_T), 0, s, x, rows, cols, ld, p.rows_per_chunk, part,
-                           maxval, (int*)argmax, tickets);
+        hipLaunchKernelGGL((colmax_kernel<1, 64, CR_T>), grid, dim3(CR_T), 0, s, x, rows, cols, ld, p.rows_per_chunk,
+                           part, maxval, (int*)argmax, tickets);
     return launch_status(who);
 }
 
