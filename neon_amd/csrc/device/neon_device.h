@@ -16,6 +16,9 @@
 #define NEON_DEVICE_H
 
 #define NEON_WAVE 64
+// accelerator complex dies of an MI355X: workgroups go to them round-robin in
+// dispatch order, and each has an L2 of its own
+#define NH_XCDS 8
 #define NEON_DEV __device__ __forceinline__
 
 typedef _Float16 nh_f16;

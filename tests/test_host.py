@@ -350,6 +350,28 @@ def test_generated_kernels_compile_for_every_dtype(tmp_path, dtype, axis):
     assert be.cache.stats["compiled"] == 4
 
 
+SHAPES_TO_GENERATE = [(1, 1), (3, 1), (1, 3), (2, 2), (7, 5), (1000, 1), (1, 1000), (1000, 2), (1000, 128),
+                      (33, 130), (513, 4), (20000, 1), (20000, 64), (64, 20000), (3, 100003), (100003, 3)]
+
+
+@pytest.mark.parametrize("shape", SHAPES_TO_GENERATE, ids=lambda s: "%dx%d" % s)
+def test_every_family_generates_for_degenerate_and_odd_shapes(pb, shape):
+    """planning and code generation (no compilation) of the trees every family
+    serves, down to single rows, single columns and 1x1: a planner or generator
+    that assumes "some operand has more than one column" fails here, not on the
+    device"""
+    x = pb.empty(shape)
+    for axis in (0, 1):
+        line = (1, shape[1]) if axis == 0 else (shape[0], 1)
+        pb.empty(shape)[:] = pb.exp(x - pb.max(x, axis=axis)) / pb.sum(pb.exp(x - pb.max(x, axis=axis)), axis=axis)
+        pb.empty(line, np.int32)[:] = pb.argmax(x, axis=axis)
+        pb.empty(line)[:] = pb.sum(x * x, axis=axis)
+        pb.empty(shape, np.float16)[:] = (x - pb.mean(x, axis=axis)) / pb.sqrt(pb.var(x, axis=axis) + 1e-3)
+    pb.empty(shape)[:] = 1.0 / (1.0 + pb.exp(-x))
+    for c in pb.choices:
+        assert "@NAME@" not in c.spec.source and c.spec.source.count("{") == c.spec.source.count("}")
+
+
 def test_stochastic_rounding_store_compiles_and_changes_the_plan(tmp_path):
     be = prebuild.PlanBackend(cache_dir=str(tmp_path / "kc"))
     x = be.empty((96, 160))
