@@ -176,6 +176,8 @@ class Runtime(object):
         self._grid = (c_uint32 * 3)()
         self._block = (c_uint32 * 3)()
         self._launch_prepared = self.lib.nh_launch_prepared
+        # the same entry point as a plain address, for callers that launch from C
+        self.launch_prepared_address = ctypes.cast(self.lib.nh_launch_prepared, c_void_p).value
 
     # -- memory ------------------------------------------------------------------
     def malloc(self, nbytes):

@@ -20,6 +20,7 @@ import numpy as np
 
 from neon_amd.backends import backend as _own
 from neon_amd.backends.hip import bf16
+from neon_amd.backends.hip import fastpath
 from neon_amd.backends.hip import runtime as hiprt
 from neon_amd.backends.hip.optree_ir import MixedAxes, Program, REDUCE, eval_const
 from neon_amd.backends.hip.planner import KernelCache, NeedsSplit, make_plan
@@ -232,7 +233,13 @@ class HIPTensorBase(object):
         engines; everything else is an op-tree kernel
         (reference nervanagpu.py:334-383)."""
         be = self.backend
-        if isinstance(value, (int, float)):
+        if isinstance(value, self._api.OpTreeNode):
+            if (be._replayer is not None and not be._fusing and be._captured is None and be._recording is None
+                    and not self.rounding and be._replay_in_c(self, value)):
+                return self              # a statement seen before: its recorded launches went out
+            # (what OpTreeNode.build("assign", ...) comes to, without inferring a shape nobody reads)
+            be.execute(self._api.OpTreeNode({"op": "assign", "shape": self.shape}, self, value))
+        elif isinstance(value, (int, float)):
             if self.is_contiguous and not be._fusing:
                 if self.size:
                     if self.dtype == bf16.bfloat16:
@@ -250,9 +257,6 @@ class HIPTensorBase(object):
                     be.rt.memcpy_d2d(self.gpudata, value.gpudata, self.nbytes)
             else:
                 self._api.OpTreeNode.build("assign", self, value)
-        elif isinstance(value, self._api.OpTreeNode):
-            # (what OpTreeNode.build("assign", ...) comes to, without inferring a shape nobody reads)
-            be.execute(self._api.OpTreeNode({"op": "assign", "shape": self.shape}, self, value))
         elif isinstance(value, np.ndarray):
             self.set(value)
         else:
@@ -412,11 +416,12 @@ class _FuseScope(object):
 
 class _Recorded(object):
     """Launches recorded for one statement group."""
-    __slots__ = ("launches", "temps", "raw", "patch", "coop", "prepared")
+    __slots__ = ("launches", "temps", "raw", "patch", "coop", "prepared", "fast")
 
     def __init__(self, launches, temps, raw, patch, coop=()):
         self.coop = coop             # cooperative plans among the launches (checked at the next synchronisation)
         self.prepared = None         # launch records, made at the first replay
+        self.fast = None             # the same records in the form the C replayer takes (with the first replay)
         self.launches = launches
         self.temps = temps           # temporaries the recorded arguments point into
         self.raw = raw               # the numbers of the trees when recorded
@@ -446,14 +451,21 @@ class _Recorded(object):
         if self.prepared is not None:
             ctypes.memmove(self.prepared[0][2], self.launches[0][3], len(buf))     # same record, new constants
         self.raw = list(raw)
+        if self.fast is not None:
+            self.fast.set_numbers(self.raw)
         return self.launches
 
-    def replay(self, rt):
-        """enqueue the recorded launches"""
+    def replay(self, rt, records_type=None):
+        """enqueue the recorded launches; the first replay fills in the launch
+        records, and -- for a statement that is kernel launches only, none of
+        them cooperative -- hands them to the C replayer (``records_type``),
+        which serves the statement from then on"""
         prepared = self.prepared
         if prepared is None:
             prepared = self.prepared = [None if kernel is None else rt.prepare(kernel, grid, block, args)
                                         for kernel, grid, block, args in self.launches]
+            if records_type is not None and not self.coop and None not in prepared:
+                self.fast = records_type([p[0].value for p in prepared], self.raw, prepared)
         for prep, launch in zip(prepared, self.launches):
             if prep is None:
                 launch[1](*launch[3])            # a recorded call of a prebuilt kernel's entry point
@@ -512,7 +524,7 @@ class NervanaHIPBase(object):
         self.cu_count = int(self.rt.props.compute_units)
         self.kernels = KernelCache(self.rt.arch.split(":")[0], cache_dir)
         self.plans = {}
-        self.plan_stats = {"hit": 0, "miss": 0, "split": 0, "launches": 0, "replayed": 0}
+        self._stats = {"hit": 0, "miss": 0, "split": 0, "launches": 0, "replayed": 0}
         self._pending = []
         self._pending_post = []       # postfix walks of the pending statements
         self._pending_sig = None      # what kind of group the pending statements form
@@ -520,6 +532,12 @@ class NervanaHIPBase(object):
         self._fuse_depth = 0
         self._captured = None
         self._launch_cache = {}      # statement-group identity -> recorded launches
+        self._replayer = self._records_type = None
+        if fastpath.enabled():
+            # repeated single statements: walk, lookup and launches in C (neon_amd/csrc/fastpath.c)
+            mod = fastpath.load()
+            self._replayer = mod.Replayer(self._launch_cache, self.tensor_cls, self.rt.launch_prepared_address)
+            self._records_type = mod.Records
         self._recording = None
         self._rec_temps = None
         self._rec_coop = None
@@ -554,7 +572,7 @@ class NervanaHIPBase(object):
                 for p in (plan if isinstance(plan, list) else [plan]):
                     p.release()
             self.plans = {}
-            self._launch_cache = {}
+            self._launch_cache.clear()       # (the C replayer holds this very dict)
             self._temp_pool = {}
             if getattr(self, "_lut_ws", None):
                 rt.free(self._lut_ws[0])
@@ -808,6 +826,8 @@ class NervanaHIPBase(object):
         if not self._fusing and self._captured is None and self._recording is None and not optree[1].rounding:
             # a single statement outside any group: ONE walk over the tree yields the replay
             # key; a statement seen before costs that walk, a dictionary lookup and its launches
+            if self._replayer is not None and self._replay_in_c(optree[1], optree[2]):
+                return optree[1]
             parts, raw = [], []
             try:
                 self._walk_key(optree, parts.append, raw.append, self.tensor_cls)
@@ -816,10 +836,10 @@ class NervanaHIPBase(object):
             except (TypeError, AttributeError, KeyError):
                 entry = None
             if entry is not None and entry.rebind(raw) is not None:
-                entry.replay(self.rt)
+                entry.replay(self.rt, self._records_type)
                 for plan in entry.coop:
                     self._coop_pending[plan.key] = plan
-                stats = self.plan_stats
+                stats = self._stats
                 stats["replayed"] += 1
                 stats["launches"] += len(entry.launches)
                 return optree[1]
@@ -835,6 +855,22 @@ class NervanaHIPBase(object):
         else:
             self._run([optree], [post])
         return optree[1]
+
+    def _replay_in_c(self, out, value):
+        """True when the C replayer issued the recorded launches of ``out[:] = value``"""
+        r = self._replayer.replay(out, value)
+        if r < 0:
+            hiprt._check(-r)
+        return r == 1
+
+    @property
+    def plan_stats(self):
+        """counters of the execution path (a snapshot; replays done in C included)"""
+        stats = dict(self._stats)
+        if self._replayer is not None:
+            stats["replayed"] += self._replayer.replayed
+            stats["launches"] += self._replayer.launches
+        return stats
 
     def _walk_key(self, node, add, num, tensor_cls):
         """postfix walk of one tree emitting the parts of ``_launch_key``"""
@@ -914,7 +950,7 @@ class NervanaHIPBase(object):
         if entry is not None:
             launches = entry.rebind(raw)
             if launches is not None:
-                entry.replay(self.rt)
+                entry.replay(self.rt, self._records_type if len(trees) == 1 else None)
                 for plan in entry.coop:
                     self._coop_pending[plan.key] = plan
                 if self._recording is not None:
@@ -922,8 +958,8 @@ class NervanaHIPBase(object):
                     self._rec_temps.extend(entry.temps)
                     self._rec_coop.extend(entry.coop)
                     self._rec_single = None
-                self.plan_stats["replayed"] += 1
-                self.plan_stats["launches"] += len(launches)
+                self._stats["replayed"] += 1
+                self._stats["launches"] += len(launches)
                 return
         outer = self._recording is None
         if outer:
@@ -962,7 +998,7 @@ class NervanaHIPBase(object):
             # a group that is exactly one launch of one program can be re-bound
             # to new constants: remember where they sit and how they derive
             self._rec_single = (plan.const_offsets(prog), prog.const_exprs) if not self._recording[:-1] else None
-        self.plan_stats["launches"] += 1
+        self._stats["launches"] += 1
 
     def _run_slow(self, trees):
         if len(trees) == 1 and not self._originals and self._stage_transposed_views(trees[0]):
@@ -976,12 +1012,12 @@ class NervanaHIPBase(object):
             key = prog.key()
             plan = self.plans.get(key)
             if plan is None:
-                self.plan_stats["miss"] += 1
+                self._stats["miss"] += 1
                 plan = make_plan(prog, self.rt, self.kernels, self.cu_count, coop=key not in self._coop_failed)
                 plan.key = key
                 self.plans[key] = plan
             else:
-                self.plan_stats["hit"] += 1
+                self._stats["hit"] += 1
             self._launch_plan(plan, prog)
         except (NeedsSplit, MixedAxes, NotImplementedError) as e:
             if self._originals:
@@ -1006,7 +1042,7 @@ class NervanaHIPBase(object):
                 return
             if isinstance(e, NotImplementedError) and not _splittable(trees[0]):
                 raise
-            self.plan_stats["split"] += 1
+            self._stats["split"] += 1
             self._run_split(trees[0])
 
     # -- bench mode (the reference brackets launches with events when its
@@ -1061,7 +1097,7 @@ class NervanaHIPBase(object):
         if self._recording is not None:
             self._recording.append((None, fn, None, args))
             self._rec_single = None
-        self.plan_stats["launches"] += 1
+        self._stats["launches"] += 1
 
     def _strided_copy(self, dst, src):
         """dst[i, j] = src[i, j] for two 2-d views of one dtype, whatever their
@@ -1180,7 +1216,7 @@ class NervanaHIPBase(object):
         key = prog.key()
         plan = self.plans.get(key)
         if plan is None:
-            self.plan_stats["miss"] += 1
+            self._stats["miss"] += 1
             try:
                 plan = make_plan(prog, self.rt, self.kernels, self.cu_count, coop=key not in self._coop_failed)
             except NeedsSplit:
@@ -1188,7 +1224,7 @@ class NervanaHIPBase(object):
             plan.key = key
             self.plans[key] = plan
         else:
-            self.plan_stats["hit"] += 1
+            self._stats["hit"] += 1
         self._launch_plan(plan, prog)
 
     def _temp(self, shape, dtype, temps):

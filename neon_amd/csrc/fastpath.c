@@ -1,0 +1,342 @@
+/* Host-side replay of a repeated single statement, as a CPython extension.
+ *
+ * A statement `out[:] = expr` that the backend has run before costs, in Python,
+ * one walk over the op-tree (the key of the launch cache), a dictionary lookup
+ * and one call through ctypes per recorded launch.  This module does the same
+ * three steps in C: `Replayer.replay(out, value)` walks the tree, builds the very
+ * key `NervanaHIPBase._launch_key` builds, looks it up in the backend's launch
+ * cache and calls `nh_launch_prepared` (include/neonhip.h) on the entry's launch
+ * records.  Anything it does not recognise -- a key that is not in the cache, an
+ * entry without prepared records, numbers that differ from the recorded ones, an
+ * operand type it does not know -- is answered with 0 and the caller takes the
+ * general Python path; nothing is decided here that the Python path would decide
+ * differently.  The role of the reference's per-call argument derivation that its
+ * own comment wants cached (neon/backends/float_ew.py:640-641).
+ *
+ * No GPU headers: the launch function is handed over as an address at set-up.
+ */
+#define PY_SSIZE_T_CLEAN
+#include <Python.h>
+#include <structmember.h>
+#include <stdint.h>
+
+typedef int (*launch_fn)(const void*);
+
+static PyObject *s_geom, *s_op, *s_axis, *s_idx, *s_fast, *s_bar, *s_assign;
+
+/* ---- Records: the launch records and numbers of one cache entry --------------------- */
+typedef struct {
+    PyObject_HEAD
+    Py_ssize_t nrec, nraw;
+    const void** recs;
+    double* raw;
+    PyObject* keep;          /* whatever owns the memory the records point into */
+} Records;
+
+static void Records_dealloc(Records* self) {
+    PyMem_Free((void*)self->recs);
+    PyMem_Free(self->raw);
+    Py_XDECREF(self->keep);
+    Py_TYPE(self)->tp_free((PyObject*)self);
+}
+
+static int fill_raw(Records* self, PyObject* seq) {
+    PyObject* fast = PySequence_Fast(seq, "numbers must be a sequence");
+    if (!fast) return -1;
+    Py_ssize_t n = PySequence_Fast_GET_SIZE(fast);
+    double* raw = (double*)PyMem_Malloc((n ? n : 1) * sizeof(double));
+    if (!raw) { Py_DECREF(fast); PyErr_NoMemory(); return -1; }
+    for (Py_ssize_t i = 0; i < n; ++i) {
+        raw[i] = PyFloat_AsDouble(PySequence_Fast_GET_ITEM(fast, i));
+        if (raw[i] == -1.0 && PyErr_Occurred()) { PyMem_Free(raw); Py_DECREF(fast); return -1; }
+    }
+    Py_DECREF(fast);
+    PyMem_Free(self->raw);
+    self->raw = raw;
+    self->nraw = n;
+    return 0;
+}
+
+static PyObject* Records_new(PyTypeObject* type, PyObject* args, PyObject* kw) {
+    PyObject *addresses, *numbers, *keep;
+    if (!PyArg_ParseTuple(args, "OOO:Records", &addresses, &numbers, &keep)) return NULL;
+    PyObject* fast = PySequence_Fast(addresses, "addresses must be a sequence");
+    if (!fast) return NULL;
+    Records* self = (Records*)type->tp_alloc(type, 0);
+    if (!self) { Py_DECREF(fast); return NULL; }
+    self->nrec = PySequence_Fast_GET_SIZE(fast);
+    self->recs = (const void**)PyMem_Malloc((self->nrec ? self->nrec : 1) * sizeof(void*));
+    if (!self->recs) { Py_DECREF(fast); Py_DECREF(self); return PyErr_NoMemory(); }
+    for (Py_ssize_t i = 0; i < self->nrec; ++i) {
+        self->recs[i] = PyLong_AsVoidPtr(PySequence_Fast_GET_ITEM(fast, i));
+        if (!self->recs[i]) {
+            if (!PyErr_Occurred()) PyErr_SetString(PyExc_ValueError, "null launch record");
+            Py_DECREF(fast); Py_DECREF(self); return NULL;
+        }
+    }
+    Py_DECREF(fast);
+    if (fill_raw(self, numbers) < 0) { Py_DECREF(self); return NULL; }
+    Py_INCREF(keep);
+    self->keep = keep;
+    return (PyObject*)self;
+}
+
+static PyObject* Records_set_numbers(Records* self, PyObject* numbers) {
+    if (fill_raw(self, numbers) < 0) return NULL;
+    Py_RETURN_NONE;
+}
+
+static PyMethodDef Records_methods[] = {
+    {"set_numbers", (PyCFunction)Records_set_numbers, METH_O,
+     "the numbers the records' argument buffers now hold"},
+    {NULL, NULL, 0, NULL}};
+
+static PyMemberDef Records_members[] = {
+    {"launches", T_PYSSIZET, offsetof(Records, nrec), READONLY, "number of launch records"},
+    {NULL, 0, 0, 0, NULL}};
+
+static PyTypeObject RecordsType = {
+    PyVarObject_HEAD_INIT(NULL, 0)
+    .tp_name = "neon_amd._fastpath.Records",
+    .tp_basicsize = sizeof(Records),
+    .tp_dealloc = (destructor)Records_dealloc,
+    .tp_flags = Py_TPFLAGS_DEFAULT,
+    .tp_doc = "Records(addresses, numbers, keep): launch records of one statement",
+    .tp_methods = Records_methods,
+    .tp_members = Records_members,
+    .tp_new = Records_new,
+};
+
+/* ---- the walk ------------------------------------------------------------------------- */
+#define MAX_PARTS 512
+#define MAX_RAW 128
+
+typedef struct {
+    PyObject* parts[MAX_PARTS];   /* owned references */
+    Py_ssize_t nparts;
+    double raw[MAX_RAW];
+    Py_ssize_t nraw;
+    PyTypeObject* tensor_cls;
+    int depth;
+} Walk;
+
+/* 0 = ok, -1 = not replayable here (a Python error may be set; the caller clears it) */
+static int push(Walk* w, PyObject* owned) {
+    if (!owned) return -1;
+    if (w->nparts >= MAX_PARTS) { Py_DECREF(owned); return -1; }
+    w->parts[w->nparts++] = owned;
+    return 0;
+}
+
+static int push_number(Walk* w, double v) {
+    if (v == -1.0 && PyErr_Occurred()) return -1;
+    if (w->nraw >= MAX_RAW) return -1;
+    w->raw[w->nraw++] = v;
+    Py_INCREF(Py_None);
+    return push(w, Py_None);
+}
+
+static int walk_node(Walk* w, PyObject* d, PyObject* left, PyObject* right);
+
+static int walk_operand(Walk* w, PyObject* x) {
+    PyTypeObject* t = Py_TYPE(x);
+    if (t == w->tensor_cls) return push(w, PyObject_GetAttr(x, s_geom));
+    if (t == &PyFloat_Type) return push_number(w, PyFloat_AS_DOUBLE(x));
+    if (t == &PyLong_Type) return push_number(w, PyLong_AsDouble(x));
+    if (x == Py_None) return 0;
+    if (PyTuple_Check(x)) {
+        if (PyTuple_GET_SIZE(x) != 3) return -1;
+        return walk_node(w, PyTuple_GET_ITEM(x, 0), PyTuple_GET_ITEM(x, 1), PyTuple_GET_ITEM(x, 2));
+    }
+    if (PyFloat_Check(x)) return push_number(w, PyFloat_AsDouble(x));
+    if (PyLong_Check(x)) return push_number(w, PyLong_AsDouble(x));
+    return -1;
+}
+
+static int walk_node(Walk* w, PyObject* d, PyObject* left, PyObject* right) {
+    if (!PyDict_Check(d) || ++w->depth > 200) return -1;
+    if (walk_operand(w, left) < 0 || walk_operand(w, right) < 0) return -1;
+    w->depth--;
+    PyObject* op = PyDict_GetItemWithError(d, s_op);             /* borrowed */
+    if (!op || !PyUnicode_Check(op)) return -1;
+    PyObject* axis = PyDict_GetItemWithError(d, s_axis);         /* borrowed */
+    if (axis) {
+        if (PyUnicode_CompareWithASCIIString(op, "onehot") == 0) {
+            PyObject* idx = PyDict_GetItemWithError(d, s_idx);
+            if (!idx) return -1;
+            PyObject* g = PyObject_GetAttr(idx, s_geom);
+            if (!g) return -1;
+            PyObject* part = PyTuple_Pack(3, op, axis, g);
+            Py_DECREF(g);
+            return push(w, part);
+        }
+        return push(w, PyTuple_Pack(2, op, axis));
+    }
+    if (PyErr_Occurred()) return -1;
+    if (PyUnicode_CompareWithASCIIString(op, "rand") == 0) return -1;     /* random trees are never replayed */
+    Py_INCREF(op);
+    return push(w, op);
+}
+
+/* ---- Replayer: one per backend instance ----------------------------------------------- */
+typedef struct {
+    PyObject_HEAD
+    PyObject* cache;              /* the backend's launch cache (dict) */
+    PyTypeObject* tensor_cls;
+    launch_fn launch;
+    long long replayed, launches;
+} Replayer;
+
+static void Replayer_dealloc(Replayer* self) {
+    Py_XDECREF(self->cache);
+    Py_XDECREF((PyObject*)self->tensor_cls);
+    Py_TYPE(self)->tp_free((PyObject*)self);
+}
+
+static PyObject* Replayer_new(PyTypeObject* type, PyObject* args, PyObject* kw) {
+    PyObject *cache, *cls, *fn;
+    if (!PyArg_ParseTuple(args, "O!O!O:Replayer", &PyDict_Type, &cache, &PyType_Type, &cls, &fn)) return NULL;
+    void* p = PyLong_AsVoidPtr(fn);
+    if (!p) {
+        if (!PyErr_Occurred()) PyErr_SetString(PyExc_ValueError, "null launch function");
+        return NULL;
+    }
+    Replayer* self = (Replayer*)type->tp_alloc(type, 0);
+    if (!self) return NULL;
+    Py_INCREF(cache);
+    Py_INCREF(cls);
+    self->cache = cache;
+    self->tensor_cls = (PyTypeObject*)cls;
+    self->launch = (launch_fn)p;
+    return (PyObject*)self;
+}
+
+/* key(out, value) -> (key tuple, list of numbers): what replay() looks up; for tests */
+static PyObject* build_key(Walk* w) {
+    Py_INCREF(s_bar);
+    if (push(w, s_bar) < 0) return NULL;
+    PyObject* key = PyTuple_New(w->nparts);
+    if (!key) return NULL;
+    for (Py_ssize_t i = 0; i < w->nparts; ++i) PyTuple_SET_ITEM(key, i, w->parts[i]);   /* steals */
+    w->nparts = 0;
+    return key;
+}
+
+static void walk_release(Walk* w) {
+    for (Py_ssize_t i = 0; i < w->nparts; ++i) Py_DECREF(w->parts[i]);
+    w->nparts = 0;
+}
+
+static int walk_statement(Replayer* self, Walk* w, PyObject* out, PyObject* value) {
+    w->nparts = w->nraw = 0;
+    w->depth = 0;
+    w->tensor_cls = self->tensor_cls;
+    if (walk_operand(w, out) < 0 || walk_operand(w, value) < 0) return -1;
+    Py_INCREF(s_assign);
+    return push(w, s_assign);
+}
+
+static PyObject* Replayer_key(Replayer* self, PyObject* args) {
+    PyObject *out, *value;
+    if (!PyArg_ParseTuple(args, "OO:key", &out, &value)) return NULL;
+    Walk w;
+    if (walk_statement(self, &w, out, value) < 0) {
+        walk_release(&w);
+        if (!PyErr_Occurred()) PyErr_SetString(PyExc_TypeError, "not replayable");
+        return NULL;
+    }
+    PyObject* key = build_key(&w);
+    if (!key) { walk_release(&w); return NULL; }
+    PyObject* nums = PyList_New(w.nraw);
+    if (!nums) { Py_DECREF(key); return NULL; }
+    for (Py_ssize_t i = 0; i < w.nraw; ++i) PyList_SET_ITEM(nums, i, PyFloat_FromDouble(w.raw[i]));
+    PyObject* r = PyTuple_Pack(2, key, nums);
+    Py_DECREF(key);
+    Py_DECREF(nums);
+    return r;
+}
+
+/* replay(out, value) -> 1: the statement's recorded launches were issued; 0: not handled here;
+ * a negative number: minus the error code nh_launch_prepared returned (launches may be partly issued) */
+static PyObject* Replayer_replay(Replayer* self, PyObject* const* args, Py_ssize_t nargs) {
+    if (nargs != 2) { PyErr_SetString(PyExc_TypeError, "replay(out, value)"); return NULL; }
+    Walk w;
+    long result = 0;
+    if (walk_statement(self, &w, args[0], args[1]) < 0) goto unhandled;
+    {
+        PyObject* key = build_key(&w);
+        if (!key) goto unhandled;
+        PyObject* entry = PyDict_GetItemWithError(self->cache, key);      /* borrowed */
+        Py_DECREF(key);
+        if (!entry) goto unhandled;
+        PyObject* recs = PyObject_GetAttr(entry, s_fast);
+        if (!recs) goto unhandled;
+        if (Py_TYPE(recs) == &RecordsType) {
+            Records* r = (Records*)recs;
+            int same = r->nraw == w.nraw;
+            for (Py_ssize_t i = 0; same && i < w.nraw; ++i) same = r->raw[i] == w.raw[i];
+            if (same) {
+                result = 1;
+                for (Py_ssize_t i = 0; i < r->nrec; ++i) {
+                    int rc = self->launch(r->recs[i]);
+                    if (rc) { result = -(long)rc; break; }
+                }
+                if (result == 1) {
+                    self->replayed += 1;
+                    self->launches += r->nrec;
+                }
+            }
+        }
+        Py_DECREF(recs);
+        return PyLong_FromLong(result);
+    }
+unhandled:
+    walk_release(&w);
+    PyErr_Clear();
+    return PyLong_FromLong(0);
+}
+
+static PyMemberDef Replayer_members[] = {
+    {"replayed", T_LONGLONG, offsetof(Replayer, replayed), 0, "statements replayed here"},
+    {"launches", T_LONGLONG, offsetof(Replayer, launches), 0, "launches issued here"},
+    {NULL, 0, 0, 0, NULL}};
+
+static PyMethodDef Replayer_methods[] = {
+    {"replay", (PyCFunction)(void (*)(void))Replayer_replay, METH_FASTCALL,
+     "replay(out, value) -> 1 issued, 0 not handled, < 0 minus the launch error code"},
+    {"key", (PyCFunction)Replayer_key, METH_VARARGS, "key(out, value) -> (cache key, numbers)"},
+    {NULL, NULL, 0, NULL}};
+
+static PyTypeObject ReplayerType = {
+    PyVarObject_HEAD_INIT(NULL, 0)
+    .tp_name = "neon_amd._fastpath.Replayer",
+    .tp_basicsize = sizeof(Replayer),
+    .tp_dealloc = (destructor)Replayer_dealloc,
+    .tp_flags = Py_TPFLAGS_DEFAULT,
+    .tp_doc = "Replayer(launch_cache, tensor_class, address of nh_launch_prepared)",
+    .tp_methods = Replayer_methods,
+    .tp_members = Replayer_members,
+    .tp_new = Replayer_new,
+};
+
+static struct PyModuleDef moduledef = {
+    PyModuleDef_HEAD_INIT, "_fastpath", "C replay of repeated op-tree statements", -1, NULL, NULL, NULL, NULL, NULL};
+
+PyMODINIT_FUNC PyInit__fastpath(void) {
+    if (PyType_Ready(&RecordsType) < 0 || PyType_Ready(&ReplayerType) < 0) return NULL;
+    PyObject* m = PyModule_Create(&moduledef);
+    if (!m) return NULL;
+    s_geom = PyUnicode_InternFromString("_geom");
+    s_op = PyUnicode_InternFromString("op");
+    s_axis = PyUnicode_InternFromString("axis");
+    s_idx = PyUnicode_InternFromString("idx");
+    s_fast = PyUnicode_InternFromString("fast");
+    s_bar = PyUnicode_InternFromString("|");
+    s_assign = PyUnicode_InternFromString("assign");
+    if (!s_geom || !s_op || !s_axis || !s_idx || !s_fast || !s_bar || !s_assign) return NULL;
+    Py_INCREF(&RecordsType);
+    Py_INCREF(&ReplayerType);
+    if (PyModule_AddObject(m, "Records", (PyObject*)&RecordsType) < 0) return NULL;
+    if (PyModule_AddObject(m, "Replayer", (PyObject*)&ReplayerType) < 0) return NULL;
+    return m;
+}

@@ -1,0 +1,236 @@
+"""The C replayer of repeated statements (neon_amd/csrc/fastpath.c) against the
+Python walk it stands in for, without a GPU: the launch function is a ctypes
+callback that only counts."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from neon_amd.backends.hip import fastpath
+from neon_amd.backends.hip.prebuild import PlanBackend, ShapeTensor
+from neon_amd.backends.nervanahip import NervanaHIPBase
+
+
+class GeomTensor(ShapeTensor):
+    """shape-only tensor carrying the layout tuple the launch key is made of"""
+    def __init__(self, *args, **kw):
+        super(GeomTensor, self).__init__(*args, **kw)
+        self._geom = (self.ptr, self.shape, self.strides, self.dtype.char, 0)
+
+
+class _Walker(object):
+    _walk_key = NervanaHIPBase._walk_key
+
+
+def python_key(out, value):
+    parts, raw = [], []
+    node = ({"op": "assign"}, out, value)
+    _Walker()._walk_key(node, parts.append, raw.append, GeomTensor)
+    parts.append("|")
+    return tuple(parts), raw
+
+
+class Entry(object):
+    def __init__(self, fast):
+        self.fast = fast
+
+
+@pytest.fixture()
+def rig():
+    mod = fastpath.load()
+    be = PlanBackend(compile_kernels=False)
+    calls = []
+    verdict = [0]
+
+    @ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p)
+    def launch(rec):
+        calls.append(rec)
+        return verdict[0]
+
+    cache = {}
+    rp = mod.Replayer(cache, GeomTensor, ctypes.cast(launch, ctypes.c_void_p).value)
+    t = lambda shape, dtype=np.float32: GeomTensor(be, shape, dtype)
+    return mod, be, rp, cache, calls, verdict, t, launch
+
+
+def trees(be, t):
+    x, y, o = t((64, 32)), t((64, 32)), t((64, 32))
+    col, row = t((64, 1)), t((1, 32))
+    idx = t((1, 32), np.int32)
+    return [
+        (o, be.sig(0.5 * x + 2.0 * y)),
+        (o, x),
+        (o, 3),
+        (o, x * 2 - 1 / y + col * row),
+        (row, be.sum(x, axis=0)),
+        (col, be.max(x - be.max(x, axis=1), axis=1)),
+        (row, be.argmax(x, axis=0)),
+        (o, be.exp(x - be.max(x, axis=0)) / be.sum(be.exp(x - be.max(x, axis=0)), axis=0)),
+        (row, be.sum(be.onehot(idx, axis=0) * be.safelog(x), axis=0)),
+        (o, -x + abs(y) ** 2.5),
+        (o, be.sqrt(be.var(x, axis=1) + 1e-6)),
+        (o, x * np.float64(0.25) + True),            # subclasses of float and int
+    ]
+
+
+def test_c_key_is_the_python_key(rig):
+    mod, be, rp, cache, calls, verdict, t, _ = rig
+    for out, value in trees(be, t):
+        want_key, want_raw = python_key(out, value)
+        key, raw = rp.key(out, value)
+        assert key == want_key and hash(key) == hash(want_key)
+        assert raw == want_raw
+
+
+def test_what_the_replayer_leaves_to_python(rig):
+    mod, be, rp, cache, calls, verdict, t, _ = rig
+    x, o = t((8, 8)), t((8, 8))
+    assert rp.replay(o, x + 1.0) == 0                        # never seen
+    assert rp.replay(o, "text") == 0 and rp.replay(o, [1, 2]) == 0
+    from neon_amd.backends.backend import OpTreeNode
+    assert rp.replay(o, OpTreeNode.build("rand", None, None) * x) == 0                  # random trees are never replayed
+    plain = ShapeTensor(be, (8, 8))
+    assert rp.replay(o, plain + 1.0) == 0                    # a tensor of another class
+    deep = x
+    for _ in range(300):
+        deep = deep + 1.0
+    assert rp.replay(o, deep) == 0                           # deeper than the C walk goes
+    with pytest.raises(TypeError):
+        rp.key(o, "text")
+    assert calls == [] and rp.replayed == 0
+
+
+def test_replay_issues_the_records_in_order(rig):
+    mod, be, rp, cache, calls, verdict, t, _ = rig
+    x, o = t((8, 8)), t((8, 8))
+    key, raw = python_key(o, 0.5 * x + 2.0)
+    keep = object()
+    recs = mod.Records([0x1000, 0x2000, 0x3000], raw, keep)
+    assert recs.launches == 3
+    cache[key] = Entry(recs)
+    assert rp.replay(o, 0.5 * x + 2.0) == 1
+    assert calls == [0x1000, 0x2000, 0x3000]
+    assert (rp.replayed, rp.launches) == (1, 3)
+    # other numbers: the Python path re-binds the constants, then tells the records
+    del calls[:]
+    assert rp.replay(o, 0.25 * x + 2.0) == 0 and calls == []
+    recs.set_numbers([0.25, 2.0])
+    assert rp.replay(o, 0.25 * x + 2.0) == 1 and len(calls) == 3
+    assert rp.replay(o, 0.5 * x + 2.0) == 0
+    # an entry that has no records yet, or something else in their place
+    cache[key] = Entry(None)
+    assert rp.replay(o, 0.25 * x + 2.0) == 0
+    cache[key] = Entry([1, 2])
+    assert rp.replay(o, 0.25 * x + 2.0) == 0
+    # the same tree over another tensor is another statement
+    cache[key] = Entry(recs)
+    assert rp.replay(t((8, 8)), 0.25 * x + 2.0) == 0
+    # a cleared cache forgets
+    cache.clear()
+    assert rp.replay(o, 0.25 * x + 2.0) == 0
+
+
+def test_launch_errors_come_back_negated(rig):
+    mod, be, rp, cache, calls, verdict, t, _ = rig
+    x, o = t((8, 8)), t((8, 8))
+    key, raw = python_key(o, x * x)
+    cache[key] = Entry(mod.Records([0x10, 0x20], raw, None))
+    verdict[0] = 7
+    assert rp.replay(o, x * x) == -7
+    assert calls == [0x10] and rp.replayed == 0              # stopped at the failing launch
+    with pytest.raises(ValueError):
+        mod.Records([0], [], None)                           # a null record is refused at construction
+    with pytest.raises(TypeError):
+        mod.Records([1], ["a"], None)
+
+
+def test_records_keep_their_owner_alive(rig):
+    import gc
+    import weakref
+    mod = rig[0]
+
+    class Owner(object):
+        pass
+    owner = Owner()
+    ref = weakref.ref(owner)
+    recs = mod.Records([0x10], [], owner)
+    del owner
+    gc.collect()
+    assert ref() is not None
+    del recs
+    gc.collect()
+    assert ref() is None
+
+
+def test_random_trees_have_no_key(rig):
+    from neon_amd.backends.backend import OpTreeNode
+    mod, be, rp, cache, calls, verdict, t, _ = rig
+    x, o = t((8, 8)), t((8, 8))
+    with pytest.raises(TypeError):
+        rp.key(o, OpTreeNode.build("rand", None, None) * x)
+
+
+# ---- on the device: the third and later calls of a statement go through the C replayer -------
+@pytest.mark.gpu
+def test_replayed_statements_match_the_oracle(hip, cpu):
+    assert hip._replayer is not None, "the C replayer is the default path"
+    rs = np.random.RandomState(5)
+    a, b = rs.randn(300, 70).astype(np.float32), rs.randn(300, 70).astype(np.float32)
+    hx, hy, ho = hip.array(a), hip.array(b), hip.empty((300, 70))
+    hred = hip.empty((1, 70))
+    cx, cy, co = cpu.array(a), cpu.array(b), cpu.empty((300, 70))
+    cred = cpu.empty((1, 70))
+    before = hip._replayer.replayed
+    stats = hip.plan_stats
+    for k in range(8):
+        scale = 0.5 if k < 5 else 0.125 * k            # the numbers change at the sixth call
+        if k == 3:                                     # the data changes, the statement does not
+            a2 = rs.randn(300, 70).astype(np.float32)
+            hx.set(a2)
+            cx.set(a2)
+        for be, x, y, o, red in ((hip, hx, hy, ho, hred), (cpu, cx, cy, co, cred)):
+            o[:] = be.sig(scale * x + 2.0 * y)
+            red[:] = be.sum(o * x, axis=0)
+        np.testing.assert_allclose(ho.get(), co.get(), rtol=1e-5, atol=1e-6)
+        np.testing.assert_allclose(hred.get(), cred.get(), rtol=1e-4, atol=1e-4)
+    # calls 0 record, 1 replay in Python and hand over the records, 2..4 run in C; the changed
+    # numbers go back through Python once (6, 7 differ from each other too)
+    assert hip._replayer.replayed - before >= 6
+    after = hip.plan_stats
+    assert after["launches"] - stats["launches"] == 16 and after["replayed"] - stats["replayed"] >= 12
+
+
+@pytest.mark.gpu
+def test_replayer_steps_aside_for_groups_rounding_and_capture(hip, cpu):
+    from neon_amd.backends.backend import Block
+    rs = np.random.RandomState(6)
+    a = rs.randn(64, 48).astype(np.float32)
+    hx, ho, hp = hip.array(a), hip.empty((64, 48)), hip.empty((64, 48))
+    for _ in range(4):
+        ho[:] = hx * 3.0
+    np.testing.assert_array_equal(ho.get(), a * np.float32(3.0))
+    # the same statement inside a fused group must join the group, not be replayed on its own
+    before = hip.plan_stats["launches"]
+    hip.begin(Block.update, 0)
+    ho[:] = hx * 3.0
+    hp[:] = ho + 1.0
+    hip.end(Block.update, 0)
+    assert hip.plan_stats["launches"] - before == 1
+    np.testing.assert_array_equal(hp.get(), a * np.float32(3.0) + np.float32(1.0))
+    # captured statements are not launched at all
+    ho.fill(0)
+    with hip.capture() as groups:
+        ho[:] = hx * 3.0
+    assert len(groups) == 1 and not ho.get().any()
+    # a stochastically rounded target never takes a recorded launch
+    h16 = hip.empty((64, 48), dtype=np.float16)
+    for _ in range(3):
+        h16[:] = hx * 3.0
+    exact = h16.get().copy()
+    h16.rounding = 4
+    h16[:] = hx * 3.0
+    got = h16.get()
+    assert np.all((got.view(np.uint16) & 0x3f) == 0) and not np.array_equal(got, exact)
+    h16.rounding = 0
+    h16[:] = hx * 3.0
+    np.testing.assert_array_equal(h16.get(), exact)
