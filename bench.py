@@ -446,11 +446,54 @@ def cpu_leg(max_seconds=25.0):
             model = [l.split(":", 1)[1].strip() for l in f if l.startswith("model name")][0]
     except Exception:
         model = "unknown"
+    del g, p, m, v, grad_h, param_h
+
+    # the other configurations on the oracle, full size, median of 5 calls each (a few seconds in all)
+    def median_s(issue, calls=5):
+        issue()
+        ts = []
+        for _ in range(calls):
+            t0 = time.perf_counter()
+            issue()
+            ts.append(time.perf_counter() - t0)
+        return float(np.median(ts))
+
+    per_config = []
+
+    def row(label, issue, nbytes, elements):
+        sec = median_s(issue)
+        per_config.append({"config": label, "us": round(sec * 1e6, 1), "gbs": round(nbytes / sec / 1e9, 2),
+                           "elements_per_s": elements / sec})
+
+    x1, y1 = (cpu.array(a) for a in configs.inputs_c1())
+    o1 = cpu.empty(configs.C1_SHAPE)
+    n1 = configs.C1_SHAPE[0] * configs.C1_SHAPE[1]
+    row("C1a", lambda: configs.c1a(cpu, o1, x1, y1), configs.bytes_c1a(), n1)
+    row("C1b", lambda: configs.c1b(cpu, o1), configs.bytes_c1b(), n1)
+    row("C1 fused", lambda: configs.c1_fused(cpu, o1, x1, y1), configs.bytes_c1a(), n1)
+    x2, o2 = cpu.array(configs.inputs_c2()[0]), cpu.empty(configs.C2_SHAPE)
+    row("C2", lambda: configs.c2_softmax(cpu, o2, x2), configs.bytes_c2(), configs.C2_SHAPE[0] * configs.C2_SHAPE[1])
+    xh, gam, bet = configs.inputs_c4()
+    # fp16 storage with fp32 arithmetic: the quantised values held as fp32, the result stored as fp16
+    x4, g4, b4 = cpu.array(xh.astype(np.float32)), cpu.array(gam), cpu.array(bet)
+    o4 = cpu.empty(configs.C4_SHAPE, dtype=np.float16)
+    row("C4", lambda: configs.c4_rownorm(cpu, o4, x4, g4, b4), configs.bytes_c4(),
+        configs.C4_SHAPE[0] * configs.C4_SHAPE[1])
+    del x4, o4, xh
+    x5h, idx = configs.inputs_c5()
+    x5 = cpu.array(x5h)
+    n5 = configs.C5_SHAPE[0] * configs.C5_SHAPE[1]
+    am, mx, ce = (cpu.empty((1, configs.C5_SHAPE[1]), dtype=dt) for dt in (np.int32, np.float32, np.float32))
+    row("C5a", lambda: configs.c5a_argmax(cpu, am, x5), configs.bytes_c5_reduce(), n5)
+    row("C5b", lambda: configs.c5b_max(cpu, mx, x5), configs.bytes_c5_reduce(), n5)
+    hot = cpu.empty(configs.C5_SHAPE)
+    hot[:] = cpu.onehot(cpu.array(idx, dtype=np.int32), axis=0)      # the oracle takes the dense one-hot only
+    row("C5c (dense one-hot)", lambda: configs.c5c_cross_entropy(cpu, ce, x5, hot), configs.bytes_c5c(), n5)
     return {"value": configs.bytes_c3(fused=True) / med / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": "%d full-size Adam steps (5000x5000 fp32) on the numpy oracle, median step %.3f s; "
                       "numpy ufuncs are single-threaded" % (len(timed), med),
             "elements_per_s": configs.C3_SHAPE[0] * configs.C3_SHAPE[1] / med,
-            "host_cpu": model, "host_cpu_count": os.cpu_count()}
+            "host_cpu": model, "host_cpu_count": os.cpu_count(), "per_config": per_config}
 
 
 def counter_pass():
