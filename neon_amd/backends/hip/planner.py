@@ -427,6 +427,12 @@ _COL_BUDGET = {1024: 40, 512: 120, 256: 300}
 
 COLSPLIT_THREADS = int(os.environ.get("NEON_HIP_CS_T", "256"))
 
+COLCOOP = os.environ.get("NEON_HIP_COLCOOP", "1") != "0"       # 0: axis-0 trees never wait between workgroups
+# Beyond this size the cooperative family (rows resident in registers, one workgroup per compute
+# unit, a waiting exchange per level) loses to stage-by-stage evaluation, whose reduction kernels
+# stream at full occupancy.  Softmax, measured: (32000,256) 28 us either way; (64000,256) 60 us
+# cooperative, 44 us in two kernels; (6000,2304) 54 against 40 us.
+COLCOOP_MAX_BYTES = int(os.environ.get("NEON_HIP_COLCOOP_MAX_MB", "48")) << 20
 ONLINE_LSE_IN_ONE_WORKGROUP = os.environ.get("NEON_HIP_ONLINE_LSE_COL", "0") != "0"
 
 
@@ -485,7 +491,7 @@ def _plan_col(prog, cu_count, coop=True):
     # strip keep their rows in registers and exchange partials between sweeps.
     # Everything must be resident at once, so the grid stays within one
     # workgroup per compute unit.
-    if coop and not (single_level and line_only):
+    if coop and COLCOOP and not (single_level and line_only) and R * C * isz <= COLCOOP_MAX_BYTES:
         # narrow strips keep the partials each workgroup has to gather small
         # (measured on (32000,256): 8 column-lanes 37 us, 16 lanes 43 us, 4 lanes
         # 41 us).  More strips than half the compute units leave no second

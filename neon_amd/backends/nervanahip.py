@@ -1155,11 +1155,16 @@ class NervanaHIPBase(object):
         out, expr = tree[1], tree[2]
         temps = []
         memo = {}
+        together = {}
 
         def lower(node, top=False):
             if not isinstance(node, self._api.OpTreeNode):
                 return node
             op = node[0]["op"]
+            if together and op in REDUCE and not top:
+                tmp = together.get(node.key())
+                if tmp is not None:
+                    return tmp
             left = lower(node[1])
             right = lower(node[2])
             if op == "dot":
@@ -1201,11 +1206,70 @@ class NervanaHIPBase(object):
             return rebuilt
 
         try:
+            # reductions along one axis, nested or side by side (softmax's max and sum of
+            # exponentials): ONE kernel that reads the operand once, where a family takes the
+            # group; otherwise one kernel per reduction, innermost first
+            reds = self._reductions_along_one_axis(expr)
+            if reds is not None and len(reds) > 1:
+                tmps = [self._temp(r[0]["shape"], np.float32, temps) for r in reds]
+                if self._run_as_one_kernel([self._api.OpTreeNode({"op": "assign"}, t, r)
+                                            for t, r in zip(tmps, reds)]):
+                    together.update((r.key(), t) for t, r in zip(tmps, reds))
             lowered = lower(expr, top=True)
             self._run_leaf(self._api.OpTreeNode({"op": "assign"}, out, lowered))
         finally:
             for t in temps:
                 self._temp_release(t)
+
+    def _reductions_along_one_axis(self, expr):
+        """the distinct reduction nodes below the root of ``expr``, innermost
+        first, when they all run along the same axis and the tree holds nothing
+        a single kernel cannot (products, transposes, random numbers); None
+        otherwise"""
+        node_cls = self._api.OpTreeNode
+        found, seen, axes = [], set(), set()
+
+        def walk(node, top):
+            if not isinstance(node, node_cls):
+                return True
+            op = node[0]["op"]
+            if op in ("dot", "transpose", "rand"):
+                return False
+            if not (walk(node[1], False) and walk(node[2], False)):
+                return False
+            if op in REDUCE and not top:
+                k = node.key()
+                if k not in seen:
+                    seen.add(k)
+                    found.append(node)
+                    axes.add(node[0].get("axis"))
+            return True
+
+        if not walk(expr, True) or len(axes) != 1 or None in axes:
+            return None
+        return found
+
+    def _run_as_one_kernel(self, trees):
+        """launch the statement group ``trees`` if one kernel can run it;
+        False, with nothing launched, if none can"""
+        try:
+            prog = Program()
+            for t in trees:
+                prog.add_statement(t)
+            prog.finalize()
+            key = prog.key()
+            plan = self.plans.get(key)
+            if plan is None:
+                plan = make_plan(prog, self.rt, self.kernels, self.cu_count, coop=key not in self._coop_failed)
+                plan.key = key
+                self.plans[key] = plan
+                self._stats["miss"] += 1
+            else:
+                self._stats["hit"] += 1
+        except (NeedsSplit, MixedAxes, NotImplementedError, ValueError, TypeError):
+            return False
+        self._launch_plan(plan, prog)
+        return True
 
     def _run_leaf(self, tree):
         if self._stage_transposed_views(tree):

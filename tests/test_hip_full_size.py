@@ -141,3 +141,61 @@ def test_c5_full_size_all_forms(pair):
             assert_close(ce.get(), cce.get(), rtol=1e-5, atol=1e-6, what="dense one-hot, pair %s" % lse)
     assert families[(True, True)] == ["colsplit"]        # one pass, nobody waits
     assert families[(False, False)] == ["colcoop"]       # three sweeps over resident rows, as written
+
+
+def test_axis0_trees_too_large_for_one_kernel_are_staged_with_their_reductions_together(pair):
+    """A matrix too tall for one workgroup's registers and too large for the
+    cooperative family: the reductions of the tree (nested or side by side)
+    run as ONE kernel over the operand, then the elementwise rest -- softmax
+    reads x twice and writes once.  Against the oracle and float64."""
+    cpu, hip = pair
+    shape = (9000, 3072)
+    rs = np.random.RandomState(77)
+    x = (rs.standard_normal(shape) * 3.0).astype(np.float32)
+    x64 = x.astype(np.float64)
+    e64 = np.exp(x64 - x64.max(axis=0))
+    sm64 = e64 / e64.sum(axis=0)
+    hx, cx = hip.array(x), cpu.array(x)
+    hout, cout = hip.empty(shape), cpu.empty(shape)
+
+    def launches(issue):
+        before = hip.plan_stats["launches"]
+        issue()
+        return hip.plan_stats["launches"] - before
+
+    for name, tree in (("softmax as written", lambda be, t: be.exp(t - be.max(t, axis=0)) /
+                        be.sum(be.exp(t - be.max(t, axis=0)), axis=0)),
+                       ("softmax, reciprocal form", lambda be, t: be.fprop_softmax(t, 0))):
+        cout[:] = tree(cpu, cx)
+        for lse, want_launches in ((True, 2), (False, 3)):
+            with rewrites(hip, lse, True):
+                assert launches(lambda: hout.__setitem__(slice(None), tree(hip, hx))) == want_launches, name
+                got = hout.get()
+                # numpy adds the 9000 terms of a column one after the other in fp32 (error up to
+                # rows x 2^-24); the device adds a tree and stays within 1e-5 of float64
+                assert rel_err(got, cout.get(), floor_frac=1e-3) < 1e-4, name
+                assert rel_err(got, sm64, floor_frac=1e-3) < 1e-5, name
+                assert np.allclose(got.sum(axis=0), 1.0, atol=1e-5)
+                # again: the recorded launches (three temporaries' worth of them) are replayed
+                hout.fill(0)
+                assert launches(lambda: hout.__setitem__(slice(None), tree(hip, hx))) == want_launches
+                assert np.array_equal(hout.get(), got)
+    # log-softmax: the same two reductions under another elementwise rest
+    with rewrites(hip, True, True):
+        n = launches(lambda: hout.__setitem__(
+            slice(None), hx - hip.max(hx, axis=0) - hip.log(hip.sum(hip.exp(hx - hip.max(hx, axis=0)), axis=0))))
+        assert n == 2
+        want = x64 - x64.max(axis=0) - np.log(e64.sum(axis=0))
+        assert_close(hout.get(), want, rtol=1e-5, atol=2e-5, what="log-softmax")
+    # two reductions side by side (no nesting): one pass for both
+    n = launches(lambda: hout.__setitem__(slice(None), (hx - hip.min(hx, axis=0)) /
+                                          (hip.max(hx, axis=0) - hip.min(hx, axis=0))))
+    assert n <= 2
+    want = (x64 - x64.min(axis=0)) / (x64.max(axis=0) - x64.min(axis=0))
+    assert_close(hout.get(), want, rtol=1e-5, atol=1e-6, what="min-max scaling")
+    # nested reductions no family takes together (variance around the mean): one kernel each
+    cout[:] = (cx - cpu.mean(cx, axis=0)) / cpu.sqrt(cpu.var(cx, axis=0) + 1e-5)
+    n = launches(lambda: hout.__setitem__(slice(None), (hx - hip.mean(hx, axis=0)) /
+                                          hip.sqrt(hip.var(hx, axis=0) + 1e-5)))
+    assert n == 3
+    assert_close(hout.get(), cout.get(), rtol=1e-4, atol=1e-5, what="column normalisation")
