@@ -750,7 +750,7 @@ class _RedGen(_Gen):
 # =====================================================================================
 # family: row  (axis 1)
 # =====================================================================================
-def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=False):
+def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=False, park_bytes=0):
     """Axis-1 reductions.  A team of LX lanes (a power of two up to 64, or the
     whole workgroup) owns one row; the workgroup holds LY rows.  A lane visits
     column tiles tx, tx+LX, ...; with ``NCH`` > 0 that loop has a fixed trip
@@ -762,6 +762,14 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
     while they fit, the others are fetched again, a few tiles at a time, in
     every sweep that reads them (batch-norm backward keeps ``x`` and re-reads
     the deltas: four passes over HBM instead of five).
+
+    ``park_bytes`` (whole-workgroup rows): LDS the workgroup may use as a second
+    tier of residence.  An operand that found no registers and is read by more
+    than one sweep leaves the tiles it fetched in its first sweep there -- every
+    lane its own, 16 bytes apart from its neighbour's, no barrier needed -- and
+    later sweeps take them back from LDS instead of memory; tiles that do not
+    fit are fetched again.  The planner grants it when every workgroup has a
+    compute unit (and its 160 KB) to itself.
 
     ``chunks`` > 1 (family ``rowcoop``; whole-workgroup rows with ``NCH`` > 0
     only): few, very long rows.  grid = (rows, chunks); workgroup (r, q) owns
@@ -786,6 +794,9 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
     assert not coop or (resident and LY == 1 and T % 64 == 0 and chunks <= T)
     words_left = [keep_words]       # None: everything is kept
     transient = set()               # nids of row operands that are not kept
+    park_left = [int(park_bytes) if (LY == 1 and NCH > 0) else 0]
+    park = {}                       # nid of a transient operand -> tiles it parks in LDS
+    parked = set()                  # ... whose tiles are in LDS by now
     params, fmt = g.param_list([("char* ws", "P"), ("long long ctr_offset", "q")] if coop else [])
     head = ('extern "C" __global__ __launch_bounds__(%d) void @NAME@(%s)\n' % (T, params))
     per_level = _levels(prog)
@@ -916,7 +927,15 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
             L("const int k = kb + u;")
             chunk_position("k")         # k beyond the row: c >= C, so ok is false
             for n in passing:
-                L(tile_load("%s[u]" % g.tile_name(n, "_s"), n))
+                name = "%s[u]" % g.tile_name(n, "_s")
+                if n.nid in parked:
+                    # (k is a compile-time number once the loops are unrolled)
+                    L("if (k < %d) %s = park%d[k][threadIdx.x]; else { %s }"
+                      % (park[n.nid], name, n.nid, tile_load(name, n)))
+                else:
+                    L(tile_load(name, n))
+                    if n.nid in park:
+                        L("if (k < %d) park%d[k][threadIdx.x] = %s;" % (park[n.nid], n.nid, name))
             L.close()
             L("#pragma unroll")
             L.open("for (int u = 0; u < %d; ++u)" % SU)
@@ -925,6 +944,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
             emit_body(tiles)
             L.close()
             L.close()
+            parked.update(n.nid for n in passing if n.nid in park)
             return
         L.open("for (int kb = 0; kb < nch; kb += %d)" % SU)
         for n in moving:
@@ -948,6 +968,20 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
     def varies_in_loop(n):
         return g.tile_width(n, 2) == 2      # tile spans columns
 
+    # how many sweeps (the final, storing one included) read each operand
+    sweeps_reading = {}
+    if park_left[0]:
+        earlier = set()
+        rounds = [[n for n in per_level.get(s_, [])] for s_ in range(nsweeps)]
+        for reds_ in rounds:
+            if reds_:
+                for leaf in g.leaf_nodes(_needed([n.args[0] for n in reds_], earlier)):
+                    sweeps_reading[leaf.nid] = sweeps_reading.get(leaf.nid, 0) + 1
+                earlier.update(n.nid for n in reds_)
+        if full_out:
+            for leaf in g.leaf_nodes(_needed([st.root for st in full_out], earlier)):
+                sweeps_reading[leaf.nid] = sweeps_reading.get(leaf.nid, 0) + 1
+
     def declare_tiles(leaves):
         """function-scope declarations needed before a sweep's loop"""
         for n in leaves:
@@ -961,6 +995,12 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
                 need = NCH * max(1, (g.tile_width(n, V) * prog.tensors[n.slot].dtype.itemsize + 3) // 4)
                 if words_left[0] is not None and need > words_left[0]:
                     transient.add(n.nid)
+                    tile_bytes = 4 * T * max(1, (g.tile_width(n, V) * prog.tensors[n.slot].dtype.itemsize + 3) // 4)
+                    fit = min(NCH, park_left[0] // tile_bytes)
+                    if fit > 0 and sweeps_reading.get(n.nid, 0) > 1:
+                        park[n.nid] = fit
+                        park_left[0] -= fit * tile_bytes
+                        L("__shared__ __attribute__((aligned(16))) %s park%d[%d][%d];" % (g.tile_type(n, V), n.nid, fit, T))
                     continue
                 if words_left[0] is not None:
                     words_left[0] -= need
@@ -1156,7 +1196,8 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
     L.close()
     return _finish("rowcoop" if coop else "row", g, head, fmt, T, 0,
                    dict(V=V, LX=LX, LY=LY, NCH=NCH, stream=bool(stream), passing=len(transient),
-                        over=len(vals), chunks=chunks, NRED=len(all_reds), tail=bool(tail)))
+                        over=len(vals), chunks=chunks, NRED=len(all_reds), tail=bool(tail),
+                        parked=sum(park.values())))
 
 
 # =====================================================================================

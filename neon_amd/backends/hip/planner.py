@@ -364,6 +364,11 @@ def _plan_ew(prog, cu_count):
     return Choice(spec, (gx, gy, 1), extras=(row_tiles,))
 
 
+# LDS a workgroup that has a compute unit to itself may use as a second tier of residence
+# (gfx950: 160 KB per compute unit; the rest is left to the reduction slots)
+ROW_PARK_BYTES = int(os.environ.get("NEON_HIP_ROW_PARK_KB", "144")) << 10
+
+
 def _plan_row(prog, cu_count, coop=True):
     R, C = prog.domain
     V = _vector_width(prog, tail_ok=True)
@@ -407,14 +412,16 @@ def _plan_row(prog, cu_count, coop=True):
                         for t in prog.tensors if t.read and t.shape[1] > 1] or [1 << 30])
         if chunks >= 2 and per <= 16 and per * smallest <= 64:
             kw = None if per * words <= 64 else 64
-            spec = codegen.gen_row(prog, V, 1024, 1, per, _streams(prog), keep_words=kw, chunks=chunks, tail=tail)
+            spec = codegen.gen_row(prog, V, 1024, 1, per, _streams(prog), keep_words=kw, chunks=chunks, tail=tail,
+                                   park_bytes=ROW_PARK_BYTES if kw else 0)
             part_bytes = R * spec.params["NRED"] * chunks * 8
             ctr_off = _ceil_div(part_bytes, 256) * 256
             return Choice(spec, (R, chunks, 1), workspace=(ctr_off + R * 8 + 4, ctr_off, 2 * R + 1),
                           status_offset=ctr_off + R * 8)
     LY = T // LX
-    spec = codegen.gen_row(prog, V, LX, LY, NCH, _streams(prog), keep_words=keep_words, tail=tail)
     gx = _ceil_div(R, LY)
+    park = ROW_PARK_BYTES if (keep_words and LY == 1 and gx <= cu_count) else 0
+    spec = codegen.gen_row(prog, V, LX, LY, NCH, _streams(prog), keep_words=keep_words, tail=tail, park_bytes=park)
     return Choice(spec, (gx, 1, 1))
 
 

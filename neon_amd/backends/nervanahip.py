@@ -939,7 +939,9 @@ class NervanaHIPBase(object):
         tree, same tensors -- replays the recorded launches, re-binding the
         constant arguments when only numbers changed (Adam's step-dependent
         learning rate).  The reference re-derived everything on every call
-        (its own TODO at float_ew.py:640-641 asks for exactly this)."""
+        (its own TODO at float_ew.py:640-641 asks for exactly this).
+        Returns the recording that now stands for the group (None when the
+        group cannot be replayed)."""
         try:
             key, raw = self._launch_key(trees, posts)
             if self._originals:
@@ -958,14 +960,15 @@ class NervanaHIPBase(object):
                     self._rec_temps.extend(entry.temps)
                     self._rec_coop.extend(entry.coop)
                     self._rec_single = None
+                    entry = None
                 self._stats["replayed"] += 1
                 self._stats["launches"] += len(launches)
-                return
+                return entry
         outer = self._recording is None
         if outer:
             self._recording, self._rec_temps, self._rec_single, self._rec_coop = [], [], None, []
             self._rec_foreign = False
-        ok = False
+        ok, made = False, None
         try:
             self._run_slow(trees)
             ok = True
@@ -978,7 +981,8 @@ class NervanaHIPBase(object):
                         self._launch_cache.clear()
                     if len(rec) != 1:
                         single = None
-                    self._launch_cache[key] = _Recorded(rec, temps, raw, single, tuple(coop))
+                    made = self._launch_cache[key] = _Recorded(rec, temps, raw, single, tuple(coop))
+        return made
 
     def _launch_plan(self, plan, prog):
         if prog.rand_count:
@@ -1521,8 +1525,40 @@ class NervanaHIPBase(object):
         self._flush()
         if self._captured is not None:
             self._captured.append(list(trees))
-        else:
-            self._run(list(trees))
+            return None
+        return self._run(list(trees))
+
+    def _call_key(self, name, tensors, numbers):
+        """identity of one call of a compound operation: the memory layout (and
+        rounding mode) of every tensor argument and the numbers.  Equal keys
+        mean the same trees over the same memory, i.e. the same launches."""
+        return (name,) + tuple((t._geom, t.rounding) for t in tensors) + tuple(numbers)
+
+    def _remember_call(self, ckey, recording):
+        if recording is not None:
+            self._launch_cache[ckey] = (recording, list(recording.raw))
+
+    def _replay_call(self, ckey):
+        """enqueue the launches recorded for an earlier identical call of a
+        compound operation, without building its trees again; False when
+        there is no such recording (or launches are being captured)"""
+        if self._captured is not None or self._recording is not None:
+            return False
+        self._flush()
+        found = self._launch_cache.get(ckey)
+        if found is None:
+            return False
+        entry, raw = found
+        if entry.raw != raw:
+            # the statement-level path has since re-bound this recording to other numbers
+            del self._launch_cache[ckey]
+            return False
+        entry.replay(self.rt)
+        for plan in entry.coop:
+            self._coop_pending[plan.key] = plan
+        self._stats["replayed"] += 1
+        self._stats["launches"] += len(entry.launches)
+        return True
 
     def compound_fprop_bn(self, x, xsum, xvar, gmean, gvar, gamma, beta, y, eps, rho,
                           compute_batch_sum, accumbeta=0.0, relu=False, threads=None, repeat=1,
@@ -1541,6 +1577,10 @@ class NervanaHIPBase(object):
             xhat = (x - gmean) / self.sqrt(gvar + eps)
             y[:] = (y * accumbeta + xhat * gamma + beta) if accumbeta != 0 else (xhat * gamma + beta)
             return
+        ckey = self._call_key("compound_fprop_bn", (x, xsum, xvar, gmean, gvar, gamma, beta, y),
+                              (float(eps), float(rho), bool(compute_batch_sum), float(accumbeta)))
+        if self._replay_call(ckey):
+            return
         st, n = self._stmt, float(x.shape[1])
         trees = []
         if compute_batch_sum:
@@ -1552,7 +1592,7 @@ class NervanaHIPBase(object):
         xhat = (x - xsum) / self.sqrt(xvar + eps)
         out = y.reshape(x.shape)
         trees.append(st(out, (xhat * gamma + beta + accumbeta * out) if accumbeta != 0 else (xhat * gamma + beta)))
-        self._run_group(trees)
+        self._remember_call(ckey, self._run_group(trees))
 
     def compound_bprop_bn(self, delta_out, grad_gamma, grad_beta, delta_in, x, xsum, xvar,
                           gamma, eps, threads=None, repeat=1, binary=False, layer=None):
@@ -1561,6 +1601,10 @@ class NervanaHIPBase(object):
         deltas from one pass over ``x`` and ``delta_in``."""
         if binary:
             raise NotImplementedError("shift-based batch norm is outside the op-tree path")
+        ckey = self._call_key("compound_bprop_bn", (delta_out, grad_gamma, grad_beta, delta_in, x, xsum, xvar, gamma),
+                              (float(eps),))
+        if self._replay_call(ckey):
+            return
         st = self._stmt
         inv_v = 1.0 / self.sqrt(xvar + eps)
         xhat = (x - xsum) * inv_v
@@ -1568,7 +1612,7 @@ class NervanaHIPBase(object):
                  st(grad_beta, self.sum(delta_in, axis=1))]
         xtmp = (xhat * grad_gamma + grad_beta) / float(x.shape[1])
         trees.append(st(delta_out.reshape(delta_in.shape), ((delta_in - xtmp) * gamma) * inv_v))
-        self._run_group(trees)
+        self._remember_call(ckey, self._run_group(trees))
 
     # -- layer-level helpers that are plain op-trees ----------------------------------------
     def consume(self, buf_index, hostlist, devlist):

@@ -622,6 +622,44 @@ def test_compound_batchnorm(pair, shape, dtype):
         assert fams
 
 
+def test_repeated_batchnorm_calls_replay_their_recorded_launches(pair):
+    """the second and later calls of compound_fprop_bn / compound_bprop_bn on the
+    same tensors take the launches recorded by the first (no trees are built);
+    new data, other numbers and other tensors must all still come out right"""
+    cpu, hip = pair
+    shape = (24, 3000)
+    rs = np.random.RandomState(9)
+    state = []
+    for be in pair:
+        vec = lambda: be.zeros((shape[0], 1))     # noqa: E731
+        state.append(dict(be=be, x=be.empty(shape), d=be.empty(shape), y=be.empty(shape), dout=be.empty(shape),
+                          xsum=vec(), xvar=vec(), gmean=vec(), gvar=vec(), gg=vec(), gb=vec(),
+                          gamma=be.array(rs.uniform(0.5, 1.5, (shape[0], 1)).astype(np.float32)),
+                          beta=be.array((rs.standard_normal((shape[0], 1)) * 0.1).astype(np.float32))))
+        rs = np.random.RandomState(9)             # same gamma / beta on both backends
+    before = hip.plan_stats["replayed"]
+    for call, rho in enumerate((0.9, 0.9, 0.9, 0.5, 0.5, 0.9)):
+        x0 = (rs.standard_normal(shape) * (1 + call) + 0.25 * call).astype(np.float32)
+        d0 = rs.standard_normal(shape).astype(np.float32)
+        out = []
+        for st in state:
+            be = st["be"]
+            st["x"].set(x0)
+            st["d"].set(d0)
+            y = st["y"] if call != 4 else be.empty(shape)        # once into another output tensor
+            be.compound_fprop_bn(st["x"], st["xsum"], st["xvar"], st["gmean"], st["gvar"], st["gamma"], st["beta"],
+                                 y, 1e-3, rho, True)
+            be.compound_bprop_bn(st["dout"], st["gg"], st["gb"], st["d"], st["x"], st["xsum"], st["xvar"],
+                                 st["gamma"], 1e-3)
+            out.append([t.get().astype(np.float64) for t in (y, st["xsum"], st["xvar"], st["gmean"], st["gvar"],
+                                                             st["dout"], st["gg"], st["gb"])])
+        for got, want, name in zip(out[1], out[0], ("y", "xmean", "xvar", "gmean", "gvar", "delta", "gg", "gb")):
+            scale = np.abs(want).max() + 1e-30
+            assert np.abs(got - want).max() <= 2e-5 * scale, (call, name)
+    # calls 1, 2 and 5 of the forward pass and 1..5 of the backward pass found their recording
+    assert hip.plan_stats["replayed"] - before >= 8
+
+
 def test_more_than_2_31_elements(hip):
     """a tensor of 46341 x 46342 fp16 (2^31 + 83k elements, 4.3 GB): fill,
     elementwise tree and both reduction axes address it with 64-bit offsets;
