@@ -367,6 +367,8 @@ def _plan_ew(prog, cu_count):
 # LDS a workgroup that has a compute unit to itself may use as a second tier of residence
 # (gfx950: 160 KB per compute unit; the rest is left to the reduction slots)
 ROW_PARK_BYTES = int(os.environ.get("NEON_HIP_ROW_PARK_KB", "144")) << 10
+ROW_SPLIT_WORDS = int(os.environ.get("NEON_HIP_SPLIT_WORDS", "64"))
+ROW_SPLIT_MAX_TILES = 32        # tiles of 1024 lanes per row that the unrolled split-residence form takes
 
 
 def _plan_row(prog, cu_count, coop=True):
@@ -398,6 +400,10 @@ def _plan_row(prog, cu_count, coop=True):
                         for t in prog.tensors if t.read and t.shape[1] > 1] or [1 << 30])
         if nch <= 16 and nch * smallest <= 64:
             LX, T, NCH, keep_words = 1024, 1024, nch, 64
+        elif nch <= ROW_SPLIT_MAX_TILES and R <= cu_count and ROW_PARK_BYTES:
+            # longer still: registers and LDS together hold (most of) one operand
+            # ((256,200704) fp16: 16 tiles in registers + 9 in LDS = the whole row)
+            LX, T, NCH, keep_words = 1024, 1024, nch, ROW_SPLIT_WORDS
     # Few, very long rows (batch norm over the 64 feature maps of an early
     # convolution): one workgroup per row would leave most compute units idle
     # and the row may not fit its registers.  Spread every row over several
