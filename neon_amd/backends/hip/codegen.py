@@ -783,8 +783,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
     first sweep there -- every lane its own, 16 bytes apart from its
     neighbour's, no barrier needed --, holds the next ones in whatever registers
     are left, and later sweeps take both back instead of going to memory; only
-    tiles beyond that are fetched again.  The planner grants it when every
-    workgroup has a compute unit (and its 160 KB) to itself.
+    tiles beyond that are fetched again.
 
     ``chunks`` > 1 (family ``rowcoop``; whole-workgroup rows with ``NCH`` > 0
     only): few, very long rows.  grid = (rows, chunks); workgroup (r, q) owns

@@ -364,8 +364,11 @@ def _plan_ew(prog, cu_count):
     return Choice(spec, (gx, gy, 1), extras=(row_tiles,))
 
 
-# LDS a workgroup that has a compute unit to itself may use as a second tier of residence
-# (gfx950: 160 KB per compute unit; the rest is left to the reduction slots)
+# LDS a 1024-lane workgroup may use as a second tier of residence (gfx950: 160 KB per compute
+# unit; the rest is left to the reduction slots).  A compute unit then holds one such workgroup
+# instead of two, which costs less than fetching the tiles again -- also with more rows than
+# compute units (batch-norm backward over (512,100352) fp16: 71 -> 57 us; forward over
+# (512,200704): 136 -> 80 us; half the LDS and two workgroups per unit: 64 / 87 us).
 ROW_PARK_BYTES = int(os.environ.get("NEON_HIP_ROW_PARK_KB", "144")) << 10
 ROW_SPLIT_WORDS = int(os.environ.get("NEON_HIP_SPLIT_WORDS", "64"))
 ROW_SPLIT_MAX_TILES = 32        # tiles of 1024 lanes per row that the unrolled split-residence form takes
@@ -400,7 +403,7 @@ def _plan_row(prog, cu_count, coop=True):
                         for t in prog.tensors if t.read and t.shape[1] > 1] or [1 << 30])
         if nch <= 16 and nch * smallest <= 64:
             LX, T, NCH, keep_words = 1024, 1024, nch, 64
-        elif nch <= ROW_SPLIT_MAX_TILES and R <= cu_count and ROW_PARK_BYTES:
+        elif nch <= ROW_SPLIT_MAX_TILES and ROW_PARK_BYTES:
             # longer still: registers and LDS together hold (most of) one operand
             # ((256,200704) fp16: 16 tiles in registers + 9 in LDS = the whole row)
             LX, T, NCH, keep_words = 1024, 1024, nch, ROW_SPLIT_WORDS
@@ -426,7 +429,7 @@ def _plan_row(prog, cu_count, coop=True):
                           status_offset=ctr_off + R * 8)
     LY = T // LX
     gx = _ceil_div(R, LY)
-    park = ROW_PARK_BYTES if (keep_words and LY == 1 and gx <= cu_count) else 0
+    park = ROW_PARK_BYTES if (keep_words and LY == 1) else 0
     spec = codegen.gen_row(prog, V, LX, LY, NCH, _streams(prog), keep_words=keep_words, tail=tail, park_bytes=park)
     return Choice(spec, (gx, 1, 1))
 

@@ -40,6 +40,7 @@ def bn_pair(be, x, d, shape, dtype):
 
 @pytest.mark.parametrize("shape,dtype", [
     ((200, 100352), np.float16),      # x resident, deltas parked (9 tiles) and held (3)
+    ((300, 100352), np.float16),      # the same with more rows than compute units
     ((130, 150528), np.float16),      # 19 tiles: one operand split between LDS and registers
     ((129, 200704), np.float16),      # 25 tiles: registers and LDS exactly full
     ((130, 100003), np.float32),      # fp32, 25 tiles, partial last tile
@@ -92,9 +93,9 @@ def test_which_forms_the_planner_picks(hip):
     assert spec.family == "rowcoop" and spec.params["parked"] > 0
     p = fprop_spec((150, 270000), f16).params
     assert p["NCH"] == 0 and p["parked"] == 0
-    # more rows than compute units: a compute unit holds two workgroups, LDS stays free
+    # more rows than compute units: the same form (one workgroup per compute unit at a time)
     p = bprop_spec((300, 100352), f16).params
-    assert p["parked"] == 0 and p["passing"] == 1
+    assert (p["parked"], p["held"], p["passing"]) == (9, 3, 1)
 
 
 @pytest.mark.parametrize("shape,dtype", [((130, 150528), np.float16), ((130, 100003), np.float32)])
