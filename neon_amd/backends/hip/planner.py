@@ -371,6 +371,7 @@ def _plan_ew(prog, cu_count):
 # (512,200704): 136 -> 80 us; half the LDS and two workgroups per unit: 64 / 87 us).
 ROW_PARK_BYTES = int(os.environ.get("NEON_HIP_ROW_PARK_KB", "144")) << 10
 ROW_SPLIT_WORDS = int(os.environ.get("NEON_HIP_SPLIT_WORDS", "64"))
+ROWCOOP_MAX_TILES = int(os.environ.get('NEON_HIP_ROWCOOP_TILES', '64'))
 ROW_SPLIT_MAX_TILES = 32        # tiles of 1024 lanes per row that the unrolled split-residence form takes
 
 
@@ -419,8 +420,14 @@ def _plan_row(prog, cu_count, coop=True):
         chunks = _ceil_div(tiles, per)
         smallest = min([max(1, (V * t.dtype.itemsize + 3) // 4)
                         for t in prog.tensors if t.read and t.shape[1] > 1] or [1 << 30])
-        if chunks >= 2 and per <= 16 and per * smallest <= 64:
-            kw = None if per * words <= 64 else 64
+        # (longer shares, where the row is swept more than once: what registers and LDS do not
+        # hold of a workgroup's share is fetched again in every sweep -- still all compute units
+        # at work instead of one per row.  Batch norm over (64,1605632) fp16: forward 304 ->
+        # 147 us, backward 372 -> 169 us; a single sweep gains nothing from it)
+        sweeps = prog.nlevels + (1 if any(st.out.shape[1] > 1 for st in prog.statements) else 0)
+        if chunks >= 2 and ((per <= 16 and per * smallest <= 64) or
+                            (per <= ROWCOOP_MAX_TILES and ROW_PARK_BYTES and sweeps >= 2)):
+            kw = None if (per <= 16 and per * words <= 64) else (64 if per <= 16 else ROW_SPLIT_WORDS)
             spec = codegen.gen_row(prog, V, 1024, 1, per, _streams(prog), keep_words=kw, chunks=chunks, tail=tail,
                                    park_bytes=ROW_PARK_BYTES if kw else 0)
             part_bytes = R * spec.params["NRED"] * chunks * 8

@@ -47,6 +47,7 @@ def bn_pair(be, x, d, shape, dtype):
     ((72, 200704), np.float16),       # few rows: three workgroups per row, each with its share resident
     ((140, 140001), np.float16),      # 18 tiles, partial last tile
     ((64, 401408), np.float16),       # few rows: four workgroups per row cooperate, each parking its share
+    ((120, 300000), np.float16),      # two workgroups per row, 19 tiles each: parked, held and fetched again
     ((150, 270000), np.float16),      # 33 tiles: beyond the unrolled form, streamed in every sweep
 ])
 def test_batch_norm_pair_over_long_rows(pair, shape, dtype):
@@ -91,6 +92,9 @@ def test_which_forms_the_planner_picks(hip):
     assert (p["NCH"], p["parked"], p["held"], p["tail"]) == (25, 9, 16, True)
     spec = bprop_spec((64, 401408), f16)
     assert spec.family == "rowcoop" and spec.params["parked"] > 0
+    spec = bprop_spec((120, 300000), f16)
+    assert spec.family == "rowcoop" and spec.params["NCH"] == 19 and spec.params["chunks"] == 2
+    assert spec.params["parked"] == 9 and spec.params["passing"] == 2
     p = fprop_spec((150, 270000), f16).params
     assert p["NCH"] == 0 and p["parked"] == 0
     # more rows than compute units: the same form (one workgroup per compute unit at a time)
