@@ -396,6 +396,8 @@ def _plan_row(prog, cu_count, coop=True):
     # two fp16 rows of batch-norm backward resident in 512-lane workgroups, 200
     # registers per lane, measured 53 us against 45 us for streaming twice)
     keep_words = None
+    # passes over the row: one per level of reductions, one more when full-shape results are stored
+    sweeps = prog.nlevels + (1 if any(st.out.shape[1] > 1 for st in prog.statements) else 0)
     if NCH == 0 and prog.nlevels + 1 >= 2:
         # the row does not fit as a whole: keep what fits of it (in order of
         # first use) in a 1024-lane workgroup and fetch the rest again per sweep
@@ -404,7 +406,7 @@ def _plan_row(prog, cu_count, coop=True):
                         for t in prog.tensors if t.read and t.shape[1] > 1] or [1 << 30])
         if nch <= 16 and nch * smallest <= 64:
             LX, T, NCH, keep_words = 1024, 1024, nch, 64
-        elif nch <= ROW_SPLIT_MAX_TILES and ROW_PARK_BYTES:
+        elif nch <= ROW_SPLIT_MAX_TILES and ROW_PARK_BYTES and sweeps >= 2:
             # longer still: registers and LDS together hold (most of) one operand
             # ((256,200704) fp16: 16 tiles in registers + 9 in LDS = the whole row)
             LX, T, NCH, keep_words = 1024, 1024, nch, ROW_SPLIT_WORDS
@@ -424,7 +426,6 @@ def _plan_row(prog, cu_count, coop=True):
         # hold of a workgroup's share is fetched again in every sweep -- still all compute units
         # at work instead of one per row.  Batch norm over (64,1605632) fp16: forward 304 ->
         # 147 us, backward 372 -> 169 us; a single sweep gains nothing from it)
-        sweeps = prog.nlevels + (1 if any(st.out.shape[1] > 1 for st in prog.statements) else 0)
         if chunks >= 2 and ((per <= 16 and per * smallest <= 64) or
                             (per <= ROWCOOP_MAX_TILES and ROW_PARK_BYTES and sweeps >= 2)):
             kw = None if (per <= 16 and per * words <= 64) else (64 if per <= 16 else ROW_SPLIT_WORDS)
