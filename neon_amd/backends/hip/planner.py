@@ -370,6 +370,16 @@ def _plan_ew(prog, cu_count):
 # compute units (batch-norm backward over (512,100352) fp16: 71 -> 57 us; forward over
 # (512,200704): 136 -> 80 us; half the LDS and two workgroups per unit: 64 / 87 us).
 ROW_PARK_BYTES = int(os.environ.get("NEON_HIP_ROW_PARK_KB", "144")) << 10
+
+
+def limit_lds(bytes_per_workgroup):
+    """tell the planner how much LDS a workgroup may have on the device in use
+    (160 KB on gfx950, which the defaults assume); called by the backend with
+    the figure the runtime reports"""
+    global ROW_PARK_BYTES
+    ROW_PARK_BYTES = max(0, min(ROW_PARK_BYTES, int(bytes_per_workgroup) - (16 << 10)))
+
+
 ROW_SPLIT_WORDS = int(os.environ.get("NEON_HIP_SPLIT_WORDS", "64"))
 ROWCOOP_MAX_TILES = int(os.environ.get('NEON_HIP_ROWCOOP_TILES', '64'))
 ROW_SPLIT_MAX_TILES = 32        # tiles of 1024 lanes per row that the unrolled split-residence form takes

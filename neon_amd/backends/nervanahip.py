@@ -23,6 +23,7 @@ from neon_amd.backends.hip import bf16
 from neon_amd.backends.hip import fastpath
 from neon_amd.backends.hip import runtime as hiprt
 from neon_amd.backends.hip.optree_ir import MixedAxes, Program, REDUCE, eval_const
+from neon_amd.backends.hip import planner
 from neon_amd.backends.hip.planner import KernelCache, NeedsSplit, make_plan
 
 logger = logging.getLogger(__name__)
@@ -522,6 +523,7 @@ class NervanaHIPBase(object):
         self.hist_bins, self.hist_offset = hist_bins, hist_offset
         self.hist_base, self.hist_map, self.hist_idx, self.hist_max = None, dict(), 0, 4 * 4096
         self.cu_count = int(self.rt.props.compute_units)
+        planner.limit_lds(self.rt.props.lds_bytes_per_block)
         self.kernels = KernelCache(self.rt.arch.split(":")[0], cache_dir)
         self.plans = {}
         self._stats = {"hit": 0, "miss": 0, "split": 0, "launches": 0, "replayed": 0}

@@ -473,3 +473,48 @@ def test_more_than_2_31_elements_stay_two_dimensional(pb):
     x, y, out = (pb.empty(small) for _ in range(3))
     ch = plan_of(pb, lambda: out.__setitem__(slice(None), x * 0.5 + y))
     assert ch.grid[0] * 256 * ch.spec.params["V"] >= small[0] * small[1]                    # flattened
+
+
+# ---- row family: LDS as a second tier of residence -------------------------------------------
+def _bn_backward_group(pb, shape, dtype=np.float16):
+    """the statements of batch-norm backward as one fused group (no device needed)"""
+    x, d, o = pb.empty(shape, dtype), pb.empty(shape, dtype), pb.empty(shape, dtype)
+    xsum, xvar, gamma, gg, gb = (pb.empty((shape[0], 1)) for _ in range(5))
+    inv_v = 1.0 / pb.sqrt(xvar + 1e-5)
+    xhat = (x - xsum) * inv_v
+    pb.begin(Block.update, 0)
+    gg[:] = pb.sum(xhat * d, axis=1)
+    gb[:] = pb.sum(d, axis=1)
+    o[:] = ((d - (xhat * gg + gb) / float(shape[1])) * gamma) * inv_v
+    pb.end(Block.update, 0)
+    return pb.choices[-1]
+
+
+def test_row_operands_without_registers_go_to_lds(tmp_path):
+    pb = prebuild.PlanBackend(cache_dir=str(tmp_path / "kc"), compile_kernels=True)      # hiprtc takes 144 KB of LDS
+    ch = _bn_backward_group(pb, (256, 100352))
+    p = ch.spec.params
+    assert ch.spec.family == "row" and (p["NCH"], p["passing"], p["parked"], p["held"]) == (13, 1, 9, 3)
+    assert "__shared__ __attribute__((aligned(16))) nh_raw<nh_f16, 8> park" in ch.spec.source
+    pb = prebuild.PlanBackend(cache_dir=str(tmp_path / "kc"), compile_kernels=False)
+    # rows of 25 tiles: one operand split between LDS and registers, the other fetched per sweep
+    p = _bn_backward_group(pb, (256, 200704)).spec.params
+    assert (p["NCH"], p["passing"], p["parked"], p["held"]) == (25, 2, 9, 16)
+    # a single sweep has nothing to come back for: streamed, no LDS
+    x, col = pb.empty((1000, 131072)), pb.empty((1000, 1))
+    p = plan_of(pb, lambda: col.__setitem__(slice(None), pb.sum(x, axis=1))).spec.params
+    assert (p["NCH"], p["parked"], p["held"]) == (0, 0, 0)
+    # few very long rows swept twice: workgroups of a row cooperate on shares beyond 16 tiles
+    ch = _bn_backward_group(pb, (64, 1605632))
+    assert ch.spec.family == "rowcoop" and ch.spec.params["NCH"] == 49 and ch.spec.params["parked"] == 9
+    # a device with 64 KB of LDS per workgroup gets 48 KB worth of parked tiles
+    saved = planner.ROW_PARK_BYTES
+    try:
+        planner.limit_lds(64 << 10)
+        p = _bn_backward_group(pb, (256, 100352)).spec.params
+        assert (p["parked"], p["held"]) == (3, 3)
+        planner.limit_lds(8 << 10)
+        p = _bn_backward_group(pb, (256, 100352)).spec.params
+        assert (p["parked"], p["held"], p["passing"]) == (0, 0, 1)
+    finally:
+        planner.ROW_PARK_BYTES = saved
