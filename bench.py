@@ -568,6 +568,57 @@ def counter_pass():
     print(json.dumps({"counter_pass": table}))
 
 
+def shape_sweep(dtype_name):
+    """Seven common trees over a grid of shapes between 8 MB and 1 GB: wall
+    clock per call through the public API, and the fraction of the HBM peak
+    the algorithmic bytes come to.  A map of where the kernel families stand
+    away from the five benchmark shapes (``python bench.py --sweep float32``)."""
+    from neon_amd.backends import gen_backend
+    be = gen_backend("hip", rng_seed=0)
+    dt = np.dtype(dtype_name)
+    isz = dt.itemsize
+
+    def per_call_us(issue, reps):
+        for _ in range(3):
+            issue()
+        be.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            issue()
+        be.synchronize()
+        return (time.perf_counter() - t0) * 1e6 / reps
+
+    names = ("x*2+1", "x+col", "sum ax0", "sum ax1", "argmax ax0", "softmax ax0", "softmax ax1")
+    print("%s storage; cells: microseconds per call / fraction of %.0f GB/s" % (dt.name, HBM_PEAK_GBS))
+    print("%-18s %s" % ("shape", " ".join("%12s" % n for n in names)))
+    dims = (64, 1000, 4096, 30000, 131072, 1048576)
+    for R in dims:
+        for C in dims:
+            n = R * C
+            if n * isz < (8 << 20) or n * isz > (1 << 30):
+                continue
+            x, o = be.empty((R, C), dtype=dt), be.empty((R, C), dtype=dt)
+            x[:] = be.rand()
+            col, row, irow = be.zeros((R, 1)), be.zeros((1, C)), be.zeros((1, C), dtype=np.int32)
+            reps = max(3, min(50, int(2e9 / (n * isz))))
+            trees = (
+                (lambda: o.__setitem__(slice(None), x * 2.0 + 1.0), 2),
+                (lambda: o.__setitem__(slice(None), x + col), 2),
+                (lambda: row.__setitem__(slice(None), be.sum(x, axis=0)), 1),
+                (lambda: col.__setitem__(slice(None), be.sum(x, axis=1)), 1),
+                (lambda: irow.__setitem__(slice(None), be.argmax(x, axis=0)), 1),
+                (lambda: o.__setitem__(slice(None), be.exp(x - be.max(x, axis=0)) /
+                                       be.sum(be.exp(x - be.max(x, axis=0)), axis=0)), 2),
+                (lambda: o.__setitem__(slice(None), be.exp(x - be.max(x, axis=1)) /
+                                       be.sum(be.exp(x - be.max(x, axis=1)), axis=1)), 2))
+            cells = []
+            for issue, passes in trees:
+                us = per_call_us(issue, reps)
+                cells.append("%6.0f/%.2f" % (us, passes * n * isz / us / 1e3 / HBM_PEAK_GBS))
+            print("%-18s %s" % ((R, C), " ".join("%12s" % c for c in cells)), flush=True)
+            del x, o
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -577,7 +628,14 @@ def main():
     ap.add_argument("--no-detail", action="store_true", help="headline only, no per-config table")
     ap.add_argument("--counter-pass", action="store_true",
                     help="short untimed run for rocprofv3 --pmc (see counter_pass)")
+    ap.add_argument("--sweep", metavar="DTYPE", default=None,
+                    help="common trees over a grid of shapes (float32 / float16), see shape_sweep")
     args = ap.parse_args()
+    if args.sweep:
+        import __graft_entry__
+        __graft_entry__.ensure_built()
+        shape_sweep(args.sweep)
+        return
     if args.counter_pass:
         counter_pass()
         return

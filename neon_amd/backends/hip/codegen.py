@@ -48,7 +48,8 @@ _UN = {"neg": "(-{0})", "abs": "__builtin_fabsf({0})", "sgn": "nh_sgn({0})",
        "log": "logf({0})", "exp2": "exp2f({0})", "log2": "log2f({0})",
        "sig": "nh_sig({0})", "sig2": "nh_sig2({0})", "tanh": "tanhf({0})",
        "tanh2": "nh_tanh2({0})", "safelog": "nh_safelog({0})",
-       "rint": "rintf({0})", "finite": "nh_finite({0})", "ident": "({0})"}
+       "rint": "rintf({0})", "finite": "nh_finite({0})", "ident": "({0})",
+       "exp_nonpos": "nh_exp_nonpos({0})"}
 _RED_OP = {"sum": "nh_op_sum", "max": "nh_op_max", "min": "nh_op_min",
            "argmax": "nh_op_argmax", "argmin": "nh_op_argmin"}
 
@@ -278,6 +279,10 @@ class _Gen(object):
                 return "nh_rand01(%s)" % word
             return "nh_sround(%s, %s, %s)" % (a[0], n.op.split(":")[1], word)
         if len(a) == 1:
+            if n.op == "exp" and EXP_OF_NONPOSITIVE and _below_its_maximum(n.args[0]):
+                # exp(x - max(x)): the argument cannot be positive, which is all nh_exp_nonpos
+                # asks for (softmax and log-sum-exp trees; 7 instructions against expf's 13)
+                return "nh_exp_nonpos({0})".format(*a)
             return _UN[n.op].format(*a)
         if n.op in ("add", "sub") and self.one_declared and any(self.is_half_leaf(x) for x in n.args):
             # widening of the fp16 operand and the addition in one instruction
@@ -386,6 +391,7 @@ RECIPROCAL_OF_BROADCAST = os.environ.get("NEON_HIP_RCP", "1") != "0"
 FMA_IN_SUMS = os.environ.get("NEON_HIP_FMA_SUMS", "1") != "0"
 # results stored as 16-bit floats: a chain of multiplications / divisions by
 # per-line values and a final per-line addend collapse into one multiply-add
+EXP_OF_NONPOSITIVE = os.environ.get("NEON_HIP_EXP_NONPOS", "1") != "0"
 AFFINE_16BIT_OUTPUTS = os.environ.get("NEON_HIP_AFFINE16", "1") != "0"
 
 
@@ -430,6 +436,14 @@ def _affine_in_line(root, constant):
     if constant(n) or n is root:
         return None
     return n, mults, addends
+
+
+def _below_its_maximum(n):
+    """n is ``v - max(v)`` along some axis: never positive (NaN aside)"""
+    if n.kind != "E" or n.op != "sub" or len(n.args) != 2:
+        return False
+    v, m = n.args
+    return m.kind == "R" and m.op == "max" and m.args[0] is v
 
 
 def _needed(targets, available):

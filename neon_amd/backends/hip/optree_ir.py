@@ -35,7 +35,10 @@ from neon_amd.backends.hip.bf16 import bfloat16
 
 
 UNARY = {"neg", "abs", "sgn", "sqrt", "sqr", "exp", "log", "exp2", "log2", "sig",
-         "sig2", "tanh", "tanh2", "safelog", "rint", "finite"}
+         "sig2", "tanh", "tanh2", "safelog", "rint", "finite",
+         # internal: exp of an argument known not to be positive (what staged evaluation makes
+         # of exp(x - max(x)) once the maximum sits in a temporary)
+         "exp_nonpos"}
 BINARY = {"add", "sub", "mul", "div", "eq", "ne", "lt", "le", "gt", "ge", "pow",
           "minimum", "maximum"}
 REDUCE = {"sum", "max", "min", "argmax", "argmin"}
@@ -62,7 +65,7 @@ def _fold_unary(op, x):
             return float(np.sqrt(x))
         if op == "sqr":
             return x * x
-        if op == "exp":
+        if op == "exp" or op == "exp_nonpos":
             return float(np.exp(x))
         if op == "log":
             return float(np.log(x))

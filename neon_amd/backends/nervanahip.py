@@ -23,7 +23,7 @@ from neon_amd.backends.hip import bf16
 from neon_amd.backends.hip import fastpath
 from neon_amd.backends.hip import runtime as hiprt
 from neon_amd.backends.hip.optree_ir import MixedAxes, Program, REDUCE, eval_const
-from neon_amd.backends.hip import planner
+from neon_amd.backends.hip import codegen, planner
 from neon_amd.backends.hip.planner import KernelCache, NeedsSplit, make_plan
 
 logger = logging.getLogger(__name__)
@@ -1162,6 +1162,7 @@ class NervanaHIPBase(object):
         temps = []
         memo = {}
         together = {}
+        nonpos_exp = codegen.EXP_OF_NONPOSITIVE
 
         def lower(node, top=False):
             if not isinstance(node, self._api.OpTreeNode):
@@ -1198,6 +1199,10 @@ class NervanaHIPBase(object):
                 tmp = self._temp(left.shape, np.float32, temps)
                 self._run([self._api.OpTreeNode({"op": "assign"}, tmp, left)])
                 return tmp.T
+            if op == "exp" and nonpos_exp and self._is_below_its_maximum(node[1]):
+                # exp(x - max(x)) keeps the cheaper exponential that a single kernel would use
+                # for it, although the maximum is a temporary by now
+                return self._api.OpTreeNode(dict(node[0], op="exp_nonpos"), left, right)
             rebuilt = self._api.OpTreeNode(node[0], left, right)
             if op in REDUCE:
                 if top:
@@ -1226,6 +1231,19 @@ class NervanaHIPBase(object):
         finally:
             for t in temps:
                 self._temp_release(t)
+
+    def _is_below_its_maximum(self, node):
+        """``node`` is ``v - max(v, axis)``: never positive"""
+        cls = self._api.OpTreeNode
+        if not isinstance(node, cls) or node[0]["op"] != "sub":
+            return False
+        v, m = node[1], node[2]
+        if not isinstance(m, cls) or m[0]["op"] != "max" or m[0].get("axis") not in (0, 1):
+            return False
+        w = m[1]
+        if isinstance(v, cls) and isinstance(w, cls):
+            return v.key() == w.key()
+        return v is w
 
     def _reductions_along_one_axis(self, expr):
         """the distinct reduction nodes below the root of ``expr``, innermost

@@ -927,3 +927,39 @@ def test_gather_views_clamp_indices_outside_the_table(hip):
     cols = hip.empty((40, 3))
     cols[:] = T.take(hip.array(np.array([[5], [6], [-2]], dtype=np.int32), dtype=np.int32), 1)
     assert np.array_equal(cols.get(), table[:, [5, 5, 0]])
+
+
+def test_exponential_of_values_below_their_maximum_is_good_to_the_last_place(hip):
+    """exp(x - max(x)) runs a shorter exponential (its argument is never
+    positive): against float64 over the whole range that yields normal
+    numbers, and the edge cases -- equal to the maximum, -inf, NaN columns"""
+    rs = np.random.RandomState(21)
+    cols = 512
+    d = -np.abs(rs.uniform(0, 87.0, (400, cols))).astype(np.float32)
+    d[0, :] = 0.0                                           # every column's maximum
+    d[1, :] = -np.logspace(-8, 1.9, cols).astype(np.float32)
+    x = d + rs.uniform(-50, 50, (1, cols)).astype(np.float32)
+    # (the difference is taken in fp32, as any fp32 evaluation takes it; the exponential of
+    # that difference is what is being checked)
+    want = np.exp((x - x.max(axis=0)).astype(np.float64))
+    out = hip.empty(x.shape)
+    out[:] = hip.exp(hip.array(x) - hip.max(hip.array(x), axis=0))
+    got = out.get().astype(np.float64)
+    normal = want > 1.2e-38
+    assert np.max(np.abs(got[normal] - want[normal]) / want[normal]) < 2.5e-7        # two units in the last place
+    assert np.all(got[~normal] <= 1.2e-38)
+    assert np.all(got[0] == 1.0)
+    # along rows, with -inf entries and a NaN row
+    y = rs.uniform(-30, 30, (64, 300)).astype(np.float32)
+    y[3, 5] = -np.inf
+    y[7, :] = -np.inf                                      # (all -inf: -inf - -inf = NaN, as in numpy)
+    y[9, 11] = np.nan
+    outy = hip.empty(y.shape)
+    outy[:] = hip.exp(hip.array(y) - hip.max(hip.array(y), axis=1))
+    with np.errstate(invalid="ignore"):
+        wy = np.exp((y - y.max(axis=1, keepdims=True)).astype(np.float64))
+    gy = outy.get()
+    assert np.array_equal(np.isnan(gy), np.isnan(wy))
+    ok = ~np.isnan(wy)
+    np.testing.assert_allclose(gy[ok], wy[ok], rtol=2.5e-7, atol=1e-38)
+    assert gy[3, 5] == 0.0

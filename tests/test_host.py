@@ -428,7 +428,7 @@ def test_softmax_reuses_the_registers_of_x_for_the_exponentials(pb):
 
     spec = plan_of(pb, lambda: out.__setitem__(slice(None), softmax(x))).spec
     assert spec.family == "col" and spec.params["over"] == 1
-    assert spec.source.count("expf(") == 1 and ".put(j, " in spec.source
+    assert spec.source.count("nh_exp_nonpos(") == 1 and "expf(" not in spec.source and ".put(j, " in spec.source
 
     spec = plan_of(pb, lambda: out.__setitem__(slice(None), softmax(x) + x)).spec
     assert spec.params["over"] == 0 and ".put(j, " not in spec.source
@@ -447,18 +447,18 @@ def test_row_softmax_reuses_registers_when_the_row_is_resident(pb):
 
     spec = plan_of(pb, lambda: out.__setitem__(slice(None), softmax(x))).spec
     assert spec.family == "row" and spec.params["NCH"] > 0 and spec.params["over"] == 1
-    assert spec.source.count("expf(") == 1
+    assert spec.source.count("nh_exp_nonpos(") == 1 and "expf(" not in spec.source
     # few rows too long for one workgroup's registers are spread over several
     # workgroups and stay resident
     xl, outl = pb.empty((16, 1 << 20)), pb.empty((16, 1 << 20))
     ch = plan_of(pb, lambda: outl.__setitem__(slice(None), softmax(xl)))
     assert ch.spec.family == "rowcoop" and ch.grid == (16, 16, 1) and ch.spec.params["over"] == 1
-    assert ch.spec.source.count("expf(") == 1
+    assert ch.spec.source.count("nh_exp_nonpos(") == 1
     # many such rows are streamed in every sweep: nothing to reuse
     xl, outl = pb.empty((512, 1 << 20)), pb.empty((512, 1 << 20))
     spec = plan_of(pb, lambda: outl.__setitem__(slice(None), softmax(xl))).spec
     assert spec.family == "row" and spec.params["NCH"] == 0 and spec.params["over"] == 0
-    assert spec.source.count("expf(") == 2
+    assert spec.source.count("nh_exp_nonpos(") == 2
 
 
 def test_more_than_2_31_elements_stay_two_dimensional(pb):
@@ -518,3 +518,17 @@ def test_row_operands_without_registers_go_to_lds(tmp_path):
         assert (p["parked"], p["held"], p["passing"]) == (0, 0, 1)
     finally:
         planner.ROW_PARK_BYTES = saved
+
+
+def test_the_cheaper_exponential_is_for_arguments_below_their_own_maximum_only(pb):
+    x, y, out = pb.empty((1000, 256)), pb.empty((1000, 256)), pb.empty((1000, 256))
+    for axis in (0, 1):
+        src = plan_of(pb, lambda: out.__setitem__(slice(None), pb.exp(x - pb.max(x, axis=axis)))).spec.source
+        assert "nh_exp_nonpos(" in src and "expf(" not in src
+        src = plan_of(pb, lambda: out.__setitem__(slice(None), pb.exp(x * 2.0 - pb.max(x * 2.0, axis=axis)))).spec.source
+        assert "nh_exp_nonpos(" in src and "expf(" not in src
+        # the maximum of something else, a minimum, the difference the other way round: expf
+        for tree in (lambda: pb.exp(x - pb.max(y, axis=axis)), lambda: pb.exp(x - pb.min(x, axis=axis)),
+                     lambda: pb.exp(pb.max(x, axis=axis) - x), lambda: pb.exp(x + pb.max(x, axis=axis))):
+            src = plan_of(pb, lambda: out.__setitem__(slice(None), tree())).spec.source
+            assert "expf(" in src and "nh_exp_nonpos(" not in src
