@@ -14,6 +14,7 @@ wherever its two backends differ.
 """
 import ctypes
 import logging
+import os
 import struct
 
 import numpy as np
@@ -1007,7 +1008,8 @@ class NervanaHIPBase(object):
         self._stats["launches"] += 1
 
     def _run_slow(self, trees):
-        if len(trees) == 1 and not self._originals and self._stage_transposed_views(trees[0]):
+        if len(trees) == 1 and not self._originals and (self._stage_transposed_views(trees[0]) or
+                                                        self._stage_folded_reduction(trees[0])):
             return
         try:
             prog = Program()
@@ -1147,6 +1149,88 @@ class NervanaHIPBase(object):
                 return dense.get(id(node), node)
 
             self._run([self._api.OpTreeNode({"op": "assign"}, out, swap(expr))])
+        finally:
+            for t in temps:
+                self._temp_release(t)
+        return True
+
+    # A lone sum / max / min along the rows of a dense matrix with few, very long rows: one
+    # workgroup per row leaves most compute units idle.  Memory is row-major, so (R, C) is also
+    # (R*q, C/q): the same reduction over that shape, then a second, tiny one over the q partial
+    # results of every row ((64,1048576) fp32: 77 -> 45 us; (16,1605632) fp16: 16 -> 9 us).
+    # (The mirror image -- a tall matrix a few columns wide, reduced down the columns as
+    # (R/q, C*q) -- was measured too and gains nothing over the split column family.)
+    FOLD_REDUCTIONS = os.environ.get("NEON_HIP_FOLD_REDUCTIONS", "1") != "0"
+
+    def _stage_folded_reduction(self, tree):
+        """Run ``out[:] = f(red(g(x, ...), axis=1))`` -- ONE sum / max / min whose
+        operand is an elementwise expression of dense full-shape tensors and
+        numbers -- through a reshaped view when the shape calls for it (see
+        above).  Returns True when the tree was run that way."""
+        if not self.FOLD_REDUCTIONS:
+            return False
+        cls = self._api.OpTreeNode
+        out, expr = tree[1], tree[2]
+        if not isinstance(expr, cls) or out.rounding or len(out.shape) != 2 or out.shape[1] != 1:
+            return False       # (a result of the full shape is swept again anyway: the cooperative rows do that)
+        reds = []
+
+        def find(node, inside):
+            """False if the tree holds anything but one reduction with a plain operand"""
+            if not isinstance(node, cls):
+                if inside and isinstance(node, HIPTensorBase):
+                    leaves.append(node)
+                return True
+            op = node[0]["op"]
+            if op in REDUCE:
+                if inside or op not in ("sum", "max", "min") or node[0].get("axis") != 1:
+                    return False
+                reds.append(node)
+                return find(node[1], True)
+            if op in ("dot", "transpose", "rand", "onehot"):
+                return False
+            return find(node[1], inside) and find(node[2], inside)
+
+        leaves = []
+        if not find(expr, False) or len(reds) != 1 or not leaves:
+            return False
+        red = reds[0]
+        axis = red[0]["axis"]
+        R, C = leaves[0].shape if len(leaves[0].shape) == 2 else (0, 0)
+        for t in leaves:
+            if t.shape != (R, C) or not t.is_contiguous or t.take_array or len(t.shape) != 2:
+                return False
+        q = 1
+        if axis == 1 and R * 3 <= self.cu_count and C >= (1 << 17):
+            # split every row into q pieces of at least 16384 elements, enough of them to
+            # give every compute unit a few rows
+            while C % (2 * q) == 0 and C // (2 * q) >= (1 << 14) and R * q < 4 * self.cu_count:
+                q *= 2
+        if q < 2:
+            return False
+        shape1, part_shape, view_shape = (R * q, C // q), (R * q, 1), (R, q)
+        temps = []
+        try:
+            views = dict((id(t), t.reshape(shape1)) for t in leaves)
+
+            def reshaped(node):
+                if isinstance(node, cls):
+                    return cls(dict(node[0], shape=shape1), reshaped(node[1]), reshaped(node[2]))
+                return views.get(id(node), node)
+
+            part = self._temp(part_shape, np.float32, temps)
+            first = cls(dict(red[0], shape=part_shape), reshaped(red[1]), None)
+            self._run([cls({"op": "assign"}, part, first)])
+            second = cls(dict(red[0]), part.reshape(view_shape), None)
+
+            def swap(node):
+                if node is red:
+                    return second
+                if isinstance(node, cls):
+                    return cls(node[0], swap(node[1]), swap(node[2]))
+                return node
+
+            self._run([cls({"op": "assign"}, out, swap(expr))])
         finally:
             for t in temps:
                 self._temp_release(t)

@@ -963,3 +963,41 @@ def test_exponential_of_values_below_their_maximum_is_good_to_the_last_place(hip
     ok = ~np.isnan(wy)
     np.testing.assert_allclose(gy[ok], wy[ok], rtol=2.5e-7, atol=1e-38)
     assert gy[3, 5] == 0.0
+
+
+@pytest.mark.parametrize("shape,axis,dtype", [((40, 262144), 1, np.float32), ((24, 393216), 1, np.float16),
+                                               ((3, 1 << 21), 1, np.float32)])
+def test_lone_reductions_over_few_very_long_rows(hip, shape, axis, dtype):
+    """few very long rows reduced along the rows: run over a reshaped view
+    plus a small second reduction (two launches); sums against float64,
+    max / min exactly"""
+    rs = np.random.RandomState(shape[0] % 13)
+    xh = rs.standard_normal(shape).astype(np.float32).astype(dtype)
+    x = hip.array(xh, dtype=dtype)
+    x64 = xh.astype(np.float64)
+    line = (shape[0], 1) if axis == 1 else (1, shape[1])
+    out = hip.empty(line)
+
+    def launches(issue):
+        before = hip.plan_stats["launches"]
+        issue()
+        return hip.plan_stats["launches"] - before
+
+    n = shape[axis]
+    assert launches(lambda: out.__setitem__(slice(None), hip.sum(x, axis=axis))) == 2
+    np.testing.assert_allclose(out.get(), x64.sum(axis=axis, keepdims=True), rtol=1e-5, atol=1e-5 * np.sqrt(n))
+    assert launches(lambda: out.__setitem__(slice(None), hip.max(x, axis=axis))) == 2
+    assert np.array_equal(out.get(), xh.max(axis=axis, keepdims=True).astype(np.float32))
+    assert launches(lambda: out.__setitem__(slice(None), hip.min(x, axis=axis))) == 2
+    assert np.array_equal(out.get(), xh.min(axis=axis, keepdims=True).astype(np.float32))
+    # an expression below the reduction and arithmetic above it (a mean of squares, shifted)
+    assert launches(lambda: out.__setitem__(slice(None), hip.sum(x * x + 1.0, axis=axis) * (1.0 / n) - 1.0)) == 2
+    np.testing.assert_allclose(out.get(), (x64 * x64).mean(axis=axis, keepdims=True), rtol=2e-5, atol=1e-6)
+    # again: replayed from the recording
+    out.fill(0)
+    assert launches(lambda: out.__setitem__(slice(None), hip.sum(x * x + 1.0, axis=axis) * (1.0 / n) - 1.0)) == 2
+    np.testing.assert_allclose(out.get(), (x64 * x64).mean(axis=axis, keepdims=True), rtol=2e-5, atol=1e-6)
+    # an index reduction keeps its own kernel
+    idx = hip.empty(line, dtype=np.int32)
+    assert launches(lambda: idx.__setitem__(slice(None), hip.argmax(x, axis=axis))) == 1
+    assert np.array_equal(idx.get(), xh.argmax(axis=axis).reshape(line))
