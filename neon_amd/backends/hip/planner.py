@@ -70,6 +70,9 @@ class KernelCache(object):
             # device-scope release / acquire around the inter-workgroup hand-offs instead of
             # the store-wait the default build relies on (see neon_device.h)
             self.header = "#define NH_FORMAL_FENCES 1\n" + self.header
+        if os.environ.get("NEON_HIP_EXACT_LSE_TERMS", "0") != "0":
+            # the terms of a running sum of exponentials each rounded like expf (see nh_exp_term)
+            self.header = "#define NH_EXACT_LSE_TERMS 1\n" + self.header
         if cache_dir is None:
             cache_dir = os.environ.get("NEON_HIP_CACHE_DIR")
         if cache_dir is None and os.environ.get("NEON_CACHE_DIR"):

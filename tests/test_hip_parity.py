@@ -1001,3 +1001,21 @@ def test_lone_reductions_over_few_very_long_rows(hip, shape, axis, dtype):
     idx = hip.empty(line, dtype=np.int32)
     assert launches(lambda: idx.__setitem__(slice(None), hip.argmax(x, axis=axis))) == 1
     assert np.array_equal(idx.get(), xh.argmax(axis=axis).reshape(line))
+
+
+def test_sum_of_exponentials_in_one_sweep_stays_within_a_few_units_of_float64(hip):
+    """the one-sweep (max, sum of exponentials) pair adds terms computed with a
+    plain product by log2(e): each term's error is weighted by the term, so
+    the SUM stays within a few 1e-7 of float64 however many terms there are
+    -- checked where the weights are worst (every term near e^-1) and over a
+    wide spread"""
+    rs = np.random.RandomState(33)
+    for rows, lo, hi in ((65536, -1.2, -0.8), (200000, -30.0, 0.0), (40000, -87.0, 0.0)):
+        x = rs.uniform(lo, hi, (rows, 64)).astype(np.float32)
+        x[rs.randint(0, rows, 64), np.arange(64)] = 0.0                 # the maximum of every column
+        out = hip.empty((1, 64))
+        dx = hip.array(x)
+        out[:] = hip.sum(hip.exp(dx - hip.max(dx, axis=0)), axis=0)
+        want = np.exp(x.astype(np.float64)).sum(axis=0)
+        got = out.get().ravel().astype(np.float64)
+        assert np.max(np.abs(got - want) / want) < 4e-7, (rows, lo, hi)
