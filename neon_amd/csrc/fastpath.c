@@ -33,7 +33,20 @@ typedef struct {
     PyObject* keep;          /* whatever owns the memory the records point into */
 } Records;
 
+/* (both types take part in cycle collection: backend -> replayer -> launch cache -> entry ->
+ * records / temporaries -> tensors -> backend is a cycle the collector has to see through) */
+static int Records_traverse(Records* self, visitproc visit, void* arg) {
+    Py_VISIT(self->keep);
+    return 0;
+}
+
+static int Records_clear(Records* self) {
+    Py_CLEAR(self->keep);
+    return 0;
+}
+
 static void Records_dealloc(Records* self) {
+    PyObject_GC_UnTrack(self);
     PyMem_Free((void*)self->recs);
     PyMem_Free(self->raw);
     Py_XDECREF(self->keep);
@@ -100,7 +113,9 @@ static PyTypeObject RecordsType = {
     .tp_name = "neon_amd._fastpath.Records",
     .tp_basicsize = sizeof(Records),
     .tp_dealloc = (destructor)Records_dealloc,
-    .tp_flags = Py_TPFLAGS_DEFAULT,
+    .tp_flags = Py_TPFLAGS_DEFAULT | Py_TPFLAGS_HAVE_GC,
+    .tp_traverse = (traverseproc)Records_traverse,
+    .tp_clear = (inquiry)Records_clear,
     .tp_doc = "Records(addresses, numbers, keep): launch records of one statement",
     .tp_methods = Records_methods,
     .tp_members = Records_members,
@@ -187,7 +202,20 @@ typedef struct {
     long long replayed, launches;
 } Replayer;
 
+static int Replayer_traverse(Replayer* self, visitproc visit, void* arg) {
+    Py_VISIT(self->cache);
+    Py_VISIT((PyObject*)self->tensor_cls);
+    return 0;
+}
+
+static int Replayer_clear(Replayer* self) {
+    Py_CLEAR(self->cache);
+    Py_CLEAR(self->tensor_cls);
+    return 0;
+}
+
 static void Replayer_dealloc(Replayer* self) {
+    PyObject_GC_UnTrack(self);
     Py_XDECREF(self->cache);
     Py_XDECREF((PyObject*)self->tensor_cls);
     Py_TYPE(self)->tp_free((PyObject*)self);
@@ -266,7 +294,7 @@ static PyObject* Replayer_replay(Replayer* self, PyObject* const* args, Py_ssize
     {
         PyObject* key = build_key(&w);
         if (!key) goto unhandled;
-        PyObject* entry = PyDict_GetItemWithError(self->cache, key);      /* borrowed */
+        PyObject* entry = self->cache ? PyDict_GetItemWithError(self->cache, key) : NULL;      /* borrowed */
         Py_DECREF(key);
         if (!entry) goto unhandled;
         PyObject* recs = PyObject_GetAttr(entry, s_fast);
@@ -312,7 +340,9 @@ static PyTypeObject ReplayerType = {
     .tp_name = "neon_amd._fastpath.Replayer",
     .tp_basicsize = sizeof(Replayer),
     .tp_dealloc = (destructor)Replayer_dealloc,
-    .tp_flags = Py_TPFLAGS_DEFAULT,
+    .tp_flags = Py_TPFLAGS_DEFAULT | Py_TPFLAGS_HAVE_GC,
+    .tp_traverse = (traverseproc)Replayer_traverse,
+    .tp_clear = (inquiry)Replayer_clear,
     .tp_doc = "Replayer(launch_cache, tensor_class, address of nh_launch_prepared)",
     .tp_methods = Replayer_methods,
     .tp_members = Replayer_members,

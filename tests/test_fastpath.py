@@ -162,6 +162,26 @@ def test_records_keep_their_owner_alive(rig):
     assert ref() is None
 
 
+def test_cycles_through_the_replayer_are_collected(rig):
+    """backend -> replayer -> launch cache -> entry -> ... -> backend: the
+    collector has to see through the C objects"""
+    import gc
+    import weakref
+    mod, be, rp, cache, calls, verdict, t, launch = rig
+
+    class Holder(object):
+        pass
+    holder = Holder()
+    own_cache = {}
+    holder.replayer = mod.Replayer(own_cache, GeomTensor, ctypes.cast(launch, ctypes.c_void_p).value)
+    holder.records = mod.Records([0x10], [], holder)
+    own_cache["entry"] = holder
+    ref = weakref.ref(holder)
+    del holder, own_cache
+    gc.collect()
+    assert ref() is None
+
+
 def test_random_trees_have_no_key(rig):
     from neon_amd.backends.backend import OpTreeNode
     mod, be, rp, cache, calls, verdict, t, _ = rig
