@@ -112,6 +112,34 @@ def test_row_normalisation_config_in_bf16(pair):
     assert np.allclose(got.std(axis=1, keepdims=True), gamma, rtol=1e-2)
 
 
+def test_batch_norm_pair_over_long_bf16_rows(pair):
+    """rows of 19 bf16 tiles: part of an operand parked in LDS, part held in
+    registers, the rest fetched again (the forms tests/test_hip_long_rows.py
+    covers for fp16 and fp32)"""
+    cpu, hip = pair
+    shape = (130, 150528)
+    rs = np.random.RandomState(8)
+    x = _q(rs.standard_normal(shape) * 2.0 + 0.5)
+    d = _q(rs.standard_normal(shape))
+    gam = rs.uniform(0.5, 1.5, (shape[0], 1)).astype(np.float32)
+    bet = (rs.standard_normal((shape[0], 1)) * 0.1).astype(np.float32)
+    res = []
+    for be, dt in ((cpu, np.float32), (hip, bfloat16)):
+        vec = lambda: be.zeros((shape[0], 1))     # noqa: E731
+        X, D = be.array(x, dtype=dt), be.array(d, dtype=dt)
+        y, dout = be.empty(shape, dtype=dt), be.empty(shape, dtype=dt)
+        xsum, xvar, gmean, gvar, gg, gb = vec(), vec(), vec(), vec(), vec(), vec()
+        be.compound_fprop_bn(X, xsum, xvar, gmean, gvar, be.array(gam), be.array(bet), y, 1e-3, 0.9, True)
+        be.compound_bprop_bn(dout, gg, gb, D, X, xsum, xvar, be.array(gam), 1e-3)
+        res.append([t.get().astype(np.float64) for t in (y, dout, xsum, xvar, gg, gb)])
+    for k, name in enumerate(("y", "delta")):
+        assert rel_err(res[1][k], _q(res[0][k]), floor_frac=1e-3) <= TOL, name
+    for k, name in ((2, "mean"), (3, "var")):
+        assert rel_err(res[1][k], res[0][k], floor_frac=1e-3) <= 2e-5, name
+    for k, name in ((4, "grad_gamma"), (5, "grad_beta")):
+        assert np.abs(res[1][k] - res[0][k]).max() <= 2e-4 * np.abs(res[0][k]).max() + 1e-2, name
+
+
 def test_stochastic_rounding_into_bf16_is_unbiased(hip):
     x = np.full((64, 4096), 1.0 + 2.0 ** -10, np.float32)            # a quarter of the way between two 4-bit neighbours
     t = hip.empty(x.shape, dtype=bfloat16)
