@@ -412,7 +412,7 @@ class _FuseScope(object):
             if exc_type is None:
                 self.be._flush()
             else:
-                self.be._pending, self.be._pending_post = [], []
+                self.be._pending, self.be._pending_post, self.be._deferred = [], [], []
         return False
 
 
@@ -529,6 +529,7 @@ class NervanaHIPBase(object):
         self.plans = {}
         self._stats = {"hit": 0, "miss": 0, "split": 0, "launches": 0, "replayed": 0}
         self._pending = []
+        self._deferred = []           # statements of the open fusion group that have not been looked at yet
         self._pending_post = []       # postfix walks of the pending statements
         self._pending_sig = None      # what kind of group the pending statements form
         self._fusing = False
@@ -569,7 +570,7 @@ class NervanaHIPBase(object):
         if rt is None:
             return
         try:
-            self._pending, self._pending_post = [], []
+            self._pending, self._pending_post, self._deferred = [], [], []
             rt.synchronize()
             for plan in self.plans.values():
                 for p in (plan if isinstance(plan, list) else [plan]):
@@ -739,6 +740,11 @@ class NervanaHIPBase(object):
                 self._flush()
 
     def _flush(self):
+        if self._deferred:
+            self._resolve_deferred()
+        self._flush_pending()
+
+    def _flush_pending(self):
         if self._pending:
             trees, self._pending = self._pending, []
             posts, self._pending_post = self._pending_post, []
@@ -846,18 +852,57 @@ class NervanaHIPBase(object):
                 stats["replayed"] += 1
                 stats["launches"] += len(entry.launches)
                 return optree[1]
+        if self._fusing and self._replayer is not None and self._captured is None and self._recording is None:
+            # inside a fusion group: just queue.  When the group ends, ONE walk in C over all
+            # its statements yields the key of the launch cache; only a group never seen before
+            # is taken apart statement by statement (_enqueue)
+            self._deferred.append(optree)
+            return optree[1]
+        self._enqueue(optree)
+        return optree[1]
+
+    def _enqueue(self, optree):
+        """a statement joins the pending fusion group, or ends it, or runs on its own"""
         post = optree.traverse([])
         if self._fusing:
             if self._can_join(optree, post):
                 self._pending.append(optree)
                 self._pending_post.append(post)
-                return optree[1]
-            self._flush()
+                return
+            self._flush_pending()
         if self._captured is not None:
             self._captured.append([optree])
         else:
             self._run([optree], [post])
-        return optree[1]
+
+    def _resolve_deferred(self):
+        """the statements queued by ``execute`` since the fusion group began: replayed at
+        once if the very same group has run before, otherwise grouped and run the long way"""
+        trees, self._deferred = self._deferred, []
+        entry = None
+        if self._captured is None and self._recording is None and not self._originals:
+            try:
+                if not any(t[1].rounding for t in trees):
+                    key, raw = self._replayer.key_group(trees)
+                    entry = self._launch_cache.get(key)
+            except (TypeError, AttributeError, KeyError):
+                entry = None
+        if entry is not None and entry.rebind(raw) is not None:
+            entry.replay(self.rt)
+            for plan in entry.coop:
+                self._coop_pending[plan.key] = plan
+            self._stats["replayed"] += 1
+            self._stats["launches"] += len(entry.launches)
+            return
+        # (statements reach _enqueue in fusing mode whatever the mode is by now: the group
+        # was written inside begin / end)
+        fusing, self._fusing = self._fusing, True
+        try:
+            for tree in trees:
+                self._enqueue(tree)
+            self._flush_pending()
+        finally:
+            self._fusing = fusing
 
     def _replay_in_c(self, out, value):
         """True when the C replayer issued the recorded launches of ``out[:] = value``"""

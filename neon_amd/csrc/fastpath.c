@@ -284,6 +284,50 @@ static PyObject* Replayer_key(Replayer* self, PyObject* args) {
     return r;
 }
 
+/* key_group(trees) -> (key tuple, list of numbers) of a GROUP of assign trees (each a 3-tuple
+ * (op dict, target, value)): the key NervanaHIPBase._launch_key builds for the group.  Raises
+ * TypeError when a tree is not replayable. */
+static PyObject* Replayer_key_group(Replayer* self, PyObject* trees) {
+    PyObject* fast = PySequence_Fast(trees, "key_group takes a sequence of assign trees");
+    if (!fast) return NULL;
+    Walk w;
+    w.nparts = w.nraw = 0;
+    w.depth = 0;
+    w.tensor_cls = self->tensor_cls;
+    Py_ssize_t n = PySequence_Fast_GET_SIZE(fast);
+    for (Py_ssize_t k = 0; k < n; ++k) {
+        PyObject* tree = PySequence_Fast_GET_ITEM(fast, k);
+        int ok = PyTuple_Check(tree) && PyTuple_GET_SIZE(tree) == 3 &&
+                 walk_node(&w, PyTuple_GET_ITEM(tree, 0), PyTuple_GET_ITEM(tree, 1), PyTuple_GET_ITEM(tree, 2)) == 0;
+        if (ok) {
+            Py_INCREF(s_bar);
+            ok = push(&w, s_bar) == 0;
+        }
+        if (!ok) {
+            walk_release(&w);
+            Py_DECREF(fast);
+            if (!PyErr_Occurred()) PyErr_SetString(PyExc_TypeError, "not replayable");
+            return NULL;
+        }
+    }
+    Py_DECREF(fast);
+    PyObject* key = PyTuple_New(w.nparts);
+    if (!key) { walk_release(&w); return NULL; }
+    for (Py_ssize_t i = 0; i < w.nparts; ++i) PyTuple_SET_ITEM(key, i, w.parts[i]);   /* steals */
+    w.nparts = 0;
+    PyObject* nums = PyList_New(w.nraw);
+    if (!nums) { Py_DECREF(key); return NULL; }
+    for (Py_ssize_t i = 0; i < w.nraw; ++i) {
+        PyObject* f = PyFloat_FromDouble(w.raw[i]);
+        if (!f) { Py_DECREF(key); Py_DECREF(nums); return NULL; }
+        PyList_SET_ITEM(nums, i, f);
+    }
+    PyObject* r = PyTuple_Pack(2, key, nums);
+    Py_DECREF(key);
+    Py_DECREF(nums);
+    return r;
+}
+
 /* replay(out, value) -> 1: the statement's recorded launches were issued; 0: not handled here;
  * a negative number: minus the error code nh_launch_prepared returned (launches may be partly issued) */
 static PyObject* Replayer_replay(Replayer* self, PyObject* const* args, Py_ssize_t nargs) {
@@ -333,6 +377,8 @@ static PyMethodDef Replayer_methods[] = {
     {"replay", (PyCFunction)(void (*)(void))Replayer_replay, METH_FASTCALL,
      "replay(out, value) -> 1 issued, 0 not handled, < 0 minus the launch error code"},
     {"key", (PyCFunction)Replayer_key, METH_VARARGS, "key(out, value) -> (cache key, numbers)"},
+    {"key_group", (PyCFunction)Replayer_key_group, METH_O,
+     "key_group(assign trees) -> (cache key of the statement group, numbers)"},
     {NULL, NULL, 0, NULL}};
 
 static PyTypeObject ReplayerType = {

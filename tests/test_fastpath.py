@@ -82,6 +82,32 @@ def test_c_key_is_the_python_key(rig):
         assert raw == want_raw
 
 
+def test_c_group_key_is_the_python_group_key(rig):
+    from neon_amd.backends.backend import OpTreeNode
+    mod, be, rp, cache, calls, verdict, t, _ = rig
+
+    class Keyer(object):
+        tensor_cls = GeomTensor
+        _launch_key = NervanaHIPBase._launch_key
+
+    pairs = trees(be, t)
+    for out, _ in pairs:
+        out.rounding = 0
+    for group in (pairs[:1], pairs[:3], pairs[3:8], pairs):
+        assigns = [OpTreeNode({"op": "assign", "shape": out.shape}, out, value) for out, value in group]
+        want_key, want_raw = Keyer()._launch_key(assigns)
+        key, raw = rp.key_group(assigns)
+        assert key == want_key and hash(key) == hash(want_key) and raw == want_raw
+    # one statement: the key replay() looks up
+    out, value = pairs[0]
+    assert rp.key_group([OpTreeNode({"op": "assign"}, out, value)]) == rp.key(out, value)
+    with pytest.raises(TypeError):
+        rp.key_group([OpTreeNode({"op": "assign"}, out, OpTreeNode.build("rand", None, None) * value)])
+    with pytest.raises(TypeError):
+        rp.key_group([(1, 2)])
+    assert rp.key_group([]) == ((), [])
+
+
 def test_what_the_replayer_leaves_to_python(rig):
     mod, be, rp, cache, calls, verdict, t, _ = rig
     x, o = t((8, 8)), t((8, 8))
@@ -254,3 +280,48 @@ def test_replayer_steps_aside_for_groups_rounding_and_capture(hip, cpu):
     h16.rounding = 0
     h16[:] = hx * 3.0
     np.testing.assert_array_equal(h16.get(), exact)
+
+
+@pytest.mark.gpu
+def test_fusion_groups_are_keyed_by_one_walk_and_still_behave(hip):
+    rs = np.random.RandomState(12)
+    x0, y0 = rs.randn(96, 40).astype(np.float32), rs.randn(96, 40).astype(np.float32)
+    x, y = hip.array(x0), hip.array(y0)
+    a, b, s = hip.empty((96, 40)), hip.empty((96, 40)), hip.empty((1, 40))
+    # the same group again and again, with other numbers and other data in between
+    for k, scale in enumerate((2.0, 2.0, 2.0, 0.5, 0.5)):
+        if k == 2:
+            x0 = rs.randn(96, 40).astype(np.float32)
+            x.set(x0)
+        before = hip.plan_stats["launches"]
+        with hip.fused():
+            a[:] = x * scale
+            b[:] = a + y
+        assert hip.plan_stats["launches"] - before == 1
+        np.testing.assert_array_equal(a.get(), x0 * np.float32(scale))
+        np.testing.assert_array_equal(b.get(), x0 * np.float32(scale) + y0)
+    # a statement that cannot join (a reduction among elementwise assigns) splits the group
+    for _ in range(3):
+        with hip.fused():
+            a[:] = x * 3.0
+            s[:] = hip.sum(a, axis=0)
+            b[:] = a - 1.0
+        np.testing.assert_array_equal(a.get(), x0 * np.float32(3.0))
+        np.testing.assert_allclose(s.get(), (x0 * np.float32(3.0)).sum(axis=0, keepdims=True), rtol=1e-5, atol=1e-5)
+        np.testing.assert_array_equal(b.get(), x0 * np.float32(3.0) - np.float32(1.0))
+    # reading a tensor inside the group sees everything written before
+    with hip.fused():
+        a[:] = x + 7.0
+        seen = a.get()
+        b[:] = a * 2.0
+    np.testing.assert_array_equal(seen, x0 + np.float32(7.0))
+    np.testing.assert_array_equal(b.get(), (x0 + np.float32(7.0)) * np.float32(2.0))
+    # an exception inside the block drops what was queued
+    a.fill(0)
+    with pytest.raises(RuntimeError):
+        with hip.fused():
+            a[:] = x + 1.0
+            raise RuntimeError("caller's")
+    assert not a.get().any()
+    a[:] = x + 1.0
+    np.testing.assert_array_equal(a.get(), x0 + np.float32(1.0))
