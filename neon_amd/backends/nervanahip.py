@@ -839,9 +839,13 @@ class NervanaHIPBase(object):
                 return optree[1]
             parts, raw = [], []
             try:
-                self._walk_key(optree, parts.append, raw.append, self.tensor_cls)
-                parts.append("|")
-                entry = self._launch_cache.get(tuple(parts))
+                if self._replayer is not None:
+                    key, raw = self._replayer.key(optree[1], optree[2])       # (the same walk, in C)
+                else:
+                    self._walk_key(optree, parts.append, raw.append, self.tensor_cls)
+                    parts.append("|")
+                    key = tuple(parts)
+                entry = self._launch_cache.get(key)
             except (TypeError, AttributeError, KeyError):
                 entry = None
             if entry is not None and entry.rebind(raw) is not None:
