@@ -19,6 +19,16 @@ from neon_amd.backends.hip.bf16 import bfloat16  # noqa: F401  (storage dtype fo
 # backend to ITS classes instead -- see nervanahip.bind
 NervanaHIP, HIPTensor = nervanahip.bind(Backend, OpTreeNode, Tensor, Block)
 
+# this package's own API copy builds its elementwise nodes in C when the extension is there
+# (a host package's API classes are its own business)
+from neon_amd.backends import backend as _api                   # noqa: E402
+from neon_amd.backends.hip import fastpath as _fastpath         # noqa: E402
+if _fastpath.enabled():
+    try:
+        _api.use_c_node_builder(_fastpath.load())
+    except ImportError:
+        pass
+
 _atexit_registered = False
 
 

@@ -44,6 +44,22 @@ class Block(object):
 
 _NO_OPERAND, _SCALAR_SHAPE = (0, 0), (1, 1)
 
+# builder of elementwise nodes in C (neon_amd/csrc/fastpath.c), installed by
+# ``use_c_node_builder``; None: nodes are built by ``OpTreeNode.build`` alone
+_c_ew_node = None
+
+
+def use_c_node_builder(module):
+    """Let ``OpTreeNode.build`` hand elementwise nodes without keyword
+    arguments to ``module.ew_node`` (same nodes, a third of the time);
+    ``None`` switches back to Python."""
+    global _c_ew_node
+    if module is None:
+        _c_ew_node = None
+        return
+    module.configure_builder(OpTreeNode, Tensor, sorted(_EW_NOT_ASSIGN))
+    _c_ew_node = module.ew_node
+
 
 def _shape_of_operand(x):
     """2-d shape an operand contributes to shape inference, None for a type
@@ -309,6 +325,12 @@ class OpTreeNode(_LazyOperators, tuple):
         surfaces in ``execute``); reduction with ``axis`` = operand shape with
         that axis set to 1; numbers are 1x1; 1-d shapes are padded to 2-d.
         """
+        if _c_ew_node is not None and out is None and not kwargs:
+            # (the common case -- an elementwise operator between tensors, nodes and numbers --
+            # built in C; None means "not mine")
+            node = _c_ew_node(op, a, b)
+            if node is not None:
+                return node
         sa, sb = _shape_of_operand(a), _shape_of_operand(b)
         if sa is None or sb is None:
             return NotImplemented

@@ -395,8 +395,106 @@ static PyTypeObject ReplayerType = {
     .tp_new = Replayer_new,
 };
 
+/* ---- elementwise node construction for the package's own API copy ---------------------- */
+/* OpTreeNode.build(op, a, b) for an elementwise op without keyword arguments, as
+ * neon_amd/backends/backend.py does it in Python (shape = per-axis maximum of the operand
+ * shapes; numbers are 1x1, a missing operand 0x0, 1-d shapes padded to 2-d).  Anything it
+ * is not sure about -- an op outside the set, an operand of an unknown type, a shape that is
+ * not one or two integers -- is answered with None and Python takes over. */
+static PyObject *b_node_cls, *b_tensor_cls, *b_ew_ops, *s_shape, *t_scalar, *t_none;
+
+static PyObject* builder_configure(PyObject* self, PyObject* args) {
+    PyObject *node_cls, *tensor_cls, *ops;
+    if (!PyArg_ParseTuple(args, "O!O!O:configure_builder", &PyType_Type, &node_cls, &PyType_Type, &tensor_cls, &ops))
+        return NULL;
+    if (!PyType_IsSubtype((PyTypeObject*)node_cls, &PyTuple_Type)) {
+        PyErr_SetString(PyExc_TypeError, "the node class must derive from tuple");
+        return NULL;
+    }
+    PyObject* frozen = PyFrozenSet_New(ops);
+    if (!frozen) return NULL;
+    Py_INCREF(node_cls); Py_XSETREF(b_node_cls, node_cls);
+    Py_INCREF(tensor_cls); Py_XSETREF(b_tensor_cls, tensor_cls);
+    Py_XSETREF(b_ew_ops, frozen);
+    Py_RETURN_NONE;
+}
+
+/* 1 = ok (rows, cols set; *keep = the operand's own 2-tuple when it has one, borrowed),
+ * 0 = let Python decide, -1 = error */
+static int operand_shape(PyObject* x, Py_ssize_t* rows, Py_ssize_t* cols, PyObject** keep) {
+    *keep = NULL;
+    if (x == Py_None) { *rows = *cols = 0; *keep = t_none; return 1; }
+    if (PyFloat_Check(x) || PyLong_Check(x)) { *rows = *cols = 1; *keep = t_scalar; return 1; }
+    PyObject* shp;
+    if (PyObject_TypeCheck(x, (PyTypeObject*)b_node_cls)) {
+        PyObject* d = PyTuple_GET_SIZE(x) == 3 ? PyTuple_GET_ITEM(x, 0) : NULL;
+        if (!d || !PyDict_Check(d)) return 0;
+        shp = PyDict_GetItemWithError(d, s_shape);       /* borrowed */
+        if (!shp) return PyErr_Occurred() ? -1 : 0;
+        Py_INCREF(shp);
+    } else if (PyObject_TypeCheck(x, (PyTypeObject*)b_tensor_cls)) {
+        shp = PyObject_GetAttr(x, s_shape);
+        if (!shp) return -1;
+    } else {
+        return 0;
+    }
+    int ok = 0;
+    if (PyTuple_Check(shp)) {
+        Py_ssize_t n = PyTuple_GET_SIZE(shp);
+        if ((n == 1 || n == 2) && PyLong_Check(PyTuple_GET_ITEM(shp, 0)) && (n == 1 || PyLong_Check(PyTuple_GET_ITEM(shp, 1)))) {
+            *rows = PyLong_AsSsize_t(PyTuple_GET_ITEM(shp, 0));
+            *cols = n == 2 ? PyLong_AsSsize_t(PyTuple_GET_ITEM(shp, 1)) : 1;
+            ok = !((*rows == -1 || *cols == -1) && PyErr_Occurred());
+            if (!ok) PyErr_Clear();
+            /* (the tuple stays alive through its owner, the operand, for as long as we use it) */
+            if (ok && n == 2) *keep = shp;
+        }
+    }
+    Py_DECREF(shp);
+    return ok;
+}
+
+static PyObject* builder_ew_node(PyObject* self, PyObject* const* args, Py_ssize_t nargs) {
+    if (nargs != 3) { PyErr_SetString(PyExc_TypeError, "ew_node(op, a, b)"); return NULL; }
+    if (!b_node_cls) Py_RETURN_NONE;
+    int known = PySet_Contains(b_ew_ops, args[0]);
+    if (known < 0) return NULL;
+    if (!known) Py_RETURN_NONE;
+    Py_ssize_t ra, ca, rb, cb;
+    PyObject *ka, *kb;
+    int ok = operand_shape(args[1], &ra, &ca, &ka);
+    if (ok > 0) ok = operand_shape(args[2], &rb, &cb, &kb);
+    if (ok < 0) return NULL;
+    if (!ok) Py_RETURN_NONE;
+    PyObject* shape;
+    if (ra == rb && ca == cb && ka) { shape = ka; Py_INCREF(shape); }
+    else if (ra >= rb && ca >= cb && ka) { shape = ka; Py_INCREF(shape); }
+    else if (rb >= ra && cb >= ca && kb) { shape = kb; Py_INCREF(shape); }
+    else shape = Py_BuildValue("(nn)", ra > rb ? ra : rb, ca > cb ? ca : cb);
+    if (!shape) return NULL;
+    PyObject* d = PyDict_New();
+    if (!d || PyDict_SetItem(d, s_op, args[0]) < 0 || PyDict_SetItem(d, s_shape, shape) < 0) {
+        Py_XDECREF(d); Py_DECREF(shape); return NULL;
+    }
+    Py_DECREF(shape);
+    PyTypeObject* cls = (PyTypeObject*)b_node_cls;
+    PyObject* node = cls->tp_alloc(cls, 3);
+    if (!node) { Py_DECREF(d); return NULL; }
+    PyTuple_SET_ITEM(node, 0, d);
+    Py_INCREF(args[1]); PyTuple_SET_ITEM(node, 1, args[1]);
+    Py_INCREF(args[2]); PyTuple_SET_ITEM(node, 2, args[2]);
+    return node;
+}
+
+static PyMethodDef module_methods[] = {
+    {"configure_builder", builder_configure, METH_VARARGS,
+     "configure_builder(node class, tensor class, elementwise op names)"},
+    {"ew_node", (PyCFunction)(void (*)(void))builder_ew_node, METH_FASTCALL,
+     "ew_node(op, a, b) -> node, or None when Python has to build it"},
+    {NULL, NULL, 0, NULL}};
+
 static struct PyModuleDef moduledef = {
-    PyModuleDef_HEAD_INIT, "_fastpath", "C replay of repeated op-tree statements", -1, NULL, NULL, NULL, NULL, NULL};
+    PyModuleDef_HEAD_INIT, "_fastpath", "C replay of repeated op-tree statements", -1, module_methods, NULL, NULL, NULL, NULL};
 
 PyMODINIT_FUNC PyInit__fastpath(void) {
     if (PyType_Ready(&RecordsType) < 0 || PyType_Ready(&ReplayerType) < 0) return NULL;
@@ -409,7 +507,11 @@ PyMODINIT_FUNC PyInit__fastpath(void) {
     s_fast = PyUnicode_InternFromString("fast");
     s_bar = PyUnicode_InternFromString("|");
     s_assign = PyUnicode_InternFromString("assign");
-    if (!s_geom || !s_op || !s_axis || !s_idx || !s_fast || !s_bar || !s_assign) return NULL;
+    s_shape = PyUnicode_InternFromString("shape");
+    t_scalar = Py_BuildValue("(ii)", 1, 1);
+    t_none = Py_BuildValue("(ii)", 0, 0);
+    if (!s_geom || !s_op || !s_axis || !s_idx || !s_fast || !s_bar || !s_assign || !s_shape || !t_scalar || !t_none)
+        return NULL;
     Py_INCREF(&RecordsType);
     Py_INCREF(&ReplayerType);
     if (PyModule_AddObject(m, "Records", (PyObject*)&RecordsType) < 0) return NULL;

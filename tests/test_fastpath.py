@@ -325,3 +325,57 @@ def test_fusion_groups_are_keyed_by_one_walk_and_still_behave(hip):
     assert not a.get().any()
     a[:] = x + 1.0
     np.testing.assert_array_equal(a.get(), x0 + np.float32(1.0))
+
+
+def test_c_node_builder_builds_the_nodes_python_builds():
+    """every elementwise op over every kind of operand pair: same node class,
+    same op dict (same key order), same operands -- or the same refusal"""
+    import neon_amd.backends  # noqa: F401  (installs the C builder on this package's API copy)
+    from neon_amd.backends import backend as api
+    from neon_amd.backends.backend import OpCollection, OpTreeNode
+    assert api._c_ew_node is not None
+    be = PlanBackend(compile_kernels=False)
+    full, col, row, one = be.empty((5, 7)), be.empty((5, 1)), be.empty((1, 7)), be.empty((1, 1))
+    vec = ShapeTensor(be, (9,))
+    vec.shape = (9,)                                     # a 1-d shape is padded
+    cube = be.empty((5, 1))
+    cube.shape = (2, 3, 4)                               # more than two axes: left to Python
+    listy = be.empty((5, 1))
+    listy.shape = [5, 7]                                 # a list, not a tuple: left to Python
+    node = full * col
+    operands = [full, col, row, one, vec, cube, listy, node, node + 1.0, 2.5, 3, True, np.float64(0.5), None, "text", [1, 2]]
+    ops = sorted(set(OpCollection.ew_ops) - {"assign"}) + ["assign", "sum", "bogus"]
+    c_builder = api._c_ew_node
+
+    def build_both(op, a, b):
+        results = []
+        for use_c in (True, False):
+            api._c_ew_node = c_builder if use_c else None
+            try:
+                results.append(OpTreeNode.build(op, a, b) if op not in ("assign", "sum") else
+                               (c_builder(op, a, b) if use_c else None))
+            except Exception as e:                       # noqa: BLE001  (compared, not handled)
+                results.append(type(e))
+        api._c_ew_node = c_builder
+        return results
+
+    checked = 0
+    for op in ops:
+        for a in operands:
+            for b in operands:
+                got, want = build_both(op, a, b)
+                if op in ("assign", "sum", "bogus"):
+                    if op != "bogus":
+                        assert got is None               # never the C builder's business
+                    else:
+                        assert got is want               # the same refusal, whichever it is
+                    continue
+                if isinstance(want, tuple):
+                    assert type(got) is type(want) is OpTreeNode, (op, a, b)
+                    assert got[0] == want[0] and list(got[0]) == list(want[0]), (op, a, b, got[0], want[0])
+                    assert type(got[0]["shape"]) is tuple
+                    assert got[1] is a and got[2] is b
+                    checked += 1
+                else:
+                    assert got is want, (op, a, b, got, want)
+    assert checked > 2000
