@@ -578,8 +578,6 @@ def _plan_col(prog, cu_count, coop=True):
         # one workgroup per compute unit (small inputs): twice the lanes, so that a SIMD has a
         # second wave to run while the first waits for its rows ((32000,256): argmax 11.0 ->
         # 10.7 us, max 8.1 -> 7.3 us); larger inputs already get several workgroups per unit
-        threads = COLSPLIT_THREADS * 2 if (per_cu == 1 and COLSPLIT_THREADS == 256) else COLSPLIT_THREADS
-        LY = threads // LX
         strips = _ceil_div(nvec, LX)
         # (the limit bounds what the last workgroup of a strip has to fold; strips
         # under 64 columns may take more chunks, as far as it takes to get two
@@ -587,7 +585,21 @@ def _plan_col(prog, cu_count, coop=True):
         cap = codegen.COLSPLIT_MAX_CHUNKS
         wide_cap = cap * max(1, 64 // (LX * V))
         cap = max(cap, min(wide_cap, _ceil_div(2 * cu_count, strips)))
-        chunks = max(1, min(cap, target // strips))
+        # Row chunks per strip: enough for one workgroup per compute unit, and beyond that no
+        # more than 32 -- every further chunk is another ticket on the strip's counter and
+        # another partial for its last workgroup to fold, which costs more than the extra
+        # workgroups bring.  Measured (max over axis 0): (30000,1000) fp16 94 chunks 27 us, 32
+        # chunks 17 us; (131072,1000) fp16 128: 69 us, 32: 60 us; (128000,1024) fp32 127: 94 us,
+        # 32: 91 us; (200704,128) fp32, four strips: 126: 22 us, 64: 18 us, 32: 23 us.
+        chunks = max(1, min(cap, max(cu_count // strips, min(32, target // strips))))
+        # few workgroups: twice the lanes each, so that a SIMD has a second wave to run while the
+        # first waits for its rows ((32000,256): max 8.1 -> 7.3 us; (802816,32) fp32 29 -> 22 us;
+        # (1000000,64) fp16 52 -> 35 us); many workgroups already overlap
+        if os.environ.get("NEON_HIP_CS_T"):
+            threads = COLSPLIT_THREADS
+        else:
+            threads = 512 if strips * chunks <= 2 * cu_count else 256
+        LY = threads // LX
         rpc = max(codegen.COLSPLIT_ROWS_IN_FLIGHT * LY, _ceil_div(R, chunks))
         rpc = _ceil_div(rpc, LY) * LY
         chunks = _ceil_div(R, rpc)
