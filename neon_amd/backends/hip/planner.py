@@ -571,7 +571,10 @@ def _plan_col(prog, cu_count, coop=True):
         # Measured: (200704,128) fp32 23 -> 21 us, fp16 26 -> 18 us, (32000,256)
         # fp32 10.1 -> 9.3 us; (200704,256) fp32 already has 512 workgroups with
         # 16 lanes and loses with 8 (36 us against 44 us).
-        LX = max(lx_min, min(16, _pow2ceil(nvec)))
+        # (wide matrices: 32 column-lanes, 512-byte row pieces -- (4096,30000) fp32 97 -> 90 us,
+        # (32000,2048) 47 -> 43 us, (30000,4096) fp16 46 -> 41 us, (4096,131072) fp16 183 -> 166 us;
+        # 64 lanes gain nothing more)
+        LX = max(lx_min, min(32 if nvec >= 256 else 16, _pow2ceil(nvec)))
         if LX == 16 and (per_cu == 1 or
                          _ceil_div(nvec, LX) * codegen.COLSPLIT_MAX_CHUNKS < min(target, 2 * cu_count)):
             LX = max(lx_min, 8)
