@@ -355,6 +355,13 @@ def _plan_ew(prog, cu_count):
         # with four rows per lane, 334 us with one -- as for the flat kernels,
         # more loads in flight per lane only add read/write turnarounds)
         UR = 1 if _streams(prog) else max(1, min(4, R // (LY * 8)))
+        if UR == 1 and R >= LY * 16:
+            # two rows per lane where a workgroup fetches a piece of a row vector for every
+            # row tile it handles (x * row over (4096,30000): 190 -> 173 us), and for very many
+            # short rows ((131072,1000) bias add: 195 -> 189 us)
+            row_vectors = any(t.read and t.shape[0] == 1 and t.shape[1] > 1 for t in prog.tensors)
+            if row_vectors or (nvec <= 256 and R > 65535 * LY):
+                UR = 2
     # one pass over far more data than the caches hold: streaming accesses
     stream = _streams(prog)
     tail = (C % V) != 0
