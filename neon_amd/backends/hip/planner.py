@@ -403,7 +403,11 @@ def _plan_row(prog, cu_count, coop=True):
     words = _words_per_tile(prog, V, 1)
     options = []
     if nvec <= 64 * 8:
-        options.append((max(1, min(64, _pow2ceil(_ceil_div(nvec, 4)))), 256))
+        # four tiles per lane, but a row's lanes together fetch at least
+        # one 128-byte line per load: with fewer, every load of a wave
+        # touches a line per row and uses a fraction of it
+        line = max(8, 32 // V)
+        options.append((max(min(line, _pow2ceil(nvec)), min(64, _pow2ceil(_ceil_div(nvec, 4)))), 256))
     options += [(256, 256), (512, 512), (1024, 1024)]
     LX, T, NCH = 1024, 1024, 0          # fallback: stream the row on every sweep
     for lx, t in options:
