@@ -778,7 +778,8 @@ class _RedGen(_Gen):
 BATCH_FENCE_TILES = int(os.environ.get("NEON_HIP_BATCH_FENCE", "16"))
 
 
-def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=False, park_bytes=0):
+def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=False, park_bytes=0,
+            max_vals=0):
     """Axis-1 reductions.  A team of LX lanes (a power of two up to 64, or the
     whole workgroup) owns one row; the workgroup holds LY rows.  A lane visits
     column tiles tx, tx+LX, ...; with ``NCH`` > 0 that loop has a fixed trip
@@ -798,6 +799,10 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
     neighbour's, no barrier needed --, holds the next ones in whatever registers
     are left, and later sweeps take both back instead of going to memory; only
     tiles beyond that are fetched again.
+
+    ``max_vals`` (with ``NCH`` > 0): how many expensive elementwise results
+    that two sweeps need may be kept in float32 registers of their own, NCH*V
+    words each (softmax over 16-bit rows: exp(x - max) once per element).
 
     ``chunks`` > 1 (family ``rowcoop``; whole-workgroup rows with ``NCH`` > 0
     only): few, very long rows.  grid = (rows, chunks); workgroup (r, q) owns
@@ -1083,7 +1088,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
 
     # expensive values that later sweeps need again take over the registers of
     # a resident float32 operand nothing else reads afterwards
-    over, vals = {}, {}
+    over, vals, own = {}, {}, set()
     if resident:
         stages = [[n.args[0] for n in per_level.get(s, [])] for s in range(nsweeps)]
         stages = [t for t in stages if t]
@@ -1094,6 +1099,9 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
             return varies_in_loop(leaf) and DTYPE_CODE[prog.tensors[leaf.slot].dtype] == "f4"
 
         over = dict((n.nid, leaf) for n, leaf in _overwriting_values(prog, stages, one_word_per_element))
+        if max_vals:
+            by_nid = dict((n.nid, n) for n in prog.nodes)
+            own = set(n.nid for n in _kept_values(prog, stages, max_vals, already=[by_nid[k] for k in over]))
 
     def stops():
         d = set(done)
@@ -1112,8 +1120,11 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
             g.declare_acc(n)
         # (an operand that did not get registers cannot lend them)
         fresh = [n for n in nodes if n.nid in over and n.nid not in vals and over[n.nid].nid not in transient]
+        fresh_own = [n for n in nodes if n.nid in own and n.nid not in vals and n.nid not in over]
+        for n in fresh_own:
+            L("float val%d[%d][%d];" % (n.nid, NCH, V))
 
-        def reduce_body(tiles, nodes=nodes, reds=reds, fresh=fresh):
+        def reduce_body(tiles, nodes=nodes, reds=reds, fresh=fresh, fresh_own=fresh_own):
             L.open("if (ok)")
             # plain sums of a packed fp16 operand: two elements per instruction, straight
             # from the tile (a partial last tile is zero-filled, so it needs no guard)
@@ -1122,7 +1133,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
             for n in pairwise:
                 L("acc%d = %s.sum_into(acc%d);" % (n.nid, tiles[n.args[0].nid], n.nid))
             reds = [n for n in reds if n not in pairwise]
-            if not reds and not fresh:
+            if not reds and not fresh and not fresh_own:
                 L.close()
                 return
             if V > 1:
@@ -1136,6 +1147,8 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
                 g.accumulate(n, ref(n.args[0]), "c + j", ref)
             for n in fresh:
                 L("keep%d[k].put(j, t%d);" % (over[n.nid].nid, n.nid))
+            for n in fresh_own:
+                L("val%d[k][j] = t%d;" % (n.nid, n.nid))
             if tail:
                 L.close()
             L.close()
@@ -1144,6 +1157,8 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
         sweep(leaves, reduce_body)
         for n in fresh:
             vals[n.nid] = "keep%d[k].get(j)" % over[n.nid].nid
+        for n in fresh_own:
+            vals[n.nid] = "val%d[k][j]" % n.nid
         for n in reds:
             op = _RED_OP[n.op]
             ty_ = "nh_pair" if n.is_index else "float"
@@ -1261,7 +1276,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
     L.close()
     return _finish("rowcoop" if coop else "row", g, head, fmt, T, 0,
                    dict(V=V, LX=LX, LY=LY, NCH=NCH, stream=bool(stream), passing=len(transient),
-                        over=len(vals), chunks=chunks, NRED=len(all_reds), tail=bool(tail),
+                        over=len([k for k in vals if k in over]), kept=len([k for k in vals if k in own]), chunks=chunks, NRED=len(all_reds), tail=bool(tail),
                         parked=sum(park.values()), held=sum(hold.values())))
 
 

@@ -395,6 +395,9 @@ ROWCOOP_MAX_TILES = int(os.environ.get('NEON_HIP_ROWCOOP_TILES', '64'))
 ROW_SPLIT_MAX_TILES = 32        # tiles of 1024 lanes per row that the unrolled split-residence form takes
 
 
+ROW_KEPT_VALUES = os.environ.get("NEON_HIP_ROW_VALS", "1") != "0"
+
+
 def _plan_row(prog, cu_count, coop=True):
     R, C = prog.domain
     V = _vector_width(prog, tail_ok=True)
@@ -462,7 +465,14 @@ def _plan_row(prog, cu_count, coop=True):
     LY = T // LX
     gx = _ceil_div(R, LY)
     park = ROW_PARK_BYTES if (keep_words and LY == 1) else 0
-    spec = codegen.gen_row(prog, V, LX, LY, NCH, _streams(prog), keep_words=keep_words, tail=tail, park_bytes=park)
+    # registers left over next to a fully resident row may hold expensive
+    # values that a later sweep needs again
+    max_vals = 0
+    if NCH and keep_words is None and sweeps >= 2 and ROW_KEPT_VALUES:
+        budget = 64 if T == 1024 else 96
+        max_vals = min(2, max(0, (budget - NCH * words) // (NCH * V)))
+    spec = codegen.gen_row(prog, V, LX, LY, NCH, _streams(prog), keep_words=keep_words, tail=tail, park_bytes=park,
+                           max_vals=max_vals)
     return Choice(spec, (gx, 1, 1))
 
 

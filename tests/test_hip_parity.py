@@ -787,6 +787,39 @@ def test_narrow_elements_with_short_rows(pair, shape, dtype):
         assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("shape", [(300, 1000), (40, 16384), (2000, 64), (77, 1003), (5, 40000)])
+def test_expensive_values_of_16bit_rows_are_kept_between_sweeps(pair, shape, dtype):
+    """softmax and friends over rows of 16-bit elements: the exponentials of the
+    summing sweep are kept in float32 registers for the sweep that stores --
+    same arithmetic as the oracle's on the widened values"""
+    from neon_amd.backends import bfloat16
+    cpu, hip = pair
+    rs = np.random.RandomState(shape[1] % 1000)
+    x32 = (rs.standard_normal(shape) * 3).astype(np.float32)
+    if dtype == "f16":
+        x16, store = x32.astype(np.float16), np.float16
+        x32 = x16.astype(np.float32)
+    else:
+        store = bfloat16
+        x32 = (x32.view(np.uint32) & np.uint32(0xFFFF0000)).view(np.float32)
+        x16 = x32
+    trees = [lambda be, t: be.exp(t - be.max(t, axis=1)) / be.sum(be.exp(t - be.max(t, axis=1)), axis=1),
+             lambda be, t: be.sig(t) / be.sum(be.sig(t), axis=1),
+             lambda be, t: be.exp(t - be.max(t, axis=1)) / be.sum(be.exp(t - be.max(t, axis=1)), axis=1)
+             + be.tanh(t) * be.max(be.tanh(t), axis=1)]
+    for k, f in enumerate(trees):
+        want = call_func(f, cpu, [x32])
+        th = hip.array(x16, dtype=store)
+        out = hip.empty(shape)
+        out[:] = f(hip, th)
+        assert_close(out.get(), want, rtol=RTOL32, atol=1e-7, what="tree %d" % k)
+        narrow = hip.empty(shape, dtype=store)
+        narrow[:] = f(hip, th)
+        assert_close(narrow.get().astype(np.float32), want, rtol=1e-3 if dtype == "f16" else 8e-3, atol=1e-7,
+                     what="tree %d, 16-bit result" % k)
+
+
 # ---- several reductions of one operand in one launch -----------------------------------------
 @pytest.mark.gpu
 def test_argmax_and_max_of_one_operand_fuse_into_one_launch(pair):
@@ -963,6 +996,30 @@ def test_exponential_of_values_below_their_maximum_is_good_to_the_last_place(hip
     ok = ~np.isnan(wy)
     np.testing.assert_allclose(gy[ok], wy[ok], rtol=2.5e-7, atol=1e-38)
     assert gy[3, 5] == 0.0
+
+
+def test_logistic_function_is_good_to_a_few_units_on_both_tails(hip):
+    """sig / sig2 are computed from e^-|x| with a Newton-refined reciprocal
+    instead of expf and a division: against float64 over the range that
+    yields normal numbers, at the edges (0, -0, +-inf, NaN, huge) and on the
+    far negative tail, where the true result is below the normal range"""
+    rs = np.random.RandomState(33)
+    x = np.concatenate([rs.uniform(-87, 87, 200000), rs.normal(0, 2, 200000), np.logspace(-30, 1.9, 20000),
+                        -np.logspace(-30, 1.9, 20000)]).astype(np.float32).reshape(-1, 1000)
+    out = hip.empty(x.shape)
+    for name, base in (("sig", np.e), ("sig2", 2.0)):
+        out[:] = getattr(hip, name)(hip.array(x))
+        want = 1.0 / (1.0 + np.power(base, -x.astype(np.float64)))
+        got = out.get().astype(np.float64)
+        assert np.max(np.abs(got - want) / want) < 4e-7, name               # three units in the last place
+    edge = np.array([[0.0, -0.0, np.inf, -np.inf, np.nan, 3e38, -3e38, 100.0, -100.0, -95.0, 17.0, -17.0]], np.float32)
+    oe = hip.empty(edge.shape)
+    oe[:] = hip.sig(hip.array(edge))
+    g = oe.get()[0]
+    assert g[0] == 0.5 and g[1] == 0.5 and g[2] == 1.0 and g[3] == 0.0 and np.isnan(g[4])
+    assert g[5] == 1.0 and g[6] == 0.0 and g[7] == 1.0
+    assert 0.0 <= g[8] <= 4e-44 and 0.0 <= g[9] <= 6e-42                     # true values are denormal
+    np.testing.assert_allclose(g[10:], 1.0 / (1.0 + np.exp(-edge[0, 10:].astype(np.float64))), rtol=4e-7)
 
 
 @pytest.mark.parametrize("shape,axis,dtype", [((40, 262144), 1, np.float32), ((24, 393216), 1, np.float16),

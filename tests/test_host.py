@@ -8,6 +8,7 @@ import re
 import numpy as np
 import pytest
 
+from neon_amd.backends import bfloat16
 from neon_amd.backends.backend import Backend, Block, OpCollection, OpTreeNode
 from neon_amd.backends.hip import codegen, planner, prebuild
 from neon_amd.backends.hip import runtime as hiprt
@@ -448,6 +449,16 @@ def test_row_softmax_reuses_registers_when_the_row_is_resident(pb):
     spec = plan_of(pb, lambda: out.__setitem__(slice(None), softmax(x))).spec
     assert spec.family == "row" and spec.params["NCH"] > 0 and spec.params["over"] == 1
     assert spec.source.count("nh_exp_nonpos(") == 1 and "expf(" not in spec.source
+    # 16-bit rows leave registers free: the exponentials get float32 registers of their own
+    for dt in (np.float16, bfloat16):
+        xh, outh = pb.empty((4096, 1000), dt), pb.empty((4096, 1000), dt)
+        spec = plan_of(pb, lambda: outh.__setitem__(slice(None), softmax(xh))).spec
+        assert spec.params["over"] == 0 and spec.params["kept"] == 1
+        assert spec.source.count("nh_exp_nonpos(") == 1 and "float val" in spec.source
+    # ... unless the row itself fills them ((64, 131072) fp16: 16 tiles of 1024 lanes)
+    xh, outh = pb.empty((512, 131072), np.float16), pb.empty((512, 131072), np.float16)
+    spec = plan_of(pb, lambda: outh.__setitem__(slice(None), softmax(xh))).spec
+    assert spec.params["NCH"] == 16 and spec.params["kept"] == 0 and spec.source.count("nh_exp_nonpos(") == 2
     # few rows too long for one workgroup's registers are spread over several
     # workgroups and stay resident
     xl, outl = pb.empty((16, 1 << 20)), pb.empty((16, 1 << 20))
