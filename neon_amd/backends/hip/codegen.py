@@ -776,6 +776,8 @@ class _RedGen(_Gen):
 # family: row  (axis 1)
 # =====================================================================================
 BATCH_FENCE_TILES = int(os.environ.get("NEON_HIP_BATCH_FENCE", "16"))
+# rows of more tiles than this: the tiles that are streamed in every sweep run as a loop, not unrolled
+ROLLED_TAIL_FROM = int(os.environ.get("NEON_HIP_ROLLED_TAIL", "32"))
 
 
 def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=False, park_bytes=0,
@@ -966,45 +968,59 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
                 L.close()
                 return
             # kept tiles come from registers, the others SU tiles at a time
-            L("#pragma unroll")
-            L.open("for (int kb = 0; kb < %d; kb += %d)" % (NCH, SU))
-            for n in passing:
-                L("%s %s[%d];" % (g.tile_type(n, V), g.tile_name(n, "_s"), SU))
-                tiles[n.nid] = "%s[u]" % g.tile_name(n, "_s")
-            L("#pragma unroll")
-            L.open("for (int u = 0; u < %d; ++u)" % SU)
-            L("const int k = kb + u;")
-            chunk_position("k")         # k beyond the row: c >= C, so ok is false
-            for n in passing:
-                name = "%s[u]" % g.tile_name(n, "_s")
-                pk, hk = park.get(n.nid, 0), hold.get(n.nid, 0)
-                # (k is a compile-time number once the loops are unrolled)
-                if n.nid in parked:
-                    L("if (k < %d) %s = park%d[k][threadIdx.x];" % (pk, name, n.nid))
-                    if hk:
-                        L("else if (k < %d) %s = hold%d[k - %d];" % (pk + hk, name, n.nid, pk))
-                    L("else { %s }" % tile_load(name, n))
-                else:
-                    L(tile_load(name, n))
-            L.close()
-            L("#pragma unroll")
-            L.open("for (int u = 0; u < %d; ++u)" % SU)
-            L("const int k = kb + u;")
-            chunk_position("k")
-            # (after the batch's loads have all been issued: a store into LDS waits for its tile)
-            for n in passing:
-                if n.nid not in parked and n.nid in park:
-                    name, pk, hk = "%s[u]" % g.tile_name(n, "_s"), park[n.nid], hold.get(n.nid, 0)
-                    L("if (k < %d) park%d[k][threadIdx.x] = %s;" % (pk, n.nid, name))
-                    if hk:
-                        L("else if (k < %d) hold%d[k - %d] = %s;" % (pk + hk, n.nid, pk, name))
-            emit_body(tiles)
-            L.close()
-            if NCH > BATCH_FENCE_TILES:
-                # long rows: without this the scheduler starts the loads of every batch of
-                # the unrolled loop at once and spills what they bring
-                L("__builtin_amdgcn_sched_barrier(0);")
-            L.close()
+            def batches(lo, hi, unrolled):
+                """tiles lo ... hi-1, SU at a time; ``unrolled``: k is a compile-time number
+                (needed to address registers and LDS slots by tile)"""
+                L("#pragma unroll" if unrolled else "#pragma unroll 1")
+                L.open("for (int kb = %d; kb < %d; kb += %d)" % (lo, hi, SU))
+                for n in passing:
+                    L("%s %s[%d];" % (g.tile_type(n, V), g.tile_name(n, "_s"), SU))
+                    tiles[n.nid] = "%s[u]" % g.tile_name(n, "_s")
+                L("#pragma unroll")
+                L.open("for (int u = 0; u < %d; ++u)" % SU)
+                L("const int k = kb + u;")
+                chunk_position("k")         # k beyond the row: c >= C, so ok is false
+                for n in passing:
+                    name = "%s[u]" % g.tile_name(n, "_s")
+                    pk, hk = park.get(n.nid, 0), hold.get(n.nid, 0)
+                    if n.nid in parked and unrolled:
+                        L("if (k < %d) %s = park%d[k][threadIdx.x];" % (pk, name, n.nid))
+                        if hk:
+                            L("else if (k < %d) %s = hold%d[k - %d];" % (pk + hk, name, n.nid, pk))
+                        L("else { %s }" % tile_load(name, n))
+                    else:
+                        L(tile_load(name, n))
+                L.close()
+                L("#pragma unroll")
+                L.open("for (int u = 0; u < %d; ++u)" % SU)
+                L("const int k = kb + u;")
+                chunk_position("k")
+                # (after the batch's loads have all been issued: a store into LDS waits for its tile)
+                for n in passing:
+                    if n.nid not in parked and n.nid in park and unrolled:
+                        name, pk, hk = "%s[u]" % g.tile_name(n, "_s"), park[n.nid], hold.get(n.nid, 0)
+                        L("if (k < %d) park%d[k][threadIdx.x] = %s;" % (pk, n.nid, name))
+                        if hk:
+                            L("else if (k < %d) hold%d[k - %d] = %s;" % (pk + hk, n.nid, pk, name))
+                emit_body(tiles)
+                L.close()
+                if NCH > BATCH_FENCE_TILES and unrolled:
+                    # long rows: without this the scheduler starts the loads of every batch of
+                    # the unrolled loop at once and spills what they bring
+                    L("__builtin_amdgcn_sched_barrier(0);")
+                L.close()
+
+            # Tiles beyond what LDS and registers hold are only ever streamed: where nothing
+            # else is addressed by tile number they run as a loop proper (64 tiles unrolled
+            # three times over made a kernel that spilled 224 registers).
+            split_at = NCH
+            if len(passing) == len(moving) and NCH > ROLLED_TAIL_FROM and not max_vals:
+                kept_tiles = max(park.get(n.nid, 0) + hold.get(n.nid, 0) for n in passing)
+                split_at = min(NCH, -(-kept_tiles // SU) * SU)
+            if split_at:
+                batches(0, split_at, True)
+            if split_at < NCH:
+                batches(split_at, NCH, False)
             parked.update(n.nid for n in passing if n.nid in park)
             return
         L.open("for (int kb = 0; kb < nch; kb += %d)" % SU)
@@ -1371,7 +1387,10 @@ def _emit_col_fold(g, L, n, LX, LY, T, V, src, dst_decl=True):
     # walking the groups in the outer loop lets them come in as one LDS read
     L("#pragma unroll")
     L("for (int j = 0; j < %d; ++j) %s[j] = %s[0][tx * %d + j];" % (V, src, buf, V))
-    L("#pragma unroll")
+    # (at most 32 LDS reads in flight: unrolled as a whole, the 15 x 8 reads of a 1024-lane
+    # workgroup with 8 values per lane were all issued ahead of the first addition and took
+    # the kernel from 56 to over 200 registers -- spilled, three times slower)
+    L("#pragma unroll %d" % max(1, 32 // V) if (WY - 1) * V > 32 else "#pragma unroll")
     L.open("for (int y = 1; y < %d; ++y)" % WY)
     L("#pragma unroll")
     L("for (int j = 0; j < %d; ++j) %s[j] = %s::f(%s[j], %s[y][tx * %d + j]);" % (V, src, op, src, buf, V))

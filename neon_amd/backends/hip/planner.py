@@ -391,8 +391,8 @@ def limit_lds(bytes_per_workgroup):
 
 
 ROW_SPLIT_WORDS = int(os.environ.get("NEON_HIP_SPLIT_WORDS", "64"))
-ROWCOOP_MAX_TILES = int(os.environ.get('NEON_HIP_ROWCOOP_TILES', '64'))
-ROW_SPLIT_MAX_TILES = 32        # tiles of 1024 lanes per row that the unrolled split-residence form takes
+ROWCOOP_MAX_TILES = int(os.environ.get('NEON_HIP_ROWCOOP_TILES', str(1 << 20)))
+ROW_SPLIT_MAX_TILES = int(os.environ.get('NEON_HIP_ROW_SPLIT_TILES', str(1 << 20)))   # tiles of 1024 lanes per row that the split-residence form takes
 
 
 ROW_KEPT_VALUES = os.environ.get("NEON_HIP_ROW_VALS", "1") != "0"
@@ -491,6 +491,10 @@ COLCOOP = os.environ.get("NEON_HIP_COLCOOP", "1") != "0"       # 0: axis-0 trees
 # stream at full occupancy.  Softmax, measured: (32000,256) 28 us either way; (64000,256) 60 us
 # cooperative, 44 us in two kernels; (6000,2304) 54 against 40 us.
 COLCOOP_MAX_BYTES = int(os.environ.get("NEON_HIP_COLCOOP_MAX_MB", "48")) << 20
+# ... and below this one its exchanges (some 8 us each, whatever the size) cost more than the extra pass
+# over a small matrix.  Softmax, cooperative / staged: (8192,1024) fp16, 16 MB: 26 / 20 us; (4096,1000)
+# fp32, 16 MB: 18.3 / 16.6; (3000,2000) fp32, 24 MB: 20.5 / 22.0; (16384,512) fp32, 32 MB: 24.3 / 26.4.
+COLCOOP_MIN_BYTES = int(os.environ.get("NEON_HIP_COLCOOP_MIN_MB", "20")) << 20
 ONLINE_LSE_IN_ONE_WORKGROUP = os.environ.get("NEON_HIP_ONLINE_LSE_COL", "0") != "0"
 
 
@@ -514,24 +518,53 @@ def _plan_col(prog, cu_count, coop=True):
     lx_pref = max(lx_min, min(64, _pow2floor(max(1, nvec // 32))))
     lx_pref = min(lx_pref, _pow2ceil(nvec))
     lx_min = min(lx_min, lx_pref)
+    def lanes_for(lx):
+        """workgroup size, row-lanes and rows per lane for strips of ``lx``
+        column-lanes, or None where the rows do not fit in registers"""
+        strips = _ceil_div(nvec, lx)
+        # many strips: small workgroups, several per compute unit; few: spend more lanes on
+        # each so that the rows-per-lane count drops and a unit has waves to switch between
+        # (tiny inputs: joining 16 waves costs more than a second row per lane -- softmax
+        # over (1000,128): 1024 lanes 5.3 us, 512 lanes 4.4 us)
+        if strips >= 4 * cu_count:
+            order = (256, 512, 1024)
+        elif strips >= 2 * cu_count:
+            order = (512, 1024, 256)
+        elif tiny:
+            order = (512, 1024, 256)
+        else:
+            order = (1024, 512, 256)
+        for T in order:
+            LY = T // lx
+            NR = _ceil_div(R, LY)
+            if LY >= 1 and NR <= 16 and NR * words <= _COL_BUDGET[T]:
+                return (T, LY, NR)
+        return None
+
     fit = None
     LX = lx_pref
+    if R <= 2048:
+        # rather strips of 32-byte row pieces than workgroups that have to wait for each other:
+        # softmax / normalisation down the columns of (2000,2048) fp16 14.6 / 14.7 us against
+        # 18.4 / 21.9 us cooperating, (1500,1024) fp32 7.6 / 7.9 against 11.0 / 13.0, (2048,8192)
+        # fp32 38 / 42 against 43 / 53 us in stages; from 3000 rows on the narrow strips lose
+        lx_min = min(lx_min, max(1, 32 // (V * isz)))
     while fit is None and LX >= lx_min:
-        strips = _ceil_div(nvec, LX)
-        # few strips: spend more lanes on each so the rows-per-lane count drops
-        # (tiny inputs: joining 16 waves costs more than a second row per lane
-        # -- softmax over (1000,128): 1024 lanes 5.3 us, 512 lanes 4.4 us)
-        for T in ((256, 512, 1024) if strips >= cu_count else (512, 1024, 256) if tiny else (1024, 512, 256)):
-            LY = T // LX
-            NR = _ceil_div(R, LY)
-            budget = _COL_BUDGET[T]
-            if NR <= 16 and NR * words <= budget:
-                fit = (T, LY, NR)
-                break
+        fit = lanes_for(LX)
         if fit is None:
             LX //= 2
     if fit is None:
         LX = lx_pref
+    # Fewer strips than compute units: narrower strips, down to 32-byte row pieces, while the
+    # rows still fit -- a strip is one workgroup, and an idle unit costs more than half-used
+    # cache lines (whose other half a neighbouring strip on the same XCD reads).  Softmax down
+    # the columns, before -> after: (512,4096) fp32 10.6 -> 6.2 us, (256,8192) 10.4 -> 6.1,
+    # (1000,1024) 10.3 -> 6.0, (1000,4096) 11.8 -> 9.5, fp16 21.3 -> 9.6, (1000,8192) fp16 23.1 -> 15.9.
+    while fit is not None and _ceil_div(nvec, LX) < cu_count and (LX // 2) * V * isz >= 32:
+        narrower = lanes_for(LX // 2)
+        if narrower is None:
+            break
+        LX, fit = LX // 2, narrower
     single_level = prog.nlevels == 1
     big = R * C >= (1 << 18)
     if fit and not (single_level and line_only and big and R >= 512):
@@ -549,7 +582,7 @@ def _plan_col(prog, cu_count, coop=True):
     # strip keep their rows in registers and exchange partials between sweeps.
     # Everything must be resident at once, so the grid stays within one
     # workgroup per compute unit.
-    if coop and COLCOOP and not (single_level and line_only) and R * C * isz <= COLCOOP_MAX_BYTES:
+    if coop and COLCOOP and not (single_level and line_only) and COLCOOP_MIN_BYTES <= R * C * isz <= COLCOOP_MAX_BYTES:
         # narrow strips keep the partials each workgroup has to gather small
         # (measured on (32000,256): 8 column-lanes 37 us, 16 lanes 43 us, 4 lanes
         # 41 us).  More strips than half the compute units leave no second
@@ -559,7 +592,10 @@ def _plan_col(prog, cu_count, coop=True):
         if strips_c <= cu_count:
             chunks = max(1, min(128, cu_count // strips_c))
             rpc0 = _ceil_div(R, chunks)
-            options = ((1024, 40), (512, 120), (256, 300))
+            # (eight values per lane: the folds' temporaries take twice the registers, and many
+            # rows per lane then spill -- (5000,5000) fp16 softmax with 27 rows per lane in 512
+            # lanes 64 us, with 53 in 256 lanes 88 us, in stages 43 us; (10000,2000) 46 / 38 us)
+            options = ((1024, 40), (512, 120), (256, 300)) if V < 8 else ((1024, 32), (512, 64))
             if os.environ.get("NEON_HIP_COOP_T"):          # tuning aid
                 options = tuple(o for o in options if o[0] == int(os.environ["NEON_HIP_COOP_T"]))
             for T, budget in options:

@@ -1338,8 +1338,10 @@ class NervanaHIPBase(object):
                 return self._api.OpTreeNode(dict(node[0], op="exp_nonpos"), left, right)
             rebuilt = self._api.OpTreeNode(node[0], left, right)
             if op in REDUCE:
-                if top:
+                if top and tuple(out.shape) == tuple(node[0]["shape"]):
                     return rebuilt
+                # (a reduction stored straight into a tensor of the operand's shape is staged
+                # like any inner one: its line of results, then the broadcast assignment)
                 k = rebuilt.key()
                 if k in memo:
                     return memo[k]

@@ -48,7 +48,9 @@ def bn_pair(be, x, d, shape, dtype):
     ((140, 140001), np.float16),      # 18 tiles, partial last tile
     ((64, 401408), np.float16),       # few rows: four workgroups per row cooperate, each parking its share
     ((120, 300000), np.float16),      # two workgroups per row, 19 tiles each: parked, held and fetched again
-    ((150, 270000), np.float16),      # 33 tiles: beyond the unrolled form, streamed in every sweep
+    ((150, 270000), np.float16),      # 33 tiles: 25 of them kept, the rest streamed by a loop proper in every sweep
+    ((140, 600000), np.float16),      # 74 tiles: the same, mostly loop
+    ((100, 540001), np.float32),      # two workgroups per row, 66 tiles each, partial last tile
 ])
 def test_batch_norm_pair_over_long_rows(pair, shape, dtype):
     cpu, hip = pair
@@ -95,14 +97,20 @@ def test_which_forms_the_planner_picks(hip):
     spec = bprop_spec((120, 300000), f16)
     assert spec.family == "rowcoop" and spec.params["NCH"] == 19 and spec.params["chunks"] == 2
     assert spec.params["parked"] == 9 and spec.params["passing"] == 2
-    p = fprop_spec((150, 270000), f16).params
-    assert p["NCH"] == 0 and p["parked"] == 0
+    spec = fprop_spec((150, 270000), f16)
+    assert (spec.params["NCH"], spec.params["parked"], spec.params["held"]) == (33, 9, 16)
+    assert "#pragma unroll 1\n    for (int kb = 28; kb < 33; kb += 4)" in spec.source
+    spec = bprop_spec((140, 600000), f16)
+    assert spec.family == "row" and spec.params["NCH"] == 74 and spec.params["passing"] == 2
+    spec = bprop_spec((100, 540001), np.float32)
+    assert spec.family == "rowcoop" and (spec.params["NCH"], spec.params["chunks"], spec.params["tail"]) == (66, 2, True)
     # more rows than compute units: the same form (one workgroup per compute unit at a time)
     p = bprop_spec((300, 100352), f16).params
     assert (p["parked"], p["held"], p["passing"]) == (9, 3, 1)
 
 
-@pytest.mark.parametrize("shape,dtype", [((130, 150528), np.float16), ((130, 100003), np.float32)])
+@pytest.mark.parametrize("shape,dtype", [((130, 150528), np.float16), ((130, 100003), np.float32),
+                                         ((135, 300001), np.float32), ((20, 1500000), np.float32)])
 def test_row_softmax_and_normalisation_over_long_rows(pair, shape, dtype):
     cpu, hip = pair
     rs = np.random.RandomState(5)

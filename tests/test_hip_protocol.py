@@ -5,6 +5,7 @@ cooperative kernel that gave up waiting."""
 import numpy as np
 import pytest
 
+from neon_amd.backends.hip import planner
 from neon_amd.backends.hip import runtime as hiprt
 from utils import assert_close
 
@@ -14,10 +15,12 @@ def _families(hip):
 
 
 @pytest.mark.gpu
-def test_soak_alternating_split_and_cooperative_launches(hip):
+def test_soak_alternating_split_and_cooperative_launches(hip, monkeypatch):
     """2100 launches, three families in turn, new random data every round
     (drawn on the device); max / argmax bit-exact against numpy, sums against
     float64; stops at the first mismatch"""
+    # (matrices this small are evaluated in stages otherwise; the protocol is what is under test)
+    monkeypatch.setattr(planner, "COLCOOP_MIN_BYTES", 0)
     xs = hip.empty((2048, 128))          # colsplit: one level, one value per column
     xc = hip.empty((20000, 64))          # colcoop: two levels over more rows than a workgroup holds
     xr = hip.empty((8, 40000))           # rowcoop: few very long rows
@@ -45,10 +48,11 @@ def test_soak_alternating_split_and_cooperative_launches(hip):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("family", ["colcoop", "rowcoop"])
-def test_a_cooperative_kernel_that_gave_up_is_reported_and_replaced(pair, family):
+def test_a_cooperative_kernel_that_gave_up_is_reported_and_replaced(pair, family, monkeypatch):
     """Nothing is made to hang: the word an aborting workgroup would leave is
     written into the plan's workspace from the host.  The next synchronisation
     raises, and from then on the tree runs without inter-workgroup waits."""
+    monkeypatch.setattr(planner, "COLCOOP_MIN_BYTES", 0)      # a small matrix, cooperating all the same
     cpu, hip = pair
     rs = np.random.RandomState(9)
     if family == "colcoop":
