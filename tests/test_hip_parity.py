@@ -545,6 +545,29 @@ def test_tall_trees_with_one_value_per_column_repeat(hip, shape):
         assert_close(ce.get().ravel(), want_ce, rtol=2e-5, atol=2e-5, what="cross-entropy, repetition %d" % rep)
 
 
+@pytest.mark.parametrize("shape,dtype", [((600000, 64), np.float16), ((540000, 48), np.float16)])
+def test_very_tall_single_strip_reductions_run_in_1024_lane_workgroups(hip, shape, dtype):
+    """one strip of columns, long row chunks, fewer workgroups than half the
+    compute units: the split column family takes 1024 lanes per workgroup;
+    max / argmax bit-exact, sums against float64, two launches on fresh data"""
+    for rep in range(2):
+        rs = np.random.RandomState(rep + 77)
+        x = rs.standard_normal(shape).astype(dtype)
+        tx = hip.array(x, dtype=dtype)
+        sm, mx, am = hip.empty((1, shape[1])), hip.empty((1, shape[1])), hip.empty((1, shape[1]), dtype=np.int32)
+        with hip.capture() as groups:
+            sm[:] = hip.sum(tx, axis=0)
+        spec = hip.time_group(groups[0], reps=1)[1].spec
+        assert spec.family == "colsplit" and spec.block == 1024
+        sm[:] = hip.sum(tx, axis=0)
+        mx[:] = hip.max(tx, axis=0)
+        am[:] = hip.argmax(tx, axis=0)
+        x64 = x.astype(np.float64)
+        assert_close(sm.get(), x64.sum(axis=0, keepdims=True), rtol=RTOL32, atol=2e-2, what="sum, repetition %d" % rep)
+        assert np.array_equal(mx.get(), x.astype(np.float32).max(axis=0, keepdims=True))
+        assert np.array_equal(am.get().ravel(), x.argmax(axis=0))
+
+
 def test_full_size_properties(hip):
     """size-independent checks at the benchmark shapes"""
     be = hip
