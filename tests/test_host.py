@@ -63,7 +63,8 @@ def test_optree_build_rules(pb):
 
 # ---- C ABI ------------------------------------------------------------------------------
 def _declared_symbols():
-    text = open(os.path.join(ROOT, "include", "neonhip.h")).read()
+    with open(os.path.join(ROOT, "include", "neonhip.h")) as f:
+        text = f.read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(nh_[a-z0-9_]+)\s*\(", text)))
 
