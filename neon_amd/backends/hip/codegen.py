@@ -775,6 +775,30 @@ class _RedGen(_Gen):
 # =====================================================================================
 # family: row  (axis 1)
 # =====================================================================================
+MERGED_MOMENTS = os.environ.get("NEON_HIP_MERGED_MOMENTS", "1") != "0"
+
+
+def _shifted_square_sum(n2, firsts):
+    """``n2`` = sum(sqr(x - a)) along the row, with ``x`` free of reductions, ``a``
+    constant along the row and ``sum(x)`` among the first sweep's reductions
+    ``firsts`` (the variance around a mean): (n2, sum(x), x, a), else None."""
+    if n2.op != "sum" or n2.is_index:
+        return None
+    e = n2.args[0]
+    if e.kind != "E" or e.op != "sqr":
+        return None
+    d = e.args[0]
+    if d.kind != "E" or d.op != "sub" or len(d.args) != 2:
+        return None
+    x, a = d.args
+    if not x.vc or x.level != 0 or a.vc or a.level > 1 or a.kind == "R" and a.is_index:
+        return None
+    for r1 in firsts:
+        if r1.op == "sum" and not r1.is_index and r1.args[0] is x:
+            return (n2, r1, x, a)
+    return None
+
+
 BATCH_FENCE_TILES = int(os.environ.get("NEON_HIP_BATCH_FENCE", "16"))
 # rows of more tiles than this: the tiles that are streamed in every sweep run as a loop, not unrolled
 ROLLED_TAIL_FROM = int(os.environ.get("NEON_HIP_ROLLED_TAIL", "32"))
@@ -899,13 +923,14 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
                     % (name, g.ld, addr, name, addr, name))
         return "if (ok) %s.%s(%s); else %s.zero();" % (name, g.ld, addr, name)
 
-    def exchange(reds):
+    def exchange(reds, riders=()):
         """join the workgroups of a row: red<id> of every reduction of this
         sweep becomes the result over the whole row, in every lane of every
-        workgroup"""
+        workgroup.  ``riders``: reductions whose per-workgroup values travel
+        along and are only fetched (g<id>), for the caller to combine"""
         exchanges[0] += 1
         L.open("if (threadIdx.x == 0)")
-        for n in reds:
+        for n in list(reds) + list(riders):
             val = ("red%d" % n.nid) if n.is_index else ("nh_pair{red%d, 0}" % n.nid)
             L("nh_part_store(&part[%d + blockIdx.y], %s);" % (red_slot[n.nid] * chunks, val))
         L.close()
@@ -925,7 +950,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
         L("if (threadIdx.x == 0) __hip_atomic_store(status, NH_COOP_ABORTED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
         L("return;")
         L.close()
-        for n in reds:
+        for n in list(reds) + list(riders):
             op = _RED_OP[n.op]
             init = ("%s::init()" % op) if n.is_index else ("nh_pair{%s::init(), 0}" % op)
             L("const nh_pair g%d = (threadIdx.x < %d) ? nh_part_load(&part[%d + threadIdx.x]) : %s;"
@@ -1124,7 +1149,80 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
         d.update(vals)
         return d
 
+    # Variance around a mean over a row that several workgroups share: instead of a second
+    # exchange for sum((x - a)^2), every workgroup takes the squares around the mean of ITS OWN
+    # part (known without waiting), and the parts combine exactly afterwards:
+    #   sum_i sum_{x in i} (x - a)^2 = sum_i [ M2_i + n_i (mean_i - a)^2 ],  M2_i = sum (x - mean_i)^2
+    # -- one exchange for both sweeps, terms that are all non-negative, and the rounding of a
+    # two-pass variance (the pairwise form of Chan, Golub and LeVeque).
+    merged = []
+    if coop and MERGED_MOMENTS and not over and not own and per_level.get(0) and per_level.get(1):
+        merged = [_shifted_square_sum(n2, per_level[0]) for n2 in per_level[1]]
+        if not all(merged):
+            merged = []
+    span = NCH * LX * V      # elements of a row that one workgroup owns
+
+    def local_second_moments():
+        """after the first sweep's fold inside the workgroup (red<sum> = this part's sum):
+        red<n2> = sum over this part of (x - this part's mean)^2"""
+        L("const long long left_ = (long long)C - (long long)blockIdx.y * %dll;" % span)
+        L("const float n_loc = (float)(left_ < %dll ? left_ : %dll);" % (span, span))
+        for n2, r1, x, a in merged:
+            L("const float mu%d = red%d / n_loc;" % (n2.nid, r1.nid))
+            vals[a.nid] = "mu%d" % n2.nid
+        seconds = [m[0] for m in merged]
+        nodes = _needed([n.args[0] for n in seconds], stops())
+        leaves = g.leaf_nodes(nodes)
+        declare_tiles(leaves)
+        for n in seconds:
+            g.declare_acc(n)
+
+        def body(tiles):
+            L.open("if (ok)")
+            if V > 1:
+                L("#pragma unroll")
+            L.open("for (int j = 0; j < %d; ++j)" % V)
+            if tail:
+                L.open("if (j < lim)")
+            ref = g.make_ref("_s", "rr", "c", V, tiles, vals)
+            g.emit_exprs(nodes, ref, stops())
+            for n in seconds:
+                g.accumulate(n, ref(n.args[0]), "c + j", ref)
+            if tail:
+                L.close()
+            L.close()
+            L.close()
+
+        sweep(leaves, body)
+        for n in seconds:
+            L("float red%d = nh_block_allreduce<nh_op_sum, %d, float>(acc%d, s_f);" % (n.nid, T // 64, n.nid))
+        for n2, r1, x, a in merged:
+            del vals[a.nid]
+
+    def combine_second_moments():
+        """after the exchange (g<id> = the parts' sums and second moments, rv<sum> final)"""
+        line_ref = g.make_ref("_s", "rr", "0", 1, dict((nid, name) for nid, name in line_tiles.items()), vals)
+        for n2, r1, x, a in merged:
+            L("float shift%d;" % n2.nid)
+            L.open("")
+            L("const int j = 0; (void)j;")
+            g.emit_exprs(_needed([a], stops()), line_ref, stops())
+            L("shift%d = %s;" % (n2.nid, line_ref(a)))
+            L.close()
+            L("float term%d = 0.0f;" % n2.nid)
+            L.open("if (threadIdx.x < %d)" % chunks)
+            L("const long long lq = (long long)C - (long long)threadIdx.x * %dll;" % span)
+            L("const float nq = (float)(lq < %dll ? lq : %dll);" % (span, span))
+            L("const float dq = g%d.v / nq - shift%d;" % (r1.nid, n2.nid))
+            L("term%d = __builtin_fmaf(nq * dq, dq, g%d.v);" % (n2.nid, n2.nid))
+            L.close()
+            L("red%d = nh_block_allreduce<nh_op_sum, %d, float>(term%d, s_f);" % (n2.nid, T // 64, n2.nid))
+            L("const float rv%d = red%d;" % (n2.nid, n2.nid))
+            done[n2.nid] = n2
+
     for s in range(nsweeps):
+        if merged and s == 1:
+            continue            # done together with the first sweep
         reds = [n for n in per_level.get(s, [])]
         if not reds:
             continue
@@ -1184,7 +1282,10 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
             else:
                 L("%s%s red%d = nh_block_allreduce<%s, %d, %s>(acc%d, %s);"
                   % (const, ty_, n.nid, op, T // 64, ty_, n.nid, "s_p" if n.is_index else "s_f"))
-        if coop:
+        if coop and merged and s == 0:
+            local_second_moments()
+            exchange(reds, riders=[m[0] for m in merged])
+        elif coop:
             exchange(reds)
         for n in reds:
             if n.is_index:
@@ -1192,6 +1293,8 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
             else:
                 L("const float rv%d = red%d;" % (n.nid, n.nid))
             done[n.nid] = n
+        if coop and merged and s == 0:
+            combine_second_moments()
 
     # outputs that have one value per row
     if line_out:

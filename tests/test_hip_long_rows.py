@@ -130,3 +130,27 @@ def test_row_softmax_and_normalisation_over_long_rows(pair, shape, dtype):
     e = np.exp(x64 - x64.max(axis=1, keepdims=True))
     assert rel_err(res[1][0], e / e.sum(axis=1, keepdims=True), floor_frac=1e-3) <= 1e-5
     assert rel_err(res[1][1], res[0][1], floor_frac=1e-3) <= (1e-3 if dtype == np.float16 else 2e-5)
+
+
+@pytest.mark.parametrize("shape", [(8, 300001), (40, 70000)])
+def test_variance_of_shared_rows_with_a_large_mean(hip, shape):
+    """rows spread over several workgroups, values far from zero (mean 100,
+    deviation 1): the parts' second moments are taken around their own means
+    and combined exactly, so the variance keeps the accuracy of a two-pass
+    evaluation -- against float64"""
+    rs = np.random.RandomState(shape[0])
+    x = (100.0 + rs.standard_normal(shape)).astype(np.float32)
+    x[0, : shape[1] // 2] += 3.0             # parts of one row with different means
+    tx = hip.array(x)
+    mean, var, out = hip.empty((shape[0], 1)), hip.empty((shape[0], 1)), hip.empty(shape)
+    with hip.fused():
+        mean[:] = hip.mean(tx, axis=1)
+        var[:] = hip.var(tx, axis=1)
+        out[:] = (tx - hip.mean(tx, axis=1)) / hip.sqrt(hip.var(tx, axis=1) + 1e-5)
+    x64 = x.astype(np.float64)
+    m64, v64 = x64.mean(axis=1, keepdims=True), x64.var(axis=1, keepdims=True)
+    assert np.abs(mean.get() - m64).max() <= 2e-5
+    assert np.abs(var.get() - v64).max() <= 2e-4 * v64.max()
+    assert np.abs(out.get() - (x64 - m64) / np.sqrt(v64 + 1e-5)).max() <= 2e-4
+    fams = set(p.spec.family for p in hip.plans.values())
+    assert "rowcoop" in fams

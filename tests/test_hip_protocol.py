@@ -16,7 +16,7 @@ def _families(hip):
 
 @pytest.mark.gpu
 def test_soak_alternating_split_and_cooperative_launches(hip, monkeypatch):
-    """2100 launches, three families in turn, new random data every round
+    """2800 launches, three families in turn, new random data every round
     (drawn on the device); max / argmax bit-exact against numpy, sums against
     float64; stops at the first mismatch"""
     # (matrices this small are evaluated in stages otherwise; the protocol is what is under test)
@@ -25,7 +25,7 @@ def test_soak_alternating_split_and_cooperative_launches(hip, monkeypatch):
     xc = hip.empty((20000, 64))          # colcoop: two levels over more rows than a workgroup holds
     xr = hip.empty((8, 40000))           # rowcoop: few very long rows
     am, mx = hip.empty((1, 128), dtype=np.int32), hip.empty((1, 128))
-    lse = hip.empty((1, 64))
+    lse, devc = hip.empty((1, 64)), hip.empty((20000, 64))
     rs_, dev = hip.empty((8, 1)), hip.empty((8, 40000))
     for rnd in range(700):
         for t in (xs, xc, xr):
@@ -33,6 +33,7 @@ def test_soak_alternating_split_and_cooperative_launches(hip, monkeypatch):
         am[:] = hip.argmax(xs, axis=0)
         mx[:] = hip.max(xs, axis=0)
         lse[:] = hip.sum(hip.exp(xc - hip.max(xc, axis=0)), axis=0)
+        devc[:] = xc - hip.mean(xc, axis=0)       # a result of the operand's shape: every workgroup waits for the column sums
         rs_[:] = hip.sum(xr, axis=1)
         dev[:] = xr - hip.mean(xr, axis=1)
         hs, hc, hr = xs.get(), xc.get().astype(np.float64), xr.get().astype(np.float64)
@@ -40,6 +41,8 @@ def test_soak_alternating_split_and_cooperative_launches(hip, monkeypatch):
         assert np.array_equal(mx.get(), hs.max(axis=0, keepdims=True)), "max, round %d" % rnd
         want = np.exp(hc - hc.max(axis=0, keepdims=True)).sum(axis=0, keepdims=True)
         assert_close(lse.get(), want, rtol=1e-5, atol=0, what="sum exp, round %d" % rnd)
+        assert_close(devc.get(), hc - hc.mean(axis=0, keepdims=True), rtol=1e-5, atol=1e-5,
+                     what="column deviation, round %d" % rnd)
         assert_close(rs_.get(), hr.sum(axis=1, keepdims=True), rtol=1e-5, atol=1e-3, what="row sum, round %d" % rnd)
         assert_close(dev.get(), hr - hr.mean(axis=1, keepdims=True), rtol=1e-5, atol=1e-5,
                      what="row deviation, round %d" % rnd)

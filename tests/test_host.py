@@ -543,6 +543,26 @@ def test_row_operands_without_registers_go_to_lds(tmp_path):
         planner.ROW_PARK_BYTES = saved
 
 
+def test_cooperating_rows_take_mean_and_variance_with_one_exchange(pb, monkeypatch):
+    """sum((x - mean)^2) over a row that several workgroups share: each takes the
+    squares around the mean of its own part, the parts are combined after the one
+    exchange that also carries the sums; other second sweeps still wait twice"""
+    x, out = pb.empty((16, 1 << 20)), pb.empty((16, 1 << 20))
+
+    def norm():
+        out[:] = (x - pb.mean(x, axis=1)) / pb.sqrt(pb.var(x, axis=1) + 1e-5)
+
+    ch = plan_of(pb, norm)
+    assert ch.spec.family == "rowcoop" and ch.spec.source.count("nh_ticket_take(ctr)") == 1
+    assert "const float mu" in ch.spec.source and "n_loc" in ch.spec.source
+    monkeypatch.setattr(codegen, "MERGED_MOMENTS", False)
+    assert plan_of(pb, norm).spec.source.count("nh_ticket_take(ctr)") == 2
+    monkeypatch.setattr(codegen, "MERGED_MOMENTS", True)
+    # a second sweep of another form (absolute deviations) needs the finished mean everywhere
+    ch = plan_of(pb, lambda: out.__setitem__(slice(None), x / pb.sum(pb.absolute(x - pb.mean(x, axis=1)), axis=1)))
+    assert ch.spec.family == "rowcoop" and ch.spec.source.count("nh_ticket_take(ctr)") == 2
+
+
 def test_the_cheaper_exponential_is_for_arguments_below_their_own_maximum_only(pb):
     x, y, out = pb.empty((1000, 256)), pb.empty((1000, 256)), pb.empty((1000, 256))
     for axis in (0, 1):
