@@ -776,6 +776,7 @@ class _RedGen(_Gen):
 # family: row  (axis 1)
 # =====================================================================================
 MERGED_MOMENTS = os.environ.get("NEON_HIP_MERGED_MOMENTS", "1") != "0"
+SHARED_FLOAT_JOIN = os.environ.get("NEON_HIP_FLOAT_JOIN", "1") != "0"   # 0: every lane joins its own columns' pieces
 
 
 def _shifted_square_sum(n2, firsts):
@@ -1461,22 +1462,24 @@ def _emit_col_fold(g, L, n, LX, LY, T, V, src, dst_decl=True):
         L.close()
     L("__syncthreads();")
     S = LX * V
-    if pair and S <= T:
-        # (value, index) and (max, sum) pairs cost ten to twenty instructions to combine:
-        # instead of every lane joining all V columns of its tile over all wave groups, P
+    if S <= T and (pair or SHARED_FLOAT_JOIN):
+        # Instead of every lane joining all V columns of its tile over all wave groups, P
         # adjacent lanes share ONE column, each takes every P-th group, a DPP all-reduce
-        # over the P lanes finishes, and the results go round through LDS
+        # over the P lanes finishes, and the results go round through LDS.  (value, index)
+        # and (max, sum) pairs cost ten to twenty instructions to combine; for plain values
+        # it is the LDS traffic that counts -- 16 waves x 4 values read by each of 1024
+        # lanes took a fifth of a softmax over (1000,4096): 9.4 -> 8.6 us, fp16 9.6 -> 7.9 us
         P = 1
         while P * 2 <= min(T // S, 64) and P < WY:
             P *= 2
         L.open("")
         L("const int fcol = threadIdx.x / %d, fk = threadIdx.x %% %d;" % (P, P))
-        L("nh_pair one = %s::init();" % op)
+        L("%s one = %s::init();" % ("nh_pair" if pair else "float", op))
         L.open("if (fcol < %d)" % S)
         L("for (int y = fk; y < %d; y += %d) one = %s::f(one, %s[y][fcol]);" % (WY, P, op, buf))
         L.close()
         if P > 1:
-            L("one = nh_wave_allreduce<%s, %d, nh_pair>(one);" % (op, P))
+            L("one = nh_wave_allreduce<%s, %d, %s>(one);" % (op, P, "nh_pair" if pair else "float"))
         L("__syncthreads();     // every piece has been read: the first row of the buffer takes the results")
         L("if (fk == 0 && fcol < %d) %s[0][fcol] = one;" % (S, buf))
         L.close()
