@@ -749,7 +749,7 @@ class _RedGen(_Gen):
             L("#pragma unroll")
             L("for (int j = 0; j < %d; ++j) acc%d[j] = %s::init();" % (self.V, n.nid, op))
         else:
-            L("%s acc%d = %s::init();" % ("nh_pair" if n.is_index else "float", n.nid, op))
+            L("%s acc%d = %s::init();" % ("nh_pair" if self.is_pair(n) else "float", n.nid, op))
 
     def accumulate(self, n, val, index, ref=None):
         """fold one element into the lane's accumulator (inside the j loop)"""
@@ -783,7 +783,7 @@ def _shifted_square_sum(n2, firsts):
     """``n2`` = sum(sqr(x - a)) along the row, with ``x`` free of reductions, ``a``
     constant along the row and ``sum(x)`` among the first sweep's reductions
     ``firsts`` (the variance around a mean): (n2, sum(x), x, a), else None."""
-    if n2.op != "sum" or n2.is_index:
+    if n2.op != "sum" or n2.is_index or n2.lse_max is not None:
         return None
     e = n2.args[0]
     if e.kind != "E" or e.op != "sqr":
@@ -878,7 +878,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
     L("const long long rr = row_ok ? r : 0;")   # address clamp for idle teams
     if not resident:
         L("const int nch = (C + %d - 1) / %d;" % (LX * V, LX * V))
-    all_reds = [n for lv in sorted(per_level) for n in per_level[lv]]
+    all_reds = g.own_reductions([n for lv in sorted(per_level) for n in per_level[lv]])
     red_slot = dict((n.nid, k) for k, n in enumerate(all_reds))
     exchanges = [0]
     if coop:
@@ -932,7 +932,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
         exchanges[0] += 1
         L.open("if (threadIdx.x == 0)")
         for n in list(reds) + list(riders):
-            val = ("red%d" % n.nid) if n.is_index else ("nh_pair{red%d, 0}" % n.nid)
+            val = ("red%d" % n.nid) if g.is_pair(n) else ("nh_pair{red%d, 0}" % n.nid)
             L("nh_part_store(&part[%d + blockIdx.y], %s);" % (red_slot[n.nid] * chunks, val))
         L.close()
         L("nh_publish_barrier();     // the partial stores have been performed")
@@ -952,13 +952,13 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
         L("return;")
         L.close()
         for n in list(reds) + list(riders):
-            op = _RED_OP[n.op]
-            init = ("%s::init()" % op) if n.is_index else ("nh_pair{%s::init(), 0}" % op)
+            op = g.red_op(n)
+            init = ("%s::init()" % op) if g.is_pair(n) else ("nh_pair{%s::init(), 0}" % op)
             L("const nh_pair g%d = (threadIdx.x < %d) ? nh_part_load(&part[%d + threadIdx.x]) : %s;"
               % (n.nid, chunks, red_slot[n.nid] * chunks, init))
         for n in reds:
-            op = _RED_OP[n.op]
-            if n.is_index:
+            op = g.red_op(n)
+            if g.is_pair(n):
                 L("red%d = nh_block_allreduce<%s, %d, nh_pair>(g%d, s_p);" % (n.nid, op, T // 64, n.nid))
             else:
                 L("red%d = nh_block_allreduce<%s, %d, float>(g%d.v, s_f);" % (n.nid, op, T // 64, n.nid))
@@ -1075,7 +1075,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
     sweeps_reading = {}
     if park_left[0]:
         earlier = set()
-        rounds = [[n for n in per_level.get(s_, [])] for s_ in range(nsweeps)]
+        rounds = [g.own_reductions(per_level.get(s_, [])) for s_ in range(nsweeps)]
         for reds_ in rounds:
             if reds_:
                 for leaf in g.leaf_nodes(_needed([n.args[0] for n in reds_], earlier)):
@@ -1132,7 +1132,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
     # a resident float32 operand nothing else reads afterwards
     over, vals, own = {}, {}, set()
     if resident:
-        stages = [[n.args[0] for n in per_level.get(s, [])] for s in range(nsweeps)]
+        stages = [[n.args[0] for n in g.own_reductions(per_level.get(s, []))] for s in range(nsweeps)]
         stages = [t for t in stages if t]
         if full_out:
             stages.append([st.root for st in full_out])
@@ -1224,7 +1224,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
     for s in range(nsweeps):
         if merged and s == 1:
             continue            # done together with the first sweep
-        reds = [n for n in per_level.get(s, [])]
+        reds = g.own_reductions(per_level.get(s, []))
         if not reds:
             continue
         args = [n.args[0] for n in reds]
@@ -1251,6 +1251,14 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
             if not reds and not fresh and not fresh_own:
                 L.close()
                 return
+            # a running (max, sum of exponentials) pair takes the tile's V values at once:
+            # one rescaling of the sum per tile instead of one per element
+            running = [n for n in reds if g.fused_max(n)]
+            for n in running:
+                L("float lv%d[%d];" % (n.nid, V))
+                if tail:
+                    L("#pragma unroll")
+                    L("for (int j = 0; j < %d; ++j) lv%d[j] = -NH_INF;" % (V, n.nid))
             if V > 1:
                 L("#pragma unroll")
             L.open("for (int j = 0; j < %d; ++j)" % V)
@@ -1259,7 +1267,10 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
             ref = g.make_ref("_s", "rr", "c", V, tiles, vals)
             g.emit_exprs(nodes, ref, stops())
             for n in reds:
-                g.accumulate(n, ref(n.args[0]), "c + j", ref)
+                if n in running:
+                    L("lv%d[j] = %s;" % (n.nid, ref(n.args[0])))
+                else:
+                    g.accumulate(n, ref(n.args[0]), "c + j", ref)
             for n in fresh:
                 L("keep%d[k].put(j, t%d);" % (over[n.nid].nid, n.nid))
             for n in fresh_own:
@@ -1267,6 +1278,8 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
             if tail:
                 L.close()
             L.close()
+            for n in running:
+                L("nh_op_lse::stepn<%d>(acc%d, lv%d);" % (V, n.nid, n.nid))
             L.close()
 
         sweep(leaves, reduce_body)
@@ -1275,14 +1288,14 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
         for n in fresh_own:
             vals[n.nid] = "val%d[k][j]" % n.nid
         for n in reds:
-            op = _RED_OP[n.op]
-            ty_ = "nh_pair" if n.is_index else "float"
+            op = g.red_op(n)
+            ty_ = "nh_pair" if g.is_pair(n) else "float"
             const = "" if coop else "const "
             if LX <= 64:
                 L("%s%s red%d = nh_wave_allreduce<%s, %d, %s>(acc%d);" % (const, ty_, n.nid, op, LX, ty_, n.nid))
             else:
                 L("%s%s red%d = nh_block_allreduce<%s, %d, %s>(acc%d, %s);"
-                  % (const, ty_, n.nid, op, T // 64, ty_, n.nid, "s_p" if n.is_index else "s_f"))
+                  % (const, ty_, n.nid, op, T // 64, ty_, n.nid, "s_p" if g.is_pair(n) else "s_f"))
         if coop and merged and s == 0:
             local_second_moments()
             exchange(reds, riders=[m[0] for m in merged])
@@ -1291,6 +1304,10 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
         for n in reds:
             if n.is_index:
                 L("const int ri%d = red%d.i;" % (n.nid, n.nid))
+            elif g.fused_max(n):
+                L("const float rv%d = red%d.v;" % (n.nid, n.nid))
+                L("const float rv%d = nh_lse_total(red%d);" % (n.lse_sum.nid, n.nid))
+                done[n.lse_sum.nid] = n.lse_sum
             else:
                 L("const float rv%d = red%d;" % (n.nid, n.nid))
             done[n.nid] = n
@@ -1439,7 +1456,7 @@ def _emit_col_fold(g, L, n, LX, LY, T, V, src, dst_decl=True):
         if n.is_index:
             L("for (int j = 0; j < %d; ++j) ri%d[j] = %s[j].i;" % (V, n.nid, src))
         elif g.fused_max(n):
-            L("for (int j = 0; j < %d; ++j) { rv%d[j] = %s[j].v; rv%d[j] = nh_lse_sum(%s[j]); }"
+            L("for (int j = 0; j < %d; ++j) { rv%d[j] = %s[j].v; rv%d[j] = nh_lse_total(%s[j]); }"
               % (V, n.nid, src, n.lse_sum.nid, src))
         else:
             L("for (int j = 0; j < %d; ++j) rv%d[j] = %s[j];" % (V, n.nid, src))
@@ -2115,7 +2132,7 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1):
         if n.is_index:
             L("for (int j = 0; j < %d; ++j) ri%d[j] = s_r%d[tx * %d + j].i;" % (V, n.nid, n.nid, V))
         elif g.fused_max(n):
-            L("for (int j = 0; j < %d; ++j) { rv%d[j] = s_r%d[tx * %d + j].v; rv%d[j] = nh_lse_sum(s_r%d[tx * %d + j]); }"
+            L("for (int j = 0; j < %d; ++j) { rv%d[j] = s_r%d[tx * %d + j].v; rv%d[j] = nh_lse_total(s_r%d[tx * %d + j]); }"
               % (V, n.nid, n.nid, V, n.lse_sum.nid, n.nid, V))
         else:
             L("for (int j = 0; j < %d; ++j) rv%d[j] = s_r%d[tx * %d + j];" % (V, n.nid, n.nid, V))

@@ -484,13 +484,12 @@ class Program(object):
         self._analyse()
         self.lse_pairs = 0
         self.gathers = 0
-        if self.axis == 0:
-            if self.online_lse:
-                self._pair_max_with_sum_of_exp()
-            if self.onehot_gather:
-                self._gather_at_hot_rows()
-            if self.lse_pairs or self.gathers:
-                self._analyse()
+        if self.axis is not None and self.online_lse:
+            self._pair_max_with_sum_of_exp()
+        if self.axis == 0 and self.onehot_gather:
+            self._gather_at_hot_rows()
+        if self.lse_pairs or self.gathers:
+            self._analyse()
         for st in self.statements:
             rs, os_ = st.root.shape, st.out.shape
             if (rs[0] not in (1, os_[0])) or (rs[1] not in (1, os_[1])):
@@ -575,6 +574,13 @@ class Program(object):
             n.lse_max = n.lse_sum = None
         self.lse_pairs = 0
         self._analyse()
+
+    def pair_lse(self):
+        """(again) one sweep for both, where the tree has the pattern"""
+        if not self.lse_pairs and self.online_lse:
+            self._pair_max_with_sum_of_exp()
+            if self.lse_pairs:
+                self._analyse()
 
     def _gather_at_hot_rows(self):
         """``sum(onehot(idx, 0) * expr, 0)`` adds one term of ``expr`` per column

@@ -399,6 +399,13 @@ ROW_KEPT_VALUES = os.environ.get("NEON_HIP_ROW_VALS", "1") != "0"
 
 
 def _plan_row(prog, cu_count, coop=True):
+    # The tiling is chosen for the tree as written.  A maximum and the sum of exponentials
+    # around it then share a sweep (a running pair) only where that saves a pass over memory
+    # or an exchange: rows that are streamed, wholly or in part; rows resident in registers
+    # are swept three times at no cost and keep the exponentials for the last sweep.
+    paired = prog.lse_pairs > 0
+    if paired:
+        prog.unpair_lse()
     R, C = prog.domain
     V = _vector_width(prog, tail_ok=True)
     tail = (C % V) != 0
@@ -456,6 +463,12 @@ def _plan_row(prog, cu_count, coop=True):
         if chunks >= 2 and ((per <= 16 and per * smallest <= 64) or
                             (per <= ROWCOOP_MAX_TILES and ROW_PARK_BYTES and sweeps >= 2)):
             kw = None if (per <= 16 and per * words <= 64) else (64 if per <= 16 else ROW_SPLIT_WORDS)
+            # (resident shares of 16-bit rows too: their exponentials cannot take over the
+            # operand's registers, so the pair costs no extra exponential and saves an exchange --
+            # (16,1605632) fp16 35.8 -> 32.3 us; fp32 shares lose 1-3 us with it)
+            narrow = any(t.read and t.shape[1] > 1 and t.dtype.itemsize < 4 for t in prog.tensors)
+            if paired and (kw is not None or narrow):
+                prog.pair_lse()
             spec = codegen.gen_row(prog, V, 1024, 1, per, _streams(prog), keep_words=kw, chunks=chunks, tail=tail,
                                    park_bytes=ROW_PARK_BYTES if kw else 0)
             part_bytes = R * spec.params["NRED"] * chunks * 8
@@ -471,6 +484,11 @@ def _plan_row(prog, cu_count, coop=True):
     if NCH and keep_words is None and sweeps >= 2 and ROW_KEPT_VALUES:
         budget = 64 if T == 1024 else 96
         max_vals = min(2, max(0, (budget - NCH * words) // (NCH * V)))
+    # (also 16-bit rows that fill the registers: with no room to keep the exponentials, the pair's
+    # one sweep is cheaper than the two it replaces -- (4096,131072) fp16 521 -> 482 us)
+    narrow = any(t.read and t.shape[1] > 1 and t.dtype.itemsize < 4 for t in prog.tensors)
+    if paired and (NCH == 0 or keep_words is not None or (max_vals == 0 and narrow)):
+        prog.pair_lse()
     spec = codegen.gen_row(prog, V, LX, LY, NCH, _streams(prog), keep_words=keep_words, tail=tail, park_bytes=park,
                            max_vals=max_vals)
     return Choice(spec, (gx, 1, 1))

@@ -473,6 +473,9 @@ struct nh_op_argmin {
 // taken as 0 instead of evaluating exp(-inf + inf).  NaN and +inf propagate
 // as in the two-sweep form (the sum becomes NaN).
 NEON_DEV float nh_lse_sum(nh_pair p) { return __builtin_bit_cast(float, p.i); }
+// The finished sum, as the two-sweep evaluation has it: where every element was
+// -inf that one adds up exp(-inf - -inf) = NaN terms.
+NEON_DEV float nh_lse_total(nh_pair p) { return (p.v == -NH_INF) ? __builtin_nanf("") : nh_lse_sum(p); }
 // exp(d) for d <= 0 (a term of a sum whose largest term is 1): the product
 // d * log2(e) is carried in two pieces so that the result is good to about a
 // unit in the last place, like expf, at half its instruction count; what

@@ -154,3 +154,35 @@ def test_variance_of_shared_rows_with_a_large_mean(hip, shape):
     assert np.abs(out.get() - (x64 - m64) / np.sqrt(v64 + 1e-5)).max() <= 2e-4
     fams = set(p.spec.family for p in hip.plans.values())
     assert "rowcoop" in fams
+
+
+@pytest.mark.parametrize("shape,dtype", [((6, 300000), np.float32), ((300, 140000), np.float32), ((5, 1200000), np.float16)])
+def test_softmax_over_streamed_rows_with_infinities_and_nans(hip, shape, dtype):
+    """rows too long for registers take maximum and sum of exponentials in one
+    sweep (a running pair): -inf entries, a row of nothing but -inf, a NaN, a
+    row whose maximum comes last -- as the three-sweep numpy evaluation has it"""
+    rs = np.random.RandomState(41)
+    x = (rs.standard_normal(shape) * 3).astype(dtype)
+    x[0, 5] = -np.inf
+    x[1, :] = -np.inf                        # -inf - -inf: NaN everywhere in the row
+    x[2, 77] = np.nan
+    x[3, -1] = 60.0                          # the running maximum jumps at the very end
+    x[4, 0] = 60.0                           # ... or is there from the start
+    tx = hip.array(x, dtype=dtype)
+    out, lse = hip.empty(shape), hip.empty((shape[0], 1))
+    out[:] = hip.exp(tx - hip.max(tx, axis=1)) / hip.sum(hip.exp(tx - hip.max(tx, axis=1)), axis=1)
+    lse[:] = hip.log(hip.sum(hip.exp(tx - hip.max(tx, axis=1)), axis=1)) + hip.max(tx, axis=1)
+    x64 = x.astype(np.float64)
+    with np.errstate(invalid="ignore"):
+        m = x64.max(axis=1, keepdims=True)
+        e = np.exp(x64 - m)
+        want = e / e.sum(axis=1, keepdims=True)
+        want_lse = np.log(e.sum(axis=1, keepdims=True)) + m
+    got, got_lse = out.get().astype(np.float64), lse.get().astype(np.float64)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.abs(got[ok] - want[ok]).max() <= 1e-5 * want[ok].max()
+    assert got[0, 5] == 0.0
+    assert np.array_equal(np.isnan(got_lse), np.isnan(want_lse))
+    okl = ~np.isnan(want_lse)
+    assert np.abs(got_lse[okl] - want_lse[okl]).max() <= 1e-5 * np.abs(want_lse[okl]).max()

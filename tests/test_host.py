@@ -466,7 +466,9 @@ def test_row_softmax_reuses_registers_when_the_row_is_resident(pb):
     # ... unless the row itself fills them ((64, 131072) fp16: 16 tiles of 1024 lanes)
     xh, outh = pb.empty((512, 131072), np.float16), pb.empty((512, 131072), np.float16)
     spec = plan_of(pb, lambda: outh.__setitem__(slice(None), softmax(xh))).spec
-    assert spec.params["NCH"] == 16 and spec.params["kept"] == 0 and spec.source.count("nh_exp_nonpos(") == 2
+    # (then maximum and sum share a sweep as a running pair instead: two sweeps, not three)
+    assert spec.params["NCH"] == 16 and spec.params["kept"] == 0
+    assert spec.source.count("nh_op_lse::stepn<8>(") == 1 and spec.source.count("nh_exp_nonpos(") == 1
     # few rows too long for one workgroup's registers are spread over several
     # workgroups and stay resident
     xl, outl = pb.empty((16, 1 << 20)), pb.empty((16, 1 << 20))
@@ -474,14 +476,26 @@ def test_row_softmax_reuses_registers_when_the_row_is_resident(pb):
     assert ch.spec.family == "rowcoop" and ch.grid == (16, 16, 1) and ch.spec.params["over"] == 1
     assert ch.spec.source.count("nh_exp_nonpos(") == 1
     # many such rows: a workgroup per row keeps the first tiles in LDS and registers and streams
-    # the rest in every sweep, as a loop proper -- nothing to lend registers
+    # the rest in every sweep, as a loop proper -- nothing to lend registers.  Maximum and sum
+    # of exponentials share the first sweep (a running pair), one pass over memory less
     xl, outl = pb.empty((512, 1 << 20)), pb.empty((512, 1 << 20))
     spec = plan_of(pb, lambda: outl.__setitem__(slice(None), softmax(xl))).spec
     assert spec.family == "row" and spec.params["over"] == 0
     assert (spec.params["NCH"], spec.params["parked"], spec.params["held"]) == (256, 9, 16)
-    assert spec.source.count("for (int kb = 0; kb < 28; kb += 4)") == 3
-    assert spec.source.count("#pragma unroll 1\n    for (int kb = 28; kb < 256; kb += 4)") == 3
-    assert spec.source.count("nh_exp_nonpos(") == 4         # two sweeps, the unrolled and the looping part of each
+    assert spec.source.count("for (int kb = 0; kb < 28; kb += 4)") == 2
+    assert spec.source.count("#pragma unroll 1\n    for (int kb = 28; kb < 256; kb += 4)") == 2
+    assert spec.source.count("nh_op_lse::stepn<4>(") == 2 and spec.source.count("nh_exp_nonpos(") == 2
+    saved = Program.__init__
+
+    def two_sweeps(self, *a, **k):
+        saved(self, *a, **k)
+        self.online_lse = False
+    try:
+        Program.__init__ = two_sweeps
+        spec = plan_of(pb, lambda: outl.__setitem__(slice(None), softmax(xl))).spec
+    finally:
+        Program.__init__ = saved
+    assert spec.source.count("for (int kb = 0; kb < 28; kb += 4)") == 3 and "stepn" not in spec.source
 
 
 def test_more_than_2_31_elements_stay_two_dimensional(pb):
