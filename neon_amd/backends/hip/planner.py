@@ -467,7 +467,9 @@ def _plan_row(prog, cu_count, coop=True):
             # operand's registers, so the pair costs no extra exponential and saves an exchange --
             # (16,1605632) fp16 35.8 -> 32.3 us; fp32 shares lose 1-3 us with it)
             narrow = any(t.read and t.shape[1] > 1 and t.dtype.itemsize < 4 for t in prog.tensors)
-            if paired and (kw is not None or narrow):
+            # (short shares excepted: folding pairs through the workgroup costs two exponentials a
+            # step, more than the exchange saved -- (64,131072) fp16, 4 tiles each: 13.8 vs 16.2 us)
+            if paired and (kw is not None or (narrow and per >= 8)):
                 prog.pair_lse()
             spec = codegen.gen_row(prog, V, 1024, 1, per, _streams(prog), keep_words=kw, chunks=chunks, tail=tail,
                                    park_bytes=ROW_PARK_BYTES if kw else 0)
