@@ -186,3 +186,27 @@ def test_softmax_over_streamed_rows_with_infinities_and_nans(hip, shape, dtype):
     assert np.array_equal(np.isnan(got_lse), np.isnan(want_lse))
     okl = ~np.isnan(want_lse)
     assert np.abs(got_lse[okl] - want_lse[okl]).max() <= 1e-5 * np.abs(want_lse[okl]).max()
+
+
+@pytest.mark.parametrize("shape,dtype", [((8, 300001), np.float32), ((20, 1200000), np.float16), ((300, 150000), np.float32)])
+def test_softmax_and_normalisation_of_one_operand_in_one_group(hip, shape, dtype):
+    """both trees over the same long rows in one fusion group: the running
+    (max, sum) pair, the sums and the parts' second moments travel in the same
+    sweep and -- where rows are shared -- the same exchange"""
+    rs = np.random.RandomState(shape[0])
+    x = (rs.standard_normal(shape) * 2 + 1).astype(dtype)
+    tx = hip.array(x, dtype=dtype)
+    sm, nm = hip.empty(shape), hip.empty(shape)
+    before = hip.plan_stats["launches"]
+    node = hip._api.OpTreeNode
+    # (handed over as one statement group, the way the compound batch-norm calls hand over theirs)
+    hip._flush()
+    hip._run([node({"op": "assign"}, sm, hip.exp(tx - hip.max(tx, axis=1)) / hip.sum(hip.exp(tx - hip.max(tx, axis=1)), axis=1)),
+              node({"op": "assign"}, nm, (tx - hip.mean(tx, axis=1)) / hip.sqrt(hip.var(tx, axis=1) + 1e-5))])
+    assert hip.plan_stats["launches"] - before == 1
+    x64 = x.astype(np.float64)
+    e = np.exp(x64 - x64.max(axis=1, keepdims=True))
+    want_sm = e / e.sum(axis=1, keepdims=True)
+    want_nm = (x64 - x64.mean(axis=1, keepdims=True)) / np.sqrt(x64.var(axis=1, keepdims=True) + 1e-5)
+    assert rel_err(sm.get().astype(np.float64), want_sm, floor_frac=1e-3) <= 2e-5
+    assert np.abs(nm.get().astype(np.float64) - want_nm).max() <= 2e-4
