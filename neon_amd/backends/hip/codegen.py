@@ -780,8 +780,8 @@ SHARED_FLOAT_JOIN = os.environ.get("NEON_HIP_FLOAT_JOIN", "1") != "0"   # 0: eve
 
 
 def _shifted_square_sum(n2, firsts):
-    """``n2`` = sum(sqr(x - a)) along the row, with ``x`` free of reductions, ``a``
-    constant along the row and ``sum(x)`` among the first sweep's reductions
+    """``n2`` = sum(sqr(x - a)) along the reduced axis, with ``x`` free of reductions, ``a``
+    constant along that axis and ``sum(x)`` among the first sweep's reductions
     ``firsts`` (the variance around a mean): (n2, sum(x), x, a), else None."""
     if n2.op != "sum" or n2.is_index or n2.lse_max is not None:
         return None
@@ -792,7 +792,8 @@ def _shifted_square_sum(n2, firsts):
     if d.kind != "E" or d.op != "sub" or len(d.args) != 2:
         return None
     x, a = d.args
-    if not x.vc or x.level != 0 or a.vc or a.level > 1 or a.kind == "R" and a.is_index:
+    along_x, along_a = (x.vc, a.vc) if n2.axis == 1 else (x.vr, a.vr)
+    if not along_x or x.level != 0 or along_a or a.level > 1 or a.kind == "R" and a.is_index:
         return None
     for r1 in firsts:
         if r1.op == "sum" and not r1.is_index and r1.args[0] is x:
@@ -1598,15 +1599,17 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False)
             L("const long long r = (long long)i * %d + ty;" % LY)
         L("const bool ok = col_ok && (r < R);")
 
-    def exchange(reds, last_one_folds=False):
+    def exchange(reds, last_one_folds=False, riders=()):
         """fold the workgroups of a strip: afterwards acc/rv/ri hold the
-        result over all rows in every lane of every workgroup.
+        result over all rows in every lane of every workgroup.  ``riders``:
+        reductions whose per-workgroup values travel along and are only
+        fetched (q<id>[][]), for the caller to combine.
 
         ``last_one_folds``: nothing but one value per column remains to be
         written, so nobody waits: the workgroup whose arrival completes the
         count gathers, folds and goes on alone, the others are done."""
         exchanges[0] += 1
-        for n in reds:
+        for n in list(reds) + list(riders):
             L("nh_pair* part%d = reinterpret_cast<nh_pair*>(ws) + (long long)%d * C;"
               % (n.nid, red_slot[n.nid] * chunks))
         L.open("if (col_ok && ty == 0)")
@@ -1614,7 +1617,7 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False)
         L.open("for (int j = 0; j < %d; ++j)" % V)
         if tail:
             L.open("if (j < clim)")
-        for n in reds:
+        for n in list(reds) + list(riders):
             if g.is_pair(n):
                 L("nh_part_store(&part%d[(long long)blockIdx.y * C + c + j], acc%d[j]);" % (n.nid, n.nid))
             else:
@@ -1633,7 +1636,7 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False)
             L("if (s_abort) return;     // not the last to arrive: the last one finishes the strip")
         else:
             exchange_wait()
-        exchange_gather(reds)
+        exchange_gather(reds, riders)
 
     def exchange_wait():
         L.open("if (threadIdx.x == 0)")
@@ -1652,9 +1655,9 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False)
         L("return;")
         L.close()
 
-    def exchange_gather(reds):
+    def exchange_gather(reds, riders=()):
         QMAX = -(-chunks // LY)
-        for n in reds:
+        for n in list(reds) + list(riders):
             L("nh_pair q%d[%d][%d];" % (n.nid, QMAX, V))
         L("#pragma unroll")
         L.open("for (int k = 0; k < %d; ++k)" % QMAX)
@@ -1662,7 +1665,7 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False)
         L("const bool live = col_ok && (q < %d);" % chunks)
         L("#pragma unroll")
         L.open("for (int j = 0; j < %d; ++j)" % V)
-        for n in reds:
+        for n in list(reds) + list(riders):
             op = g.red_op(n)
             init = ("%s::init()" % op) if g.is_pair(n) else ("nh_pair{%s::init(), 0}" % op)
             L("q%d[k][j] = (live%s) ? nh_part_load(&part%d[(long long)q * C + c + j]) : %s;"
@@ -1765,8 +1768,85 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False)
             if n.nid in kept_ids and n.nid not in vals and n.nid not in over:
                 L("float val%d[%d][%d];" % (n.nid, NR, V))
 
+    # Variance around a mean down columns that several workgroups share: as in the row family,
+    # every workgroup takes the squares around the mean of its own rows, and one exchange
+    # carries sums and second moments; sum_i [ M2_i + n_i (mean_i - a)^2 ] afterwards.
+    merged = []
+    if coop and MERGED_MOMENTS and not over and not kept and per_level.get(0) and per_level.get(1):
+        merged = [_shifted_square_sum(n2, g.own_reductions(per_level[0])) for n2 in g.own_reductions(per_level[1])]
+        if not merged or not all(merged):
+            merged = []
+    share = NR * LY      # rows of a strip that one workgroup owns
+
+    def local_second_moments():
+        L("const long long left_ = (long long)R - (long long)blockIdx.y * %dll;" % share)
+        L("const float n_loc = (float)(left_ < %dll ? left_ : %dll);" % (share, share))
+        for n2, r1, x, a in merged:
+            L("float mu%d[%d];" % (n2.nid, V))
+            L("#pragma unroll")
+            L("for (int j = 0; j < %d; ++j) mu%d[j] = rv%d[j] / n_loc;" % (V, n2.nid, r1.nid))
+            vals[a.nid] = "mu%d[j]" % n2.nid
+        seconds = [m[0] for m in merged]
+        nodes = _needed([n.args[0] for n in seconds], stops())
+        leaves = g.leaf_nodes(nodes)
+        declare_tiles(leaves)
+        for n in seconds:
+            g.declare_acc(n)
+        tiles = load_leaves(leaves)
+        row_loop_open()
+        L.open("if (ok)")
+        if V > 1:
+            L("#pragma unroll")
+        L.open("for (int j = 0; j < %d; ++j)" % V)
+        ref = g.make_ref("_s", "r", "cc", V, tiles, vals)
+        g.emit_exprs(nodes, ref, stops())
+        for n in seconds:
+            g.accumulate(n, ref(n.args[0]), "r", ref)
+        L.close()
+        L.close()
+        L.close()
+        for n in seconds:
+            _emit_col_fold(g, L, n, LX, LY, T, V, "acc%d" % n.nid)
+        for n2, r1, x, a in merged:
+            del vals[a.nid]
+
+    def combine_second_moments():
+        QMAX = -(-chunks // LY)
+        for n2, r1, x, a in merged:
+            L("float shift%d[%d];" % (n2.nid, V))
+            if V > 1:
+                L("#pragma unroll")
+            L.open("for (int j = 0; j < %d; ++j)" % V)
+            ref = g.make_ref("_s", "0", "cc", V, dict(line_tiles), vals)
+            g.emit_exprs(_needed([a], stops()), ref, stops())
+            L("shift%d[j] = %s;" % (n2.nid, ref(a)))
+            L.close()
+            L("#pragma unroll")
+            L("for (int j = 0; j < %d; ++j) acc%d[j] = 0.0f;" % (V, n2.nid))
+            L("#pragma unroll")
+            L.open("for (int k = 0; k < %d; ++k)" % QMAX)
+            L("const int q = ty + k * %d;" % LY)
+            L.open("if (col_ok && q < %d)" % chunks)
+            L("const long long lq = (long long)R - (long long)q * %dll;" % share)
+            L("const float nq = (float)(lq < %dll ? lq : %dll);" % (share, share))
+            L("#pragma unroll")
+            L.open("for (int j = 0; j < %d; ++j)" % V)
+            if tail:
+                L.open("if (j < clim)")
+            L("const float dq = q%d[k][j].v / nq - shift%d[j];" % (r1.nid, n2.nid))
+            L("acc%d[j] += __builtin_fmaf(nq * dq, dq, q%d[k][j].v);" % (n2.nid, n2.nid))
+            if tail:
+                L.close()
+            L.close()
+            L.close()
+            L.close()
+            _emit_col_fold(g, L, n2, LX, LY, T, V, "acc%d" % n2.nid, dst_decl=False)
+            done[n2.nid] = n2
+
     ticket_finish = False
     for s in range(nsweeps):
+        if merged and s == 1:
+            continue            # done together with the first sweep
         reds = g.own_reductions(per_level.get(s, []))
         if not reds:
             continue
@@ -1832,8 +1912,14 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False)
             if g.fused_max(n):
                 done[n.lse_sum.nid] = n.lse_sum
         if coop:
-            ticket_finish = not full_out and not any(per_level.get(k) for k in range(s + 1, nsweeps))
-            exchange(reds, last_one_folds=ticket_finish)
+            later = [k for k in range(s + 1, nsweeps) if per_level.get(k) and not (merged and k == 1)]
+            ticket_finish = not full_out and not later
+            if merged and s == 0:
+                local_second_moments()
+                exchange(reds, last_one_folds=ticket_finish, riders=[m[0] for m in merged])
+                combine_second_moments()
+            else:
+                exchange(reds, last_one_folds=ticket_finish)
 
     if line_out:
         roots = [st.root for st in line_out]

@@ -557,7 +557,7 @@ def test_row_operands_without_registers_go_to_lds(tmp_path):
         planner.ROW_PARK_BYTES = saved
 
 
-def test_cooperating_rows_take_mean_and_variance_with_one_exchange(pb, monkeypatch):
+def test_cooperating_workgroups_take_mean_and_variance_with_one_exchange(pb, monkeypatch):
     """sum((x - mean)^2) over a row that several workgroups share: each takes the
     squares around the mean of its own part, the parts are combined after the one
     exchange that also carries the sums; other second sweeps still wait twice"""
@@ -571,6 +571,17 @@ def test_cooperating_rows_take_mean_and_variance_with_one_exchange(pb, monkeypat
     assert "const float mu" in ch.spec.source and "n_loc" in ch.spec.source
     monkeypatch.setattr(codegen, "MERGED_MOMENTS", False)
     assert plan_of(pb, norm).spec.source.count("nh_ticket_take(ctr)") == 2
+    monkeypatch.setattr(codegen, "MERGED_MOMENTS", True)
+    # the same down columns that several workgroups share
+    xc, outc = pb.empty((32000, 256)), pb.empty((32000, 256))
+
+    def colnorm():
+        outc[:] = (xc - pb.mean(xc, axis=0)) / pb.sqrt(pb.var(xc, axis=0) + 1e-5)
+
+    ch = plan_of(pb, colnorm)
+    assert ch.spec.family == "colcoop" and ch.spec.source.count("nh_ticket_take(ctr)") == 1
+    monkeypatch.setattr(codegen, "MERGED_MOMENTS", False)
+    assert plan_of(pb, colnorm).spec.source.count("nh_ticket_take(ctr)") == 2
     monkeypatch.setattr(codegen, "MERGED_MOMENTS", True)
     # a second sweep of another form (absolute deviations) needs the finished mean everywhere
     ch = plan_of(pb, lambda: out.__setitem__(slice(None), x / pb.sum(pb.absolute(x - pb.mean(x, axis=1)), axis=1)))
