@@ -532,8 +532,14 @@ class NervanaHIPBase(object):
         self._deferred = []           # statements of the open fusion group that have not been looked at yet
         self._pending_post = []       # postfix walks of the pending statements
         self._pending_sig = None      # what kind of group the pending statements form
+        self._pending_vectors = []    # row / column vectors the pending elementwise statements read
+        self._sig_vectors = ()
         self._fusing = False
         self._fuse_depth = 0
+        blocks = getattr(self._api, "Block", None)
+        self._fusion_blocks = tuple(getattr(blocks, name) for name in ("update", "minibatch") if hasattr(blocks, name))
+        if os.environ.get("NEON_HIP_FUSE_MINIBATCH", "1") == "0":
+            self._fusion_blocks = self._fusion_blocks[:1]
         self._captured = None
         self._launch_cache = {}      # statement-group identity -> recorded launches
         self._replayer = self._records_type = None
@@ -636,9 +642,11 @@ class NervanaHIPBase(object):
         self.rng_set_state((self.init_rng_state, self.init_rng_state_dev))
 
     def rng_get_state(self):
+        self._flush()           # pending statements draw their counters when they are launched
         return (self.rng.get_state(), (self._rng_dev_seed, self._rng_dev_counter))
 
     def rng_set_state(self, rng_states):
+        self._flush()
         if len(rng_states) != 2 or not isinstance(rng_states[1], tuple) or len(rng_states[1]) != 2:
             # a host-only state (e.g. saved by the CPU backend)
             self.rng_reset()
@@ -726,14 +734,21 @@ class NervanaHIPBase(object):
         return _FuseScope(self)
 
     def begin(self, block, identifier):
-        """``Block.update`` opens a fusion group (the reference documents
-        begin/end as optimisation hints, backend.py:671-709)."""
-        if block == self._api.Block.update:
+        """``Block.update`` and ``Block.minibatch`` open a fusion region (the
+        reference documents begin/end as optimisation hints, backend.py:671-709,
+        and brackets every minibatch of its training and evaluation loops with
+        them, models/model.py:204-217, 763-807): consecutive elementwise
+        statements over one shape -- a bias added and an activation applied, an
+        optimizer's update of one parameter -- run as one kernel.  Anything
+        that is not such a statement (a product, a copy to the host, a
+        compound call) first runs what is pending, so the order of effects is
+        that of the program."""
+        if block in self._fusion_blocks:
             self._fuse_depth += 1
             self._fusing = True
 
     def end(self, block, identifier):
-        if block == self._api.Block.update and self._fuse_depth > 0:
+        if block in self._fusion_blocks and self._fuse_depth > 0:
             self._fuse_depth -= 1
             if self._fuse_depth == 0:
                 self._fusing = False
@@ -769,11 +784,23 @@ class NervanaHIPBase(object):
         sig = self._group_signature(tree, post)
         if sig is None:
             return False
+        vectors = self._sig_vectors
         if not self._pending:
+            if sig[0] == "ew" and vectors and any(v.get_original_base() is tree[1].get_original_base() for v in vectors):
+                return False
             self._pending_sig = sig
+            self._pending_vectors = list(vectors)
             return True
         if sig != self._pending_sig:
             return False
+        if sig[0] == "ew" and (vectors or self._pending_vectors):
+            # row / column vectors are read by lanes other than the one that would write them:
+            # none of them may live in a tensor that a statement of the group writes
+            outs = set(id(q[1].get_original_base()) for q in self._pending)
+            outs.add(id(tree[1].get_original_base()))
+            if any(id(v.get_original_base()) in outs for v in list(vectors) + self._pending_vectors):
+                return False
+            self._pending_vectors.extend(vectors)
         if sig[0] == "red":
             # results are written while operands are still being read by other
             # workgroups: a result that lives inside an operand would be a race
@@ -792,6 +819,8 @@ class NervanaHIPBase(object):
         tensor_cls = self.tensor_cls
         axis = None
         full = None
+        others = []
+        self._sig_vectors = ()
         for p in post:
             tp = type(p)
             if tp is dict:
@@ -812,15 +841,23 @@ class NervanaHIPBase(object):
                 elif not p.is_contiguous or len(p.shape) != 2:
                     return None
                 elif p.shape != shape:
+                    others.append(p)
                     if full is None:
                         full = p.shape
                     elif p.shape != full and p.shape != shape:
-                        return None
+                        full = ()           # several other shapes: only an elementwise group may take them
         if axis is None:
-            # purely elementwise: no one-hot either (its index vector has another shape)
-            if full is not None or any(type(p) is dict and p["op"] == "onehot" for p in post):
+            # purely elementwise: no one-hot either (its index vector has another shape); operands
+            # of another shape must be row or column vectors of the group's shape (a bias)
+            if any(type(p) is dict and p["op"] == "onehot" for p in post) or len(shape) != 2:
                 return None
+            for p in others:
+                if p.shape[0] not in (1, shape[0]) or p.shape[1] not in (1, shape[1]):
+                    return None
+            self._sig_vectors = tuple(others)
             return ("ew", shape)
+        if full == ():
+            return None
         if full is None or len(shape) != 2 or out.rounding or not out.is_contiguous:
             return None
         line = (1, full[1]) if axis == 0 else (full[0], 1)
@@ -869,11 +906,14 @@ class NervanaHIPBase(object):
         """a statement joins the pending fusion group, or ends it, or runs on its own"""
         post = optree.traverse([])
         if self._fusing:
-            if self._can_join(optree, post):
-                self._pending.append(optree)
-                self._pending_post.append(post)
-                return
-            self._flush_pending()
+            for attempt in (0, 1):
+                if self._can_join(optree, post):
+                    self._pending.append(optree)
+                    self._pending_post.append(post)
+                    return
+                if attempt == 0 and not self._pending:
+                    break
+                self._flush_pending()       # ... and the statement may open the next group
         if self._captured is not None:
             self._captured.append([optree])
         else:

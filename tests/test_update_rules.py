@@ -119,3 +119,55 @@ def test_adam_fp16_parameters_hip_matches_oracle(pair):
         # device (a later statement reads what an earlier one stored): 1e-3 relative
         assert_close(g.astype(np.float32), w.astype(np.float16).astype(np.float32), rtol=1e-3, atol=1e-6,
                      what="adam f16")
+
+
+@pytest.mark.gpu
+def test_statements_inside_a_minibatch_block_fuse_and_keep_program_order(pair):
+    """The reference brackets every minibatch with begin / end(Block.minibatch)
+    (models/model.py:204-217): inside, consecutive elementwise statements over
+    one shape run as one kernel, and whatever is not such a statement -- a
+    product, a copy to the host, a reduction -- sees what the program wrote
+    before it.  The sequence below (bias + activation, a product, a momentum
+    update of two parameters, a host read in the middle) against the oracle
+    and against the same sequence outside any block."""
+    from neon_amd.backends.backend import Block
+    rs = np.random.RandomState(11)
+    w0, x0, b0 = rs.standard_normal((64, 48)).astype(np.float32), rs.standard_normal((48, 32)).astype(np.float32), \
+        rs.standard_normal((64, 1)).astype(np.float32)
+    g0, g1 = rs.standard_normal((64, 48)).astype(np.float32), rs.standard_normal((64, 1)).astype(np.float32)
+
+    def program(be, block):
+        w, x, b = be.array(w0), be.array(x0), be.array(b0)
+        gw, gb = be.array(g0), be.array(g1)
+        vw, vb = be.zeros((64, 48)), be.zeros((64, 1))
+        y, act, probe = be.empty((64, 32)), be.empty((64, 32)), be.empty((64, 32))
+        launches = []
+        for step in range(3):
+            before = be.plan_stats["launches"] if hasattr(be, "plan_stats") and be.plan_stats else 0
+            if block:
+                be.begin(Block.minibatch, step)
+            be.compound_dot(w, x, y)
+            y[:] = y + b                       # bias ...
+            act[:] = be.maximum(y, 0) + 0.1 * be.minimum(y, 0)      # ... and activation: one kernel
+            probe[:] = act * 2.0
+            seen = probe.get()                 # a host read inside the block sees all of it
+            vw[:] = 0.9 * vw - 0.01 * gw
+            w[:] = w + vw
+            vb[:] = 0.9 * vb - 0.01 * gb
+            b[:] = b + vb
+            if block:
+                be.end(Block.minibatch, step)
+            if hasattr(be, "plan_stats") and be.plan_stats:
+                launches.append(be.plan_stats["launches"] - before)
+        return [t.get() for t in (w, b, vw, vb, act)] + [seen], launches
+
+    cpu, hip = pair
+    want, _ = program(cpu, True)
+    plain, n_plain = program(hip, False)
+    fused, n_fused = program(hip, True)
+    for a, b_, c in zip(want, plain, fused):
+        assert_close(b_, a, rtol=1e-5, atol=1e-6, what="outside a block")
+        assert_close(c, a, rtol=1e-5, atol=1e-6, what="inside a minibatch block")
+    # three elementwise statements after the product fuse into one launch, the four update
+    # statements into two (two shapes): 7 statements, 3 kernels
+    assert n_plain[-1] == 7 and n_fused[-1] == 3, (n_plain, n_fused)
