@@ -171,3 +171,39 @@ def test_statements_inside_a_minibatch_block_fuse_and_keep_program_order(pair):
     # three elementwise statements after the product fuse into one launch, the four update
     # statements into two (two shapes): 7 statements, 3 kernels
     assert n_plain[-1] == 7 and n_fused[-1] == 3, (n_plain, n_fused)
+
+
+@pytest.mark.gpu
+def test_vectors_read_inside_a_group_must_not_live_in_a_tensor_the_group_writes(pair):
+    """row / column vectors are read by lanes other than the ones that would
+    write them: a statement whose vector operand is a row of another
+    statement's output does not join that statement's group"""
+    rs = np.random.RandomState(12)
+    a0, b0 = rs.standard_normal((40, 96)).astype(np.float32), rs.standard_normal((40, 96)).astype(np.float32)
+    r0, c0 = rs.standard_normal((1, 96)).astype(np.float32), rs.standard_normal((40, 1)).astype(np.float32)
+    res, counts = [], []
+    for be in pair:
+        a, b, row, col = be.array(a0), be.array(b0), be.array(r0), be.array(c0)
+        out1, out2 = be.empty((40, 96)), be.empty((40, 96))
+        n0 = be.plan_stats["launches"] if getattr(be, "plan_stats", None) else 0
+        with be.fused() if hasattr(be, "fused") else _Null():
+            out1[:] = a * row + col                 # independent vectors: these two share a kernel
+            out2[:] = out1 - b * col
+        n1 = be.plan_stats["launches"] if getattr(be, "plan_stats", None) else 0
+        with be.fused() if hasattr(be, "fused") else _Null():
+            a[:] = a + 1.0                          # writes a ...
+            out2[:] = b + a[3:4, :]                 # ... whose row 3 every lane of this statement reads
+        n2 = be.plan_stats["launches"] if getattr(be, "plan_stats", None) else 0
+        res.append([t.get() for t in (out1, out2, a)])
+        counts.append((n1 - n0, n2 - n1))
+    for w, g in zip(*res):
+        assert_close(g, w, rtol=1e-5, atol=1e-6)
+    assert counts[1] == (1, 2)
+
+
+class _Null(object):
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
