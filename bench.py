@@ -194,6 +194,15 @@ def gpu_leg(steps, warmup, detail=True):
             reps=20)
     measure("C3 Adam as 3 assigns, 3 kernels (5000,5000) f32",
             lambda: configs.c3_adam_step(be, p, g, m, v, t + 2), configs.bytes_c3(fused=False), n3, reps=20)
+
+    def adam_in_minibatch():
+        # the optimizer's statements as written, inside the hint that the reference's
+        # training loop puts round every minibatch (models/model.py:204-217)
+        be.begin(Block.minibatch, 0)
+        configs.c3_adam_step(be, p, g, m, v, t + 2)
+        be.end(Block.minibatch, 0)
+    measure("C3 Adam as 3 assigns inside a minibatch block (5000,5000) f32", adam_in_minibatch,
+            configs.bytes_c3(fused=True), n3, reps=20)
     # C4
     x4h, gh, bh = configs.inputs_c4()
     x4, o4 = be.array(x4h, dtype=np.float16), be.empty(configs.C4_SHAPE, dtype=np.float16)
