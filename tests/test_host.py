@@ -600,3 +600,67 @@ def test_the_cheaper_exponential_is_for_arguments_below_their_own_maximum_only(p
                      lambda: pb.exp(pb.max(x, axis=axis) - x), lambda: pb.exp(x + pb.max(x, axis=axis))):
             src = plan_of(pb, lambda: out.__setitem__(slice(None), tree())).spec.source
             assert "expf(" in src and "nh_exp_nonpos(" not in src
+
+
+# ---- launch shapes away from the benchmark configurations ---------------------------------
+def _softmax(pb, x, axis):
+    e = pb.exp(x - pb.max(x, axis=axis))
+    return e / pb.sum(e, axis=axis)
+
+
+def _norm(pb, x, axis):
+    return (x - pb.mean(x, axis=axis)) / pb.sqrt(pb.var(x, axis=axis) + 1e-5)
+
+
+def test_short_rows_get_teams_that_fetch_whole_cache_lines(pb):
+    """four tiles per lane, but never fewer lanes per row than fetch 128 bytes per load"""
+    for shape, dtype, want in (((100000, 64), np.float32, (8, 2)), ((100000, 64), np.float16, (8, 1)),
+                               ((50000, 32), np.float32, (8, 1)), ((20000, 256), np.float32, (16, 4)),
+                               ((20000, 1000), np.float32, (64, 4))):
+        x, out = pb.empty(shape, dtype), pb.empty(shape, dtype)
+        p = plan_of(pb, lambda: out.__setitem__(slice(None), _softmax(pb, x, 1))).spec.params
+        assert (p["LX"], p["NCH"]) == want, (shape, dtype, p)
+
+
+def test_column_strips_narrow_until_every_compute_unit_has_one(pb):
+    """the widest strip whose rows fit in registers, then narrower ones -- down to 32-byte
+    row pieces -- while there are fewer strips than compute units"""
+    for shape, dtype, strips, lx in (((512, 4096), np.float32, 256, 4), ((256, 8192), np.float32, 256, 8),
+                                     ((1000, 4096), np.float16, 256, 2), ((1000, 65536), np.float32, 2048, 8)):
+        x, out = pb.empty(shape, dtype), pb.empty(shape, dtype)
+        ch = plan_of(pb, lambda: out.__setitem__(slice(None), _softmax(pb, x, 0)))
+        assert ch.spec.family == "col" and ch.grid[0] == strips and ch.spec.params["LX"] == lx, (shape, ch.grid, ch.spec.params)
+    # up to 2048 rows narrow strips are preferred to workgroups that wait for each other
+    x, out = pb.empty((2000, 2048), np.float16), pb.empty((2000, 2048), np.float16)
+    assert plan_of(pb, lambda: out.__setitem__(slice(None), _norm(pb, x, 0))).spec.family == "col"
+
+
+def test_the_cooperative_column_family_is_for_matrices_of_20_to_48_megabytes(pb):
+    x, out = pb.empty((32000, 256)), pb.empty((32000, 256))                  # 32 MB
+    assert plan_of(pb, lambda: out.__setitem__(slice(None), _softmax(pb, x, 0))).spec.family == "colcoop"
+    for shape in ((4096, 1000), (30000, 1000)):                              # 16 MB, 120 MB: in stages
+        x, out = pb.empty(shape), pb.empty(shape)
+        with pytest.raises(planner.NeedsSplit):
+            out[:] = _softmax(pb, x, 0)
+    # 16-bit matrices whose rows per lane would overflow the registers of a cooperating workgroup
+    x, out = pb.empty((5000, 5000), np.float16), pb.empty((5000, 5000), np.float16)
+    with pytest.raises(planner.NeedsSplit):
+        out[:] = _softmax(pb, x, 0)
+
+
+def test_one_tall_strip_of_long_chunks_takes_1024_lanes(pb):
+    x, line = pb.empty((600000, 64), np.float16), pb.empty((1, 64))
+    ch = plan_of(pb, lambda: line.__setitem__(slice(None), pb.sum(x, axis=0)))
+    assert ch.spec.family == "colsplit" and ch.spec.block == 1024 and ch.grid[0] == 1
+    x = pb.empty((32000, 256))
+    ch = plan_of(pb, lambda: pb.empty((1, 256)).__setitem__(slice(None), pb.max(x, axis=0)))
+    assert ch.spec.family == "colsplit" and ch.spec.block == 512
+
+
+def test_the_join_of_the_waves_reads_lds_in_batches(pb):
+    """(waves - 1) x V reads issued all at once took a 1024-lane kernel with eight values
+    per lane to over 200 registers; plain values are joined like pairs, a column shared by
+    adjacent lanes"""
+    x, out = pb.empty((32000, 256)), pb.empty((32000, 256))
+    src = plan_of(pb, lambda: out.__setitem__(slice(None), _norm(pb, x, 0))).spec.source
+    assert "const int fcol = threadIdx.x / " in src and "for (int y = 1; y < 16; ++y)" not in src
