@@ -131,6 +131,19 @@ def test_cse_and_levels(pb):
     assert sm.lse_max.op == "max" and sm.lse_max.lse_sum is sm and sm.level == sm.lse_max.level == 1
     p.unpair_lse()
     assert p.lse_pairs == 0 and p.nlevels == 2 and sm.lse_max is None and sm.level == 2
+    # ... and the planner may take it up again (twice is once)
+    p.pair_lse()
+    p.pair_lse()
+    assert p.lse_pairs == 1 and p.nlevels == 1 and sm.lse_max.op == "max"
+    # the same along rows; the row planner decides by residence whether to keep it
+    y, outy = pb.empty((64, 4096)), pb.empty((64, 4096))
+    q = _prog(pb, lambda: outy.__setitem__(slice(None), pb.exp(y - pb.max(y, axis=1)) /
+                                           pb.sum(pb.exp(y - pb.max(y, axis=1)), axis=1)))
+    assert q.axis == 1 and q.lse_pairs == 1 and q.nlevels == 1
+    # a sum of exponentials around something else than the maximum of the same operand is no pair
+    r = _prog(pb, lambda: outy.__setitem__(slice(None), pb.exp(y - pb.max(y * 2.0, axis=1)) /
+                                           pb.sum(pb.exp(y - pb.max(y * 2.0, axis=1)), axis=1)))
+    assert r.lse_pairs == 0 and r.nlevels == 2
 
 
 def test_sum_over_a_one_hot_becomes_a_gather(pb):
