@@ -677,3 +677,19 @@ def test_the_join_of_the_waves_reads_lds_in_batches(pb):
     x, out = pb.empty((32000, 256)), pb.empty((32000, 256))
     src = plan_of(pb, lambda: out.__setitem__(slice(None), _norm(pb, x, 0))).spec.source
     assert "const int fcol = threadIdx.x / " in src and "for (int y = 1; y < 16; ++y)" not in src
+
+
+def test_rows_pair_maximum_and_sum_only_where_it_saves_a_pass_or_an_exchange(pb):
+    def paired(shape, dtype):
+        x, out = pb.empty(shape, dtype), pb.empty(shape, dtype)
+        ch = plan_of(pb, lambda: out.__setitem__(slice(None), _softmax(pb, x, 1)))
+        return ch.spec.family, "nh_op_lse::stepn" in ch.spec.source
+
+    assert paired((4096, 1000), np.float32) == ("row", False)          # resident: three sweeps over registers
+    assert paired((4096, 4096), np.float16) == ("row", False)          # resident, exponentials kept in spare registers
+    assert paired((512, 131072), np.float16) == ("row", True)          # resident but no register left to keep them
+    assert paired((1000, 262144), np.float32) == ("row", True)         # partly streamed
+    assert paired((64, 1048576), np.float32) == ("rowcoop", True)      # shares that do not fit
+    assert paired((16, 1048576), np.float32) == ("rowcoop", False)     # resident fp32 shares: exponentials take x's registers
+    assert paired((16, 1605632), np.float16) == ("rowcoop", True)      # resident 16-bit shares of 13 tiles: one exchange less
+    assert paired((64, 131072), np.float16) == ("rowcoop", False)      # ... but not shares of 4 tiles
