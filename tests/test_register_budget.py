@@ -67,3 +67,18 @@ def test_generated_kernels_do_not_spill(tmp_path, what, shape, dtype, tree, axis
     # 512 registers per lane of a SIMD, shared by the waves of the workgroups resident on it
     budget = 128 if spec.block == 1024 else 256 if spec.block == 512 else 512
     assert spill == 0 and scratch == 0 and vgprs <= budget, (what, vgprs, spill, scratch)
+
+
+def test_benchmark_kernels_do_not_spill(tmp_path):
+    """every kernel of the benchmark op-trees (the ones the build step pre-compiles)"""
+    be = prebuild.PlanBackend(cache_dir=str(tmp_path / "kc"), compile_kernels=False)
+    prebuild.benchmark_statements(be)
+    seen = set()
+    for ch in be.choices:
+        if ch.spec.name in seen:
+            continue
+        seen.add(ch.spec.name)
+        vgprs, spill, scratch = _usage(ch.spec.source, tmp_path)
+        budget = 128 if ch.spec.block == 1024 else 256 if ch.spec.block == 512 else 512
+        assert spill == 0 and scratch == 0 and vgprs <= budget, (ch.spec.family, ch.spec.params, vgprs, spill, scratch)
+    assert len(seen) >= 8
