@@ -31,22 +31,29 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch from rocprofv3 counters (FETCH_SIZE and WRITE_SIZE, each scaled by what the same
-# counter reads for a plain copy kernel of known size) cannot be read from inside this process: they are
-# collected by two `rocprofv3 --pmc` runs of `bench.py --counter-pass` and kept, with the commands, in the
-# summary below, whose last line is machine-readable.
+# Figures that cannot be read from inside this process come from the committed rocprofv3 summaries (written by
+# `python -m neon_amd.profile_summary` from profiled runs of `bench.py --counter-pass` / `--trace-pass`; each
+# summary quotes its commands).  They are looked up by the NAME of the kernel that has just been timed here: when
+# the generator has changed since a summary was made, the name differs and the figure is null, never stale.
 TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "hbm_traffic_all_configs_pmc.txt")
+DURATION_SUMMARY = {"hot": os.path.join(ROOT, "profiles", "kernel_durations_hot_kernel_trace.txt"),
+                    "cold": os.path.join(ROOT, "profiles", "kernel_durations_cold_kernel_trace.txt")}
 
 
-def measured_traffic(label):
-    """HBM bytes per launch of the kernel behind ``label`` from the committed
-    counter summary, or None when there is none"""
-    try:
-        with open(TRAFFIC_SUMMARY) as f:
-            lines = [l for l in f if l.startswith("json: ")]
-        return json.loads(lines[-1][6:])[label]["traffic_bytes"]
-    except (IOError, OSError, IndexError, KeyError, ValueError):
-        return None
+def measured_traffic(kernel_name):
+    """HBM bytes per launch of ``kernel_name`` (FETCH_SIZE + WRITE_SIZE, each scaled by a
+    copy kernel of known size) from the committed counter summary, or None"""
+    from neon_amd.profile_summary import lookup
+    rec = lookup(TRAFFIC_SUMMARY, kernel_name)
+    return rec["traffic_bytes"] if rec else None
+
+
+def rocprof_us(kernel_name, mode="hot"):
+    """median rocprofv3 kernel duration (>= 50 launches after >= 10 warm-ups) of
+    ``kernel_name`` from the committed kernel-trace summary, or None"""
+    from neon_amd.profile_summary import lookup
+    rec = lookup(DURATION_SUMMARY[mode], kernel_name)
+    return rec["median_us"] if rec else None
 
 
 COLD_BYTES = 768 << 20         # tensor sets rotated through by the cold-cache rows
@@ -67,7 +74,122 @@ def _fresh(be, shape, dtype=np.float32, fill=None, rs=None, scale=1.0, shift=0.0
     return t
 
 
-def gpu_leg(steps, warmup, detail=True):
+
+class Case(object):
+    """One benchmark op-tree: ``make(k)`` allocates the k-th set of its tensors
+    (set 0 holds exactly the seeded inputs of ``neon_amd.configs``; the others
+    the same values rolled by k, so that every set of a cold-cache rotation is
+    random data too), ``issue(*tensors)`` states the tree."""
+
+    def __init__(self, label, nbytes, elements, make, issue, cold=True, reps=50):
+        self.label, self.nbytes, self.elements = label, nbytes, elements
+        self.make, self.issue, self.cold, self.reps = make, issue, cold, reps
+
+    def nsets(self):
+        return max(3, min(600, -(-COLD_BYTES // self.nbytes)))
+
+
+def baseline_cases(be):
+    """the trees of the five benchmark configurations at their full shapes,
+    plus the two floor kernels (the same structures on next to no data)"""
+    from neon_amd import configs
+    from neon_amd.backends.backend import Block
+    f32, f16, i32 = np.float32, np.float16, np.int32
+    roll = lambda a, k, axis=0: a if k == 0 else np.roll(a, 13 * k, axis=axis)
+    cases = []
+    host = {}
+
+    def inputs(name):
+        if name not in host:
+            host[name] = getattr(configs, "inputs_" + name)()
+        return host[name]
+
+    n1 = configs.C1_SHAPE[0] * configs.C1_SHAPE[1]
+
+    def make_c1(k):
+        x, y = inputs("c1")
+        return be.empty(configs.C1_SHAPE), be.array(roll(x, k)), be.array(roll(y, k))
+    cases.append(Case("C1 fused sig(0.5x+2y) (4096,128) f32", configs.bytes_c1a(), n1, make_c1,
+                      lambda o, x, y: configs.c1_fused(be, o, x, y)))
+    cases.append(Case("C1a 0.5x+2y (4096,128) f32", configs.bytes_c1a(), n1, make_c1,
+                      lambda o, x, y: configs.c1a(be, o, x, y)))
+
+    def make_c1b(k):
+        o = be.array(roll(inputs("c1")[0], k))
+        return (o,)
+    cases.append(Case("C1b sig in place (4096,128) f32", configs.bytes_c1b(), n1, make_c1b, lambda o: configs.c1b(be, o)))
+
+    def make_c2(k):
+        return be.empty(configs.C2_SHAPE), be.array(roll(inputs("c2")[0], k))
+    cases.append(Case("C2 softmax axis0 (1000,128) f32", configs.bytes_c2(), configs.C2_SHAPE[0] * configs.C2_SHAPE[1],
+                      make_c2, lambda o, x: configs.c2_softmax(be, o, x)))
+
+    n3 = configs.C3_SHAPE[0] * configs.C3_SHAPE[1]
+    step = [0]
+
+    def make_c3(k):
+        grad, param = inputs("c3")
+        tensors = be.array(param), be.array(grad), be.zeros(configs.C3_SHAPE), be.zeros(configs.C3_SHAPE)
+        host.pop("c3")
+        return tensors
+
+    def adam(p, g, m, v):
+        step[0] += 1
+        be.begin(Block.update, step[0])
+        configs.c3_adam_step(be, p, g, m, v, step[0])
+        be.end(Block.update, step[0])
+    # (700 MB per launch: far beyond every cache, so one set is already a cold run)
+    cases.append(Case("C3 Adam fused, 1 kernel (5000,5000) f32", configs.bytes_c3(fused=True), n3, make_c3, adam,
+                      cold=False, reps=20))
+
+    n4 = configs.C4_SHAPE[0] * configs.C4_SHAPE[1]
+    shared = {}
+
+    def make_c4(k):
+        x, gamma, beta = inputs("c4")
+        if "g4" not in shared:
+            shared["g4"], shared["b4"] = be.array(gamma), be.array(beta)
+        return (be.empty(configs.C4_SHAPE, dtype=f16), be.array(roll(x, k, axis=1), dtype=f16), shared["g4"], shared["b4"])
+    cases.append(Case("C4 rownorm (256,100352) f16", configs.bytes_c4(), n4, make_c4,
+                      lambda o, x, g, b: configs.c4_rownorm(be, o, x, g, b), reps=30))
+
+    n5 = configs.C5_SHAPE[0] * configs.C5_SHAPE[1]
+    line = (1, configs.C5_SHAPE[1])
+
+    def make_c5(dtype):
+        def make(k):
+            x, idx = inputs("c5")
+            if "i5" not in shared:
+                shared["i5"] = be.array(idx, dtype=i32)
+            return be.empty(line, dtype=dtype), be.array(roll(x, k))
+        return make
+    cases.append(Case("C5a argmax axis0 (32000,256) f32", configs.bytes_c5_reduce(), n5, make_c5(i32),
+                      lambda o, x: configs.c5a_argmax(be, o, x)))
+    cases.append(Case("C5b max axis0 (32000,256) f32", configs.bytes_c5_reduce(), n5, make_c5(f32),
+                      lambda o, x: configs.c5b_max(be, o, x)))
+    cases.append(Case("C5c cross-entropy axis0 (32000,256) f32, in-kernel one-hot", configs.bytes_c5c(), n5, make_c5(f32),
+                      lambda o, x: configs.c5c_cross_entropy(be, o, x, be.onehot(shared["i5"], axis=0))))
+    # floors of the latency-bound rows: what a launch, one trip to memory and back and (for the split
+    # column reduction) the publish / ticket / fold hand-off cost when there is next to nothing to stream
+    cases.append(Case("floor: elementwise kernel on 4 KB", 8192, 1024,
+                      lambda k: (be.empty((1, 1024)), be.zeros((1, 1024))),
+                      lambda o, x: o.__setitem__(slice(None), x * 2.0), cold=False))
+    cases.append(Case("floor: split column max on 1 MB (8192,32)", 4 * 8192 * 32, 8192 * 32,
+                      lambda k: (be.empty((1, 32)), be.zeros((8192, 32))),
+                      lambda o, x: o.__setitem__(slice(None), be.max(x, axis=0)), cold=False))
+    return cases
+
+
+def case_plan(be, case, tensors):
+    """the launch plan of a single-kernel case"""
+    with be.capture() as grp:
+        case.issue(*tensors)
+    assert len(grp) == 1, "%s is not one kernel" % case.label
+    _, plan = be.time_group(grp[0], reps=1)
+    return plan
+
+
+def gpu_leg(steps, warmup, detail=True, no_cold=False, hot_cold_only=False):
     from neon_amd import configs
     from neon_amd.backends import gen_backend
     from neon_amd.backends.backend import Block
@@ -111,8 +233,8 @@ def gpu_leg(steps, warmup, detail=True):
     ms, plan = be.time_group(groups[0], reps=max(steps, 5))
     out["roofline"] = {"bound": "hbm", "achieved": step_bytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
                        "unit": "GB/s", "frac": step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                       "traffic": measured_traffic("C3 fused Adam"), "kernel": plan.spec.name, "kernel_ms": ms,
-                       "algorithmic_bytes": step_bytes}
+                       "traffic": measured_traffic(plan.spec.name), "kernel": plan.spec.name, "kernel_ms": ms,
+                       "kernel_us_rocprof": rocprof_us(plan.spec.name, "hot"), "algorithmic_bytes": step_bytes}
     if not detail:
         return out, be
 
@@ -133,22 +255,34 @@ def gpu_leg(steps, warmup, detail=True):
         be.synchronize()
         return (time.perf_counter() - t0) * 1e3 / reps
 
+    def finish(row, nbytes, elements, mode="hot"):
+        row["gbs"] = nbytes / (row["ms"] * 1e-3) / 1e9
+        row["frac_of_hbm_peak"] = row["gbs"] / HBM_PEAK_GBS
+        row["elements_per_s"] = elements / (row["ms"] * 1e-3) if elements else None
+        # the same kernel's median duration in the committed rocprofv3 kernel trace (by kernel name)
+        us = rocprof_us(row["kernel"], mode) if row.get("kernel") else None
+        row["kernel_us_rocprof"] = us
+        row["frac_rocprof"] = (nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS) if us else None
+        row["traffic"] = measured_traffic(row["kernel"]) if row.get("kernel") else None
+        rows.append(row)
+
     def measure(label, issue, nbytes, elements, reps=50):
         from neon_amd.backends.hip.planner import NeedsSplit
         from neon_amd.backends.hip.optree_ir import MixedAxes
         with be.capture() as grp:
             issue()
-        row = {"config": label, "bytes": nbytes}
+        row = {"config": label, "bytes": nbytes, "kernel": None}
         try:
-            total, names = 0.0, []
+            total, names, kernels = 0.0, [], []
             for trees in grp:
                 ms_k, pl = be.time_group(trees, reps=reps)
                 total += ms_k
+                kernels.append(pl.spec.name)
                 names.append("%s[%s]" % (pl.spec.family, ",".join(
                     "%s=%s" % kv for kv in sorted(pl.spec.params.items())
                     if kv[0] in ("V", "LX", "LY", "NCH", "NR"))))
             row.update({"kernels": len(grp), "ms": total, "timing": "HIP events around back-to-back launches",
-                        "plan": " + ".join(names)})
+                        "plan": " + ".join(names), "kernel": kernels[0] if len(kernels) == 1 else None})
         except (NeedsSplit, MixedAxes):
             before = be.plan_stats["launches"]
             issue()
@@ -156,42 +290,56 @@ def gpu_leg(steps, warmup, detail=True):
             row["ms"] = api_ms(issue, reps)
             row["timing"] = "wall clock per API call (several kernels through temporaries)"
         row["api_ms"] = api_ms(issue, reps)
-        row["gbs"] = nbytes / (row["ms"] * 1e-3) / 1e9
-        row["frac_of_hbm_peak"] = row["gbs"] / HBM_PEAK_GBS
-        row["elements_per_s"] = elements / (row["ms"] * 1e-3)
-        rows.append(row)
+        finish(row, nbytes, elements)
+
+    # the same trees with cold caches: each launch works on another set of tensors, enough sets
+    # (>= 768 MB in total) that neither the L2s nor the 256 MB memory-side cache hold them
+    def measure_cold(case):
+        nsets = case.nsets()
+        sets = [case.make(k) for k in range(nsets)]
+        groups = []
+        for tensors in sets:
+            with be.capture() as grp:
+                case.issue(*tensors)
+            assert len(grp) == 1, "cold rows are single-kernel trees"
+            groups.append(grp[0])
+        be.time_group_sets(groups, reps=nsets)                    # touch every buffer once
+        ms_k, pl = be.time_group_sets(groups, reps=max(2 * nsets, 60))
+        finish({"config": case.label + " [cold]", "bytes": case.nbytes, "kernels": 1, "ms": ms_k, "api_ms": None,
+                "timing": "HIP events around launches rotating over %d tensor sets of seeded random data" % nsets,
+                "plan": pl.spec.family, "kernel": pl.spec.name}, case.nbytes, case.elements, mode="cold")
+        del sets, groups
+
+    for case in baseline_cases(be):
+        if case.label.startswith("C3"):
+            tensors = (p, g, m, v)          # the headline's tensors (400 MB) serve
+        else:
+            tensors = case.make(0)
+        measure(case.label + ("" if case.nbytes > (256 << 20) or case.label.startswith("floor") else " [cache-hot]"),
+                lambda: case.issue(*tensors), case.nbytes, case.elements, reps=case.reps)
+        del tensors
+        if case.cold and not no_cold:
+            measure_cold(case)
+    if hot_cold_only:
+        out["per_config"] = rows
+        return out, be
 
     rs = np.random.RandomState(11)
-    # C1
-    x1, y1 = (be.array(a) for a in configs.inputs_c1())
-    o1 = be.empty(configs.C1_SHAPE)
-    n1 = configs.C1_SHAPE[0] * configs.C1_SHAPE[1]
-    measure("C1a 0.5x+2y (4096,128) f32 [cache-hot]", lambda: configs.c1a(be, o1, x1, y1), configs.bytes_c1a(), n1)
-    measure("C1b sig in place (4096,128) f32 [cache-hot]", lambda: configs.c1b(be, o1), configs.bytes_c1b(), n1)
-    measure("C1 fused sig(0.5x+2y) (4096,128) f32 [cache-hot]", lambda: configs.c1_fused(be, o1, x1, y1),
-            configs.bytes_c1a(), n1)
+    n3 = configs.C3_SHAPE[0] * configs.C3_SHAPE[1]
+    # the trees whose working set fits in cache, at >= 256 MB (what the same kernels do when bandwidth is the limit)
     big = (16384, 4096)   # 256 MiB per tensor
     xb, yb, ob = _fresh(be, big, rs=rs), _fresh(be, big, rs=rs), be.empty(big)
     nb = big[0] * big[1]
     measure("C1a scaled (16384,4096) f32", lambda: configs.c1a(be, ob, xb, yb), configs.bytes_c1a(big), nb, reps=10)
     measure("C1b scaled (16384,4096) f32", lambda: configs.c1b(be, ob), configs.bytes_c1b(big), nb, reps=10)
-    # C2
-    (x2h,) = configs.inputs_c2()
-    x2, o2 = be.array(x2h), be.empty(configs.C2_SHAPE)
-    measure("C2 softmax axis0 (1000,128) f32 [cache-hot]", lambda: configs.c2_softmax(be, o2, x2),
-            configs.bytes_c2(), x2h.size)
+    del yb, xb
     wide = (1000, 65536)  # same depth, 512x the columns: 262 MB per tensor
-    del yb
-    xw = be.empty(wide)
-    xw[:] = 0.001
+    xw = _fresh(be, wide, rs=rs, scale=3.0)
     ow = ob.share(wide)
     measure("C2 softmax axis0 scaled (1000,65536) f32", lambda: configs.c2_softmax(be, ow, xw),
             configs.bytes_c2(wide), wide[0] * wide[1], reps=10)
-    del xw, ow, xb, ob
-    # C3
-    n3 = configs.C3_SHAPE[0] * configs.C3_SHAPE[1]
-    measure("C3 Adam fused, 1 kernel (5000,5000) f32", lambda: adam_step(t + 2), configs.bytes_c3(fused=True), n3,
-            reps=20)
+    del xw, ow, ob
+    # C3 as the API states it
     measure("C3 Adam as 3 assigns, 3 kernels (5000,5000) f32",
             lambda: configs.c3_adam_step(be, p, g, m, v, t + 2), configs.bytes_c3(fused=False), n3, reps=20)
 
@@ -203,87 +351,29 @@ def gpu_leg(steps, warmup, detail=True):
         be.end(Block.minibatch, 0)
     measure("C3 Adam as 3 assigns inside a minibatch block (5000,5000) f32", adam_in_minibatch,
             configs.bytes_c3(fused=True), n3, reps=20)
-    # C4
+    # C4 on bfloat16 storage; C5a and C5b in one launch
+    from neon_amd.backends import bfloat16
     x4h, gh, bh = configs.inputs_c4()
     x4, o4 = be.array(x4h, dtype=np.float16), be.empty(configs.C4_SHAPE, dtype=np.float16)
     g4, b4 = be.array(gh), be.array(bh)
-    measure("C4 rownorm (256,100352) f16", lambda: configs.c4_rownorm(be, o4, x4, g4, b4), configs.bytes_c4(),
-            x4h.size, reps=30)
     del x4h
-    # C5
+    x4b, o4b = be.empty(configs.C4_SHAPE, dtype=bfloat16), be.empty(configs.C4_SHAPE, dtype=bfloat16)
+    x4b[:] = x4
+    measure("C4 rownorm (256,100352) bf16", lambda: configs.c4_rownorm(be, o4b, x4b, g4, b4), configs.bytes_c4(),
+            configs.C4_SHAPE[0] * configs.C4_SHAPE[1], reps=30)
+    del x4b, o4b
     x5h, i5h = configs.inputs_c5()
     x5 = be.array(x5h)
-    i5 = be.array(i5h, dtype=np.int32)
     am = be.empty((1, configs.C5_SHAPE[1]), dtype=np.int32)
-    mx, ce = be.empty((1, configs.C5_SHAPE[1])), be.empty((1, configs.C5_SHAPE[1]))
+    mx = be.empty((1, configs.C5_SHAPE[1]))
     n5 = x5h.size
     del x5h
-    measure("C5a argmax axis0 (32000,256) f32", lambda: configs.c5a_argmax(be, am, x5), configs.bytes_c5_reduce(), n5)
-    measure("C5b max axis0 (32000,256) f32", lambda: configs.c5b_max(be, mx, x5), configs.bytes_c5_reduce(), n5)
-    measure("C5c cross-entropy axis0 (32000,256) f32, in-kernel one-hot",
-            lambda: configs.c5c_cross_entropy(be, ce, x5, be.onehot(i5, axis=0)), configs.bytes_c5c(), n5)
 
     def c5ab():
         with be.fused():
             configs.c5a_argmax(be, am, x5)
             configs.c5b_max(be, mx, x5)
     measure("C5a+b argmax and max in one launch (32000,256) f32", c5ab, configs.bytes_c5_reduce() + 4 * configs.C5_SHAPE[1], n5)
-    # C4 on bfloat16 storage
-    from neon_amd.backends import bfloat16
-    x4b, o4b = be.empty(configs.C4_SHAPE, dtype=bfloat16), be.empty(configs.C4_SHAPE, dtype=bfloat16)
-    x4b[:] = x4
-    measure("C4 rownorm (256,100352) bf16", lambda: configs.c4_rownorm(be, o4b, x4b, g4, b4), configs.bytes_c4(),
-            configs.C4_SHAPE[0] * configs.C4_SHAPE[1], reps=30)
-    del x4b, o4b
-    # floors of the latency-bound rows: the same kernel structures on next to no data -- what a
-    # launch, one trip to memory and back, and (for the split column reductions) the
-    # publish / ticket / fold hand-off cost when there is nothing to stream
-    tiny_x, tiny_o = be.zeros((1, 1024)), be.empty((1, 1024))
-    measure("floor: elementwise kernel on 4 KB", lambda: tiny_o.__setitem__(slice(None), tiny_x * 2.0), 8192, 1024)
-    small = be.zeros((8192, 32))
-    small_o = be.empty((1, 32))
-    measure("floor: split column max on 1 MB (8192,32)", lambda: small_o.__setitem__(slice(None), be.max(small, axis=0)),
-            4 * 8192 * 32, 8192 * 32)
-    # ---- the same trees with cold caches: each launch works on another set of tensors, enough
-    #      sets (>= 768 MB in total) that neither the L2s nor the 256 MB memory-side cache hold them
-    def measure_cold(label, make_set, issue, nbytes, elements):
-        nsets = max(3, min(600, -(-COLD_BYTES // nbytes)))
-        sets = [make_set() for _ in range(nsets)]
-        groups = []
-        for tensors in sets:
-            with be.capture() as grp:
-                issue(*tensors)
-            assert len(grp) == 1, "cold rows are single-kernel trees"
-            groups.append(grp[0])
-        be.time_group_sets(groups, reps=nsets)                    # touch every buffer once
-        ms_k, pl = be.time_group_sets(groups, reps=max(2 * nsets, 60))
-        rows.append({"config": label, "bytes": nbytes, "kernels": 1, "ms": ms_k, "api_ms": None,
-                     "timing": "HIP events around launches rotating over %d tensor sets" % nsets,
-                     "plan": pl.spec.family, "gbs": nbytes / (ms_k * 1e-3) / 1e9,
-                     "frac_of_hbm_peak": nbytes / (ms_k * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "elements_per_s": elements / (ms_k * 1e-3)})
-        del sets, groups
-
-    f16, i32 = np.float16, np.int32
-    measure_cold("C1 fused sig(0.5x+2y) (4096,128) f32 [cold]",
-                 lambda: (be.empty(configs.C1_SHAPE), be.zeros(configs.C1_SHAPE), be.zeros(configs.C1_SHAPE)),
-                 lambda o, x, y: configs.c1_fused(be, o, x, y), configs.bytes_c1a(), n1)
-    measure_cold("C2 softmax axis0 (1000,128) f32 [cold]",
-                 lambda: (be.empty(configs.C2_SHAPE), be.zeros(configs.C2_SHAPE)),
-                 lambda o, x: configs.c2_softmax(be, o, x), configs.bytes_c2(), configs.C2_SHAPE[0] * configs.C2_SHAPE[1])
-    measure_cold("C4 rownorm (256,100352) f16 [cold]",
-                 lambda: (be.empty(configs.C4_SHAPE, dtype=f16), be.zeros(configs.C4_SHAPE, dtype=f16)),
-                 lambda o, x: configs.c4_rownorm(be, o, x, g4, b4), configs.bytes_c4(),
-                 configs.C4_SHAPE[0] * configs.C4_SHAPE[1])
-    measure_cold("C5a argmax axis0 (32000,256) f32 [cold]",
-                 lambda: (be.empty((1, configs.C5_SHAPE[1]), dtype=i32), be.zeros(configs.C5_SHAPE)),
-                 lambda o, x: configs.c5a_argmax(be, o, x), configs.bytes_c5_reduce(), n5)
-    measure_cold("C5b max axis0 (32000,256) f32 [cold]",
-                 lambda: (be.empty((1, configs.C5_SHAPE[1])), be.zeros(configs.C5_SHAPE)),
-                 lambda o, x: configs.c5b_max(be, o, x), configs.bytes_c5_reduce(), n5)
-    measure_cold("C5c cross-entropy axis0 (32000,256) f32 [cold]",
-                 lambda: (be.empty((1, configs.C5_SHAPE[1])), be.zeros(configs.C5_SHAPE)),
-                 lambda o, x: configs.c5c_cross_entropy(be, o, x, be.onehot(i5, axis=0)), configs.bytes_c5c(), n5)
     # ---- the prebuilt hand-written kernels behind the direct C-ABI entry points ------------
     lib = rt.lib
     e0, e1 = rt.event(), rt.event()
@@ -512,14 +602,14 @@ def counter_pass():
     plain copy kernel of known size (the calibration: 100 MB read, 100 MB
     written) and of the kernel behind every benchmark configuration and the
     batch-norm pair.  Prints which kernel belongs to which configuration and
-    its algorithmic bytes."""
+    its algorithmic bytes (the table ``neon_amd.profile_summary`` joins with
+    the counter files)."""
     from neon_amd import configs
     from neon_amd.backends import gen_backend
-    from neon_amd.backends.backend import Block
     be = gen_backend("hip", rng_seed=0)
     be.bsz = 1
     rs = np.random.RandomState(3)
-    f16, i32 = np.float16, np.int32
+    f16 = np.float16
     table = []
 
     def run(label, nbytes, issue, reps=3):
@@ -531,50 +621,67 @@ def counter_pass():
             issue()
             be.synchronize()
         table.append({"label": label, "kernel": plan.spec.name, "family": plan.spec.family,
-                      "algorithmic_bytes": nbytes})
+                      "algorithmic_bytes": nbytes, "warmup": 0, "launches": reps + 1})
 
-    g = _fresh(be, configs.C3_SHAPE, rs=rs, scale=1e-2)
-    p = _fresh(be, configs.C3_SHAPE, rs=rs, scale=0.05)
-    m, v = be.zeros(configs.C3_SHAPE), be.zeros(configs.C3_SHAPE)
-    run("copy (calibration)", 200000000, lambda: m.__setitem__(slice(None), g * 1.0))
-    v[:] = 0
-    m[:] = 0
-    step = [0]
-
-    def adam():
-        step[0] += 1
-        be.begin(Block.update, step[0])
-        configs.c3_adam_step(be, p, g, m, v, step[0])
-        be.end(Block.update, step[0])
-    run("C3 fused Adam", configs.bytes_c3(fused=True), adam)
-    del g, p, m, v
-    x1, y1 = (be.array(a) for a in configs.inputs_c1())
-    o1 = be.empty(configs.C1_SHAPE)
-    run("C1 fused sig(0.5x+2y)", configs.bytes_c1a(), lambda: configs.c1_fused(be, o1, x1, y1))
-    x2, o2 = be.array(configs.inputs_c2()[0]), be.empty(configs.C2_SHAPE)
-    run("C2 softmax", configs.bytes_c2(), lambda: configs.c2_softmax(be, o2, x2))
+    src = _fresh(be, configs.C3_SHAPE, rs=rs, scale=1e-2)
+    dst = be.empty(configs.C3_SHAPE)
+    run("copy (calibration)", 200000000, lambda: dst.__setitem__(slice(None), src * 1.0))
+    del src, dst
+    for case in baseline_cases(be):
+        if case.label.startswith("floor"):
+            continue
+        tensors = case.make(0)
+        run(case.label, case.nbytes, lambda: case.issue(*tensors))
+        del tensors
+    K, N = configs.C4_SHAPE
     x4 = _fresh(be, configs.C4_SHAPE, dtype=f16, rs=rs, scale=2.0, shift=0.5)
     o4 = be.empty(configs.C4_SHAPE, dtype=f16)
-    g4, b4 = be.ones((configs.C4_SHAPE[0], 1)), be.zeros((configs.C4_SHAPE[0], 1))
-    run("C4 rownorm f16", configs.bytes_c4(), lambda: configs.c4_rownorm(be, o4, x4, g4, b4))
-    K, N = configs.C4_SHAPE
     vec = lambda fill: _fresh(be, (K, 1), fill=fill)
     xsum, xvar, gmean, gvar, gamma, beta = vec(0.0), vec(0.0), vec(0.0), vec(1.0), vec(1.0), vec(0.0)
-    run("BN fprop f16", 2 * K * N * 2, lambda: be.compound_fprop_bn(x4, xsum, xvar, gmean, gvar, gamma, beta, o4,
-                                                                    1e-5, 0.9, True))
+    run("BN fprop (256,100352) f16", 2 * K * N * 2,
+        lambda: be.compound_fprop_bn(x4, xsum, xvar, gmean, gvar, gamma, beta, o4, 1e-5, 0.9, True))
     delta = _fresh(be, (K, N), dtype=f16, rs=rs, scale=0.1)
     gg, gb = vec(0.0), vec(0.0)
-    run("BN bprop f16", 3 * K * N * 2, lambda: be.compound_bprop_bn(o4, gg, gb, delta, x4, xsum, xvar, gamma, 1e-5))
-    del x4, o4, delta
-    x5 = _fresh(be, configs.C5_SHAPE, rs=rs, scale=4.0)
-    i5 = be.array(rs.randint(0, configs.C5_SHAPE[0], size=(1, configs.C5_SHAPE[1])).astype(i32), dtype=i32)
-    am = be.empty((1, configs.C5_SHAPE[1]), dtype=i32)
-    mx, ce = be.empty((1, configs.C5_SHAPE[1])), be.empty((1, configs.C5_SHAPE[1]))
-    run("C5a argmax", configs.bytes_c5_reduce(), lambda: configs.c5a_argmax(be, am, x5))
-    run("C5b max", configs.bytes_c5_reduce(), lambda: configs.c5b_max(be, mx, x5))
-    run("C5c cross-entropy", configs.bytes_c5c(),
-        lambda: configs.c5c_cross_entropy(be, ce, x5, be.onehot(i5, axis=0)))
-    print(json.dumps({"counter_pass": table}))
+    run("BN bprop (256,100352) f16", 3 * K * N * 2,
+        lambda: be.compound_bprop_bn(o4, gg, gb, delta, x4, xsum, xvar, gamma, 1e-5))
+    print(json.dumps({"pass": "counters", "rows": table}))
+
+
+TRACE_WARMUP, TRACE_LAUNCHES = 12, 60
+
+
+def trace_pass(mode):
+    """The program behind the kernel-duration summaries
+    (``rocprofv3 --kernel-trace -- python3 bench.py --trace-pass hot``, then
+    ``cold``): for every benchmark configuration TRACE_WARMUP warm-up launches
+    and TRACE_LAUNCHES measured ones of its kernel, through the public API --
+    ``hot`` on one set of tensors, ``cold`` rotating over enough sets (>= 768 MB
+    of seeded random data) that no launch finds its operands in a cache, every
+    set touched during the warm-up.  Prints the table that
+    ``neon_amd.profile_summary durations`` joins with the trace."""
+    from neon_amd.backends import gen_backend
+    be = gen_backend("hip", rng_seed=0)
+    be.bsz = 1
+    table = []
+    for case in baseline_cases(be):
+        if mode == "cold" and not case.cold:
+            continue
+        nsets = case.nsets() if mode == "cold" else 1
+        sets = [case.make(k) for k in range(nsets)]
+        plan = case_plan(be, case, sets[0])
+        warm = max(TRACE_WARMUP, nsets)
+        for i in range(warm + TRACE_LAUNCHES):
+            case.issue(*sets[i % nsets])
+        be.synchronize()
+        table.append({"label": case.label + (" [cold, %d sets]" % nsets if mode == "cold" else ""),
+                      "kernel": plan.spec.name, "family": plan.spec.family, "algorithmic_bytes": case.nbytes,
+                      "warmup": warm + 1, "launches": TRACE_LAUNCHES})        # (+1: the launch that made the plan)
+        del sets
+    what = ("every launch on the same tensors (cache-hot where the working set fits a cache)" if mode == "hot" else
+            "launches rotating over >= 768 MB of distinct tensor sets (cold caches)")
+    note = ("Back-to-back launches through the public API, no synchronisation in between." if mode == "hot" else
+            "Sets hold the configuration's seeded inputs rolled by 13 rows per set: random data in every launch.")
+    print(json.dumps({"pass": mode, "what": what, "note": note, "rows": table}))
 
 
 def shape_sweep(dtype_name):
@@ -637,6 +744,11 @@ def main():
     ap.add_argument("--no-detail", action="store_true", help="headline only, no per-config table")
     ap.add_argument("--counter-pass", action="store_true",
                     help="short untimed run for rocprofv3 --pmc (see counter_pass)")
+    ap.add_argument("--trace-pass", choices=("hot", "cold"), default=None,
+                    help="the launches a rocprofv3 --kernel-trace run summarises (see trace_pass)")
+    ap.add_argument("--no-cold", action="store_true", help="skip the cold-cache rows")
+    ap.add_argument("--configs-only", action="store_true",
+                    help="headline + the benchmark configurations (hot and cold), none of the widened rows")
     ap.add_argument("--sweep", metavar="DTYPE", default=None,
                     help="common trees over a grid of shapes (float32 / float16), see shape_sweep")
     args = ap.parse_args()
@@ -645,8 +757,13 @@ def main():
         __graft_entry__.ensure_built()
         shape_sweep(args.sweep)
         return
-    if args.counter_pass:
-        counter_pass()
+    if args.counter_pass or args.trace_pass:
+        import __graft_entry__
+        __graft_entry__.ensure_built()
+        if args.counter_pass:
+            counter_pass()
+        else:
+            trace_pass(args.trace_pass)
         return
     if args.gpus != 1:
         print("bench.py measures one MI355X; --gpus %d is not supported (the op-tree path has no "
@@ -655,7 +772,8 @@ def main():
 
     import __graft_entry__
     __graft_entry__.ensure_built()
-    gpu, be = gpu_leg(args.steps, args.warmup, detail=not args.no_detail)
+    gpu, be = gpu_leg(args.steps, args.warmup, detail=not args.no_detail, no_cold=args.no_cold,
+                      hot_cold_only=args.configs_only)
     cpu = None if args.no_cpu else cpu_leg()
     line = {
         "metric": "fused op-tree HBM GB/s (% of MI355X peak) + elements/s vs CPU backend",
@@ -673,19 +791,44 @@ def main():
     }
     if cpu:
         line["gpu_over_cpu"] = gpu["value_gbs"] / cpu["value"]
-    if "per_config" in gpu:
-        # the readable table goes to stderr; the JSON line keeps short rows
-        print("%-72s %9s %9s %7s  %s" % ("config", "kernel us", "API us", "of peak", "plan"), file=sys.stderr)
-        for r in gpu["per_config"]:
-            print("%-72s %9.2f %9s %7.3f  %s" % (r["config"][:72], r["ms"] * 1e3,
-                                                 ("%.2f" % (r["api_ms"] * 1e3)) if r.get("api_ms") else "-",
-                                                 r["frac_of_hbm_peak"], r["plan"]), file=sys.stderr)
-        line["per_config"] = [{"config": r["config"], "us": round(r["ms"] * 1e3, 3),
-                               "api_us": round(r["api_ms"] * 1e3, 3) if r.get("api_ms") else None,
-                               "bytes": r["bytes"], "gbs": round(r["gbs"], 1), "frac": round(r["frac_of_hbm_peak"], 4),
-                               "kernels": r["kernels"], "plan": r["plan"].split("[")[0] if "+" not in r["plan"] else r["plan"]}
-                              for r in gpu["per_config"]]
+    per_config = gpu.get("per_config")
+    if per_config:
+        def short(r):
+            d = {"config": r["config"], "us": round(r["ms"] * 1e3, 3),
+                 "api_us": round(r["api_ms"] * 1e3, 3) if r.get("api_ms") else None,
+                 "bytes": r["bytes"], "gbs": round(r["gbs"], 1), "frac": round(r["frac_of_hbm_peak"], 4),
+                 "kernels": r["kernels"], "plan": r["plan"].split("[")[0] if "+" not in r["plan"] else r["plan"]}
+            if r.get("kernel"):
+                d["kernel"] = r["kernel"]
+                d["kernel_us_rocprof"] = r.get("kernel_us_rocprof")
+                d["frac_rocprof"] = round(r["frac_rocprof"], 4) if r.get("frac_rocprof") else None
+                d["traffic"] = r.get("traffic")
+            return d
+        line["per_config"] = [short(r) for r in per_config]
     print(json.dumps(line))
+    sys.stdout.flush()
+    if per_config:
+        # The readable table goes to stderr AFTER the JSON line, the benchmark configurations last, so that
+        # a reader who keeps only the end of the output still has them.  `events us` = HIP events around
+        # back-to-back launches (includes the dispatch gap between launches); `rocprof us` = median kernel
+        # duration of the same kernel (by name) in the committed rocprofv3 kernel trace, `-` when the
+        # committed summary was made from another version of the kernel.
+        fmt = "%-68s %9s %8s %10s %8s %8s  %s"
+        named = lambda r: r["config"][:2] in ("C1", "C2", "C3", "C4", "C5") and "scaled" not in r["config"] \
+            and "prebuilt" not in r["config"] and "bf16" not in r["config"] and "assigns" not in r["config"] \
+            and "C5a+b" not in r["config"]
+        for title, sel in (("operations around the path, scaled instances, prebuilt entry points", lambda r: not named(r)),
+                           ("benchmark configurations (fractions of 8 TB/s on algorithmic bytes)", named)):
+            print("\n" + title, file=sys.stderr)
+            print(fmt % ("config", "events us", "of peak", "rocprof us", "of peak", "API us", "plan"), file=sys.stderr)
+            for r in per_config:
+                if not sel(r):
+                    continue
+                ru, rf = r.get("kernel_us_rocprof"), r.get("frac_rocprof")
+                print(fmt % (r["config"][:68], "%.2f" % (r["ms"] * 1e3), "%.3f" % r["frac_of_hbm_peak"],
+                             ("%.2f" % ru) if ru else "-", ("%.3f" % rf) if rf else "-",
+                             ("%.2f" % (r["api_ms"] * 1e3)) if r.get("api_ms") else "-", r["plan"][:40]), file=sys.stderr)
+        sys.stderr.flush()
 
 
 if __name__ == "__main__":

@@ -201,9 +201,10 @@ int nh_colmax_argmax_f32(float* maxval, int32_t* argmax, const float* x,
  * NH_STATIC_SCRATCH_BYTES that every device holds from library load until the
  * process ends.  There is no counterpart in the reference (PyCUDA allocates
  * freely; neon/backends/nervanagpu.py:87,147).  Shapes whose partials do not
- * fit (16 KiB of tickets + row chunks * cols * 8 bytes; the launch geometry
- * keeps that within the array for every matrix whose row length is a multiple
- * of four, and for other row lengths up to about 8000 columns) are refused
+ * fit (256 KiB of tickets, a 64-byte line per column strip, + row chunks *
+ * cols * 8 bytes; the launch geometry keeps that within the array for every
+ * matrix whose row length is a multiple of four, and for other row lengths
+ * up to about 6000 columns) are refused
  * with NH_EINVAL before anything is launched.  All calls on one device
  * share the array: calls that overlap in time on one device (different
  * streams or threads) race; calls on one stream are safe back to back (the

@@ -30,6 +30,7 @@ constant slot, ``R``, ``C``, then family-specific extras.
 """
 import hashlib
 import os
+import re
 
 from neon_amd.backends.hip.optree_ir import DTYPE_CODE, used_nodes
 
@@ -460,13 +461,29 @@ def _needed(targets, available):
     return [seen[k] for k in sorted(seen)]
 
 
-def _kernel_name(family, source_body):
-    return "nk_%s_%s" % (family, hashlib.sha1(source_body.encode()).hexdigest()[:16])
+KERNEL_NAME_OPS = 10      # operators spelled out in a kernel's name (the reference: 15, float_ew.py:478-479)
+
+
+def _kernel_name(family, source_body, prog=None):
+    """``nk_<family>_<operators>_<hash>``: the tree's operators in evaluation
+    order, so that a profiler row can be read without a side table (the
+    reference joins its op names the same way, float_ew.py:478-479, 590), then
+    a hash of the generated text."""
+    ops = []
+    if prog is not None:
+        for n in used_nodes([st.root for st in prog.statements]):
+            if n.kind in ("E", "R", "G", "H") and n.op:
+                ops.append(re.sub(r"\W", "", n.op))
+    if len(ops) > KERNEL_NAME_OPS:
+        ops = ops[:KERNEL_NAME_OPS] + ["etc"]
+    if not ops:
+        ops = ["copy"]
+    return "nk_%s_%s_%s" % (family, "_".join(ops), hashlib.sha1(source_body.encode()).hexdigest()[:12])
 
 
 def _finish(family, g, head, fmt, block, lds, params):
     body = g.L.text()
-    name = _kernel_name(family, head + body + repr(sorted(params.items())))
+    name = _kernel_name(family, head + body + repr(sorted(params.items())), g.prog)
     src = head.replace("@NAME@", name) + body
     return Spec(family, name, src, fmt, block, lds, params)
 
@@ -1998,30 +2015,51 @@ COLSPLIT_MAX_CHUNKS = 128
 
 
 COLSPLIT_FOLD_BATCH = 4
+# fewest rows a lane of the split column family takes from its chunk
+COLSPLIT_ROWS_IN_FLIGHT = 4
+# Rows a lane of the split column family loads at once (all issued before the first is used), and
+# rows of such a batch that a pair reduction takes at a time; the former times the words a row
+# position costs bounds the registers held.  Measured on (32000,256) fp32, max / argmax /
+# cross-entropy in microseconds: 4 rows 5.2 / 6.9 / 8.3, 8 rows 5.2 / 6.5 / 7.8, 16 rows (pairs
+# 16 at a time) 5.6 / 6.7 / 8.2, 16 rows (pairs 4 at a time) 5.6 / 7.3 / 8.5.
+COLSPLIT_BATCH_ROWS = 8
+COLSPLIT_SUBBATCH_ROWS = 8
+COLSPLIT_BATCH_WORDS = 64
+# The ticket counters of neighbouring strips sit this many 32-bit words apart.  Atomics on one
+# cache line are served one after the other, whichever words of it they address: with the
+# counters of all strips in one line, the 256 workgroups of an (8 strips x 32 chunks) grid queued
+# behind each other for 2 us (max over (32000,256): 7.3 -> 5.1 us with a line per strip).
+TICKET_STRIDE_WORDS = 64
 
 
-COLSPLIT_ROWS_IN_FLIGHT = int(os.environ.get("NEON_HIP_CS_U", "4"))
-
-
-def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1):
+def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, NB=4, multi=True):
     """One level of axis-0 reductions over a tall matrix.  grid = (column
-    strips, row chunks).  Each workgroup reduces its chunk, leaves one partial
-    per column in the workspace and takes a ticket; the workgroup that draws
-    the last ticket of its strip folds the partials, evaluates the statements
-    (one value per column) and stores them.  Tickets live in the workspace,
-    start at zero and are reset by their last user.
+    strips, row chunks); a workgroup is LX column-lanes x LY row-lanes.
+    ``multi``: more than one chunk per strip.
+
+    Sweep.  A lane takes its rows NR at a time: all NR loads are issued before
+    the first value is used (a chunk of at most NR * LY rows is fetched in ONE
+    round of requests).  Pair reductions then take the rows NB at a time: a
+    maximum per element and one scan for its first position for
+    arg-reductions, one local maximum and one exponential per element for the
+    running (max, sum) pair.  Only a batch that reaches beyond the chunk takes
+    the row-by-row form.
 
     The part after the sweep is a chain of dependent steps on a few values, so
-    it is kept short rather than wide (measured on (32000,256) argmax: 14.4 ->
-    9.7 us): the row-lanes of a wave fold by lane exchanges, LDS joins the
-    waves with ONE lane per column doing the join and publishing that column's
-    partial; in the last workgroup P adjacent lanes share a column, each takes
-    every P-th chunk (``fold_batch`` loads in flight) and a DPP all-reduce over
-    the P lanes finishes -- no second pass through LDS.  Results reach the
-    lanes that evaluate the statements through LDS.
+    it is kept short rather than wide: the row-lanes of a wave fold by lane
+    exchanges (arg-reductions as 64-bit keys, nh_arg_key: a merge is an
+    integer maximum), LDS joins the waves with ONE lane per column doing the
+    join and -- with several chunks per strip -- publishing that column's
+    partial; then the workgroup takes a ticket, and the one that draws the
+    strip's last ticket folds the partials: P adjacent lanes share a column,
+    each takes every P-th chunk (``fold_batch`` loads in flight), a DPP
+    all-reduce over the P lanes finishes.  Results reach the lanes that
+    evaluate the statements through LDS.
 
     Extra parameters: ``rows_per_chunk``, workspace pointer (partials first,
-    tickets after ``ticket_offset`` bytes)."""
+    then one ticket per strip, TICKET_STRIDE_WORDS words apart, after
+    ``ticket_offset`` bytes; tickets start at zero and are reset by their
+    last user)."""
     assert prog.nlevels == 1
     g = _RedGen(prog, V, stream, "colsplit")
     g.col_tail = bool(tail)     # partial last column tile, as in gen_col
@@ -2030,7 +2068,8 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1):
     S = LX * V                  # columns of a strip
     assert LX < 64 and T % 64 == 0 and S <= T
     WY = T // 64
-    P = min(T // S, 64)         # lanes per column in the last workgroup's fold
+    P = min(T // S, 64)         # lanes per column in the folding workgroup
+    NB = max(1, min(NB, NR))
     params, fmt = g.param_list([("int rows_per_chunk", "i"), ("char* ws", "P"),
                                 ("long long ticket_offset", "q")])
     head = ('extern "C" __global__ __launch_bounds__(%d) void @NAME@(%s)\n' % (T, params))
@@ -2038,16 +2077,19 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1):
     for st in prog.statements:
         assert st.out.shape[0] == 1
     done = {}
-
+    # what the stages after a lane's own sweep merge with: arg-reductions travel as keys
+    fold_op = dict((n.nid, "nh_op_key" if n.is_index else g.red_op(n)) for n in reds)
     L.open("")
-    lds = 4
+    lds = 16
     for n in reds:
         ty_ = "nh_pair" if g.is_pair(n) else "float"
         L("__shared__ __attribute__((aligned(16))) %s s_w%d[%d][%d];" % (ty_, n.nid, WY, S))
+        lds += WY * S * (8 if g.is_pair(n) else 4)
         L("__shared__ __attribute__((aligned(16))) %s s_r%d[%d];" % (ty_, n.nid, S))
-        lds += (WY + 1) * S * (8 if g.is_pair(n) else 4)
+        lds += S * (8 if g.is_pair(n) else 4)
     L("__shared__ int s_last;")
     g.declare_one()
+    L("const int nchunks = gridDim.y;")
     L("const int tx = threadIdx.x %% %d, ty = threadIdx.x / %d;" % (LX, LX))
     L("const long long c0 = (long long)blockIdx.x * %d;" % S)
     L("const long long c = c0 + tx * %d;" % V)
@@ -2058,7 +2100,6 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1):
         L("const int clim = cfull ? %d : (col_ok ? (int)(C - c) : 0);" % V)
     L("const long long r0 = (long long)blockIdx.y * rows_per_chunk;")
     L("const long long r1 = (r0 + rows_per_chunk < R) ? (r0 + rows_per_chunk) : (long long)R;")
-    L("const int nchunks = gridDim.y;")
     g.pos = ("0", "c")
     g.emit_gather_prefetch(_needed([st.root for st in prog.statements], set(n.nid for n in prog.nodes if n.kind == "R")),
                            V, "col_ok && ty == 0")
@@ -2067,144 +2108,145 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1):
     leaves = g.leaf_nodes(nodes)
     for n in reds:
         g.declare_acc(n)
-    U = COLSPLIT_ROWS_IN_FLIGHT
-    # main loop: U independent rows in flight per lane
+    # reductions that take several rows as a whole
+    batched = [n for n in reds if g.is_pair(n) and NB > 1]
     L.open("if (col_ok)")
-    L("long long r = r0 + ty;")
-    L.open("for (; r + %d < r1; r += %d)" % ((U - 1) * LY, U * LY))
-    for u in range(U):
+    L.open("for (long long rb = r0 + ty; rb < r1; rb += %d)" % (NR * LY))
+    # -- a whole batch inside the chunk: every load first
+    L.open("if (rb + %d < r1)" % ((NR - 1) * LY))
+    for u in range(NR):
         for n in leaves:
-            g.emit_load(n, "r + %d" % (u * LY), "c", V, "_%d" % u)
-    # running (max, sum of exponentials) pairs take the U rows of a step at once:
-    # one rescaling of the sum per step instead of one per row
-    batched = [n for n in reds if g.fused_max(n) and U > 1]
-    if batched:
+            g.emit_load(n, "rb + %d" % (u * LY), "c", V, "_%d" % u)
+    for b0 in range(0, NR, NB):
+        nb = min(NB, NR - b0)
         if V > 1:
             L("#pragma unroll")
         L.open("for (int j = 0; j < %d; ++j)" % V)
         for n in batched:
-            L("float lv%d[%d];" % (n.nid, U))
-        for u in range(U):
+            L("float lv%d[%d];" % (n.nid, nb))
+        for u in range(b0, b0 + nb):
             L.open("")
-            ref = g.make_ref("_%d" % u, "r + %d" % (u * LY), "c", V)
+            ref = g.make_ref("_%d" % u, "rb + %d" % (u * LY), "c", V)
             g.emit_exprs(nodes, ref, {})
             for n in reds:
                 if n in batched:
-                    L("lv%d[%d] = %s;" % (n.nid, u, ref(n.args[0])))
+                    L("lv%d[%d] = %s;" % (n.nid, u - b0, ref(n.args[0])))
                 else:
-                    g.accumulate(n, ref(n.args[0]), "r + %d" % (u * LY), ref)
+                    g.accumulate(n, ref(n.args[0]), "rb + %d" % (u * LY), ref)
             L.close()
         for n in batched:
-            L("nh_op_lse::stepn<%d>(acc%d[j], lv%d);" % (U, n.nid, n.nid))
+            if g.fused_max(n):
+                L("nh_op_lse::stepn<%d>(acc%d[j], lv%d);" % (nb, n.nid, n.nid))
+            else:
+                L("%s::stepn<%d>(acc%d[j], lv%d, (int)rb + %d, %d);" % (g.red_op(n), nb, n.nid, n.nid, b0 * LY, LY))
         L.close()
-    else:
-        for u in range(U):
-            if V > 1:
-                L("#pragma unroll")
-            L.open("for (int j = 0; j < %d; ++j)" % V)
-            ref = g.make_ref("_%d" % u, "r + %d" % (u * LY), "c", V)
-            g.emit_exprs(nodes, ref, {})
-            for n in reds:
-                g.accumulate(n, ref(n.args[0]), "r + %d" % (u * LY), ref)
-            L.close()
     L.close()
-    L.open("for (; r < r1; r += %d)" % LY)
-    for n in leaves:
-        g.emit_load(n, "r", "c", V, "_t")
-    if V > 1:
-        L("#pragma unroll")
-    L.open("for (int j = 0; j < %d; ++j)" % V)
-    ref = g.make_ref("_t", "r", "c", V)
-    g.emit_exprs(nodes, ref, {})
-    for n in reds:
-        g.accumulate(n, ref(n.args[0]), "r", ref)
+    # -- a batch that reaches beyond the chunk: the rows that exist, one by one (loads first all the same)
+    L.open("else")
+    for u in range(NR):
+        for n in leaves:
+            L("%s %s;" % (g.tile_type(n, V), g.tile_name(n, "_%d" % u)))
+            L.open("if (rb + %d < r1)" % (u * LY))
+            L(g.load_stmt(g.tile_name(n, "_%d" % u), n, "rb + %d" % (u * LY), "c", V))
+            L.close()
+            L("else %s.zero();" % g.tile_name(n, "_%d" % u))
+    for u in range(NR):
+        L.open("if (rb + %d < r1)" % (u * LY))
+        if V > 1:
+            L("#pragma unroll")
+        L.open("for (int j = 0; j < %d; ++j)" % V)
+        ref = g.make_ref("_%d" % u, "rb + %d" % (u * LY), "c", V)
+        g.emit_exprs(nodes, ref, {})
+        for n in reds:
+            g.accumulate(n, ref(n.args[0]), "rb + %d" % (u * LY), ref)
+        L.close()
+        L.close()
     L.close()
     L.close()
     L.close()
     # -- after the sweep ---------------------------------------------------------------
+    for n in reds:
+        if n.is_index:
+            L("#pragma unroll")
+            L("for (int j = 0; j < %d; ++j) acc%d[j] = nh_arg_key<%s>(acc%d[j]);" % (V, n.nid, g.red_op(n), n.nid))
     steps = (64 // LX).bit_length() - 1
     VK = max(1, V >> steps)             # values a lane still holds after the wave's row-lanes have folded
-    for n in reds:
-        L.open("")
-        L("const int j0 = nh_col_wave_fold<%s, %d, %d>(acc%d);" % (g.red_op(n), V, LX, n.nid))
-        L.open("if ((threadIdx.x & 63) < %d)" % (LX * (V // VK)))
+    holders = LX * (V // VK)            # ... and the lanes of a wave that hold distinct columns
+    L("int j0[%d];" % len(reds))
+    for k, n in enumerate(reds):
+        L("j0[%d] = nh_col_wave_fold<%s, %d, %d>(acc%d);" % (k, fold_op[n.nid], V, LX, n.nid))
+    # the waves join through LDS, one lane per column
+    L.open("if ((threadIdx.x & 63) < %d)" % holders)
+    for k, n in enumerate(reds):
         L("#pragma unroll")
-        L("for (int j = 0; j < %d; ++j) s_w%d[threadIdx.x >> 6][tx * %d + j0 + j] = acc%d[j];" % (VK, n.nid, V, n.nid))
-        L.close()
-        L.close()
+        L("for (int j = 0; j < %d; ++j) s_w%d[threadIdx.x >> 6][tx * %d + j0[%d] + j] = acc%d[j];" % (VK, n.nid, V, k, n.nid))
+    L.close()
     L("__syncthreads();")
-    # one lane per column joins the waves
     for n in reds:
-        L("%s one%d = %s::init();" % ("nh_pair" if g.is_pair(n) else "float", n.nid, g.red_op(n)))
+        L("%s one%d = %s::init();" % ("nh_pair" if g.is_pair(n) else "float", n.nid, fold_op[n.nid]))
     L.open("if (threadIdx.x < %d)" % S)
     for n in reds:
         L("one%d = s_w%d[0][threadIdx.x];" % (n.nid, n.nid))
         if WY > 1:
             L("#pragma unroll")
             L("for (int y = 1; y < %d; ++y) one%d = %s::f(one%d, s_w%d[y][threadIdx.x]);"
-              % (WY, n.nid, g.red_op(n), n.nid, n.nid))
+              % (WY, n.nid, fold_op[n.nid], n.nid, n.nid))
     L.close()
-
-    # partial buffers: reduction k occupies [k*nchunks*C, (k+1)*nchunks*C) entries
-    # of 8 bytes (value, index)
-    L.open("if (nchunks > 1)")
-    for k, n in enumerate(reds):
-        L("nh_pair* part%d = reinterpret_cast<nh_pair*>(ws) + (long long)%d * nchunks * C;" % (n.nid, k))
-    L("unsigned int* tickets = reinterpret_cast<unsigned int*>(ws + ticket_offset);")
-    L.open("if (threadIdx.x < %d && c0 + threadIdx.x < C)" % S)
-    for n in reds:
-        val = ("one%d" % n.nid) if g.is_pair(n) else ("nh_pair{one%d, 0}" % n.nid)
-        L("nh_part_store(&part%d[(long long)blockIdx.y * C + c0 + threadIdx.x], %s);" % (n.nid, val))
-    L.close()
-    # The partials were written through to device-coherent memory
-    # (nh_part_store); every lane waits for its own stores before the barrier
-    # (nh_publish_barrier), lane 0 then takes the ticket, and the last
-    # workgroup reads the partials past its L2 (nh_part_load).
-    L("nh_publish_barrier();")
-    L.open("if (threadIdx.x == 0)")
-    L("const unsigned int t = nh_ticket_take(&tickets[blockIdx.x]);")
-    L("s_last = (t == (unsigned int)(nchunks - 1));")
-    L.close()
-    L("__syncthreads();")
-    L("if (!s_last) return;")
-    # the last workgroup: P adjacent lanes per column, lane k0 of them takes chunks
-    # k0, k0 + P, ..., QB of them in flight at a time
-    QB = max(1, int(fold_batch))
-    L("const int fcol = threadIdx.x / %d, k0 = threadIdx.x %% %d;" % (P, P))
-    L("const bool fold_ok = (fcol < %d) && (c0 + fcol < C);" % S)
-    for n in reds:
-        L("one%d = %s::init();" % (n.nid, g.red_op(n)))
-    L.open("for (int kb = k0; kb < nchunks; kb += %d)" % (P * QB))
-    for n in reds:
-        L("nh_pair q%d[%d];" % (n.nid, QB))
-    L("#pragma unroll")
-    L.open("for (int k = 0; k < %d; ++k)" % QB)
-    L("const int q = kb + k * %d;" % P)
-    for n in reds:
-        op = g.red_op(n)
-        init = ("%s::init()" % op) if g.is_pair(n) else ("nh_pair{%s::init(), 0}" % op)
-        L("q%d[k] = (fold_ok && q < nchunks) ? nh_part_load(&part%d[(long long)q * C + c0 + fcol]) : %s;"
-          % (n.nid, n.nid, init))
-    L.close()
-    L("#pragma unroll")
-    L.open("for (int k = 0; k < %d; ++k)" % QB)
-    for n in reds:
-        L("one%d = %s::f(one%d, q%d[k]%s);" % (n.nid, g.red_op(n), n.nid, n.nid, "" if g.is_pair(n) else ".v"))
-    L.close()
-    L.close()
-    for n in reds:
-        ty_ = "nh_pair" if g.is_pair(n) else "float"
-        L("one%d = nh_wave_allreduce<%s, %d, %s>(one%d);" % (n.nid, g.red_op(n), P, ty_, n.nid))
-    L("if (threadIdx.x == 0) nh_ticket_reset(&tickets[blockIdx.x]);")
-    L.open("if (k0 == 0 && fcol < %d)" % S)
-    for n in reds:
-        L("s_r%d[fcol] = one%d;" % (n.nid, n.nid))
-    L.close()
-    L.close()
-    L.open("else if (threadIdx.x < %d)" % S)
-    for n in reds:
-        L("s_r%d[threadIdx.x] = one%d;" % (n.nid, n.nid))
-    L.close()
+    if multi:
+        # partial buffers: reduction k occupies [k*nchunks*C, (k+1)*nchunks*C) entries of 8 bytes
+        for k, n in enumerate(reds):
+            L("nh_pair* part%d = reinterpret_cast<nh_pair*>(ws) + (long long)%d * nchunks * C;" % (n.nid, k))
+        L("unsigned int* const ticket = reinterpret_cast<unsigned int*>(ws + ticket_offset) + %d * blockIdx.x;" % TICKET_STRIDE_WORDS)
+        L.open("if (threadIdx.x < %d && c0 + threadIdx.x < C)" % S)
+        for n in reds:
+            val = ("one%d" % n.nid) if g.is_pair(n) else ("nh_pair{one%d, 0}" % n.nid)
+            L("nh_part_store(&part%d[(long long)blockIdx.y * C + c0 + threadIdx.x], %s);" % (n.nid, val))
+        L.close()
+        # The partials were written through to device-coherent memory (nh_part_store); every
+        # lane waits for its own stores before the barrier (nh_publish_barrier), lane 0 then
+        # takes the ticket, and the last workgroup reads the partials past its L2 (nh_part_load).
+        L("nh_publish_barrier();")
+        L("if (threadIdx.x == 0) s_last = (nh_ticket_take(ticket) == (unsigned int)(nchunks - 1));")
+        L("__syncthreads();")
+        L("if (!s_last) return;")
+        # the last workgroup: P adjacent lanes per column, lane i of them takes chunks
+        # i, i + P, ..., QB of them in flight at a time
+        QB = max(1, int(fold_batch))
+        L("const int fcol = threadIdx.x / %d, flane = threadIdx.x %% %d;" % (P, P))
+        L("const bool fold_ok = (fcol < %d) && (c0 + fcol < C);" % S)
+        for n in reds:
+            L("one%d = %s::init();" % (n.nid, fold_op[n.nid]))
+        L.open("for (int kb = flane; kb < nchunks; kb += %d)" % (P * QB))
+        for n in reds:
+            L("nh_pair q%d[%d];" % (n.nid, QB))
+        L("#pragma unroll")
+        L.open("for (int k = 0; k < %d; ++k)" % QB)
+        L("const int q = kb + k * %d;" % P)
+        for n in reds:
+            op = fold_op[n.nid]
+            init = ("%s::init()" % op) if g.is_pair(n) else ("nh_pair{%s::init(), 0}" % op)
+            L("q%d[k] = (fold_ok && q < nchunks) ? nh_part_load(&part%d[(long long)q * C + c0 + fcol]) : %s;"
+              % (n.nid, n.nid, init))
+        L.close()
+        L("#pragma unroll")
+        L.open("for (int k = 0; k < %d; ++k)" % QB)
+        for n in reds:
+            L("one%d = %s::f(one%d, q%d[k]%s);" % (n.nid, fold_op[n.nid], n.nid, n.nid, "" if g.is_pair(n) else ".v"))
+        L.close()
+        L.close()
+        for n in reds:
+            ty_ = "nh_pair" if g.is_pair(n) else "float"
+            L("one%d = nh_wave_allreduce<%s, %d, %s>(one%d);" % (n.nid, fold_op[n.nid], P, ty_, n.nid))
+        L("if (threadIdx.x == 0) nh_ticket_reset(ticket);")
+        L.open("if (flane == 0 && fcol < %d)" % S)
+        for n in reds:
+            L("s_r%d[fcol] = one%d;" % (n.nid, n.nid))
+        L.close()
+    else:
+        L.open("if (threadIdx.x < %d)" % S)
+        for n in reds:
+            L("s_r%d[threadIdx.x] = one%d;" % (n.nid, n.nid))
+        L.close()
     L("__syncthreads();")
     # the lanes that evaluate the statements pick up the V columns of their tile
     for n in reds:
@@ -2216,7 +2258,7 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1):
             L("float rv%d[%d];" % (n.lse_sum.nid, V))
         L("#pragma unroll")
         if n.is_index:
-            L("for (int j = 0; j < %d; ++j) ri%d[j] = s_r%d[tx * %d + j].i;" % (V, n.nid, n.nid, V))
+            L("for (int j = 0; j < %d; ++j) ri%d[j] = nh_key_index(s_r%d[tx * %d + j]);" % (V, n.nid, n.nid, V))
         elif g.fused_max(n):
             L("for (int j = 0; j < %d; ++j) { rv%d[j] = s_r%d[tx * %d + j].v; rv%d[j] = nh_lse_total(s_r%d[tx * %d + j]); }"
               % (V, n.nid, n.nid, V, n.lse_sum.nid, n.nid, V))
@@ -2250,4 +2292,5 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1):
     L.close()
     L.close()
     return _finish("colsplit", g, head, fmt, T, lds,
-                   dict(V=V, LX=LX, LY=LY, NRED=len(reds), stream=bool(stream), tail=bool(tail)))
+                   dict(V=V, LX=LX, LY=LY, NR=NR, NB=NB, NRED=len(reds), multi=bool(multi),
+                        stream=bool(stream), tail=bool(tail)))

@@ -684,20 +684,25 @@ def _plan_col(prog, cu_count, coop=True):
                 # ((1048576,64) fp16, one strip of 128 chunks: sum 31.3 -> 27.4 us, argmax 47.7 -> 36.4)
                 threads = 1024
         LY = threads // LX
-        rpc = max(codegen.COLSPLIT_ROWS_IN_FLIGHT * LY, _ceil_div(R, chunks))
-        rpc = _ceil_div(rpc, LY) * LY
+        # rows a lane fetches at once and reduces as one batch: as many as the registers take
+        # (COLSPLIT_BATCH_WORDS words of resident tiles), at most what a chunk gives a lane.
+        # A chunk is a whole number of such batches, so that only the matrix's last chunk
+        # meets its end inside one.
+        per_lane = max(codegen.COLSPLIT_ROWS_IN_FLIGHT, _ceil_div(max(1, _ceil_div(R, chunks)), LY))
+        NR = max(1, min(codegen.COLSPLIT_BATCH_ROWS, codegen.COLSPLIT_BATCH_WORDS // words, per_lane))
+        rpc = _ceil_div(per_lane, NR) * NR * LY
         chunks = _ceil_div(R, rpc)
         if chunks > 65535:
             raise ValueError("tensor too large for one launch")
         # partials a lane of the last workgroup has in flight: P = lanes per column there
         lanes_per_column = min(threads // (LX * V), 64)
         fold_batch = max(1, min(codegen.COLSPLIT_FOLD_BATCH, _ceil_div(chunks, lanes_per_column)))
-        spec = codegen.gen_colsplit(prog, V, LX, LY, _streams(prog), tail=tail, fold_batch=fold_batch)
-        nred = spec.params["NRED"]
-        part_bytes = nred * chunks * C * 8
+        spec = codegen.gen_colsplit(prog, V, LX, LY, _streams(prog), tail=tail, fold_batch=fold_batch, NR=NR,
+                                    NB=codegen.COLSPLIT_SUBBATCH_ROWS, multi=chunks > 1)
+        part_bytes = spec.params["NRED"] * chunks * C * 8
         ticket_off = _ceil_div(part_bytes, 256) * 256
-        ws_bytes = ticket_off + strips * 4
+        ws_bytes = ticket_off + strips * 4 * codegen.TICKET_STRIDE_WORDS
         return Choice(spec, (strips, chunks, 1), extras=(rpc,),
-                      workspace=(ws_bytes, ticket_off, strips))
+                      workspace=(ws_bytes, ticket_off, strips * codegen.TICKET_STRIDE_WORDS))
 
     raise NeedsSplit()

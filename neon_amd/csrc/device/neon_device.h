@@ -453,6 +453,25 @@ struct nh_op_argmax {
     // !(v <= a.v) holds for a larger value and for a NaN on either side; a NaN
     // already held (a.v != a.v) stays
     static NEON_DEV void step(nh_pair& a, float v, int i) { if (!(v <= a.v) && (a.v == a.v)) { a.v = v; a.i = i; } }
+    // N elements at once, x[k] sitting at index i0 + k * stride (increasing): one maximum per
+    // element, then -- only when the batch beats what is held -- a scan for the first
+    // position of that maximum (of the first NaN when there is one)
+    template <int N> static NEON_DEV void stepn(nh_pair& a, const float (&x)[N], int i0, int stride) {
+        float m = x[0];
+#pragma unroll
+        for (int k = 1; k < N; ++k) m = nh_max(m, x[k]);
+        if (!(m <= a.v) && (a.v == a.v)) {
+            int k0 = N - 1;
+            if (__builtin_expect(m != m, 0)) {
+#pragma unroll
+                for (int k = N - 2; k >= 0; --k) k0 = (x[k] != x[k]) ? k : k0;
+            } else {
+#pragma unroll
+                for (int k = N - 2; k >= 0; --k) k0 = (x[k] == m) ? k : k0;
+            }
+            a.v = m; a.i = i0 + k0 * stride;
+        }
+    }
 };
 struct nh_op_argmin {
     static NEON_DEV nh_pair init() { nh_pair p; p.v = NH_INF; p.i = 0; return p; }
@@ -462,6 +481,53 @@ struct nh_op_argmin {
         nh_pair r; r.v = take_b ? b.v : a.v; r.i = take_b ? b.i : a.i; return r;
     }
     static NEON_DEV void step(nh_pair& a, float v, int i) { if (!(v >= a.v) && (a.v == a.v)) { a.v = v; a.i = i; } }
+    template <int N> static NEON_DEV void stepn(nh_pair& a, const float (&x)[N], int i0, int stride) {
+        float m = x[0];
+#pragma unroll
+        for (int k = 1; k < N; ++k) m = nh_min(m, x[k]);
+        if (!(m >= a.v) && (a.v == a.v)) {
+            int k0 = N - 1;
+            if (__builtin_expect(m != m, 0)) {
+#pragma unroll
+                for (int k = N - 2; k >= 0; --k) k0 = (x[k] != x[k]) ? k : k0;
+            } else {
+#pragma unroll
+                for (int k = N - 2; k >= 0; --k) k0 = (x[k] == m) ? k : k0;
+            }
+            a.v = m; a.i = i0 + k0 * stride;
+        }
+    }
+};
+
+// An arg-reduction's (value, index) as ONE 64-bit key whose unsigned order is the
+// reduction's preference -- high word: the value mapped to an unsigned integer that
+// grows with it (argmax) or shrinks with it (argmin), -0 taken as +0, any NaN as
+// the largest key; low word: ~index, so that among equal values the lower index
+// wins.  Merging two keys is a 64-bit maximum (three instructions, no branches),
+// which is what every stage after a lane's own sweep uses: lane exchanges, the
+// join of the waves, the partials between workgroups.  Carried in an nh_pair
+// (v = bits of the high word, i = low word).
+NEON_DEV nh_u32 nh_ordered_bits(float v) {
+    const nh_u32 u = __builtin_bit_cast(nh_u32, v + 0.0f);
+    return u ^ ((nh_u32)((int)u >> 31) | 0x80000000u);
+}
+template <class OP> NEON_DEV nh_pair nh_arg_key(nh_pair p);
+template <> NEON_DEV nh_pair nh_arg_key<nh_op_argmax>(nh_pair p) {
+    const nh_u32 k = (p.v != p.v) ? 0xFFFFFFFFu : nh_ordered_bits(p.v);
+    nh_pair r; r.v = __builtin_bit_cast(float, k); r.i = ~p.i; return r;
+}
+template <> NEON_DEV nh_pair nh_arg_key<nh_op_argmin>(nh_pair p) {
+    const nh_u32 k = (p.v != p.v) ? 0xFFFFFFFFu : ~nh_ordered_bits(p.v);
+    nh_pair r; r.v = __builtin_bit_cast(float, k); r.i = ~p.i; return r;
+}
+NEON_DEV int nh_key_index(nh_pair k) { return ~k.i; }
+struct nh_op_key {
+    static NEON_DEV nh_pair init() { nh_pair p; p.v = __builtin_bit_cast(float, 0u); p.i = 0; return p; }
+    static NEON_DEV nh_pair f(nh_pair a, nh_pair b) {
+        const unsigned long long ka = ((unsigned long long)__builtin_bit_cast(nh_u32, a.v) << 32) | (nh_u32)a.i;
+        const unsigned long long kb = ((unsigned long long)__builtin_bit_cast(nh_u32, b.v) << 32) | (nh_u32)b.i;
+        return (kb > ka) ? b : a;
+    }
 };
 
 // Running log-sum-exp state of a column: v = maximum so far, i = the bits of
@@ -524,10 +590,16 @@ NEON_DEV float nh_exp_term(float d) {
 }
 struct nh_op_lse {
     static NEON_DEV nh_pair init() { nh_pair p; p.v = -NH_INF; p.i = 0; return p; }    // bits of +0.0f
+    // the state with the larger maximum keeps its sum, the other one's is scaled by
+    // e^(smaller - larger): one exponential per merge
     static NEON_DEV nh_pair f(nh_pair a, nh_pair b) {
         const float m = nh_max(a.v, b.v);
+        const float lo = nh_min(a.v, b.v);
         const float mz = (m == -NH_INF) ? 0.0f : m;
-        const float s = nh_lse_sum(a) * nh_exp_nonpos(a.v - mz) + nh_lse_sum(b) * nh_exp_nonpos(b.v - mz);
+        const bool a_top = a.v >= b.v;
+        const float s_top = a_top ? nh_lse_sum(a) : nh_lse_sum(b);
+        const float s_low = a_top ? nh_lse_sum(b) : nh_lse_sum(a);
+        const float s = __builtin_fmaf(s_low, nh_exp_nonpos(lo - mz), s_top);
         nh_pair r; r.v = m; r.i = __builtin_bit_cast(int, s); return r;
     }
     static NEON_DEV void step(nh_pair& a, float x) {

@@ -255,13 +255,17 @@ constexpr int CR_U = 4;                   // rows in flight per lane
 constexpr int CR_FOLD_BATCH = 4;          // partials in flight per lane in the final fold
 constexpr int CR_MAX_STRIPS = 4096;
 constexpr int CR_MAX_CHUNKS = 128;
+// The tickets of neighbouring strips sit a 64-byte line apart: atomics on one line are served
+// one after the other whichever words of it they address, and with the tickets of all strips in
+// one line the workgroups of a (32000 x 256) launch queued behind each other for two microseconds.
+constexpr int CR_TICKET_STRIDE = 16;
 
-__device__ unsigned int g_cr_tickets[CR_MAX_STRIPS];  // zero at load; each strip's last workgroup resets its ticket
+__device__ unsigned int g_cr_tickets[CR_MAX_STRIPS * CR_TICKET_STRIDE];  // zero at load; each strip's last workgroup resets its ticket
 
 // Scratch of the entry point that allocates nothing: tickets first, partials
 // after them.  One copy per device, alive until the process ends; host code
 // reaches it through the address hipGetSymbolAddress returns for the device.
-constexpr size_t CR_STATIC_TICKET_BYTES = (size_t)CR_MAX_STRIPS * sizeof(unsigned int);
+constexpr size_t CR_STATIC_TICKET_BYTES = (size_t)CR_MAX_STRIPS * CR_TICKET_STRIDE * sizeof(unsigned int);
 static __device__ __align__(256) unsigned char scratch[NH_STATIC_SCRATCH_BYTES];
 
 // Join the row-lanes of the workgroup: the row-lanes of a wave fold with lane
@@ -348,7 +352,7 @@ __global__ __launch_bounds__(T) void colmax_kernel(const float* __restrict__ x, 
         if (writer) nh_part_store(&part[(size_t)blockIdx.y * cols + c0 + tid], one);
         nh_publish_barrier();     // every lane's partial stores have been performed before the ticket is taken
         if (tid == 0) {
-            const unsigned int t = nh_ticket_take(&tickets[blockIdx.x]);
+            const unsigned int t = nh_ticket_take(&tickets[blockIdx.x * CR_TICKET_STRIDE]);
             s_last = (t == nchunks - 1);
         }
         __syncthreads();
@@ -371,7 +375,7 @@ __global__ __launch_bounds__(T) void colmax_kernel(const float* __restrict__ x, 
             for (int k = 0; k < CR_FOLD_BATCH; ++k) one = nh_op_argmax::f(one, q[k]);
         }
         one = nh_wave_allreduce<nh_op_argmax, P, nh_pair>(one);
-        if (tid == 0) nh_ticket_reset(&tickets[blockIdx.x]);  // ready for the next launch on this stream
+        if (tid == 0) nh_ticket_reset(&tickets[blockIdx.x * CR_TICKET_STRIDE]);  // ready for the next launch on this stream
         writer = k0 == 0 && fold_ok;
     }
     if (writer) {
@@ -932,7 +936,8 @@ int nh_colmax_argmax_f32_static(float* maxval, int32_t* argmax, const float* x, 
     hipStream_t s = (hipStream_t)stream;
     if (p.chunks > 1) {
         // the area keeps whatever the last call left: tickets have to start at zero
-        hipLaunchKernelGGL(cr_clear_tickets_kernel, dim3((p.strips + 255) / 256), dim3(256), 0, s, tickets, p.strips);
+        const uint32_t words = p.strips * CR_TICKET_STRIDE;
+        hipLaunchKernelGGL(cr_clear_tickets_kernel, dim3((words + 255) / 256), dim3(256), 0, s, tickets, words);
         if (int rc = launch_status("nh_colmax_argmax_f32_static: clearing the tickets")) return rc;
     }
     return colmax_launch("nh_colmax_argmax_f32_static", maxval, argmax, x, rows, cols, ld, p, part, tickets, s);

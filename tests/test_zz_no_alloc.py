@@ -50,7 +50,7 @@ def test_static_scratch_entry_point_matches_the_workspace_one(hip):
 
 def test_static_scratch_entry_point_refuses_what_does_not_fit(hip):
     rt, lib = hip.rt, hip.rt.lib
-    rows, cols = 9000, 8190           # row length not a multiple of four: 16 chunks x 8190 columns x 8 bytes > 1 MiB
+    rows, cols = 9000, 8190           # row length not a multiple of four: 16 chunks x 8190 columns x 8 bytes > the 768 KiB behind the tickets
     dx = rt.malloc(rows * cols * 4)
     out = rt.malloc(4 * cols)
     try:
