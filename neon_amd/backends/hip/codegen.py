@@ -2184,23 +2184,36 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
     L("__syncthreads();")
     for n in reds:
         L("%s one%d = %s::init();" % ("nh_pair" if g.is_pair(n) else "float", n.nid, fold_op[n.nid]))
-    L.open("if (threadIdx.x < %d)" % S)
-    for n in reds:
-        L("one%d = s_w%d[0][threadIdx.x];" % (n.nid, n.nid))
-        if WY > 1:
-            L("#pragma unroll")
-            L("for (int y = 1; y < %d; ++y) one%d = %s::f(one%d, s_w%d[y][threadIdx.x]);"
-              % (WY, n.nid, fold_op[n.nid], n.nid, n.nid))
-    L.close()
+    # WY adjacent lanes share a column, each brings one wave's piece, a DPP all-reduce joins
+    # them: log2(WY) dependent merges instead of WY - 1 (pair merges are long chains)
+    spread = 1 < WY <= 16 and S * WY <= T and WY & (WY - 1) == 0
+    if spread:
+        L("const int jcol = threadIdx.x / %d;" % WY)
+        L("const bool joins = (threadIdx.x %% %d) == 0 && jcol < %d;" % (WY, S))
+        for n in reds:
+            ty_ = "nh_pair" if g.is_pair(n) else "float"
+            L("if (jcol < %d) one%d = s_w%d[threadIdx.x %% %d][jcol];" % (S, n.nid, n.nid, WY))
+            L("one%d = nh_wave_allreduce<%s, %d, %s>(one%d);" % (n.nid, fold_op[n.nid], WY, ty_, n.nid))
+    else:
+        L("const int jcol = threadIdx.x;")
+        L("const bool joins = threadIdx.x < %d;" % S)
+        L.open("if (joins)")
+        for n in reds:
+            L("one%d = s_w%d[0][threadIdx.x];" % (n.nid, n.nid))
+            if WY > 1:
+                L("#pragma unroll")
+                L("for (int y = 1; y < %d; ++y) one%d = %s::f(one%d, s_w%d[y][threadIdx.x]);"
+                  % (WY, n.nid, fold_op[n.nid], n.nid, n.nid))
+        L.close()
     if multi:
         # partial buffers: reduction k occupies [k*nchunks*C, (k+1)*nchunks*C) entries of 8 bytes
         for k, n in enumerate(reds):
             L("nh_pair* part%d = reinterpret_cast<nh_pair*>(ws) + (long long)%d * nchunks * C;" % (n.nid, k))
         L("unsigned int* const ticket = reinterpret_cast<unsigned int*>(ws + ticket_offset) + %d * blockIdx.x;" % TICKET_STRIDE_WORDS)
-        L.open("if (threadIdx.x < %d && c0 + threadIdx.x < C)" % S)
+        L.open("if (joins && c0 + jcol < C)")
         for n in reds:
             val = ("one%d" % n.nid) if g.is_pair(n) else ("nh_pair{one%d, 0}" % n.nid)
-            L("nh_part_store(&part%d[(long long)blockIdx.y * C + c0 + threadIdx.x], %s);" % (n.nid, val))
+            L("nh_part_store(&part%d[(long long)blockIdx.y * C + c0 + jcol], %s);" % (n.nid, val))
         L.close()
         # The partials were written through to device-coherent memory (nh_part_store); every
         # lane waits for its own stores before the barrier (nh_publish_barrier), lane 0 then
@@ -2243,9 +2256,9 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
             L("s_r%d[fcol] = one%d;" % (n.nid, n.nid))
         L.close()
     else:
-        L.open("if (threadIdx.x < %d)" % S)
+        L.open("if (joins)")
         for n in reds:
-            L("s_r%d[threadIdx.x] = one%d;" % (n.nid, n.nid))
+            L("s_r%d[jcol] = one%d;" % (n.nid, n.nid))
         L.close()
     L("__syncthreads();")
     # the lanes that evaluate the statements pick up the V columns of their tile

@@ -591,7 +591,7 @@ NEON_DEV float nh_exp_term(float d) {
 struct nh_op_lse {
     static NEON_DEV nh_pair init() { nh_pair p; p.v = -NH_INF; p.i = 0; return p; }    // bits of +0.0f
     // the state with the larger maximum keeps its sum, the other one's is scaled by
-    // e^(smaller - larger): one exponential per merge
+    // e^(smaller - larger): one exponential per merge, a term of the sum like any other
     static NEON_DEV nh_pair f(nh_pair a, nh_pair b) {
         const float m = nh_max(a.v, b.v);
         const float lo = nh_min(a.v, b.v);
@@ -599,7 +599,7 @@ struct nh_op_lse {
         const bool a_top = a.v >= b.v;
         const float s_top = a_top ? nh_lse_sum(a) : nh_lse_sum(b);
         const float s_low = a_top ? nh_lse_sum(b) : nh_lse_sum(a);
-        const float s = __builtin_fmaf(s_low, nh_exp_nonpos(lo - mz), s_top);
+        const float s = __builtin_fmaf(s_low, nh_exp_term(lo - mz), s_top);
         nh_pair r; r.v = m; r.i = __builtin_bit_cast(int, s); return r;
     }
     static NEON_DEV void step(nh_pair& a, float x) {
