@@ -665,6 +665,59 @@ class Program(object):
     def overlapping_slots(self):
         return self._alias_signature()
 
+    def output_hazards(self):
+        """Written slots whose memory overlaps that of ANOTHER slot of the
+        program (one that is read or written through a different view:
+        different start, shape or strides -- the same view is the same slot).
+        A kernel gives no order between the lanes that write such an output
+        and the lanes that read or write the overlapping elements, whereas the
+        reference's CPU backend finishes the right-hand side before it stores
+        (nervanacpu.py:476-477: ``left[:] = right`` on a finished array).
+        Gather / scatter views count by the whole axis they index."""
+        spans = []
+        for t in self.tensors:
+            isz = t.dtype.itemsize
+            lo = hi = 0
+            for axis, (n, st) in enumerate(zip(t.shape, t.strides)):
+                if t.take_axis == axis and t.take_extent:
+                    n = t.take_extent
+                if n > 1:
+                    if st >= 0:
+                        hi += (n - 1) * st
+                    else:
+                        lo += (n - 1) * st
+            spans.append((t.ptr + lo * isz, t.ptr + (hi + 1) * isz))
+        def line_of_its_operand(w, o):
+            """``w`` holds one value per line of the reduction axis and sits INSIDE the
+            full-shape operand ``o``, each value in the very line it is computed from
+            (``x[0:1, :] = max(x, axis=0)``, ``x[:, 0:1] = sum(x, axis=1)``): every family
+            stores a line's results after the last read of that line, and no lane of
+            another line ever touches it"""
+            ax = self.axis
+            if ax is None or w.take_axis is not None or o.take_axis is not None or o.written:
+                return False
+            if w.shape[ax] != 1 or w.shape[1 - ax] != o.shape[1 - ax] or o.shape != tuple(self.domain):
+                return False
+            if w.strides[1 - ax] != o.strides[1 - ax] or w.dtype != o.dtype:
+                return False
+            step = o.strides[ax] * o.dtype.itemsize
+            off = w.ptr - o.ptr
+            return step > 0 and off % step == 0 and 0 <= off // step < o.shape[ax]
+
+        hazards = []
+        for w in self.tensors:
+            if not w.written:
+                continue
+            a = spans[w.index]
+            for o in self.tensors:
+                if o is w or not (o.read or o.written or o.index in self.index_slots):
+                    continue
+                b = spans[o.index]
+                if a[0] < b[1] and b[0] < a[1] and not line_of_its_operand(w, o):
+                    hazards.append(w)
+                    break
+        return hazards
+
 
 def build_program(optrees):
     prog = Program()

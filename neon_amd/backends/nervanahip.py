@@ -254,7 +254,8 @@ class HIPTensorBase(object):
                 self._api.OpTreeNode.build("assign", self, value)
         elif isinstance(value, HIPTensorBase):
             if (self.is_contiguous and value.is_contiguous and self.dtype == value.dtype and
-                    self.shape == value.shape and not be._fusing):
+                    self.shape == value.shape and not be._fusing and
+                    (value.gpudata == self.gpudata or not _overlap(self, value))):
                 if self.nbytes:
                     be.rt.memcpy_d2d(self.gpudata, value.gpudata, self.nbytes)
             else:
@@ -784,6 +785,8 @@ class NervanaHIPBase(object):
         sig = self._group_signature(tree, post)
         if sig is None:
             return False
+        if sig[0] == "ew" and not self._joins_without_overlap(tree, post):
+            return False
         vectors = self._sig_vectors
         if not self._pending:
             if sig[0] == "ew" and vectors and any(v.get_original_base() is tree[1].get_original_base() for v in vectors):
@@ -811,6 +814,35 @@ class NervanaHIPBase(object):
                     if isinstance(p, HIPTensorBase) and p.size > 1 and id(p.get_original_base()) in bases \
                             and not any(p is o for o in outs):
                         return False
+        return True
+
+    def _joins_without_overlap(self, tree, post):
+        """An elementwise group runs as one kernel in which a lane reads and
+        writes its own elements only, in statement order -- which is numpy's
+        statement-by-statement result as long as no tensor that the group
+        WRITES shares memory with another tensor of the group through a
+        different view (``x[1:11] = 2*y`` followed by ``z[:] = x[0:10] + 1``:
+        the lane of row i would read x row i before the lane of row i-1 has
+        written it).  The same view of the same memory is the same elements and
+        is fine.  False: ``tree`` must not join (it opens the next group, or, if
+        it overlaps within itself, runs alone through a temporary)."""
+        tensor_cls = self.tensor_cls
+        out = tree[1]
+        mine = [p for p in post if type(p) is tensor_cls]
+        for p in mine:                       # within the statement itself
+            if p is not out and p._geom != out._geom and _overlap(p, out):
+                return False
+        if not self._pending:
+            return True
+        written = [q[1] for q in self._pending]
+        touched = [p for grp_post in self._pending_post for p in grp_post if type(p) is tensor_cls] + written
+        for w in written:                    # what the group writes against everything new
+            for p in mine + [out]:
+                if p._geom != w._geom and _overlap(p, w):
+                    return False
+        for p in touched:                    # what the new statement writes against the group
+            if p._geom != out._geom and _overlap(p, out):
+                return False
         return True
 
     def _group_signature(self, tree, post):
@@ -1106,6 +1138,17 @@ class NervanaHIPBase(object):
             for t in trees:
                 prog.add_statement(t)
             prog.finalize()
+            if not self._originals and prog.output_hazards():
+                # an output overlaps another operand through a different view
+                # (``x[:] = y + x[2:3, :]``): the right-hand side is finished in a
+                # temporary before anything is stored, as numpy finishes it
+                if len(trees) != 1:
+                    for t in trees:
+                        self._run([t])
+                else:
+                    self._stats["staged"] = self._stats.get("staged", 0) + 1
+                    self._run_through_temporary(trees[0])
+                return
             key = prog.key()
             plan = self.plans.get(key)
             if plan is None:
@@ -1141,6 +1184,22 @@ class NervanaHIPBase(object):
                 raise
             self._stats["split"] += 1
             self._run_split(trees[0])
+
+    def _run_through_temporary(self, tree):
+        """``out[:] = expr`` with the whole right-hand side evaluated into a
+        pooled temporary of the output's shape and storage type first (one
+        conversion, as a direct store would make), then copied into place."""
+        out, expr = tree[1], tree[2]
+        node = self._api.OpTreeNode
+        temps = []
+        try:
+            # a stochastically rounded output draws its random numbers in the copy
+            tmp = self._temp(out.shape, np.float32 if out.rounding else out.dtype, temps)
+            self._run([node({"op": "assign"}, tmp, expr)])
+            self._run([node({"op": "assign"}, out, tmp)])
+        finally:
+            for t in temps:
+                self._temp_release(t)
 
     # -- bench mode (the reference brackets launches with events when its
     #    ``bench`` flag is set, float_ew.py:917-938) -------------------------------------
@@ -1222,7 +1281,7 @@ class NervanaHIPBase(object):
         if not views:
             return False
         if (expr is leaves[0] and isinstance(expr, HIPTensorBase) and out.is_contiguous and not out.rounding
-                and out.dtype == expr.dtype and out.shape == expr.shape and out.gpudata != expr.gpudata):
+                and out.dtype == expr.dtype and out.shape == expr.shape and not _overlap(out, expr)):
             self._strided_copy(out, expr)
             return True
         temps = []
@@ -1476,6 +1535,10 @@ class NervanaHIPBase(object):
         prog = Program()
         prog.add_statement(tree)
         prog.finalize()
+        if prog.output_hazards():
+            self._stats["staged"] = self._stats.get("staged", 0) + 1
+            self._run_through_temporary(tree)
+            return
         key = prog.key()
         plan = self.plans.get(key)
         if plan is None:
@@ -1932,6 +1995,29 @@ def __getattr__(name):
         pair = bind()
         return pair[0] if name == "NervanaHIP" else pair[1]
     raise AttributeError("module %r has no attribute %r" % (__name__, name))
+
+
+def _byte_span(t):
+    """[first, last + 1) byte addresses a tensor view can touch; a gather /
+    scatter view counts by the whole axis it indexes"""
+    lo = hi = 0
+    take = t.take_array[1] if t.take_array else None
+    for axis, (n, st) in enumerate(zip(t.shape, t.strides)):
+        if axis == take and t.take_extent:
+            n = t.take_extent
+        if n > 1:
+            if st >= 0:
+                hi += (n - 1) * st
+            else:
+                lo += (n - 1) * st
+    isz = t.dtype.itemsize
+    return t.gpudata + lo * isz, t.gpudata + (hi + 1) * isz
+
+
+def _overlap(a, b):
+    """two tensor views share at least part of their memory range"""
+    sa, sb = _byte_span(a), _byte_span(b)
+    return sa[0] < sb[1] and sb[0] < sa[1]
 
 
 def _matrix_geometry(rows, cols, sr, sc):

@@ -693,3 +693,73 @@ def test_rows_pair_maximum_and_sum_only_where_it_saves_a_pass_or_an_exchange(pb)
     assert paired((16, 1048576), np.float32) == ("rowcoop", False)     # resident fp32 shares: exponentials take x's registers
     assert paired((16, 1605632), np.float16) == ("rowcoop", True)      # resident 16-bit shares of 13 tiles: one exchange less
     assert paired((64, 131072), np.float16) == ("rowcoop", False)      # ... but not shares of 4 tiles
+
+
+# ---- outputs that overlap operands through another view ---------------------------------
+def test_output_hazards_are_found_by_byte_range(pb):
+    """a written slot that shares memory with another slot of the program
+    through a different view (reference semantics: nervanacpu.py:476-477, the
+    right-hand side is finished before the store)"""
+    base = 1 << 32
+    x = prebuild.ShapeTensor(pb, (12, 8), ptr=base)
+    y = prebuild.ShapeTensor(pb, (12, 8), ptr=base + (1 << 20))
+    row = prebuild.ShapeTensor(pb, (1, 8), ptr=base + 2 * 8 * 4, base=x)             # x[2:3, :]
+    col = prebuild.ShapeTensor(pb, (12, 1), ptr=base + 4, strides=(8, 1), base=x)    # x[:, 1:2]
+    shifted = prebuild.ShapeTensor(pb, (10, 8), ptr=base + 8 * 4, base=x)            # x[1:11]
+    head = prebuild.ShapeTensor(pb, (10, 8), ptr=base, base=x)                       # x[0:10]
+    tree = lambda out, value: OpTreeNode({"op": "assign"}, out, value)
+
+    def hazards(*stmts):
+        prog = Program()
+        for st in stmts:
+            prog.add_statement(st)
+        return [t.index for t in prog.finalize().output_hazards()]
+
+    assert hazards(tree(x, y + x)) == []                      # same elements: fine
+    assert hazards(tree(x, y * 2.0)) == []
+    assert hazards(tree(x, y + row)) == [0]                   # x[:] = y + x[2:3, :]
+    assert hazards(tree(x, y * col)) == [0]                   # x[:] = y * x[:, 1:2]
+    assert hazards(tree(col, pb.sum(x, axis=1))) == []        # a line's result stored inside that very line: fine
+    assert hazards(tree(row, pb.max(x, axis=0))) == []
+    assert hazards(tree(col, pb.sum(x * y, axis=1) * 2.0)) == []
+    assert hazards(tree(x, x - pb.max(x, axis=0) + row)) == [0]       # ... but not a full-shape result
+    assert hazards(tree(shifted, head)) == [0]                # x[1:11] = x[0:10]
+    assert hazards(tree(y, x + row)) == []                    # overlapping READS are no hazard
+
+
+def test_fusion_group_refuses_statements_that_overlap_through_other_views():
+    """_can_join on stub tensors (no device): the lanes of a fused elementwise
+    kernel only ever touch their own elements, so a tensor the group writes
+    may not meet another tensor of the group through a different view"""
+    from neon_amd.backends import NervanaHIP
+    be = object.__new__(NervanaHIP)
+    be._pending, be._pending_post, be._pending_sig = [], [], None
+    be._pending_vectors, be._sig_vectors = [], ()
+    T = be.tensor_cls
+    base = 1 << 32
+    x = T(be, (12, 8), gpudata=base)
+    y = T(be, (10, 8), gpudata=base + (1 << 20))
+    z = T(be, (10, 8), gpudata=base + (2 << 20))
+    w = T(be, (10, 8), gpudata=base + (3 << 20))
+    tree = lambda out, value: OpTreeNode({"op": "assign"}, out, value)
+
+    def offer(t):
+        post = t.traverse([])
+        ok = be._can_join(t, post)
+        if ok:
+            be._pending.append(t)
+            be._pending_post.append(post)
+        return ok
+
+    assert offer(tree(x[1:11], y * 2.0))                      # opens the group
+    assert offer(tree(w, x[1:11] + 1.0))                      # the same view of x: the same elements
+    assert not offer(tree(z, x[0:10] + 1.0))                  # x shifted by a row: other lanes' elements
+    assert not offer(tree(x[0:10], z * 1.0))                  # writing over what the group has written, shifted
+    be._pending, be._pending_post = [], []
+    assert offer(tree(z, y * 2.0))
+    inside_z = T(be, (1, 1), gpudata=z.gpudata + 29 * 4)      # one element in the interior of a written tensor
+    inside_y = T(be, (1, 1), gpudata=y.gpudata + 29 * 4)      # ... of a tensor that is only read: fine
+    assert not offer(tree(w, w + inside_z))
+    assert offer(tree(w, w + inside_y))
+    be._pending, be._pending_post = [], []
+    assert not offer(tree(x[1:11], x[0:10] * 2.0))            # overlaps within itself: never fused
