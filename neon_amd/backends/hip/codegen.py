@@ -278,6 +278,8 @@ class _Gen(object):
                     % (streams, n.slot, "true" if aligned else "false", r, c, streams))
             if n.op == "rand":
                 return "nh_rand01(%s)" % word
+            if n.op == "sround:int":
+                return "nh_sround_int(%s, %s)" % (a[0], word)
             return "nh_sround(%s, %s, %s)" % (a[0], n.op.split(":")[1], word)
         if len(a) == 1:
             if n.op == "exp" and EXP_OF_NONPOSITIVE and _below_its_maximum(n.args[0]):

@@ -6,8 +6,9 @@ import importlib.machinery
 import importlib.util
 import os
 
-_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)))),
-                     "lib", "_fastpath.so")
+# (NEON_HIP_FASTPATH_LIB names another build of the extension: the sanitizer test runs one)
+_PATH = os.environ.get("NEON_HIP_FASTPATH_LIB") or os.path.join(
+    os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)))), "lib", "_fastpath.so")
 _module = None
 
 

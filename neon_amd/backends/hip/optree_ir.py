@@ -161,7 +161,8 @@ class MixedAxes(ValueError):
 def stochastic_bits(tensor):
     """Mantissa bits a store into ``tensor`` rounds to stochastically, 0 for
     the ordinary round-to-nearest store (reference float_ew.py:832-844: True
-    means 10, at most 15 for float32 and 10 for float16 targets)."""
+    means 10, at most 15 for float32 and 10 for float16 targets); ``"int"``
+    for signed integer targets, which round to whole numbers."""
     rounding = getattr(tensor, "rounding", 0)
     if not rounding:
         return 0
@@ -172,6 +173,10 @@ def stochastic_bits(tensor):
         cap = 10
     elif dtype == bfloat16:
         cap = 7
+    elif dtype.kind == "i":
+        # signed integer targets round to whole numbers, whatever number of bits is asked for
+        # (reference cuda_templates.py:236-286: fp32_to_int32_rand / int16 / int8)
+        return "int"
     else:
         raise NotImplementedError("stochastic rounding into %s tensors" % dtype)
     return 10 if rounding is True else max(1, min(int(rounding), cap))
@@ -377,7 +382,7 @@ class Program(object):
             self.key_parts.append(("sround", bits))
             value_node = root
             root = self._intern(("sround", ordinal),
-                                lambda: Node("E", op="sround:%d" % bits, args=(value_node,), slot=ordinal,
+                                lambda: Node("E", op="sround:%s" % bits, args=(value_node,), slot=ordinal,
                                              axis=out_slot.index))     # axis field: the slot stored to
         out_slot.written = True
         st = Statement(out_slot, root)

@@ -62,13 +62,18 @@ def _ceil_div(a, b):
 # (the role of neon/backends/util/source_module.py:16-22 for the reference)
 # ---------------------------------------------------------------------------------------
 class KernelCache(object):
-    def __init__(self, arch, cache_dir=None):
+    def __init__(self, arch, cache_dir=None, formal_fences=None):
         self.arch = arch
         with open(hiprt.DEVICE_HEADER) as f:
             self.header = f.read()
-        if os.environ.get("NEON_HIP_FORMAL_FENCES", "0") != "0":
-            # device-scope release / acquire around the inter-workgroup hand-offs instead of
-            # the store-wait the default build relies on (see neon_device.h)
+        if formal_fences is None:
+            # The default hand-off between workgroups leans on how gfx950 acknowledges write-through
+            # stores (see neon_device.h); on any other part the kernels are built with the
+            # device-scope release / acquire fences the language's memory model asks for.
+            formal_fences = (os.environ.get("NEON_HIP_FORMAL_FENCES", "0") != "0"
+                             or not arch.startswith("gfx950"))
+        self.formal_fences = bool(formal_fences)
+        if self.formal_fences:
             self.header = "#define NH_FORMAL_FENCES 1\n" + self.header
         if os.environ.get("NEON_HIP_EXACT_LSE_TERMS", "0") != "0":
             # the terms of a running sum of exponentials each rounded like expf (see nh_exp_term)

@@ -28,6 +28,11 @@ from neon_amd.backends.hip import codegen, planner
 from neon_amd.backends.hip.planner import KernelCache, NeedsSplit, make_plan
 
 logger = logging.getLogger(__name__)
+# the level the reference prints its per-launch timings at (neon/__init__.py:36-44: above WARNING,
+# so they show without any logging set-up)
+DISPLAY_LEVEL = 41
+if logging.getLevelName(DISPLAY_LEVEL) == "Level %d" % DISPLAY_LEVEL:
+    logging.addLevelName(DISPLAY_LEVEL, "DISPLAY")
 
 _none_slice = slice(None, None, None)
 _DTYPES = (np.float16, np.float32, np.uint8, np.int8, np.uint16, np.int16,
@@ -237,7 +242,7 @@ class HIPTensorBase(object):
         be = self.backend
         if isinstance(value, self._api.OpTreeNode):
             if (be._replayer is not None and not be._fusing and be._captured is None and be._recording is None
-                    and not self.rounding and be._replay_in_c(self, value)):
+                    and not self.rounding and not be.bench and be._replay_in_c(self, value)):
                 return self              # a statement seen before: its recorded launches went out
             # (what OpTreeNode.build("assign", ...) comes to, without inferring a shape nobody reads)
             be.execute(self._api.OpTreeNode({"op": "assign", "shape": self.shape}, self, value))
@@ -519,7 +524,8 @@ class NervanaHIPBase(object):
         self.device_type = 1
         self.device_id = device_id or 0
         self.round_mode = None
-        self.bench = bench
+        self.bench = bench            # truthy: every launch is timed and reported (see _launch_plan)
+        self._bench_events = None
         self.stream = None
         self.use_pinned_mem = False
         self.hist_bins, self.hist_offset = hist_bins, hist_offset
@@ -545,10 +551,17 @@ class NervanaHIPBase(object):
         self._launch_cache = {}      # statement-group identity -> recorded launches
         self._replayer = self._records_type = None
         if fastpath.enabled():
-            # repeated single statements: walk, lookup and launches in C (neon_amd/csrc/fastpath.c)
-            mod = fastpath.load()
-            self._replayer = mod.Replayer(self._launch_cache, self.tensor_cls, self.rt.launch_prepared_address)
-            self._records_type = mod.Records
+            # repeated single statements: walk, lookup and launches in C (neon_amd/csrc/fastpath.c).
+            # Without the extension the same walk and lookup happen in Python: slower per call,
+            # the same launches.
+            try:
+                mod = fastpath.load()
+            except ImportError as e:
+                logger.warning("running without the C replayer: %s", e)
+                mod = None
+            if mod is not None:
+                self._replayer = mod.Replayer(self._launch_cache, self.tensor_cls, self.rt.launch_prepared_address)
+                self._records_type = mod.Records
         self._recording = None
         self._rec_temps = None
         self._rec_coop = None
@@ -620,6 +633,8 @@ class NervanaHIPBase(object):
         if failed:
             self._launch_cache.clear()       # recorded launches of the abandoned plans must not be replayed
             self.rt.synchronize()
+            for key in failed:               # nothing launches them any more: their workspaces go back
+                pending[key].release()
             raise hiprt.HipError(hiprt.NH_ECOOP, "a cooperative kernel gave up waiting for its other workgroups "
                                  "(%d plan(s)): results since the last synchronisation are invalid; these "
                                  "op-trees now run without inter-workgroup waits" % len(failed))
@@ -901,7 +916,8 @@ class NervanaHIPBase(object):
     def execute(self, optree):
         """Run ``assign(out, expr)`` (reference nervanagpu.py:1255-1283)."""
         assert optree[0]["op"] == "assign"
-        if not self._fusing and self._captured is None and self._recording is None and not optree[1].rounding:
+        if (not self._fusing and self._captured is None and self._recording is None and not optree[1].rounding
+                and not self.bench):
             # a single statement outside any group: ONE walk over the tree yields the replay
             # key; a statement seen before costs that walk, a dictionary lookup and its launches
             if self._replayer is not None and self._replay_in_c(optree[1], optree[2]):
@@ -925,7 +941,8 @@ class NervanaHIPBase(object):
                 stats["replayed"] += 1
                 stats["launches"] += len(entry.launches)
                 return optree[1]
-        if self._fusing and self._replayer is not None and self._captured is None and self._recording is None:
+        if (self._fusing and self._replayer is not None and self._captured is None and self._recording is None
+                and not self.bench):
             # inside a fusion group: just queue.  When the group ends, ONE walk in C over all
             # its statements yields the key of the launch cache; only a group never seen before
             # is taken apart statement by statement (_enqueue)
@@ -1067,6 +1084,8 @@ class NervanaHIPBase(object):
         Returns the recording that now stands for the group (None when the
         group cannot be replayed)."""
         try:
+            if self.bench:
+                raise TypeError("bench mode times every launch: nothing is replayed")
             key, raw = self._launch_key(trees, posts)
             if self._originals:
                 key = key + ("reads-before-group",)
@@ -1116,7 +1135,25 @@ class NervanaHIPBase(object):
             prog.rng_args = (self._rng_dev_seed, self._rng_dev_counter)
             self._rng_dev_counter += n
         args = plan.pack(prog)
-        self.rt.launch_packed(plan.kernel, plan.grid, plan.block, args)
+        if self.bench:
+            # the reference's bench mode (float_ew.py:917-938): events round the launch, one
+            # line per launch -- here with the bytes the statement group has to move (every
+            # tensor once per direction) and what that comes to per second
+            if self._bench_events is None:
+                self._bench_events = (self.rt.event(), self.rt.event())
+            e0, e1 = self._bench_events
+            self.rt.event_record(e0)
+            self.rt.launch_packed(plan.kernel, plan.grid, plan.block, args)
+            self.rt.event_record(e1)
+            self.rt.event_sync(e1)
+            msecs = self.rt.event_elapsed_ms(e0, e1)
+            nbytes = sum(t.dtype.itemsize * t.shape[0] * t.shape[1] * (int(t.read) + int(t.written))
+                         for t in prog.tensors)
+            logger.log(DISPLAY_LEVEL, "%7.3f msecs %8.1f GB/s shape(%d,%d) grid(%d,%d) blk(%d) %s",
+                       msecs, nbytes / max(msecs, 1e-6) * 1e-6, plan.domain[0], plan.domain[1],
+                       plan.grid[0], plan.grid[1], plan.block[0], plan.spec.name)
+        else:
+            self.rt.launch_packed(plan.kernel, plan.grid, plan.block, args)
         if plan.status_ptr is not None:
             self._coop_pending[plan.key] = plan
             if self._rec_coop is not None:
@@ -1800,7 +1837,7 @@ class NervanaHIPBase(object):
         """enqueue the launches recorded for an earlier identical call of a
         compound operation, without building its trees again; False when
         there is no such recording (or launches are being captured)"""
-        if self._captured is not None or self._recording is not None:
+        if self._captured is not None or self._recording is not None or self.bench:
             return False
         self._flush()
         found = self._launch_cache.get(ckey)

@@ -405,6 +405,18 @@ NEON_DEV float nh_sround(float x, int bits, nh_u32 rnd) {
     return __builtin_bit_cast(float, (b + noise) & (0xffffffffu << drop));
 }
 
+// Stochastic rounding to a whole number (stores into signed integer tensors;
+// the reference adds a uniform fraction with the value's sign, rounding toward
+// zero, and truncates: cuda_templates.py:236-286).  x = n + f with n = trunc(x):
+// the result is n, or the next whole number away from zero with probability
+// |f| -- decided by comparing |f| with a uniform 24-bit fraction, every step
+// exact, so the expectation is x.  The store then converts an integral value.
+NEON_DEV float nh_sround_int(float x, nh_u32 rnd) {
+    const float n = __builtin_truncf(x);
+    const float f = __builtin_fabsf(x - n);
+    return (nh_rand01(rnd) < f) ? n + __builtin_copysignf(1.0f, x) : n;
+}
+
 // ---------------------------------------------------------------------------
 // DPP lane permutations.  Every lane of the wave must be active at the call.
 // ---------------------------------------------------------------------------

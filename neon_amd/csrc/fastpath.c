@@ -277,7 +277,11 @@ static PyObject* Replayer_key(Replayer* self, PyObject* args) {
     if (!key) { walk_release(&w); return NULL; }
     PyObject* nums = PyList_New(w.nraw);
     if (!nums) { Py_DECREF(key); return NULL; }
-    for (Py_ssize_t i = 0; i < w.nraw; ++i) PyList_SET_ITEM(nums, i, PyFloat_FromDouble(w.raw[i]));
+    for (Py_ssize_t i = 0; i < w.nraw; ++i) {
+        PyObject* f = PyFloat_FromDouble(w.raw[i]);
+        if (!f) { Py_DECREF(key); Py_DECREF(nums); return NULL; }
+        PyList_SET_ITEM(nums, i, f);
+    }
     PyObject* r = PyTuple_Pack(2, key, nums);
     Py_DECREF(key);
     Py_DECREF(nums);
@@ -329,7 +333,8 @@ static PyObject* Replayer_key_group(Replayer* self, PyObject* trees) {
 }
 
 /* replay(out, value) -> 1: the statement's recorded launches were issued; 0: not handled here;
- * a negative number: minus the error code nh_launch_prepared returned (launches may be partly issued) */
+ * a negative number: minus the error code nh_launch_prepared returned (launches may be partly
+ * issued; the recording has been dropped from the cache) */
 static PyObject* Replayer_replay(Replayer* self, PyObject* const* args, Py_ssize_t nargs) {
     if (nargs != 2) { PyErr_SetString(PyExc_TypeError, "replay(out, value)"); return NULL; }
     Walk w;
@@ -339,10 +344,9 @@ static PyObject* Replayer_replay(Replayer* self, PyObject* const* args, Py_ssize
         PyObject* key = build_key(&w);
         if (!key) goto unhandled;
         PyObject* entry = self->cache ? PyDict_GetItemWithError(self->cache, key) : NULL;      /* borrowed */
-        Py_DECREF(key);
-        if (!entry) goto unhandled;
+        if (!entry) { Py_DECREF(key); goto unhandled; }
         PyObject* recs = PyObject_GetAttr(entry, s_fast);
-        if (!recs) goto unhandled;
+        if (!recs) { Py_DECREF(key); goto unhandled; }
         if (Py_TYPE(recs) == &RecordsType) {
             Records* r = (Records*)recs;
             int same = r->nraw == w.nraw;
@@ -356,10 +360,14 @@ static PyObject* Replayer_replay(Replayer* self, PyObject* const* args, Py_ssize
                 if (result == 1) {
                     self->replayed += 1;
                     self->launches += r->nrec;
+                } else if (PyDict_DelItem(self->cache, key) < 0) {
+                    /* a recording whose launch failed is not offered again (the caller raises) */
+                    PyErr_Clear();
                 }
             }
         }
         Py_DECREF(recs);
+        Py_DECREF(key);
         return PyLong_FromLong(result);
     }
 unhandled:

@@ -160,3 +160,51 @@ def test_foreign_update_block_fuses(fhip):
     for layer_kernel in ("conv_layer", "fprop_pool"):
         with pytest.raises(NotImplementedError):
             getattr(fhip, layer_kernel)()
+
+
+def test_every_name_of_the_reference_surface_is_supplied():
+    """tests/golden/api_surface.json holds the names read off the reference
+    (abstract_backend.py:40-1428: 68 abstract methods; backend.py:45-435: the
+    Tensor class; backend.py:437-1680: what its Backend class itself defines).
+    A host laid out the same way -- an abstract class declaring all 68, a
+    Backend below it defining what the reference's Backend defines -- is bound,
+    and nothing may be left abstract; the tensor class answers every Tensor
+    method, and overrides every one that the reference's base class only
+    raises from."""
+    import abc
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "api_surface.json")) as f:
+        surface = json.load(f)
+    assert len(surface["abstract_methods"]) == 68
+
+    def stub():
+        def method(self, *args, **kwargs):
+            raise NotImplementedError()
+        return method                     # (abc.abstractmethod marks the function object itself)
+
+    declared = dict((name, abc.abstractmethod(stub())) for name in surface["abstract_methods"])
+    AbstractHost = F.Registry("AbstractHost", (F.Backend,), dict(declared, __module__=F.__name__))
+    in_backend_py = dict((name, stub()) for name in surface["backend_methods"] if name in declared)
+    HostBackend = F.Registry("HostBackend", (AbstractHost,), dict(in_backend_py, __module__=F.__name__))
+    left_to_the_concrete_backend = set(surface["abstract_methods"]) - set(in_backend_py)
+    assert {"empty", "array", "zeros", "ones", "empty_like", "zeros_like", "compound_dot", "gen_rng",
+            "rng_reset", "fprop_conv", "make_binary_mask"} <= left_to_the_concrete_backend
+    first = F.Backend.backends.get("hip")
+    try:
+        NervanaHIP, HIPTensor = nervanahip.bind(HostBackend, F.Node, F.Tensor, F.Block)
+        assert NervanaHIP.__abstractmethods__ == frozenset(), sorted(NervanaHIP.__abstractmethods__)
+        for name in left_to_the_concrete_backend:
+            assert name in vars(nervanahip.NervanaHIPBase), name
+    finally:
+        if first is not None:
+            F.Backend.backends["hip"] = first
+    missing = [name for name in surface["tensor_methods"] if not hasattr(nervanahip.HIPTensorBase, name)
+               and not hasattr(own.Tensor, name)]
+    assert missing == [], missing
+    own_tensor = nervanahip.bind()[1]
+    for name in surface["tensor_abstract"]:
+        if name == "_assign" or not name.startswith("_") or name in ("__getitem__", "__setitem__", "__len__",
+                                                                      "__str__", "__repr__"):
+            assert name in vars(nervanahip.HIPTensorBase), "%s is only a stub in the base class" % name
+    assert callable(getattr(own_tensor, "dimension_reorder", None)) or "dimension_reorder" not in surface["tensor_methods"]

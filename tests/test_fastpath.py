@@ -379,3 +379,39 @@ def test_c_node_builder_builds_the_nodes_python_builds():
                 else:
                     assert got is want, (op, a, b, got, want)
     assert checked > 2000
+
+
+def test_the_extension_is_clean_under_address_and_undefined_behaviour_sanitizers(tmp_path):
+    """fastpath.c built with -fsanitize=address,undefined and this file's CPU
+    tests (key walks, node builder, records, error paths) run against that
+    build in a child process with the sanitizer runtime preloaded: no report"""
+    import os
+    import shutil
+    import subprocess
+    import sys
+    import sysconfig
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    runtime = subprocess.run([gcc, "-print-file-name=libasan.so"], capture_output=True, text=True).stdout.strip()
+    if not os.path.isabs(runtime) or not os.path.exists(runtime):
+        pytest.skip("no address sanitizer runtime")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    lib = str(tmp_path / "_fastpath.so")
+    build = subprocess.run([gcc, "-O1", "-g", "-fPIC", "-shared", "-fsanitize=address,undefined",
+                            "-fno-omit-frame-pointer", "-I" + sysconfig.get_paths()["include"],
+                            os.path.join(root, "neon_amd", "csrc", "fastpath.c"), "-o", lib],
+                           capture_output=True, text=True)
+    assert build.returncode == 0, build.stderr[-2000:]
+    env = dict(os.environ)
+    env["NEON_HIP_FASTPATH_LIB"] = lib
+    env["LD_PRELOAD"] = runtime + (":" + env["LD_PRELOAD"] if env.get("LD_PRELOAD") else "")
+    env["ASAN_OPTIONS"] = "detect_leaks=0:verify_asan_link_order=0:abort_on_error=0"
+    env["UBSAN_OPTIONS"] = "print_stacktrace=1"
+    run = subprocess.run([sys.executable, "-m", "pytest", os.path.abspath(__file__), "-q", "-m", "not gpu",
+                          "-p", "no:cacheprovider", "-k", "not sanitizers"], cwd=root, env=env,
+                         capture_output=True, text=True, timeout=600)
+    report = run.stdout[-3000:] + run.stderr[-3000:]
+    assert run.returncode == 0, report
+    assert "AddressSanitizer" not in report and "runtime error:" not in report, report
+    assert " passed" in run.stdout

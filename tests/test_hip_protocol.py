@@ -50,6 +50,45 @@ def test_soak_alternating_split_and_cooperative_launches(hip, monkeypatch):
 
 
 @pytest.mark.gpu
+def test_the_hand_offs_built_with_release_and_acquire_fences(hip, monkeypatch):
+    """the variant parts other than gfx950 get by default (device-scope release
+    before a counter update, acquire after reading it): the same three
+    families, compiled with it, against numpy"""
+    monkeypatch.setattr(planner, "COLCOOP_MIN_BYTES", 0)
+    hip.synchronize()
+    kernels, plans, cache = hip.kernels, hip.plans, dict(hip._launch_cache)
+    hip.kernels = planner.KernelCache(kernels.arch, formal_fences=True)
+    assert hip.kernels.formal_fences and "#define NH_FORMAL_FENCES 1" in hip.kernels.header
+    hip.plans = {}
+    hip._launch_cache.clear()
+    try:
+        xs, xc, xr = hip.empty((2048, 128)), hip.empty((20000, 64)), hip.empty((8, 40000))
+        am, mx = hip.empty((1, 128), dtype=np.int32), hip.empty((1, 128))
+        devc, dev = hip.empty((20000, 64)), hip.empty((8, 40000))
+        for rnd in range(3):
+            for t in (xs, xc, xr):
+                t[:] = hip.rand() * 8.0 - 4.0
+            am[:] = hip.argmax(xs, axis=0)
+            mx[:] = hip.max(xs, axis=0)
+            devc[:] = xc - hip.mean(xc, axis=0)
+            dev[:] = xr - hip.mean(xr, axis=1)
+            hs, hc, hr = xs.get(), xc.get().astype(np.float64), xr.get().astype(np.float64)
+            assert np.array_equal(am.get(), hs.argmax(axis=0).reshape(1, -1).astype(np.int32))
+            assert np.array_equal(mx.get(), hs.max(axis=0, keepdims=True))
+            assert_close(devc.get(), hc - hc.mean(axis=0, keepdims=True), rtol=1e-5, atol=1e-5)
+            assert_close(dev.get(), hr - hr.mean(axis=1, keepdims=True), rtol=1e-5, atol=1e-5)
+        assert {"colsplit", "colcoop", "rowcoop"} <= _families(hip)
+    finally:
+        hip.synchronize()
+        for plan in hip.plans.values():
+            for p_ in (plan if isinstance(plan, list) else [plan]):
+                p_.release()
+        hip.kernels, hip.plans = kernels, plans
+        hip._launch_cache.clear()
+        hip._launch_cache.update(cache)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("family", ["colcoop", "rowcoop"])
 def test_a_cooperative_kernel_that_gave_up_is_reported_and_replaced(pair, family, monkeypatch):
     """Nothing is made to hang: the word an aborting workgroup would leave is

@@ -126,6 +126,32 @@ def test_sr_unbiased_neighbours(hip, dtype, bits):
     assert np.all(err <= 5 * 0.5 * ulp / np.sqrt(cols) + 1e-7)
 
 
+@pytest.mark.parametrize("dtype", [np.int32, np.int16, np.int8], ids=["i32", "i16", "i8"])
+def test_sr_into_integer_tensors_is_unbiased(hip, dtype):
+    """stores into signed integer tensors with ``rounding`` set go to one of the
+    two neighbouring whole numbers, the farther one from zero with probability
+    equal to the fraction (reference cuda_templates.py:236-286); whole numbers
+    stay as they are"""
+    rs = np.random.RandomState(12)
+    rows, cols = 64, 8192
+    x = (rs.rand(rows, 1) * 100.0 * np.where(rs.rand(rows, 1) < 0.5, -1, 1)).astype(np.float32)
+    x[:4, 0] = [3.0, -7.0, 0.0, 99.0]
+    out = hip.empty((rows, cols), dtype=dtype)
+    out.rounding = True
+    out[:] = hip.array(x) + hip.zeros((1, cols))           # each row: one value, 8192 draws
+    got = out.get().astype(np.float64)
+    lo = np.trunc(x)
+    hi = lo + np.sign(x) * (x != lo)
+    assert np.all((got == lo) | (got == hi))
+    assert np.all(got[:4] == x[:4])
+    err = np.abs(got.mean(axis=1, keepdims=True) - x)
+    assert np.all(err <= 5 * 0.5 / np.sqrt(cols) + 1e-6)
+    # without the attribute the store truncates, as the CPU backend's cast does
+    plain = hip.empty((rows, cols), dtype=dtype)
+    plain[:] = hip.array(x) + hip.zeros((1, cols))
+    assert np.array_equal(plain.get(), np.broadcast_to(np.trunc(x), (rows, cols)).astype(dtype))
+
+
 def test_sr_leaves_representable_values_and_specials(hip):
     x = np.array([[0.0, 1.0, -2.5, 0.75, np.inf, -np.inf, np.nan, 1024.0]], dtype=np.float32)
     out = hip.empty(x.shape, dtype=np.float32)

@@ -172,3 +172,30 @@ def test_copy_transpose_axes_given_as_a_list(hip):
     hip.copy_transpose(x, out, axes=[2, 0, 1])
     assert np.array_equal(out.get(), a.transpose(2, 0, 1))
     assert isinstance(x[0].T, type(x)) and isinstance((x[0] * 2).T, OpTreeNode)
+
+
+@pytest.mark.gpu
+def test_bench_mode_reports_every_launch(caplog):
+    """``bench=True``: events round every launch and one line per launch with
+    time, bytes per second, shape, grid, block and the kernel's name
+    (reference float_ew.py:917-938 prints `msecs shape blk,thd name`)"""
+    import logging
+    from neon_amd.backends import NervanaHIP
+    from neon_amd.backends import nervanahip
+    be = NervanaHIP(rng_seed=0, bench=True)
+    try:
+        x = be.array(np.arange(64 * 256, dtype=np.float32).reshape(64, 256))
+        out, line = be.empty((64, 256)), be.empty((1, 256))
+        with caplog.at_level(nervanahip.DISPLAY_LEVEL, logger=nervanahip.logger.name):
+            caplog.clear()
+            for _ in range(3):                    # repeated statements are timed too: nothing is replayed
+                out[:] = x * 2.0 + 1.0
+            line[:] = be.max(x, axis=0)
+        lines = [r.getMessage() for r in caplog.records if r.levelno == nervanahip.DISPLAY_LEVEL]
+        assert len(lines) == 4
+        assert all("msecs" in l and "GB/s" in l and "shape(" in l and "grid(" in l and "blk(" in l for l in lines)
+        assert "nk_ew_mul_add" in lines[0] and "_max_" in lines[3]
+        np.testing.assert_array_equal(out.get(), np.arange(64 * 256, dtype=np.float32).reshape(64, 256) * 2.0 + 1.0)
+        assert logging.getLevelName(nervanahip.DISPLAY_LEVEL) == "DISPLAY"
+    finally:
+        be.cleanup_backend()
