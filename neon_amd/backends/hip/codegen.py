@@ -55,6 +55,13 @@ _RED_OP = {"sum": "nh_op_sum", "max": "nh_op_max", "min": "nh_op_min",
            "argmax": "nh_op_argmax", "argmin": "nh_op_argmin"}
 
 
+# The ticket counters of neighbouring strips (rows, for the cooperating row family) sit this many 32-bit words apart.  Atomics on one
+# cache line are served one after the other, whichever words of it they address: with the
+# counters of all strips in one line, the 256 workgroups of an (8 strips x 32 chunks) grid queued
+# behind each other for 2 us (max over (32000,256): 7.3 -> 5.1 us with a line per strip).
+TICKET_STRIDE_WORDS = 64
+
+
 # Streaming kernels (working set far beyond the caches) read with non-temporal
 # loads.  Their stores are ordinary ones, except in the row family: measured
 # on the 7-stream fused Adam update, non-temporal loads with ordinary stores
@@ -903,8 +910,9 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
     exchanges = [0]
     if coop:
         L("__shared__ int s_abort;")
-        L("unsigned int* ctr = reinterpret_cast<unsigned int*>(ws + ctr_offset) + 2 * blockIdx.x;")
-        L("unsigned int* status = reinterpret_cast<unsigned int*>(ws + ctr_offset) + 2 * gridDim.x;")
+        # (the counters of neighbouring lines a cache line apart, see TICKET_STRIDE_WORDS)
+        L("unsigned int* ctr = reinterpret_cast<unsigned int*>(ws + ctr_offset) + %d * blockIdx.x;" % TICKET_STRIDE_WORDS)
+        L("unsigned int* status = reinterpret_cast<unsigned int*>(ws + ctr_offset) + %d * gridDim.x;" % TICKET_STRIDE_WORDS)
         L("nh_pair* part = reinterpret_cast<nh_pair*>(ws) + (long long)blockIdx.x * %d;" % (len(all_reds) * chunks))
 
     SU = 4      # column tiles in flight per lane when the row is streamed
@@ -1182,12 +1190,60 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
         if not all(merged):
             merged = []
     span = NCH * LX * V      # elements of a row that one workgroup owns
+    # The same identity with the LANES of one workgroup as the parts, for rows that sit in
+    # registers whole: every lane accumulates sum(x - s) and sum((x - s)^2) around a value s of
+    # its own (the first element it holds) WHILE ITS TILES ARRIVE, in the sweep that adds up x;
+    # once the row's sum is known a lane's share of sum((x - a)^2) is M2 + n (mean - a)^2 from
+    # those two numbers, and the second pass over the registers -- a microsecond and a half
+    # between the last load and the first store of a (256, 100352) fp16 normalisation, during
+    # which the memory system idles -- is gone.  Rounding: that of a two-pass variance inside
+    # every lane's share (its s is one of its own values), exact combination across lanes.
+    # (the workgroups of a shared row take their OWN part's second moment the same way)
+    coop_lane = []
+    if (merged and resident and keep_words is None
+            and all(m[2].kind == "T" and varies_in_loop(m[2]) for m in merged)):
+        coop_lane = merged
+    lane_merged = []
+    if (not coop and MERGED_MOMENTS and resident and LX > 64 and keep_words is None and not over and not own
+            and per_level.get(0) and per_level.get(1)):
+        lane_merged = [_shifted_square_sum(n2, per_level[0]) for n2 in per_level[1]]
+        if not all(lane_merged) or any(m[2].kind != "T" or not varies_in_loop(m[2]) for m in lane_merged):
+            lane_merged = []
+
+    def derived(x):
+        # 16-bit operands (eight elements per load: the sweep is bound by instruction issue):
+        # sum(x - s) is taken from the lane's plain sum, sum(x) - n s, instead of being added up
+        # element by element.  What the subtraction cancels is bounded by what 11-bit inputs
+        # can hold (|mean| / spread below 2^11, or the spread is quantisation noise anyway).
+        return prog.tensors[x.slot].dtype.itemsize == 2
+
+    def lane_share(n2, r1, x, about):
+        """``term_`` = this lane's share of sum((x - about)^2) from what it gathered while its
+        tiles arrived (sh: its reference value, sa: sum(x - sh), sb: sum((x - sh)^2), cnt):
+        M2 + n (mean - about)^2; nothing for a lane without elements"""
+        L("const float a_ = %s;" % about)
+        if derived(x):
+            L("sa%d = __builtin_fmaf(-cnt%d, sh%d, acc%d);" % (n2.nid, n2.nid, n2.nid, r1.nid))
+        L("const float inv_ = (cnt%d > 0.0f) ? 1.0f / cnt%d : 0.0f;" % (n2.nid, n2.nid))
+        L("const float mu_ = sa%d * inv_;" % n2.nid)
+        L("const float m2_ = nh_max(sb%d - sa%d * mu_, 0.0f);" % (n2.nid, n2.nid))
+        L("const float e_ = (sh%d + mu_) - a_;" % n2.nid)
+        L("const float term_ = (cnt%d > 0.0f) ? __builtin_fmaf(cnt%d * e_, e_, m2_) : 0.0f;" % (n2.nid, n2.nid))
 
     def local_second_moments():
         """after the first sweep's fold inside the workgroup (red<sum> = this part's sum):
         red<n2> = sum over this part of (x - this part's mean)^2"""
         L("const long long left_ = (long long)C - (long long)blockIdx.y * %dll;" % span)
         L("const float n_loc = (float)(left_ < %dll ? left_ : %dll);" % (span, span))
+        if coop_lane:
+            # from what every lane gathered during the first sweep: no second pass over the registers
+            for n2, r1, x, a in merged:
+                L("float red%d;" % n2.nid)
+                L.open("")
+                lane_share(n2, r1, x, "red%d / n_loc" % r1.nid)
+                L("red%d = nh_block_allreduce<nh_op_sum, %d, float>(term_, s_f);" % (n2.nid, T // 64))
+                L.close()
+            return
         for n2, r1, x, a in merged:
             L("const float mu%d = red%d / n_loc;" % (n2.nid, r1.nid))
             vals[a.nid] = "mu%d" % n2.nid
@@ -1242,7 +1298,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
             done[n2.nid] = n2
 
     for s in range(nsweeps):
-        if merged and s == 1:
+        if (merged or lane_merged) and s == 1:
             continue            # done together with the first sweep
         reds = g.own_reductions(per_level.get(s, []))
         if not reds:
@@ -1258,9 +1314,33 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
         fresh_own = [n for n in nodes if n.nid in own and n.nid not in vals and n.nid not in over]
         for n in fresh_own:
             L("float val%d[%d][%d];" % (n.nid, NCH, V))
+        riding = (lane_merged or coop_lane) if s == 0 else []
 
-        def reduce_body(tiles, nodes=nodes, reds=reds, fresh=fresh, fresh_own=fresh_own):
+        for n2, r1, x, a in riding:
+            L("float sh%d = 0.0f, sa%d = 0.0f, sb%d = 0.0f, cnt%d = 0.0f;" % (n2.nid, n2.nid, n2.nid, n2.nid))
+
+        def reduce_body(tiles, nodes=nodes, reds=reds, fresh=fresh, fresh_own=fresh_own, riding=riding):
             L.open("if (ok)")
+            for n2, r1, x, a in riding:
+                # the lane's own reference value: the first element it holds
+                L("if (k == 0) sh%d = %s.get(0);" % (n2.nid, tiles[x.nid]))
+                L("cnt%d += %s;" % (n2.nid, ("(float)lim" if tail else "%d.0f" % V)))
+                if V > 1:
+                    L("#pragma unroll")
+                L.open("for (int j = 0; j < %d; ++j)" % V)
+                if tail:
+                    L.open("if (j < lim)")
+                xv = "%s.get(j)" % tiles[x.nid]
+                if g.is_half_leaf(x) and g.one_declared:
+                    L("const float d_ = __builtin_fmaf(%s, nh_one, -sh%d);" % (xv, n2.nid))
+                else:
+                    L("const float d_ = %s - sh%d;" % (xv, n2.nid))
+                if not derived(x):
+                    L("sa%d += d_;" % n2.nid)
+                L("sb%d = __builtin_fmaf(d_, d_, sb%d);" % (n2.nid, n2.nid))
+                if tail:
+                    L.close()
+                L.close()
             # plain sums of a packed fp16 operand: two elements per instruction, straight
             # from the tile (a partial last tile is zero-filled, so it needs no guard)
             pairwise = [n for n in reds if n.op == "sum" and g.is_half_leaf(n.args[0]) and V % 2 == 0
@@ -1333,6 +1413,17 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
             done[n.nid] = n
         if coop and merged and s == 0:
             combine_second_moments()
+        if riding and not coop:
+            line_ref = g.make_ref("_s", "rr", "0", 1, dict((nid, name) for nid, name in line_tiles.items()), vals)
+            for n2, r1, x, a in riding:
+                L("float rv%d;" % n2.nid)
+                L.open("")
+                L("const int j = 0; (void)j;")
+                g.emit_exprs(_needed([a], stops()), line_ref, stops())
+                lane_share(n2, r1, x, line_ref(a))
+                L("rv%d = nh_block_allreduce<nh_op_sum, %d, float>(term_, s_f);" % (n2.nid, T // 64))
+                L.close()
+                done[n2.nid] = n2
 
     # outputs that have one value per row
     if line_out:
@@ -1434,7 +1525,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
     return _finish("rowcoop" if coop else "row", g, head, fmt, T, 0,
                    dict(V=V, LX=LX, LY=LY, NCH=NCH, stream=bool(stream), passing=len(transient),
                         over=len([k for k in vals if k in over]), kept=len([k for k in vals if k in own]), chunks=chunks, NRED=len(all_reds), tail=bool(tail),
-                        parked=sum(park.values()), held=sum(hold.values())))
+                        parked=sum(park.values()), held=sum(hold.values()), lane_moments=len(lane_merged)))
 
 
 # =====================================================================================
@@ -1603,8 +1694,9 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False)
         L("const int clim = cfull ? %d : (col_ok ? (int)(C - c) : 0);" % V)
     if coop:
         L("__shared__ int s_abort;")
-        L("unsigned int* ctr = reinterpret_cast<unsigned int*>(ws + ctr_offset) + 2 * blockIdx.x;")
-        L("unsigned int* status = reinterpret_cast<unsigned int*>(ws + ctr_offset) + 2 * gridDim.x;")
+        # (the counters of neighbouring lines a cache line apart, see TICKET_STRIDE_WORDS)
+        L("unsigned int* ctr = reinterpret_cast<unsigned int*>(ws + ctr_offset) + %d * blockIdx.x;" % TICKET_STRIDE_WORDS)
+        L("unsigned int* status = reinterpret_cast<unsigned int*>(ws + ctr_offset) + %d * gridDim.x;" % TICKET_STRIDE_WORDS)
     all_reds = g.own_reductions([n for lv in sorted(per_level) for n in per_level[lv]])
     red_slot = dict((n.nid, k) for k, n in enumerate(all_reds))
     exchanges = [0]
@@ -2027,11 +2119,6 @@ COLSPLIT_ROWS_IN_FLIGHT = 4
 COLSPLIT_BATCH_ROWS = 8
 COLSPLIT_SUBBATCH_ROWS = 8
 COLSPLIT_BATCH_WORDS = 64
-# The ticket counters of neighbouring strips sit this many 32-bit words apart.  Atomics on one
-# cache line are served one after the other, whichever words of it they address: with the
-# counters of all strips in one line, the 256 workgroups of an (8 strips x 32 chunks) grid queued
-# behind each other for 2 us (max over (32000,256): 7.3 -> 5.1 us with a line per strip).
-TICKET_STRIDE_WORDS = 64
 
 
 def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, NB=4, multi=True):

@@ -480,8 +480,9 @@ def _plan_row(prog, cu_count, coop=True):
                                    park_bytes=ROW_PARK_BYTES if kw else 0)
             part_bytes = R * spec.params["NRED"] * chunks * 8
             ctr_off = _ceil_div(part_bytes, 256) * 256
-            return Choice(spec, (R, chunks, 1), workspace=(ctr_off + R * 8 + 4, ctr_off, 2 * R + 1),
-                          status_offset=ctr_off + R * 8)
+            stride = codegen.TICKET_STRIDE_WORDS      # arrivals and departures of a row; rows a cache line apart
+            return Choice(spec, (R, chunks, 1), workspace=(ctr_off + (R * stride + 1) * 4, ctr_off, R * stride + 1),
+                          status_offset=ctr_off + R * stride * 4)
     LY = T // LX
     gx = _ceil_div(R, LY)
     park = ROW_PARK_BYTES if (keep_words and LY == 1) else 0
@@ -636,8 +637,9 @@ def _plan_col(prog, cu_count, coop=True):
                     part_bytes = spec.params["NRED"] * chunks * C * 8
                     ctr_off = _ceil_div(part_bytes, 256) * 256
                     return Choice(spec, (strips_c, chunks, 1),
-                                  workspace=(ctr_off + strips_c * 8 + 4, ctr_off, 2 * strips_c + 1),
-                                  status_offset=ctr_off + strips_c * 8)
+                                  workspace=(ctr_off + (strips_c * codegen.TICKET_STRIDE_WORDS + 1) * 4, ctr_off,
+                                             strips_c * codegen.TICKET_STRIDE_WORDS + 1),
+                                  status_offset=ctr_off + strips_c * codegen.TICKET_STRIDE_WORDS * 4)
 
     # (b) one level, one value per column, many rows: split rows over workgroups
     if single_level and line_only:
