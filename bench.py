@@ -644,6 +644,21 @@ def counter_pass():
     gg, gb = vec(0.0), vec(0.0)
     run("BN bprop (256,100352) f16", 3 * K * N * 2,
         lambda: be.compound_bprop_bn(o4, gg, gb, delta, x4, xsum, xvar, gamma, 1e-5))
+    del x4, o4, delta
+
+    # the two prebuilt kernels that go through LDS (their names are the compiler's: matched by a part)
+    def run_prebuilt(label, part, nbytes, call, reps=3):
+        for _ in range(reps + 1):
+            call()
+            be.synchronize()
+        table.append({"label": label, "kernel": None, "kernel_contains": part, "family": "prebuilt",
+                      "algorithmic_bytes": nbytes, "warmup": 0, "launches": reps + 1})
+    a32 = _fresh(be, configs.C3_SHAPE, rs=rs)
+    run_prebuilt("hist log2 (5000,5000) f32", "hist_log2_kernel", a32.size * 4, lambda: a32.hist("bench"))
+    sq = (8192, 8192)
+    t_in, t_out = _fresh(be, sq, rs=rs), be.empty(sq)
+    run_prebuilt("copy_transpose (8192,8192) f32", "transpose_tile", 2 * sq[0] * sq[1] * 4,
+                 lambda: be.copy_transpose(t_in, t_out))
     print(json.dumps({"pass": "counters", "rows": table}))
 
 

@@ -1677,13 +1677,21 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False)
     g.declare_one()
     L("const int tx = threadIdx.x %% %d, ty = threadIdx.x / %d;" % (LX, LX))
     wide = [t.dtype.itemsize for t in prog.tensors if t.shape[1] > 1]
-    if not coop and wide and LX * V * max(wide) < 128:
+    xcd_runs = bool(not coop and wide and LX * V * max(wide) < 128)
+    if xcd_runs:
         # Strips narrower than a cache line: neighbouring strips read the same lines.  Workgroups
         # are handed to the 8 XCDs (each with its own L2) round-robin, so consecutive strips
-        # would each pull those lines into a different L2; give every XCD a contiguous run of
-        # strips instead (softmax over (1000,128): 8x -> 2x the matrix fetched from memory).
-        L("const unsigned int strip = (gridDim.x % NH_XCDS == 0) ? (blockIdx.x % NH_XCDS) * (gridDim.x / NH_XCDS) "
-          "+ blockIdx.x / NH_XCDS : blockIdx.x;")
+        # would each pull those lines into a different L2.  Every XCD gets a contiguous run of
+        # strips instead, and a run is whole 128-byte lines: with fewer strips than that needs,
+        # fewer XCDs take part and the grid carries workgroups that leave at once (col_grid;
+        # softmax over (1000,128), memory traffic over the matrix's bytes: 5.1 with strips dealt
+        # round-robin, 1.6 with runs of half a line, 1.0 with whole lines on 4 of the 8 XCDs).
+        L("const unsigned int nstrips = (unsigned int)((C + %d) / %d);" % (LX * V - 1, LX * V))
+        L("unsigned int nx = nstrips / %du;" % max(1, 128 // (LX * V * max(wide))))
+        L("nx = nx < 1u ? 1u : (nx > NH_XCDS ? NH_XCDS : nx);")
+        L("const unsigned int per_xcd = (nstrips + nx - 1u) / nx;")
+        L("if (blockIdx.x % NH_XCDS >= nx || blockIdx.x / NH_XCDS >= per_xcd) return;")
+        L("const unsigned int strip = (blockIdx.x % NH_XCDS) * per_xcd + blockIdx.x / NH_XCDS;")
     else:
         L("const unsigned int strip = blockIdx.x;")
     L("const long long c = ((long long)strip * %d + tx) * %d;" % (LX, V))
@@ -2099,7 +2107,22 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False)
     L.close()
     return _finish("colcoop" if coop else "col", g, head, fmt, T, lds,
                    dict(V=V, LX=LX, LY=LY, NR=NR, stream=bool(stream), chunks=chunks,
-                        NRED=len(all_reds), kept=len(kept), over=len(over), tail=bool(tail)))
+                        NRED=len(all_reds), kept=len(kept), over=len(over), tail=bool(tail),
+                        line_strips=(max(1, 128 // (LX * V * max(wide))) if xcd_runs else 0)))
+
+
+def col_grid(spec, strips, xcds=8):
+    """workgroups a ``col`` kernel is launched with: one per strip, or -- strips narrower than
+    a cache line, dealt to the XCDs in runs of whole lines -- eight times the longest run"""
+    spl = spec.params.get("line_strips", 0)
+    if not spl:
+        return strips
+    nx = max(1, min(xcds, strips // spl))
+    return xcds * _ceil(strips, nx)
+
+
+def _ceil(a, b):
+    return -(-a // b)
 
 
 # (more chunks do not help tall narrow matrices: the one workgroup per strip that

@@ -602,7 +602,7 @@ def _plan_col(prog, cu_count, coop=True):
         budget = _COL_BUDGET[T]
         spare = max(0, (budget - NR * words) // (NR * V))
         spec = codegen.gen_col(prog, V, LX, LY, NR, _streams(prog), max_vals=min(2, spare), tail=tail)
-        return Choice(spec, (_ceil_div(nvec, LX), 1, 1))
+        return Choice(spec, (codegen.col_grid(spec, _ceil_div(nvec, LX)), 1, 1))
 
     # (c) deeper trees (or full-shape results) over many rows: the workgroups of a
     # strip keep their rows in registers and exchange partials between sweeps.

@@ -13,6 +13,7 @@ after the generator changed yields nothing instead of a stale number.
     python -m neon_amd.profile_summary durations --csv K.csv --log pass.log --out profiles/X.txt --command "..."
     python -m neon_amd.profile_summary traffic --fetch F.csv --write W.csv --log pass.log --out ... --command "..." --command "..."
     python -m neon_amd.profile_summary issue --csv S1.csv --csv S2.csv --log pass.log --out ... --command "..."
+    python -m neon_amd.profile_summary lds --csv L.csv --log pass.log --out ... --command "..."
 
 The metric for durations is the one the kernels are judged by: rocprofv3
 kernel duration (end - start timestamp of the dispatch), median over the
@@ -108,11 +109,20 @@ def _counters(csv_path):
     return agg
 
 
+def _resolve(rows, names):
+    """rows of prebuilt kernels name a part of the compiler's kernel name: fill in the full one"""
+    for r in rows:
+        if not r.get("kernel") and r.get("kernel_contains"):
+            found = [n for n in names if r["kernel_contains"] in n]
+            r["kernel"] = found[0] if found else r["kernel_contains"]
+    return rows
+
+
 def traffic(fetch_csv, write_csv, table, out_path, commands):
     """FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each scaled by what the same
     counter reads for the pass's plain copy kernel of known size"""
     fetch, write = _counters(fetch_csv), _counters(write_csv)
-    rows = table["rows"]
+    rows = _resolve(table["rows"], list(fetch))
     cal = rows[0]
     assert cal["label"].startswith("copy"), "the first row of a counter pass is the calibration copy"
     kib = cal["algorithmic_bytes"] / 2 / 1024.0
@@ -133,7 +143,7 @@ def traffic(fetch_csv, write_csv, table, out_path, commands):
     out.append("  FETCH_SIZE  %9.0f KiB reported for %.0f KiB read     -> scale factor %.4f" % (f_cal, kib, fs))
     out.append("  WRITE_SIZE  %9.0f KiB reported for %.0f KiB written  -> scale factor %.4f" % (w_cal, kib, ws))
     out.append("")
-    out.append("%-24s %12s %12s %12s %12s %7s  %s" % ("configuration", "FETCH KiB", "WRITE KiB", "HBM bytes", "algorithmic",
+    out.append("%-30s %12s %12s %12s %12s %7s  %s" % ("configuration", "FETCH KiB", "WRITE KiB", "HBM bytes", "algorithmic",
                                                "ratio", "kernel"))
     for r in rows[1:]:
         try:
@@ -142,8 +152,8 @@ def traffic(fetch_csv, write_csv, table, out_path, commands):
             out.append("%-24s  (kernel %s not in the counter files)" % (r["label"], r["kernel"]))
             continue
         total = (f * fs + w * ws) * 1024.0
-        out.append("%-24s %12.0f %12.0f %12.0f %12d %7.3f  %s" % (r["label"][:24], f, w, total, r["algorithmic_bytes"],
-                                                                 total / r["algorithmic_bytes"], r["kernel"]))
+        out.append("%-30s %12.0f %12.0f %12.0f %12d %7.3f  %s" % (r["label"][:30], f, w, total, r["algorithmic_bytes"],
+                                                                 total / r["algorithmic_bytes"], r["kernel"][:90]))
         js[r["kernel"]] = {"label": r["label"], "traffic_bytes": round(total), "algorithmic_bytes": r["algorithmic_bytes"],
                            "ratio": round(total / r["algorithmic_bytes"], 4)}
     out.append("")
@@ -164,6 +174,7 @@ def issue(csv_paths, table, out_path, commands, cu_count=256, clock_ghz=2.4):
         for name, per in _counters(p).items():
             for cname, vals in per.items():
                 agg[name][cname] = sum(vals) / len(vals)
+    _resolve(table["rows"], list(agg))
     out, js = [], {}
     out.append("Issue-side counters of the benchmark kernels, rocprofv3 on one MI355X (gfx950)")
     out.append("")
@@ -197,9 +208,45 @@ def issue(csv_paths, table, out_path, commands, cu_count=256, clock_ghz=2.4):
     return js
 
 
+def lds(csv_paths, table, out_path, commands):
+    """LDS instruction and conflict counters of the kernels that stage data in LDS"""
+    agg = collections.defaultdict(dict)
+    for p in csv_paths:
+        for name, per in _counters(p).items():
+            for cname, vals in per.items():
+                agg[name][cname] = sum(vals) / len(vals)
+    _resolve(table["rows"], list(agg))
+    out, js = [], {}
+    out.append("LDS counters, rocprofv3 on one MI355X (gfx950)")
+    out.append("")
+    out.append("command (from the repository root on the GPU box; TMPDIR=/tmp):")
+    for c in commands:
+        out.append("  " + c)
+    out.append("")
+    out.append("Per dispatch (mean over the pass's launches).  LDS/wave = SQ_INSTS_LDS / SQ_WAVES; conflict = the share of")
+    out.append("the cycles the LDS was addressing (SQ_LDS_IDX_ACTIVE) that went to bank conflicts (SQ_LDS_BANK_CONFLICT).")
+    out.append("")
+    out.append("%-32s %8s %9s %14s %14s %9s  %s" % ("operation", "waves", "LDS/wave", "idx active cyc", "conflict cyc", "conflict",
+                                             "kernel"))
+    for r in table["rows"]:
+        c = agg.get(r["kernel"])
+        if not c or not c.get("SQ_WAVES") or not c.get("SQ_INSTS_LDS"):
+            continue
+        act, conf = c.get("SQ_LDS_IDX_ACTIVE", 0.0), c.get("SQ_LDS_BANK_CONFLICT", 0.0)
+        out.append("%-32s %8d %9.1f %14.0f %14.0f %8.1f%%  %s" % (r["label"][:32], c["SQ_WAVES"], c["SQ_INSTS_LDS"] / c["SQ_WAVES"],
+                                                              act, conf, 100.0 * conf / act if act else 0.0, r["kernel"][:80]))
+        js[r["kernel"]] = {"label": r["label"], "lds_per_wave": round(c["SQ_INSTS_LDS"] / c["SQ_WAVES"], 1),
+                           "bank_conflict_share": round(conf / act, 4) if act else None}
+    out.append("")
+    out.append("json: " + json.dumps(js))
+    with open(out_path, "w") as f:
+        f.write("\n".join(out) + "\n")
+    return js
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
-    ap.add_argument("kind", choices=("durations", "traffic", "issue"))
+    ap.add_argument("kind", choices=("durations", "traffic", "issue", "lds"))
     ap.add_argument("--csv", action="append", default=[])
     ap.add_argument("--fetch")
     ap.add_argument("--write")
@@ -212,6 +259,8 @@ def main(argv=None):
         js = durations(args.csv[0], table, args.out, args.command)
     elif args.kind == "traffic":
         js = traffic(args.fetch, args.write, table, args.out, args.command)
+    elif args.kind == "lds":
+        js = lds(args.csv, table, args.out, args.command)
     else:
         js = issue(args.csv, table, args.out, args.command)
     print("%s: %d kernels -> %s" % (args.kind, len(js), args.out))

@@ -157,3 +157,37 @@ def test_hist_log2_entry_point(dev, n, skew, dtype, nbins, offset):
     with np.errstate(divide="ignore", invalid="ignore"):
         want, _ = np.histogram(np.rint(np.log2(np.abs(a[skew:].astype(np.float32)))), bins=edges)
     assert np.array_equal(got, want.astype(np.int32))
+
+
+@pytest.mark.parametrize("nbins,offset,shift", [(64, -48, 0), (63, -126, 0), (7, -3, 0), (64, 63, 0), (64, -48, 4),
+                                                 (5, -2, 4), (64, 64, 0), (40, -127, 0)])
+def test_hist_log2_bin_edges(dev, nbins, offset, shift):
+    """the values whose bin the last bit decides: the two fp32 neighbours of
+    sqrt(2) * 2^k (the lower rounds down, the upper up), exact powers of two,
+    the largest and smallest normal numbers, denormals, zeros, infinities and
+    NaNs -- against rint(log2|x|) evaluated in float64, which separates the
+    neighbours of sqrt(2) by 10^8 of its own roundings.  Covers the kernel that
+    bins by exponent and mantissa, the two argument ranges that must fall back
+    to the logarithm kernels, an odd number of bins and a result buffer that is
+    only 4-byte aligned (no paired adds)."""
+    ks = np.arange(-126, 128)
+    below = (np.float32(np.sqrt(2.0)) * np.exp2(ks)).astype(np.float32)         # 0x3FB504F3 * 2^k < sqrt(2) * 2^k
+    above = np.nextafter(below, np.float32(np.inf)).astype(np.float32)
+    assert np.all(below.astype(np.float64) < np.sqrt(2.0) * np.exp2(ks.astype(np.float64)))
+    specials = np.array([0.0, -0.0, 1e-45, 1e-40, -1e-39, 1.1754942e-38, 1.17549435e-38, 3.4028235e38, -3.4028235e38,
+                         np.inf, -np.inf, np.nan, -np.nan], dtype=np.float32)
+    quiet = np.array([0x7fc00000, 0xffc00001, 0x7f800001, 0x7fffffff], dtype=np.uint32).view(np.float32)
+    a = np.concatenate([below, -above, np.exp2(ks).astype(np.float32), specials, quiet,
+                        np.random.RandomState(3).randn(4096).astype(np.float32)]).astype(np.float32)
+    a = np.tile(a, 3)[:-5]                                                       # a scalar tail as well
+    x = dev.put(a)
+    base = dev.alloc(4 * nbins + 16)
+    hist = base + shift
+    ok(dev.lib, dev.lib.nh_hist_log2(c_void_p(hist), c_void_p(x), 4, a.size, nbins, offset, None))
+    got = dev.get(hist, (nbins,), np.int32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        b = np.rint(np.log2(np.abs(a.astype(np.float64)))) - offset
+    counted = b <= nbins                                                          # false for NaN
+    bins = np.clip(np.where(counted, b, 0), 0, nbins - 1).astype(np.int64)
+    want = np.bincount(bins[counted], minlength=nbins)
+    assert np.array_equal(got, want.astype(np.int32))
