@@ -654,7 +654,7 @@ def counter_pass():
         table.append({"label": label, "kernel": None, "kernel_contains": part, "family": "prebuilt",
                       "algorithmic_bytes": nbytes, "warmup": 0, "launches": reps + 1})
     a32 = _fresh(be, configs.C3_SHAPE, rs=rs)
-    run_prebuilt("hist log2 (5000,5000) f32", "hist_log2_kernel", a32.size * 4, lambda: a32.hist("bench"))
+    run_prebuilt("hist log2 (5000,5000) f32", "hist_", a32.size * 4, lambda: a32.hist("bench"))
     sq = (8192, 8192)
     t_in, t_out = _fresh(be, sq, rs=rs), be.empty(sq)
     run_prebuilt("copy_transpose (8192,8192) f32", "transpose_tile", 2 * sq[0] * sq[1] * 4,

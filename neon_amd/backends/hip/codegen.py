@@ -1642,7 +1642,7 @@ def _col_lds(L, LX, LY, T, V, any_index):
     return WY * pitch * (4 + (8 if any_index else 0))
 
 
-def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False):
+def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False, runs=False):
     """Axis-0 reductions with the rows resident in registers (LX column-lanes x
     LY row-lanes per workgroup, NR rows per lane).
 
@@ -1677,7 +1677,7 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False)
     g.declare_one()
     L("const int tx = threadIdx.x %% %d, ty = threadIdx.x / %d;" % (LX, LX))
     wide = [t.dtype.itemsize for t in prog.tensors if t.shape[1] > 1]
-    xcd_runs = bool(not coop and wide and LX * V * max(wide) < 128)
+    xcd_runs = bool(not coop and wide and (runs or LX * V * max(wide) < 128))
     if xcd_runs:
         # Strips narrower than a cache line: neighbouring strips read the same lines.  Workgroups
         # are handed to the 8 XCDs (each with its own L2) round-robin, so consecutive strips
@@ -1686,12 +1686,16 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False)
         # fewer XCDs take part and the grid carries workgroups that leave at once (col_grid;
         # softmax over (1000,128), memory traffic over the matrix's bytes: 5.1 with strips dealt
         # round-robin, 1.6 with runs of half a line, 1.0 with whole lines on 4 of the 8 XCDs).
+        # ``runs``: the same for strips of whole lines when the rows are not a multiple of 128
+        # bytes long -- every second row piece then straddles two lines and shares each with
+        # the neighbouring strip (softmax down (1000,30000) fp32 read 1.5 times its bytes).
         L("const unsigned int nstrips = (unsigned int)((C + %d) / %d);" % (LX * V - 1, LX * V))
         L("unsigned int nx = nstrips / %du;" % max(1, 128 // (LX * V * max(wide))))
         L("nx = nx < 1u ? 1u : (nx > NH_XCDS ? NH_XCDS : nx);")
         L("const unsigned int per_xcd = (nstrips + nx - 1u) / nx;")
         L("if (blockIdx.x % NH_XCDS >= nx || blockIdx.x / NH_XCDS >= per_xcd) return;")
         L("const unsigned int strip = (blockIdx.x % NH_XCDS) * per_xcd + blockIdx.x / NH_XCDS;")
+        L("if (strip >= nstrips) return;")
     else:
         L("const unsigned int strip = blockIdx.x;")
     L("const long long c = ((long long)strip * %d + tx) * %d;" % (LX, V))
@@ -1714,9 +1718,14 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False)
         L.open("for (int i = 0; i < %d; ++i)" % NR)
         if coop:
             L("const long long r = ((long long)blockIdx.y * %d + i) * %d + ty;" % (NR, LY))
+            L("const bool ok = col_ok && (r < R);")
         else:
+            # Only a lane's last row can lie past the end (the planner takes NR = ceil(R / LY)), so
+            # after unrolling the other rows carry no test and no branch.  Lanes past the last column
+            # compute on the first columns' values (cc) and are kept from storing.  Measured, softmax
+            # down the columns: (64,1048576) fp32 93 -> 88 us, (512,65536) 55 -> 52 us.
             L("const long long r = (long long)i * %d + ty;" % LY)
-        L("const bool ok = col_ok && (r < R);")
+            L("const bool ok = (i < %d) || (r < R);" % (NR - 1))
 
     def exchange(reds, last_one_folds=False, riders=()):
         """fold the workgroups of a strip: afterwards acc/rv/ri hold the
@@ -2088,7 +2097,8 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False)
                 L("o%d.set(j, %s);" % (st.out.index, ref(st.root)))
         L.close()
         for st in full_out:
-            L(g.store_stmt("o%d" % st.out.index, g.st, g.addr(st.out, "r", "c"), V if st.out.shape[1] > 1 else 1))
+            stmt = g.store_stmt("o%d" % st.out.index, g.st, g.addr(st.out, "r", "c"), V if st.out.shape[1] > 1 else 1)
+            L(stmt if coop else "if (col_ok) { %s }" % stmt)
         L.close()
         L.close()
     if coop and ticket_finish:

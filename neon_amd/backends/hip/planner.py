@@ -601,7 +601,10 @@ def _plan_col(prog, cu_count, coop=True):
             prog.unpair_lse()
         budget = _COL_BUDGET[T]
         spare = max(0, (budget - NR * words) // (NR * V))
-        spec = codegen.gen_col(prog, V, LX, LY, NR, _streams(prog), max_vals=min(2, spare), tail=tail)
+        assert (NR - 1) * LY < R <= NR * LY      # the kernels test only a lane's last row against R
+        # rows that are no whole number of cache lines: neighbouring strips share lines, keep them on one XCD
+        runs = (C * isz) % 128 != 0 and LX * V * isz >= 128 and _ceil_div(nvec, LX) >= 64
+        spec = codegen.gen_col(prog, V, LX, LY, NR, _streams(prog), max_vals=min(2, spare), tail=tail, runs=runs)
         return Choice(spec, (codegen.col_grid(spec, _ceil_div(nvec, LX)), 1, 1))
 
     # (c) deeper trees (or full-shape results) over many rows: the workgroups of a
