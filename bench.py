@@ -13,10 +13,20 @@ be.end`` calls, inputs resident in HBM, stream synchronised on both sides.
 around the same K launches.  ``per_config`` lists every benchmark op-tree
 (elementwise + sigmoid, softmax, Adam fused and as three kernels, fp16 row
 normalisation, argmax / max / cross-entropy over a 32000-row vocabulary) with
-the same event timing, a scaled-up (>= 256 MB) instance of the trees whose
-working set fits in cache, and cold-cache timings of those trees (launches
-rotating over >= 768 MB of distinct tensors).  ``cpu_baseline`` times the numpy oracle on the same
-Adam step on this machine's host cores.
+the same event timing, and cold-cache timings of those trees (launches
+rotating over >= 768 MB of distinct tensors holding seeded random data).
+Each row also carries ``kernel_us_rocprof`` -- the median rocprofv3 kernel
+duration of the same kernel from the committed summaries under ``profiles/``
+-- and ``traffic``, the HBM bytes per launch from hardware counters; both are
+looked up by kernel name and are null when the summaries were made from
+other kernels.  ``cpu_baseline`` times the numpy oracle on the same Adam step
+on this machine's host cores.
+
+Other modes (each the program behind one of the summaries in ``profiles/``):
+``--trace-pass hot|cold`` (rocprofv3 --kernel-trace), ``--counter-pass``
+(rocprofv3 --pmc), ``--sweep DTYPE`` (wall clock over a grid of shapes),
+``--configs-only`` / ``--no-cold`` (shorter tables).  The per-configuration
+tables go to stderr after the JSON line, the benchmark configurations last.
 """
 import argparse
 import json
@@ -692,11 +702,64 @@ def trace_pass(mode):
                       "kernel": plan.spec.name, "family": plan.spec.family, "algorithmic_bytes": case.nbytes,
                       "warmup": warm + 1, "launches": TRACE_LAUNCHES})        # (+1: the launch that made the plan)
         del sets
+    if mode == "hot":
+        _trace_support_rows(be, table)
     what = ("every launch on the same tensors (cache-hot where the working set fits a cache)" if mode == "hot" else
             "launches rotating over >= 768 MB of distinct tensor sets (cold caches)")
     note = ("Back-to-back launches through the public API, no synchronisation in between." if mode == "hot" else
             "Sets hold the configuration's seeded inputs rolled by 13 rows per set: random data in every launch.")
     print(json.dumps({"pass": mode, "what": what, "note": note, "rows": table}))
+
+
+def _trace_support_rows(be, table):
+    """hot-pass rows beyond the benchmark configurations: the batch-norm pair on both of its
+    shapes (one workgroup per row, and several cooperating workgroups per row), softmax down
+    cooperating column strips, and the two prebuilt kernels that stage data in LDS"""
+    from neon_amd import configs
+    rs = np.random.RandomState(3)
+    f16 = np.float16
+
+    def generated(label, nbytes, issue):
+        with be.capture() as grp:
+            issue()
+        assert len(grp) == 1, label
+        _, plan = be.time_group(grp[0], reps=1)
+        for _ in range(TRACE_WARMUP + TRACE_LAUNCHES):
+            issue()
+        be.synchronize()
+        table.append({"label": label, "kernel": plan.spec.name, "family": plan.spec.family, "algorithmic_bytes": nbytes,
+                      "warmup": TRACE_WARMUP + 1, "launches": TRACE_LAUNCHES})   # (+1: the launch that made the plan)
+
+    def prebuilt(label, part, nbytes, call):
+        for _ in range(TRACE_WARMUP + TRACE_LAUNCHES):
+            call()
+        be.synchronize()
+        table.append({"label": label, "kernel": None, "kernel_contains": part, "family": "prebuilt",
+                      "algorithmic_bytes": nbytes, "warmup": TRACE_WARMUP, "launches": TRACE_LAUNCHES})
+
+    for K, N in (configs.C4_SHAPE, (64, 401408)):
+        x = _fresh(be, (K, N), dtype=f16, rs=rs, scale=2.0, shift=0.5)
+        y = be.empty((K, N), dtype=f16)
+        vec = lambda fill: _fresh(be, (K, 1), fill=fill)
+        xsum, xvar, gmean, gvar, gamma, beta = vec(0.0), vec(0.0), vec(0.0), vec(1.0), vec(1.0), vec(0.0)
+        generated("BN fprop (%d,%d) f16" % (K, N), 2 * K * N * 2,
+                  lambda: be.compound_fprop_bn(x, xsum, xvar, gmean, gvar, gamma, beta, y, 1e-5, 0.9, True))
+        delta = _fresh(be, (K, N), dtype=f16, rs=rs, scale=0.1)
+        dout, gg, gb = be.empty((K, N), dtype=f16), vec(0.0), vec(0.0)
+        generated("BN bprop (%d,%d) f16" % (K, N), 3 * K * N * 2,
+                  lambda: be.compound_bprop_bn(dout, gg, gb, delta, x, xsum, xvar, gamma, 1e-5))
+        del x, y, delta, dout
+    xs = _fresh(be, configs.C5_SHAPE, rs=rs)
+    ys = be.empty(configs.C5_SHAPE)
+    generated("softmax axis0 (32000,256) f32", 2 * xs.size * 4, lambda: configs.c2_softmax(be, ys, xs))
+    del xs, ys
+    a32 = _fresh(be, configs.C3_SHAPE, rs=rs)
+    prebuilt("hist log2 (5000,5000) f32", "hist_", a32.size * 4, lambda: a32.hist("bench"))
+    del a32
+    sq = (8192, 8192)
+    t_in, t_out = _fresh(be, sq, rs=rs), be.empty(sq)
+    prebuilt("copy_transpose (8192,8192) f32", "transpose_tile", 2 * sq[0] * sq[1] * 4,
+             lambda: be.copy_transpose(t_in, t_out))
 
 
 def shape_sweep(dtype_name):

@@ -62,6 +62,7 @@ def _dispatches(csv_path):
 
 def durations(csv_path, table, out_path, commands):
     per_kernel = _dispatches(csv_path)
+    _resolve(table["rows"], list(per_kernel))
     taken = collections.defaultdict(int)       # launches of a kernel already assigned to earlier rows
     lines, js = [], {}
     mode = table["pass"]
@@ -88,7 +89,7 @@ def durations(csv_path, table, out_path, commands):
         med = statistics.median(meas) / 1e3
         frac = row["algorithmic_bytes"] / (med * 1e-6) / 8e12
         lines.append("%-52s %5d %5d %9.2f %9.2f %9.2f %7.3f  %s" % (row["label"][:52], warm, len(meas), med,
-                                                                  min(meas) / 1e3, max(meas) / 1e3, frac, name))
+                                                                  min(meas) / 1e3, max(meas) / 1e3, frac, name[:100]))
         rec = {"label": row["label"], "median_us": round(med, 3), "min_us": round(min(meas) / 1e3, 3),
                "max_us": round(max(meas) / 1e3, 3), "calls": len(meas), "algorithmic_bytes": row["algorithmic_bytes"],
                "frac": round(frac, 4), "pass": mode}
