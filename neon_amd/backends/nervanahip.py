@@ -481,6 +481,42 @@ class _Recorded(object):
                 rt.launch_prepared(prep)
 
 
+class _RecordedSplit(object):
+    """A stretch of queued statements that runs as several groups (two shapes, a reduction
+    between elementwise statements): the groups' recordings in order, each with its share of
+    the stretch's numbers.  Stands in the launch cache under the key of the whole stretch, so
+    that the next identical stretch is served by one keyed lookup."""
+    __slots__ = ("parts", "coop")
+
+    def __init__(self, parts):
+        self.parts = parts           # [(recording, first number, one past its last number)]
+        self.coop = tuple(plan for rec, _, _ in parts for plan in rec.coop)
+
+    @property
+    def launches(self):
+        return [launch for rec, _, _ in self.parts for launch in rec.launches]
+
+    @property
+    def temps(self):
+        return [t for rec, _, _ in self.parts for t in rec.temps]
+
+    @property
+    def raw(self):
+        return [x for rec, _, _ in self.parts for x in rec.raw]
+
+    def rebind(self, raw):
+        if raw is None or (self.parts and len(raw) != self.parts[-1][2]):
+            return None
+        for rec, a, b in self.parts:
+            if rec.rebind(raw[a:b]) is None:
+                return None
+        return self.launches
+
+    def replay(self, rt, records_type=None):
+        for rec, _, _ in self.parts:
+            rec.replay(rt)
+
+
 class _CaptureScope(object):
     def __init__(self, be):
         self.be = be
@@ -526,6 +562,7 @@ class NervanaHIPBase(object):
         self.round_mode = None
         self.bench = bench            # truthy: every launch is timed and reported (see _launch_plan)
         self._bench_events = None
+        self._split_log = None        # recordings of the groups a deferred stretch falls into (_resolve_deferred)
         self.stream = None
         self.use_pinned_mem = False
         self.hist_bins, self.hist_offset = hist_bins, hist_offset
@@ -782,7 +819,9 @@ class NervanaHIPBase(object):
             if self._captured is not None:
                 self._captured.append(trees)
             else:
-                self._run(trees, posts)
+                made = self._run(trees, posts)
+                if self._split_log is not None:
+                    self._split_log.append(made)
 
     _NOT_FUSABLE = frozenset(REDUCE) | {"dot", "transpose", "onehot"}
     _NEVER_FUSABLE = frozenset({"dot", "transpose", "rand"})
@@ -966,14 +1005,16 @@ class NervanaHIPBase(object):
         if self._captured is not None:
             self._captured.append([optree])
         else:
-            self._run([optree], [post])
+            made = self._run([optree], [post])
+            if self._split_log is not None:
+                self._split_log.append(made)
 
     def _resolve_deferred(self):
         """the statements queued by ``execute`` since the fusion group began: replayed at
         once if the very same group has run before, otherwise grouped and run the long way"""
         trees, self._deferred = self._deferred, []
-        entry = None
-        if self._captured is None and self._recording is None and not self._originals:
+        entry = key = raw = None
+        if self._captured is None and self._recording is None and not self._originals and not self.bench:
             try:
                 if not any(t[1].rounding for t in trees):
                     key, raw = self._replayer.key_group(trees)
@@ -990,12 +1031,22 @@ class NervanaHIPBase(object):
         # (statements reach _enqueue in fusing mode whatever the mode is by now: the group
         # was written inside begin / end)
         fusing, self._fusing = self._fusing, True
+        log = self._split_log = [] if key is not None else None
         try:
             for tree in trees:
                 self._enqueue(tree)
             self._flush_pending()
         finally:
             self._fusing = fusing
+            self._split_log = None
+        if log is not None and len(log) > 1 and None not in log:
+            # the stretch fell into several groups: remember them under the stretch's key
+            parts, at = [], 0
+            for rec in log:
+                parts.append((rec, at, at + len(rec.raw)))
+                at += len(rec.raw)
+            if at == len(raw) and [x for rec in log for x in rec.raw] == list(raw):
+                self._launch_cache[key] = _RecordedSplit(parts)
 
     def _replay_in_c(self, out, value):
         """True when the C replayer issued the recorded launches of ``out[:] = value``"""

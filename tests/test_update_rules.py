@@ -207,3 +207,41 @@ class _Null(object):
 
     def __exit__(self, *exc):
         return False
+
+
+@pytest.mark.gpu
+def test_a_stretch_that_falls_into_several_groups_is_replayed_as_one_recording(hip):
+    """two shapes and a reduction between elementwise statements: the stretch runs
+    as four groups; from the second identical minibatch on it is served by ONE
+    keyed lookup (a split recording under the stretch's key), with the numbers
+    of every group re-bound -- results against numpy for five steps with a
+    step-dependent rate"""
+    from neon_amd.backends.backend import Block
+    from neon_amd.backends.nervanahip import _RecordedSplit
+    be = hip
+    rs = np.random.RandomState(21)
+    w0, g0 = rs.standard_normal((96, 40)).astype(np.float32), rs.standard_normal((96, 40)).astype(np.float32)
+    b0, h0 = rs.standard_normal((96, 1)).astype(np.float32), rs.standard_normal((96, 1)).astype(np.float32)
+    w, g, b, h = be.array(w0), be.array(g0), be.array(b0), be.array(h0)
+    norm, out = be.empty((96, 1)), be.empty((96, 40))
+    wn, bn = w0.copy(), b0.copy()
+    for step in range(5):
+        lr = np.float32(0.1 / (step + 1))
+        replayed = be.plan_stats["replayed"]
+        be.begin(Block.minibatch, step)
+        w[:] = w - float(lr) * g                 # shape (96,40)
+        b[:] = b - float(lr) * h                 # shape (96,1): another group
+        norm[:] = be.sum(w * w, axis=1)          # a reduction: a group of its own
+        out[:] = w * float(step + 2) + b         # elementwise again
+        be.end(Block.minibatch, step)
+        wn = wn - lr * g0
+        bn = bn - lr * h0
+        assert_close(w.get(), wn, rtol=1e-5, atol=1e-6, what="w, step %d" % step)
+        assert_close(b.get(), bn, rtol=1e-5, atol=1e-6, what="b, step %d" % step)
+        assert_close(norm.get(), (wn * wn).sum(axis=1, keepdims=True), rtol=1e-5, atol=1e-5, what="norm, step %d" % step)
+        assert_close(out.get(), wn * np.float32(step + 2) + bn, rtol=1e-5, atol=1e-5, what="out, step %d" % step)
+        if step >= 1 and be._replayer is not None:
+            # one replay for the whole stretch, not one per group
+            assert be.plan_stats["replayed"] - replayed == 1, (step, be.plan_stats["replayed"] - replayed)
+    if be._replayer is not None:
+        assert any(isinstance(e, _RecordedSplit) and len(e.parts) >= 3 for e in be._launch_cache.values())
