@@ -2149,6 +2149,15 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False,
                         line_strips=(max(1, 128 // (LX * V * max(wide))) if xcd_runs else 0)))
 
 
+def colsplit_grid(spec, strips, chunks, xcds=8):
+    """launch grid of a ``colsplit`` kernel: (strips, chunks), or -- built with ``runs`` -- one
+    dimension of XCDs x strips per XCD x chunks"""
+    if not spec.params.get("runs"):
+        return (strips, chunks, 1)
+    nx = min(strips, xcds)
+    return (xcds * _ceil(strips, nx) * chunks, 1, 1)
+
+
 def col_grid(spec, strips, xcds=8):
     """workgroups a ``col`` kernel is launched with: one per strip, or -- strips narrower than
     a cache line, dealt to the XCDs in runs of whole lines -- eight times the longest run"""
@@ -2182,10 +2191,16 @@ COLSPLIT_SUBBATCH_ROWS = 8
 COLSPLIT_BATCH_WORDS = 64
 
 
-def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, NB=4, multi=True):
+def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, NB=4, multi=True, runs=False):
     """One level of axis-0 reductions over a tall matrix.  grid = (column
     strips, row chunks); a workgroup is LX column-lanes x LY row-lanes.
     ``multi``: more than one chunk per strip.
+
+    ``runs`` (rows that are no whole number of cache lines, where the row
+    pieces of neighbouring strips share lines): a one-dimensional grid (see
+    colsplit_grid) in which every XCD owns a contiguous run of strips and
+    takes them chunk by chunk, so that neighbours run side by side behind one
+    L2; surplus workgroups leave at once.
 
     Sweep.  A lane takes its rows NR at a time: all NR loads are issued before
     the first value is used (a chunk of at most NR * LY rows is fetched in ONE
@@ -2239,16 +2254,26 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
         lds += S * (8 if g.is_pair(n) else 4)
     L("__shared__ int s_last;")
     g.declare_one()
-    L("const int nchunks = gridDim.y;")
+    if runs:
+        L("const int nchunks = (int)(((long long)R + rows_per_chunk - 1) / rows_per_chunk);")
+        L("const unsigned int nstrips = (unsigned int)((C + %d) / %d);" % (S - 1, S))
+        L("const unsigned int nx = nstrips < NH_XCDS ? nstrips : NH_XCDS;")
+        L("const unsigned int per_xcd = (nstrips + nx - 1u) / nx;")
+        L("const unsigned int slot = blockIdx.x / NH_XCDS;")
+        L("const unsigned int strip = (blockIdx.x % NH_XCDS) * per_xcd + slot % per_xcd, chunk = slot / per_xcd;")
+        L("if (blockIdx.x % NH_XCDS >= nx || strip >= nstrips || chunk >= (unsigned int)nchunks) return;")
+    else:
+        L("const int nchunks = gridDim.y;")
+        L("const unsigned int strip = blockIdx.x, chunk = blockIdx.y;")
     L("const int tx = threadIdx.x %% %d, ty = threadIdx.x / %d;" % (LX, LX))
-    L("const long long c0 = (long long)blockIdx.x * %d;" % S)
+    L("const long long c0 = (long long)strip * %d;" % S)
     L("const long long c = c0 + tx * %d;" % V)
     L("const bool col_ok = c < C;")
     L("const long long cc = col_ok ? c : 0;")
     if tail:
         L("const bool cfull = c + %d <= C;" % V)
         L("const int clim = cfull ? %d : (col_ok ? (int)(C - c) : 0);" % V)
-    L("const long long r0 = (long long)blockIdx.y * rows_per_chunk;")
+    L("const long long r0 = (long long)chunk * rows_per_chunk;")
     L("const long long r1 = (r0 + rows_per_chunk < R) ? (r0 + rows_per_chunk) : (long long)R;")
     g.pos = ("0", "c")
     g.emit_gather_prefetch(_needed([st.root for st in prog.statements], set(n.nid for n in prog.nodes if n.kind == "R")),
@@ -2359,11 +2384,11 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
         # partial buffers: reduction k occupies [k*nchunks*C, (k+1)*nchunks*C) entries of 8 bytes
         for k, n in enumerate(reds):
             L("nh_pair* part%d = reinterpret_cast<nh_pair*>(ws) + (long long)%d * nchunks * C;" % (n.nid, k))
-        L("unsigned int* const ticket = reinterpret_cast<unsigned int*>(ws + ticket_offset) + %d * blockIdx.x;" % TICKET_STRIDE_WORDS)
+        L("unsigned int* const ticket = reinterpret_cast<unsigned int*>(ws + ticket_offset) + %d * strip;" % TICKET_STRIDE_WORDS)
         L.open("if (joins && c0 + jcol < C)")
         for n in reds:
             val = ("one%d" % n.nid) if g.is_pair(n) else ("nh_pair{one%d, 0}" % n.nid)
-            L("nh_part_store(&part%d[(long long)blockIdx.y * C + c0 + jcol], %s);" % (n.nid, val))
+            L("nh_part_store(&part%d[(long long)chunk * C + c0 + jcol], %s);" % (n.nid, val))
         L.close()
         # The partials were written through to device-coherent memory (nh_part_store); every
         # lane waits for its own stores before the barrier (nh_publish_barrier), lane 0 then
@@ -2456,4 +2481,4 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
     L.close()
     return _finish("colsplit", g, head, fmt, T, lds,
                    dict(V=V, LX=LX, LY=LY, NR=NR, NB=NB, NRED=len(reds), multi=bool(multi),
-                        stream=bool(stream), tail=bool(tail)))
+                        stream=bool(stream), tail=bool(tail), runs=bool(runs)))

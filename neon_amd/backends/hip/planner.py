@@ -511,6 +511,7 @@ _COL_BUDGET = {1024: 40, 512: 120, 256: 300}
 
 COLSPLIT_THREADS = int(os.environ.get("NEON_HIP_CS_T", "256"))
 
+COLSPLIT_RUNS = os.environ.get("NEON_HIP_COLSPLIT_RUNS", "1") != "0"
 COLCOOP = os.environ.get("NEON_HIP_COLCOOP", "1") != "0"       # 0: axis-0 trees never wait between workgroups
 # Beyond this size the cooperative family (rows resident in registers, one workgroup per compute
 # unit, a waiting exchange per level) loses to stage-by-stage evaluation, whose reduction kernels
@@ -707,12 +708,14 @@ def _plan_col(prog, cu_count, coop=True):
         # partials a lane of the last workgroup has in flight: P = lanes per column there
         lanes_per_column = min(threads // (LX * V), 64)
         fold_batch = max(1, min(codegen.COLSPLIT_FOLD_BATCH, _ceil_div(chunks, lanes_per_column)))
+        # rows that are no whole number of cache lines: the row pieces of neighbouring strips share lines
+        runs = COLSPLIT_RUNS and (C * isz) % 128 != 0 and strips >= 16 and chunks > 1
         spec = codegen.gen_colsplit(prog, V, LX, LY, _streams(prog), tail=tail, fold_batch=fold_batch, NR=NR,
-                                    NB=codegen.COLSPLIT_SUBBATCH_ROWS, multi=chunks > 1)
+                                    NB=codegen.COLSPLIT_SUBBATCH_ROWS, multi=chunks > 1, runs=runs)
         part_bytes = spec.params["NRED"] * chunks * C * 8
         ticket_off = _ceil_div(part_bytes, 256) * 256
         ws_bytes = ticket_off + strips * 4 * codegen.TICKET_STRIDE_WORDS
-        return Choice(spec, (strips, chunks, 1), extras=(rpc,),
+        return Choice(spec, codegen.colsplit_grid(spec, strips, chunks), extras=(rpc,),
                       workspace=(ws_bytes, ticket_off, strips * codegen.TICKET_STRIDE_WORDS))
 
     raise NeedsSplit()

@@ -1099,3 +1099,33 @@ def test_sum_of_exponentials_in_one_sweep_stays_within_a_few_units_of_float64(hi
         want = np.exp(x.astype(np.float64)).sum(axis=0)
         got = out.get().ravel().astype(np.float64)
         assert np.max(np.abs(got - want) / want) < 4e-7, (rows, lo, hi)
+
+
+@pytest.mark.parametrize("shape,dtype", [((9000, 2100), np.float32), ((20000, 2040), np.float16), ((5000, 4110), np.float32)])
+def test_split_column_reductions_with_strips_dealt_to_xcds_in_runs(hip, shape, dtype):
+    """rows that are no whole number of cache lines: the split column family
+    runs on a one-dimensional grid in which every XCD owns a run of strips
+    (surplus workgroups leave at once; the ticket of a strip still counts its
+    chunks).  sum / max / argmax / cross-entropy style log-sum-exp against
+    numpy, twice on fresh data."""
+    for rep in range(2):
+        rs = np.random.RandomState(rep + 31)
+        x = rs.standard_normal(shape).astype(dtype)
+        x[rs.randint(0, shape[0], 50), rs.randint(0, shape[1], 50)] = 3.5         # ties for argmax
+        tx = hip.array(x, dtype=dtype)
+        sm, mx, lse = (hip.empty((1, shape[1])) for _ in range(3))
+        am = hip.empty((1, shape[1]), dtype=np.int32)
+        with hip.capture() as groups:
+            sm[:] = hip.sum(tx, axis=0)
+        spec = hip.time_group(groups[0], reps=1)[1].spec
+        assert spec.family == "colsplit" and spec.params["runs"], spec.params
+        sm[:] = hip.sum(tx, axis=0)
+        mx[:] = hip.max(tx, axis=0)
+        am[:] = hip.argmax(tx, axis=0)
+        lse[:] = hip.log(hip.sum(hip.exp(tx - hip.max(tx, axis=0)), axis=0)) + hip.max(tx, axis=0)
+        x64 = x.astype(np.float64)
+        assert_close(sm.get(), x64.sum(axis=0, keepdims=True), rtol=RTOL32, atol=2e-3 * np.sqrt(shape[0]), what="sum")
+        assert np.array_equal(mx.get(), x.astype(np.float32).max(axis=0, keepdims=True))
+        assert np.array_equal(am.get().ravel(), x.argmax(axis=0))
+        m = x64.max(axis=0)
+        assert_close(lse.get().ravel(), np.log(np.exp(x64 - m).sum(axis=0)) + m, rtol=RTOL32, atol=1e-5, what="log-sum-exp")
