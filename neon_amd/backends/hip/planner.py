@@ -518,6 +518,7 @@ COLCOOP = os.environ.get("NEON_HIP_COLCOOP", "1") != "0"       # 0: axis-0 trees
 # stream at full occupancy.  Softmax, measured: (32000,256) 28 us either way; (64000,256) 60 us
 # cooperative, 44 us in two kernels; (6000,2304) 54 against 40 us.
 COLCOOP_MAX_BYTES = int(os.environ.get("NEON_HIP_COLCOOP_MAX_MB", "48")) << 20
+COLCOOP_MAX_BYTES_512 = max(COLCOOP_MAX_BYTES, int(os.environ.get("NEON_HIP_COLCOOP_MAX_MB_512", "72")) << 20)
 # ... and below this one its exchanges (some 8 us each, whatever the size) cost more than the extra pass
 # over a small matrix.  Softmax, cooperative / staged: (8192,1024) fp16, 16 MB: 26 / 20 us; (4096,1000)
 # fp32, 16 MB: 18.3 / 16.6; (3000,2000) fp32, 24 MB: 20.5 / 22.0; (16384,512) fp32, 32 MB: 24.3 / 26.4.
@@ -612,7 +613,7 @@ def _plan_col(prog, cu_count, coop=True):
     # strip keep their rows in registers and exchange partials between sweeps.
     # Everything must be resident at once, so the grid stays within one
     # workgroup per compute unit.
-    if coop and COLCOOP and not (single_level and line_only) and COLCOOP_MIN_BYTES <= R * C * isz <= COLCOOP_MAX_BYTES:
+    if coop and COLCOOP and not (single_level and line_only) and COLCOOP_MIN_BYTES <= R * C * isz <= COLCOOP_MAX_BYTES_512:
         # narrow strips keep the partials each workgroup has to gather small
         # (measured on (32000,256): 8 column-lanes 37 us, 16 lanes 43 us, 4 lanes
         # 41 us).  More strips than half the compute units leave no second
@@ -628,6 +629,12 @@ def _plan_col(prog, cu_count, coop=True):
             options = ((1024, 40), (512, 120), (256, 300)) if V < 8 else ((1024, 32), (512, 64))
             if os.environ.get("NEON_HIP_COOP_T"):          # tuning aid
                 options = tuple(o for o in options if o[0] == int(os.environ["NEON_HIP_COOP_T"]))
+            if R * C * isz > COLCOOP_MAX_BYTES:
+                # beyond that size only while the rows still fit workgroups of 512 lanes and more: with 256
+                # lanes (60+ rows a lane) the cooperative form loses to stages again -- softmax, cooperative /
+                # staged: (60000,256) 34.6 / 40.8 us, (14000,1024) 31.9 / 37.6, (3500,4096) 32.6 / 37.4,
+                # (28000,512) 32.5 / 38.5, but (6000,2304) 43.9 / 35.6 and (4096,4096) 46.7 / 42.1 in 256 lanes
+                options = tuple(o for o in options if o[0] >= 512)
             for T, budget in options:
                 LY = T // lxc
                 NR = _ceil_div(rpc0, LY)
