@@ -26,7 +26,8 @@ int launch_status(const char* what) {
 }
 
 // ---------------------------------------------------------------------------
-// Streaming elementwise kernels: 256 threads, one vector of V floats per lane
+// Streaming elementwise kernels: 512 threads (the Adam update over 25 M
+// parameters: 105.2 us with 256, 103.6 us with 512), one vector of V floats per lane
 // and tensor (every wave touches 1 KiB contiguous per instruction), all loads
 // issued before the first use.  One vector per lane measured fastest for the
 // 7-stream Adam update (more in flight per lane only adds read/write
@@ -34,7 +35,7 @@ int launch_status(const char* what) {
 // loads and written with ordinary stores (measured: 6.7 TB/s on the Adam
 // update against 5.9 TB/s with non-temporal stores as well).
 // ---------------------------------------------------------------------------
-constexpr int EW_T = 256;
+constexpr int EW_T = 512;
 constexpr size_t EW_STREAM_BYTES = (size_t)256 << 20;
 
 template <int V, bool NT> __device__ __forceinline__ void ew_ld(const float* p, float (&r)[V]) {

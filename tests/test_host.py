@@ -284,7 +284,7 @@ def test_shape_class_selection(pb):
     f32, f16 = np.float32, np.float16
     x, y, o = pb.empty((4096, 128)), pb.empty((4096, 128)), pb.empty((4096, 128))
     ch = plan_of(pb, lambda: o.__setitem__(slice(None), 0.5 * x + 2.0 * y))
-    assert ch.spec.family == "ew" and ch.spec.params["V"] == 4 and ch.grid[0] == 512
+    assert ch.spec.family == "ew" and ch.spec.params["V"] == 4 and ch.grid[0] == 256 and ch.spec.block == 512
     col, row = pb.empty((4096, 1)), pb.empty((1, 128))
     ch = plan_of(pb, lambda: o.__setitem__(slice(None), x * col + row))
     assert ch.spec.family == "ew" and ch.spec.params["LY"] > 1            # 2-d tiling for broadcasts
@@ -522,7 +522,7 @@ def test_more_than_2_31_elements_stay_two_dimensional(pb):
     assert pb.choices[-1].grid[0] * spec.params["LX"] * spec.params["V"] < 2 * big[1]      # a row, not the whole tensor
     x, y, out = (pb.empty(small) for _ in range(3))
     ch = plan_of(pb, lambda: out.__setitem__(slice(None), x * 0.5 + y))
-    assert ch.grid[0] * 256 * ch.spec.params["V"] >= small[0] * small[1]                    # flattened
+    assert ch.grid[0] * ch.spec.block * ch.spec.params["V"] >= small[0] * small[1] and ch.grid[1] == 1   # flattened
 
 
 # ---- row family: LDS as a second tier of residence -------------------------------------------
