@@ -2152,10 +2152,14 @@ def gen_col(prog, V, LX, LY, NR, stream=False, chunks=1, max_vals=0, tail=False,
 def colsplit_grid(spec, strips, chunks, xcds=8):
     """launch grid of a ``colsplit`` kernel: (strips, chunks), or -- built with ``runs`` -- one
     dimension of XCDs x strips per XCD x chunks"""
-    if not spec.params.get("runs"):
+    ls = int(spec.params.get("runs") or 0)
+    if not ls:
         return (strips, chunks, 1)
-    nx = min(strips, xcds)
-    return (xcds * _ceil(strips, nx) * chunks, 1, 1)
+    if ls < 0:
+        return (xcds * strips * _ceil(chunks, xcds), 1, 1)
+    lines = _ceil(strips, ls)
+    nx = min(lines, xcds)
+    return (xcds * _ceil(lines, nx) * ls * chunks, 1, 1)
 
 
 def col_grid(spec, strips, xcds=8):
@@ -2197,10 +2201,13 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
     ``multi``: more than one chunk per strip.
 
     ``runs`` (rows that are no whole number of cache lines, where the row
-    pieces of neighbouring strips share lines): a one-dimensional grid (see
-    colsplit_grid) in which every XCD owns a contiguous run of strips and
-    takes them chunk by chunk, so that neighbours run side by side behind one
-    L2; surplus workgroups leave at once.
+    pieces of neighbouring strips share lines; or strips narrower than a
+    line, ``runs`` of them per line): a one-dimensional grid (see
+    colsplit_grid) in which the strips that share lines run side by side
+    behind one L2.  Negative: every XCD takes whole row chunks with all their
+    strips (eight chunks and more); positive: every XCD owns a contiguous run
+    of strips -- whole lines -- and takes them chunk by chunk.  Surplus
+    workgroups leave at once.
 
     Sweep.  A lane takes its rows NR at a time: all NR loads are issued before
     the first value is used (a chunk of at most NR * LY rows is fetched in ONE
@@ -2254,11 +2261,20 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
         lds += S * (8 if g.is_pair(n) else 4)
     L("__shared__ int s_last;")
     g.declare_one()
-    if runs:
+    if runs < 0:
+        # every XCD takes whole row chunks (chunk = 8 * round + XCD), all strips of a chunk side by side
         L("const int nchunks = (int)(((long long)R + rows_per_chunk - 1) / rows_per_chunk);")
         L("const unsigned int nstrips = (unsigned int)((C + %d) / %d);" % (S - 1, S))
-        L("const unsigned int nx = nstrips < NH_XCDS ? nstrips : NH_XCDS;")
-        L("const unsigned int per_xcd = (nstrips + nx - 1u) / nx;")
+        L("const unsigned int slot = blockIdx.x / NH_XCDS;")
+        L("const unsigned int strip = slot % nstrips, chunk = (slot / nstrips) * NH_XCDS + blockIdx.x % NH_XCDS;")
+        L("if (chunk >= (unsigned int)nchunks) return;")
+    elif runs:
+        L("const int nchunks = (int)(((long long)R + rows_per_chunk - 1) / rows_per_chunk);")
+        L("const unsigned int nstrips = (unsigned int)((C + %d) / %d);" % (S - 1, S))
+        ls = int(runs)                # strips that share a cache line (1: strips of whole lines)
+        L("const unsigned int nlines = (nstrips + %du) / %du;" % (ls - 1, ls))
+        L("const unsigned int nx = nlines < NH_XCDS ? nlines : NH_XCDS;")
+        L("const unsigned int per_xcd = ((nlines + nx - 1u) / nx) * %du;" % ls)
         L("const unsigned int slot = blockIdx.x / NH_XCDS;")
         L("const unsigned int strip = (blockIdx.x % NH_XCDS) * per_xcd + slot % per_xcd, chunk = slot / per_xcd;")
         L("if (blockIdx.x % NH_XCDS >= nx || strip >= nstrips || chunk >= (unsigned int)nchunks) return;")
@@ -2481,4 +2497,4 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
     L.close()
     return _finish("colsplit", g, head, fmt, T, lds,
                    dict(V=V, LX=LX, LY=LY, NR=NR, NB=NB, NRED=len(reds), multi=bool(multi),
-                        stream=bool(stream), tail=bool(tail), runs=bool(runs)))
+                        stream=bool(stream), tail=bool(tail), runs=int(runs)))

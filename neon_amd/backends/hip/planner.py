@@ -679,6 +679,8 @@ def _plan_col(prog, cu_count, coop=True):
         if LX == 16 and (per_cu == 1 or
                          _ceil_div(nvec, LX) * codegen.COLSPLIT_MAX_CHUNKS < min(target, 2 * cu_count)):
             LX = max(lx_min, 8)
+        if os.environ.get("NEON_HIP_CS_LX"):               # tuning aid
+            LX = int(os.environ["NEON_HIP_CS_LX"])
         # one workgroup per compute unit (small inputs): twice the lanes, so that a SIMD has a
         # second wave to run while the first waits for its rows ((32000,256): argmax 11.0 ->
         # 10.7 us, max 8.1 -> 7.3 us); larger inputs already get several workgroups per unit
@@ -722,7 +724,19 @@ def _plan_col(prog, cu_count, coop=True):
         lanes_per_column = min(threads // (LX * V), 64)
         fold_batch = max(1, min(codegen.COLSPLIT_FOLD_BATCH, _ceil_div(chunks, lanes_per_column)))
         # rows that are no whole number of cache lines: the row pieces of neighbouring strips share lines
-        runs = COLSPLIT_RUNS and (C * isz) % 128 != 0 and strips >= 16 and chunks > 1
+        # Rows that are no whole number of cache lines: the row pieces of neighbouring strips share lines.
+        # Many strips: every XCD a contiguous run of them; few strips and eight chunks or more: every XCD
+        # whole chunks.  Sum over axis 0, (strips, chunks) grid / runs of strips / whole chunks:
+        # (4096,30000) fp32 86 / 80 / 83 us, (131072,1000) fp32 111 / 104 / 97 us, fp16 60 / 60 / 50 us.
+        runs = 0
+        if COLSPLIT_RUNS and chunks > 1 and strips > 1:
+            narrow = LX * V * isz < 128                # (strips narrower than a cache line: tuning aid only)
+            if (narrow or (C * isz) % 128 != 0) and chunks >= 8 and strips < 64:
+                runs = -1
+            elif narrow:
+                runs = 128 // (LX * V * isz)
+            elif (C * isz) % 128 != 0 and strips >= 16:
+                runs = 1
         spec = codegen.gen_colsplit(prog, V, LX, LY, _streams(prog), tail=tail, fold_batch=fold_batch, NR=NR,
                                     NB=codegen.COLSPLIT_SUBBATCH_ROWS, multi=chunks > 1, runs=runs)
         part_bytes = spec.params["NRED"] * chunks * C * 8

@@ -1101,7 +1101,7 @@ def test_sum_of_exponentials_in_one_sweep_stays_within_a_few_units_of_float64(hi
         assert np.max(np.abs(got - want) / want) < 4e-7, (rows, lo, hi)
 
 
-@pytest.mark.parametrize("shape,dtype", [((9000, 2100), np.float32), ((20000, 2040), np.float16), ((5000, 4110), np.float32)])
+@pytest.mark.parametrize("shape,dtype", [((9000, 2100), np.float32), ((20000, 2040), np.float16), ((5000, 4110), np.float32), ((60000, 1000), np.float32), ((3000, 9000), np.float32)])
 def test_split_column_reductions_with_strips_dealt_to_xcds_in_runs(hip, shape, dtype):
     """rows that are no whole number of cache lines: the split column family
     runs on a one-dimensional grid in which every XCD owns a run of strips
