@@ -60,6 +60,7 @@ _RED_OP = {"sum": "nh_op_sum", "max": "nh_op_max", "min": "nh_op_min",
 # counters of all strips in one line, the 256 workgroups of an (8 strips x 32 chunks) grid queued
 # behind each other for 2 us (max over (32000,256): 7.3 -> 5.1 us with a line per strip).
 LOCAL_EXP_REUSE = os.environ.get("NEON_HIP_LOCAL_EXP_REUSE", "1") != "0"
+TAGGED_EXCHANGE = os.environ.get("NEON_HIP_TAGGED_EXCHANGE", "1") != "0"
 TICKET_STRIDE_WORDS = 64
 
 
@@ -909,12 +910,25 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
     all_reds = g.own_reductions([n for lv in sorted(per_level) for n in per_level[lv]])
     red_slot = dict((n.nid, k) for k, n in enumerate(all_reds))
     exchanges = [0]
+    # Exchanges of plain float partials carry a tag in the pair's unused index word: a workgroup's
+    # (value, tag) is ONE 8-byte atomic store, so whoever sees the tag has the value -- no wait for the
+    # store's acknowledgement, no counter, no separate fetch.  The tag is the one the workgroup's own
+    # slot held at kernel start plus one: every launch writes every slot exactly once, so all slots of
+    # a plan carry the same tag between launches (the plan's workspace starts zeroed), and nothing has
+    # to be re-armed at the end.  One round trip instead of three.
+    tagged = bool(coop and TAGGED_EXCHANGE and all_reds and not any(g.is_pair(n) for n in all_reds)
+                  and chunks <= 64 and len(all_reds) <= 8)
     if coop:
         L("__shared__ int s_abort;")
         # (the counters of neighbouring lines a cache line apart, see TICKET_STRIDE_WORDS)
         L("unsigned int* ctr = reinterpret_cast<unsigned int*>(ws + ctr_offset) + %d * blockIdx.x;" % TICKET_STRIDE_WORDS)
         L("unsigned int* status = reinterpret_cast<unsigned int*>(ws + ctr_offset) + %d * gridDim.x;" % TICKET_STRIDE_WORDS)
         L("nh_pair* part = reinterpret_cast<nh_pair*>(ws) + (long long)blockIdx.x * %d;" % (len(all_reds) * chunks))
+    if tagged:
+        L("__shared__ float s_x[8];")
+        L("int tag = 0;")
+        L("if (threadIdx.x < 64) tag = nh_part_load(&part[blockIdx.y]).i + 1;     // (in flight while the row is fetched)")
+        L("if (threadIdx.x == 0) s_abort = 0;     // (the workgroup meets at a barrier before it is read)")
 
     SU = 4      # column tiles in flight per lane when the row is streamed
     NCHP = -(-NCH // SU) * SU
@@ -959,6 +973,40 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
         workgroup.  ``riders``: reductions whose per-workgroup values travel
         along and are only fetched (g<id>), for the caller to combine"""
         exchanges[0] += 1
+        if tagged:
+            both = list(reds) + list(riders)
+            L.open("if (threadIdx.x == 0)")
+            for n in both:
+                L("nh_part_store(&part[%d + blockIdx.y], nh_pair{red%d, tag});" % (red_slot[n.nid] * chunks, n.nid))
+            L.close()
+            for n in both:
+                L("nh_pair g%d = nh_pair{%s::init(), 0};" % (n.nid, g.red_op(n)))
+            L.open("if (threadIdx.x < %d)" % chunks)
+            L("unsigned int spins = 0;")
+            L.open("for (;;)")
+            for n in both:
+                L("g%d = nh_part_load(&part[%d + threadIdx.x]);" % (n.nid, red_slot[n.nid] * chunks))
+            L("if (%s) break;" % " && ".join("g%d.i == tag" % n.nid for n in both))
+            L("__builtin_amdgcn_s_sleep(2);")
+            L("if (++spins > NH_SPIN_LIMIT) { s_abort = 1; break; }")
+            L.close()
+            L.close()
+            L.open("if (threadIdx.x < 64)")
+            for k, n in enumerate(reds):
+                L("const float w%d = nh_wave_allreduce<%s, 64, float>((threadIdx.x < %d) ? g%d.v : %s::init());"
+                  % (n.nid, g.red_op(n), chunks, n.nid, g.red_op(n)))
+                L("if (threadIdx.x == 0) s_x[%d] = w%d;" % (k, n.nid))
+            L.close()
+            L("__syncthreads();")
+            L.open("if (s_abort)")
+            L("// the other workgroups never showed up: leave word for the host and give up rather than hang")
+            L("if (threadIdx.x == 0) __hip_atomic_store(status, NH_COOP_ABORTED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
+            L("return;")
+            L.close()
+            for k, n in enumerate(reds):
+                L("red%d = s_x[%d];" % (n.nid, k))
+            L("__syncthreads();     // s_x is free again")
+            return
         L.open("if (threadIdx.x == 0)")
         for n in list(reds) + list(riders):
             val = ("red%d" % n.nid) if g.is_pair(n) else ("nh_pair{red%d, 0}" % n.nid)
@@ -1512,7 +1560,7 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
             L.close()
 
         sweep(leaves, store_body)
-    if coop:
+    if coop and not tagged:
         # the last workgroup of the row to get here has seen everyone pass the
         # final wait: it re-arms both counters for the next launch
         L.open("if (threadIdx.x == 0)")
@@ -1526,7 +1574,8 @@ def gen_row(prog, V, LX, LY, NCH, stream=False, keep_words=None, chunks=1, tail=
     return _finish("rowcoop" if coop else "row", g, head, fmt, T, 0,
                    dict(V=V, LX=LX, LY=LY, NCH=NCH, stream=bool(stream), passing=len(transient),
                         over=len([k for k in vals if k in over]), kept=len([k for k in vals if k in own]), chunks=chunks, NRED=len(all_reds), tail=bool(tail),
-                        parked=sum(park.values()), held=sum(hold.values()), lane_moments=len(lane_merged)))
+                        parked=sum(park.values()), held=sum(hold.values()), lane_moments=len(lane_merged),
+                        tagged=tagged))
 
 
 # =====================================================================================

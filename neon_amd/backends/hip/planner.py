@@ -335,6 +335,8 @@ def make_plan(prog, rt, cache, cu_count, coop=True):
         ws_bytes, ticket_off, n_tickets = ch.workspace
         ws = rt.malloc(ws_bytes)
         rt.memset(ws + ticket_off, 0, n_tickets, 4)   # tickets start at zero and reset themselves
+        if ch.spec.params.get("tagged"):
+            rt.memset(ws, 0, ticket_off // 4, 4)      # tagged partials: every slot's tag starts at zero
         extras = extras + (ws, ticket_off)
         if ch.status_offset is not None:
             status, counters = ws + ch.status_offset, (ws + ticket_off, n_tickets)

@@ -580,11 +580,22 @@ def test_cooperating_workgroups_take_mean_and_variance_with_one_exchange(pb, mon
         out[:] = (x - pb.mean(x, axis=1)) / pb.sqrt(pb.var(x, axis=1) + 1e-5)
 
     ch = plan_of(pb, norm)
-    assert ch.spec.family == "rowcoop" and ch.spec.source.count("nh_ticket_take(ctr)") == 1
+    # (float partials of cooperating rows travel tagged: an exchange is one polling loop, no ticket)
+    waits = lambda spec: spec.source.count("nh_ticket_take(ctr)") + spec.source.count("s_x is free again")
+    assert ch.spec.family == "rowcoop" and waits(ch.spec) == 1 and ch.spec.params["tagged"]
+    assert "nh_ticket_take" not in ch.spec.source and "ctr + 1" not in ch.spec.source
     assert "const float mu" in ch.spec.source and "n_loc" in ch.spec.source
     monkeypatch.setattr(codegen, "MERGED_MOMENTS", False)
-    assert plan_of(pb, norm).spec.source.count("nh_ticket_take(ctr)") == 2
+    assert waits(plan_of(pb, norm).spec) == 2
     monkeypatch.setattr(codegen, "MERGED_MOMENTS", True)
+    monkeypatch.setattr(codegen, "TAGGED_EXCHANGE", False)
+    assert plan_of(pb, norm).spec.source.count("nh_ticket_take(ctr)") == 1
+    monkeypatch.setattr(codegen, "TAGGED_EXCHANGE", True)
+    # a row maximum with its position travels as a (value, index) pair: no room for a tag
+    am = pb.empty((16, 1), dtype=np.int32)
+    ch = plan_of(pb, lambda: am.__setitem__(slice(None), pb.argmax(x, axis=1)))
+    if ch.spec.family == "rowcoop":
+        assert not ch.spec.params["tagged"] and "nh_ticket_take(ctr)" in ch.spec.source
     # the same down columns that several workgroups share
     xc, outc = pb.empty((32000, 256)), pb.empty((32000, 256))
 
@@ -598,7 +609,7 @@ def test_cooperating_workgroups_take_mean_and_variance_with_one_exchange(pb, mon
     monkeypatch.setattr(codegen, "MERGED_MOMENTS", True)
     # a second sweep of another form (absolute deviations) needs the finished mean everywhere
     ch = plan_of(pb, lambda: out.__setitem__(slice(None), x / pb.sum(pb.absolute(x - pb.mean(x, axis=1)), axis=1)))
-    assert ch.spec.family == "rowcoop" and ch.spec.source.count("nh_ticket_take(ctr)") == 2
+    assert ch.spec.family == "rowcoop" and waits(ch.spec) == 2
 
 
 def test_the_cheaper_exponential_is_for_arguments_below_their_own_maximum_only(pb):
