@@ -1,7 +1,9 @@
 """Tensors beyond 2^31 elements and 2^32 bytes: element offsets, flattened
 extents and grid sizes must not wrap anywhere between the tree and the kernel.
 The data is drawn on the device and checked window by window against numpy on
-the host (no host array of the full size is ever made)."""
+the host (no host array of the full size is ever made).  The file name sorts
+behind the other suites: these tests move 5 GB through the device and run
+last but for the allocation-free entry point's."""
 import numpy as np
 import pytest
 
