@@ -219,7 +219,10 @@ int nh_colmax_argmax_f32_static(float* maxval, int32_t* argmax, const float* x,
  * first): bin 0 reaches down to -inf, bin k >= 1 holds offset+k, the last bin
  * also offset+nbins, larger magnitudes and NaN are not counted -- the binning
  * of Tensor.hist on the CPU backend (neon/backends/nervanacpu.py:424-445);
- * replaces kernel_histo / _compute_hist (neon/backends/float_ew.py:1070-1158). */
+ * replaces kernel_histo / _compute_hist (neon/backends/float_ew.py:1070-1158).
+ * rint(log2|x|) is taken from the exponent and mantissa bits, i.e. correctly
+ * rounded: for the two fp32 neighbours of sqrt(2) * 2^k a log2f-based binning
+ * decides by the last bit of its logarithm.                                  */
 int nh_hist_log2(int32_t* hist, const void* x, int itemsize, size_t n, int nbins,
                  int offset, void* stream);
 
