@@ -199,3 +199,71 @@ def test_axis0_trees_too_large_for_one_kernel_are_staged_with_their_reductions_t
                                           hip.sqrt(hip.var(hx, axis=0) + 1e-5)))
     assert n == 3
     assert_close(hout.get(), cout.get(), rtol=1e-4, atol=1e-5, what="column normalisation")
+
+
+def test_all_configurations_against_formulas_written_in_numpy_float64(hip):
+    """The five configurations at full shape against the formulas themselves,
+    evaluated in numpy float64 with nothing of this package between the inputs
+    and the expected values (the oracle shares its op builders with the
+    product; this test does not).  fp32 results within 1e-5 (sums of many terms
+    with the 2 eps sum|x| allowance), fp16 storage within one fp16 step, indices
+    and maxima bit for bit."""
+    be = hip
+    # C1: 0.5 x + 2 y, then the logistic function in place; and both as one statement
+    x, y = configs.inputs_c1()
+    X, Y, out, fused = be.array(x), be.array(y), be.empty(x.shape), be.empty(x.shape)
+    configs.c1a(be, out, X, Y)
+    lin = out.get()
+    assert np.array_equal(lin, np.float32(0.5) * x + np.float32(2.0) * y)          # two exact scalings and one rounding
+    configs.c1b(be, out)
+    configs.c1_fused(be, fused, X, Y)
+    sig = 1.0 / (1.0 + np.exp(-(0.5 * x.astype(np.float64) + 2.0 * y.astype(np.float64))))
+    assert_close(out.get(), sig, rtol=1e-5, atol=1e-7, what="C1b")
+    assert_close(fused.get(), sig, rtol=1e-5, atol=1e-7, what="C1 fused")
+    # C2: softmax down the columns
+    (x2,) = configs.inputs_c2()
+    o2 = be.empty(x2.shape)
+    configs.c2_softmax(be, o2, be.array(x2))
+    e = np.exp(x2.astype(np.float64) - x2.astype(np.float64).max(axis=0))
+    assert_close(o2.get(), e / e.sum(axis=0), rtol=1e-5, atol=1e-9, what="C2")
+    # C3: three Adam steps, float64 state carried alongside
+    grad, param = configs.inputs_c3()
+    p, g, m, v = be.array(param), be.array(grad), be.zeros(param.shape), be.zeros(param.shape)
+    p64, g64 = param.astype(np.float64), grad.astype(np.float64)
+    m64, v64 = np.zeros_like(p64), np.zeros_like(p64)
+    a = configs.ADAM
+    for t in range(1, 4):
+        be.begin(Block.update, t)
+        configs.c3_adam_step(be, p, g, m, v, t)
+        be.end(Block.update, t)
+        l = a["lr"] * np.sqrt(1 - a["beta2"] ** t) / (1 - a["beta1"] ** t)
+        m64 = m64 * a["beta1"] + (1. - a["beta1"]) * g64
+        v64 = v64 * a["beta2"] + (1. - a["beta2"]) * g64 * g64
+        p64 = p64 - (l * m64) / (np.sqrt(v64) + a["eps"])
+    assert_close(m.get(), m64, rtol=1e-5, atol=1e-9, what="C3 m")
+    assert_close(v.get(), v64, rtol=1e-5, atol=1e-12, what="C3 v")
+    assert_close(p.get(), p64, rtol=1e-5, atol=1e-7, what="C3 param")
+    del p, g, m, v, p64, g64, m64, v64
+    # C4: row normalisation of fp16 data, fp16 result
+    x4, gamma, beta = configs.inputs_c4()
+    o4 = be.empty(x4.shape, dtype=np.float16)
+    configs.c4_rownorm(be, o4, be.array(x4, dtype=np.float16), be.array(gamma), be.array(beta))
+    x64 = x4.astype(np.float64)
+    want = gamma * (x64 - x64.mean(axis=1, keepdims=True)) / np.sqrt(x64.var(axis=1, keepdims=True) + 1e-5) + beta
+    got = o4.get().astype(np.float64)
+    scale = np.maximum(np.abs(want), 1e-3 * np.abs(want).max())
+    assert (np.abs(got - want) / scale).max() < 1e-3
+    del o4, x64, want, got
+    # C5: argmax, max, cross-entropy down 32000 rows
+    x5, idx = configs.inputs_c5()
+    X5 = be.array(x5)
+    am, mx, ce = be.empty((1, 256), dtype=np.int32), be.empty((1, 256)), be.empty((1, 256))
+    configs.c5a_argmax(be, am, X5)
+    configs.c5b_max(be, mx, X5)
+    configs.c5c_cross_entropy(be, ce, X5, be.onehot(be.array(idx, dtype=np.int32), axis=0))
+    assert np.array_equal(am.get().ravel(), x5.argmax(axis=0))
+    assert np.array_equal(mx.get().ravel(), x5.max(axis=0))
+    x64 = x5.astype(np.float64)
+    m64 = x64.max(axis=0)
+    ce64 = np.log(np.exp(x64 - m64).sum(axis=0)) + m64 - x64[idx.ravel(), np.arange(256)]
+    assert_close(ce.get().ravel(), ce64, rtol=1e-5, atol=1e-5, what="C5c")
