@@ -2244,7 +2244,8 @@ COLSPLIT_SUBBATCH_ROWS = 8
 COLSPLIT_BATCH_WORDS = 64
 
 
-def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, NB=4, multi=True, runs=False):
+def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, NB=4, multi=True, runs=False,
+                 lookback=False):
     """One level of axis-0 reductions over a tall matrix.  grid = (column
     strips, row chunks); a workgroup is LX column-lanes x LY row-lanes.
     ``multi``: more than one chunk per strip.
@@ -2310,6 +2311,10 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
         lds += S * (8 if g.is_pair(n) else 4)
     L("__shared__ int s_last;")
     g.declare_one()
+    lookback = bool(lookback and multi and not runs and V * 64 <= T)
+    if lookback:
+        L("__shared__ unsigned int s_tag;")
+        L("__shared__ int s_abort;")
     if runs < 0:
         # every XCD takes whole row chunks (chunk = 8 * round + XCD), all strips of a chunk side by side
         L("const int nchunks = (int)(((long long)R + rows_per_chunk - 1) / rows_per_chunk);")
@@ -2340,6 +2345,11 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
         L("const int clim = cfull ? %d : (col_ok ? (int)(C - c) : 0);" % V)
     L("const long long r0 = (long long)chunk * rows_per_chunk;")
     L("const long long r1 = (r0 + rows_per_chunk < R) ? (r0 + rows_per_chunk) : (long long)R;")
+    if lookback:
+        # the tag of this launch: what this workgroup's own first record carried, flipped (every launch
+        # writes every record once; the workspace starts zeroed).  Loaded now, needed after the sweep.
+        L("nh_pair own_ = nh_pair{0.0f, 0};")
+        L("if (threadIdx.x == 0) own_ = nh_part_load(reinterpret_cast<const nh_pair*>(ws) + (long long)chunk * C + c0);")
     g.pos = ("0", "c")
     g.emit_gather_prefetch(_needed([st.root for st in prog.statements], set(n.nid for n in prog.nodes if n.kind == "R")),
                            V, "col_ok && ty == 0")
@@ -2421,6 +2431,8 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
         L("#pragma unroll")
         L("for (int j = 0; j < %d; ++j) s_w%d[threadIdx.x >> 6][tx * %d + j0[%d] + j] = acc%d[j];" % (VK, n.nid, V, k, n.nid))
     L.close()
+    if lookback:
+        L("if (threadIdx.x == 0) { s_tag = ((nh_u32)own_.i >> 31) ^ 1u; s_abort = 0; }")
     L("__syncthreads();")
     for n in reds:
         L("%s one%d = %s::init();" % ("nh_pair" if g.is_pair(n) else "float", n.nid, fold_op[n.nid]))
@@ -2450,11 +2462,55 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
         for k, n in enumerate(reds):
             L("nh_pair* part%d = reinterpret_cast<nh_pair*>(ws) + (long long)%d * nchunks * C;" % (n.nid, k))
         L("unsigned int* const ticket = reinterpret_cast<unsigned int*>(ws + ticket_offset) + %d * strip;" % TICKET_STRIDE_WORDS)
+        if lookback:
+            L("const nh_u32 tag = s_tag;")
         L.open("if (joins && c0 + jcol < C)")
         for n in reds:
             val = ("one%d" % n.nid) if g.is_pair(n) else ("nh_pair{one%d, 0}" % n.nid)
+            if lookback:
+                val = "nh_tag_put(%s, tag)" % val
             L("nh_part_store(&part%d[(long long)chunk * C + c0 + jcol], %s);" % (n.nid, val))
         L.close()
+    if multi and lookback:
+        # Tagged records instead of a ticket: (value, tag) is one 8-byte atomic store, so whoever sees the
+        # tag has the value.  The strip's LAST %d chunks each finish one tile of V columns: a wave per
+        # column polls the records of all chunks, a wave-wide fold, and the lane that owns the tile
+        # evaluates the statements.  Everybody else is done after its stores.  The finishing workgroups
+        # have the highest block numbers, so none of them starts before every other workgroup of the
+        # grid has been handed to a compute unit: they cannot keep a producer from running.
+        G = S // V
+        L("const int grp = (int)chunk - (nchunks - %d);" % G)
+        L("if (grp < 0) return;")
+        L("const int pw = threadIdx.x >> 6, pq = threadIdx.x & 63;")
+        L("const long long pc = c0 + grp * %d + pw;" % V)
+        L("const bool polls = (pw < %d) && (pq < nchunks) && (pc < C);" % V)
+        for n in reds:
+            L("nh_pair rec%d = nh_pair{0.0f, 0};" % n.nid)
+        L.open("if (polls)")
+        L("unsigned int spins = 0;")
+        L.open("for (;;)")
+        for n in reds:
+            L("rec%d = nh_part_load(&part%d[(long long)pq * C + pc]);" % (n.nid, n.nid))
+        L("if (%s) break;" % " && ".join("nh_tag_is(rec%d, tag)" % n.nid for n in reds))
+        L("__builtin_amdgcn_s_sleep(1);")
+        L("if (++spins > NH_SPIN_LIMIT) { s_abort = 1; break; }")
+        L.close()
+        L.close()
+        for n in reds:
+            op = fold_op[n.nid]
+            if n.is_index:
+                L("rec%d.i = (int)((nh_u32)rec%d.i | 0x80000000u);" % (n.nid, n.nid))
+            elif g.is_pair(n):
+                L("rec%d.i = (int)((nh_u32)rec%d.i & 0x7fffffffu);" % (n.nid, n.nid))
+            if g.is_pair(n):
+                L("one%d = nh_wave_allreduce<%s, 64, nh_pair>(polls ? rec%d : %s::init());" % (n.nid, op, n.nid, op))
+            else:
+                L("one%d = nh_wave_allreduce<%s, 64, float>(polls ? rec%d.v : %s::init());" % (n.nid, op, n.nid, op))
+        L.open("if (pq == 0 && pw < %d)" % V)
+        for n in reds:
+            L("s_r%d[grp * %d + pw] = one%d;" % (n.nid, V, n.nid))
+        L.close()
+    elif multi:
         # The partials were written through to device-coherent memory (nh_part_store); every
         # lane waits for its own stores before the barrier (nh_publish_barrier), lane 0 then
         # takes the ticket, and the last workgroup reads the partials past its L2 (nh_part_load).
@@ -2501,6 +2557,14 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
             L("s_r%d[jcol] = one%d;" % (n.nid, n.nid))
         L.close()
     L("__syncthreads();")
+    if multi and lookback:
+        # a record never came (its workgroup was not running within the wait's bound): no result for
+        # this tile, and the host is told through the plan's status word
+        L.open("if (s_abort)")
+        L("unsigned int* status = reinterpret_cast<unsigned int*>(ws + ticket_offset) + %d * gridDim.x;" % TICKET_STRIDE_WORDS)
+        L("if (threadIdx.x == 0) __hip_atomic_store(status, NH_COOP_ABORTED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
+        L("return;")
+        L.close()
     # the lanes that evaluate the statements pick up the V columns of their tile
     for n in reds:
         if n.is_index:
@@ -2524,7 +2588,7 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
     roots = [st.root for st in prog.statements]
     nodes = _needed(roots, done)
     leaves = g.leaf_nodes(nodes)
-    L.open("if (col_ok && ty == 0)")
+    L.open("if (col_ok && ty == 0%s)" % (" && tx == grp" if (multi and lookback) else ""))
     for n in leaves:
         g.emit_load(n, "0", "c", V, "_l")
     for st in prog.statements:
@@ -2546,4 +2610,4 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
     L.close()
     return _finish("colsplit", g, head, fmt, T, lds,
                    dict(V=V, LX=LX, LY=LY, NR=NR, NB=NB, NRED=len(reds), multi=bool(multi),
-                        stream=bool(stream), tail=bool(tail), runs=int(runs)))
+                        stream=bool(stream), tail=bool(tail), runs=int(runs), lookback=bool(lookback and multi)))

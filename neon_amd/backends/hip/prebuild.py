@@ -76,6 +76,7 @@ class PlanBackend(Backend):
         self.cache = planner.KernelCache(arch, cache_dir)
         self.compile_kernels = compile_kernels
         self.choices = []          # Choice per executed statement group
+        self.coop = True           # False: plan as for a program whose inter-workgroup wait once expired
         self._pending = []
         self._fusing = False
 
@@ -113,7 +114,7 @@ class PlanBackend(Backend):
         for t in trees:
             prog.add_statement(t)
         prog.finalize()
-        ch = planner.choose(prog, self.cu_count)
+        ch = planner.choose(prog, self.cu_count, self.coop)
         if self.compile_kernels:
             self.cache.code_object(ch.spec)
         self.choices.append(ch)

@@ -465,15 +465,17 @@ class _Recorded(object):
 
     def replay(self, rt, records_type=None):
         """enqueue the recorded launches; the first replay fills in the launch
-        records, and -- for a statement that is kernel launches only, none of
-        them cooperative -- hands them to the C replayer (``records_type``),
-        which serves the statement from then on"""
+        records, and -- for a statement that is kernel launches only -- hands
+        them to the C replayer (``records_type``), which serves the statement
+        from then on (and notes its cooperative plans as launched, like the
+        callers of this method do)"""
         prepared = self.prepared
         if prepared is None:
             prepared = self.prepared = [None if kernel is None else rt.prepare(kernel, grid, block, args)
                                         for kernel, grid, block, args in self.launches]
-            if records_type is not None and not self.coop and None not in prepared:
-                self.fast = records_type([p[0].value for p in prepared], self.raw, prepared)
+            if records_type is not None and None not in prepared:
+                self.fast = records_type([p[0].value for p in prepared], self.raw, prepared,
+                                         tuple((plan.key, plan) for plan in self.coop) or None)
         for prep, launch in zip(prepared, self.launches):
             if prep is None:
                 launch[1](*launch[3])            # a recorded call of a prebuilt kernel's entry point
@@ -586,6 +588,11 @@ class NervanaHIPBase(object):
             self._fusion_blocks = self._fusion_blocks[:1]
         self._captured = None
         self._launch_cache = {}      # statement-group identity -> recorded launches
+        # cooperative plans (workgroups that wait for one another) launched since the
+        # last look at their status words, and the program keys whose plan gave up
+        # (the C replayer holds this very dict: emptied in place, never replaced)
+        self._coop_pending = {}
+        self._coop_failed = set()
         self._replayer = self._records_type = None
         if fastpath.enabled():
             # repeated single statements: walk, lookup and launches in C (neon_amd/csrc/fastpath.c).
@@ -597,7 +604,8 @@ class NervanaHIPBase(object):
                 logger.warning("running without the C replayer: %s", e)
                 mod = None
             if mod is not None:
-                self._replayer = mod.Replayer(self._launch_cache, self.tensor_cls, self.rt.launch_prepared_address)
+                self._replayer = mod.Replayer(self._launch_cache, self.tensor_cls, self.rt.launch_prepared_address,
+                                              self._coop_pending)
                 self._records_type = mod.Records
         self._recording = None
         self._rec_temps = None
@@ -608,10 +616,6 @@ class NervanaHIPBase(object):
         self._rec_single = None
         self._temp_pool = {}
         self._live_allocs = 0
-        # cooperative plans (workgroups that wait for one another) launched since the
-        # last look at their status words, and the program keys whose plan gave up
-        self._coop_pending = {}
-        self._coop_failed = set()
 
     # -- memory ---------------------------------------------------------------------
     def _mem_alloc(self, nbytes):
@@ -656,7 +660,8 @@ class NervanaHIPBase(object):
         families that never wait (stage by stage where one kernel cannot)."""
         if not self._coop_pending:
             return
-        pending, self._coop_pending = self._coop_pending, {}
+        pending = dict(self._coop_pending)
+        self._coop_pending.clear()
         failed = []
         word = np.zeros(1, np.uint32)
         for key, plan in pending.items():

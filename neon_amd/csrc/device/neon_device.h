@@ -674,6 +674,11 @@ NEON_DEV nh_pair nh_part_load(const nh_pair* p) {
     return __builtin_bit_cast(nh_pair, __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p),
                                                          __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
 }
+// A tag in bit 31 of a record's second word: free for float partials (the word is unused), for
+// arg-reduction keys (the word is ~index with index < 2^31, so the bit is always 1 and is put back)
+// and for (max, sum) pairs (the word holds the bits of a sum >= 0; a NaN loses its sign).
+NEON_DEV nh_pair nh_tag_put(nh_pair p, nh_u32 tag) { p.i = (int)(((nh_u32)p.i & 0x7fffffffu) | (tag << 31)); return p; }
+NEON_DEV bool nh_tag_is(nh_pair p, nh_u32 tag) { return ((nh_u32)p.i >> 31) == tag; }
 // All threads of the workgroup call it, after the last nh_part_store.
 NEON_DEV void nh_publish_barrier() {
 #if NH_FORMAL_FENCES

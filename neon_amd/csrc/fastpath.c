@@ -31,17 +31,21 @@ typedef struct {
     const void** recs;
     double* raw;
     PyObject* keep;          /* whatever owns the memory the records point into */
+    PyObject* coop;          /* NULL, or a tuple of (key, plan): plans whose workgroups wait for one another,
+                              * to be entered into the replayer's table of plans to check after each replay */
 } Records;
 
 /* (both types take part in cycle collection: backend -> replayer -> launch cache -> entry ->
  * records / temporaries -> tensors -> backend is a cycle the collector has to see through) */
 static int Records_traverse(Records* self, visitproc visit, void* arg) {
     Py_VISIT(self->keep);
+    Py_VISIT(self->coop);
     return 0;
 }
 
 static int Records_clear(Records* self) {
     Py_CLEAR(self->keep);
+    Py_CLEAR(self->coop);
     return 0;
 }
 
@@ -50,6 +54,7 @@ static void Records_dealloc(Records* self) {
     PyMem_Free((void*)self->recs);
     PyMem_Free(self->raw);
     Py_XDECREF(self->keep);
+    Py_XDECREF(self->coop);
     Py_TYPE(self)->tp_free((PyObject*)self);
 }
 
@@ -71,8 +76,17 @@ static int fill_raw(Records* self, PyObject* seq) {
 }
 
 static PyObject* Records_new(PyTypeObject* type, PyObject* args, PyObject* kw) {
-    PyObject *addresses, *numbers, *keep;
-    if (!PyArg_ParseTuple(args, "OOO:Records", &addresses, &numbers, &keep)) return NULL;
+    PyObject *addresses, *numbers, *keep, *coop = NULL;
+    if (!PyArg_ParseTuple(args, "OOO|O:Records", &addresses, &numbers, &keep, &coop)) return NULL;
+    if (coop == Py_None) coop = NULL;
+    if (coop) {
+        int ok = PyTuple_Check(coop);
+        for (Py_ssize_t i = 0; ok && i < PyTuple_GET_SIZE(coop); ++i) {
+            PyObject* item = PyTuple_GET_ITEM(coop, i);
+            ok = PyTuple_Check(item) && PyTuple_GET_SIZE(item) == 2;
+        }
+        if (!ok) { PyErr_SetString(PyExc_TypeError, "coop must be a tuple of (key, plan) pairs"); return NULL; }
+    }
     PyObject* fast = PySequence_Fast(addresses, "addresses must be a sequence");
     if (!fast) return NULL;
     Records* self = (Records*)type->tp_alloc(type, 0);
@@ -91,6 +105,8 @@ static PyObject* Records_new(PyTypeObject* type, PyObject* args, PyObject* kw) {
     if (fill_raw(self, numbers) < 0) { Py_DECREF(self); return NULL; }
     Py_INCREF(keep);
     self->keep = keep;
+    Py_XINCREF(coop);
+    self->coop = coop;
     return (PyObject*)self;
 }
 
@@ -116,7 +132,7 @@ static PyTypeObject RecordsType = {
     .tp_flags = Py_TPFLAGS_DEFAULT | Py_TPFLAGS_HAVE_GC,
     .tp_traverse = (traverseproc)Records_traverse,
     .tp_clear = (inquiry)Records_clear,
-    .tp_doc = "Records(addresses, numbers, keep): launch records of one statement",
+    .tp_doc = "Records(addresses, numbers, keep[, coop]): launch records of one statement",
     .tp_methods = Records_methods,
     .tp_members = Records_members,
     .tp_new = Records_new,
@@ -199,18 +215,22 @@ typedef struct {
     PyObject* cache;              /* the backend's launch cache (dict) */
     PyTypeObject* tensor_cls;
     launch_fn launch;
+    PyObject* pending;            /* NULL, or the backend's dict of cooperative plans launched since it last
+                                   * looked at their status words */
     long long replayed, launches;
 } Replayer;
 
 static int Replayer_traverse(Replayer* self, visitproc visit, void* arg) {
     Py_VISIT(self->cache);
     Py_VISIT((PyObject*)self->tensor_cls);
+    Py_VISIT(self->pending);
     return 0;
 }
 
 static int Replayer_clear(Replayer* self) {
     Py_CLEAR(self->cache);
     Py_CLEAR(self->tensor_cls);
+    Py_CLEAR(self->pending);
     return 0;
 }
 
@@ -218,12 +238,14 @@ static void Replayer_dealloc(Replayer* self) {
     PyObject_GC_UnTrack(self);
     Py_XDECREF(self->cache);
     Py_XDECREF((PyObject*)self->tensor_cls);
+    Py_XDECREF(self->pending);
     Py_TYPE(self)->tp_free((PyObject*)self);
 }
 
 static PyObject* Replayer_new(PyTypeObject* type, PyObject* args, PyObject* kw) {
-    PyObject *cache, *cls, *fn;
-    if (!PyArg_ParseTuple(args, "O!O!O:Replayer", &PyDict_Type, &cache, &PyType_Type, &cls, &fn)) return NULL;
+    PyObject *cache, *cls, *fn, *pending = NULL;
+    if (!PyArg_ParseTuple(args, "O!O!O|O!:Replayer", &PyDict_Type, &cache, &PyType_Type, &cls, &fn,
+                          &PyDict_Type, &pending)) return NULL;
     void* p = PyLong_AsVoidPtr(fn);
     if (!p) {
         if (!PyErr_Occurred()) PyErr_SetString(PyExc_ValueError, "null launch function");
@@ -236,6 +258,8 @@ static PyObject* Replayer_new(PyTypeObject* type, PyObject* args, PyObject* kw) 
     self->cache = cache;
     self->tensor_cls = (PyTypeObject*)cls;
     self->launch = (launch_fn)p;
+    Py_XINCREF(pending);
+    self->pending = pending;
     return (PyObject*)self;
 }
 
@@ -351,11 +375,22 @@ static PyObject* Replayer_replay(Replayer* self, PyObject* const* args, Py_ssize
             Records* r = (Records*)recs;
             int same = r->nraw == w.nraw;
             for (Py_ssize_t i = 0; same && i < w.nraw; ++i) same = r->raw[i] == w.raw[i];
+            if (same && r->coop && !self->pending) same = 0;       /* nowhere to note the plans: not handled here */
             if (same) {
                 result = 1;
                 for (Py_ssize_t i = 0; i < r->nrec; ++i) {
                     int rc = self->launch(r->recs[i]);
                     if (rc) { result = -(long)rc; break; }
+                }
+                if (result == 1 && r->coop) {
+                    for (Py_ssize_t i = 0; i < PyTuple_GET_SIZE(r->coop); ++i) {
+                        PyObject* item = PyTuple_GET_ITEM(r->coop, i);
+                        if (PyDict_SetItem(self->pending, PyTuple_GET_ITEM(item, 0), PyTuple_GET_ITEM(item, 1)) < 0) {
+                            Py_DECREF(recs);
+                            Py_DECREF(key);
+                            return NULL;
+                        }
+                    }
                 }
                 if (result == 1) {
                     self->replayed += 1;
@@ -397,7 +432,7 @@ static PyTypeObject ReplayerType = {
     .tp_flags = Py_TPFLAGS_DEFAULT | Py_TPFLAGS_HAVE_GC,
     .tp_traverse = (traverseproc)Replayer_traverse,
     .tp_clear = (inquiry)Replayer_clear,
-    .tp_doc = "Replayer(launch_cache, tensor_class, address of nh_launch_prepared)",
+    .tp_doc = "Replayer(launch_cache, tensor_class, address of nh_launch_prepared[, pending cooperative plans])",
     .tp_methods = Replayer_methods,
     .tp_members = Replayer_members,
     .tp_new = Replayer_new,

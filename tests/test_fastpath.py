@@ -156,6 +156,36 @@ def test_replay_issues_the_records_in_order(rig):
     assert rp.replay(o, 0.25 * x + 2.0) == 0
 
 
+def test_replay_notes_the_cooperative_plans_it_launched(rig):
+    """records may carry (key, plan) pairs of kernels whose workgroups wait
+    for one another: every replay enters them in the dict the replayer was
+    given, where the backend finds them at its next synchronisation"""
+    mod, be, rp, cache, calls, verdict, t, launch = rig
+    x, o = t((8, 8)), t((8, 8))
+    key, raw = python_key(o, x * x)
+    plan_a, plan_b = object(), object()
+    recs = mod.Records([0x10, 0x20], raw, None, (("a", plan_a), ("b", plan_b)))
+    cache[key] = Entry(recs)
+    assert rp.replay(o, x * x) == 0 and calls == []          # this replayer has nowhere to note them
+    pending = {}
+    rp2 = mod.Replayer(cache, GeomTensor, ctypes.cast(launch, ctypes.c_void_p).value, pending)
+    assert rp2.replay(o, x * x) == 1 and calls == [0x10, 0x20]
+    assert pending == {"a": plan_a, "b": plan_b}
+    pending.clear()                                          # (the backend empties it in place)
+    assert rp2.replay(o, x * x) == 1 and pending == {"a": plan_a, "b": plan_b}
+    verdict[0] = 3
+    pending.clear()
+    assert rp2.replay(o, x * x) == -3 and pending == {}       # nothing noted for a launch that failed
+    verdict[0] = 0
+    cache[key] = Entry(mod.Records([0x10], raw, None, None)) # no cooperative plans: as without the argument
+    assert rp.replay(o, x * x) == 1
+    for bad in ([("a", plan_a)], (("a",),), ("ab",), 5):
+        with pytest.raises(TypeError):
+            mod.Records([0x10], raw, None, bad)
+    with pytest.raises(TypeError):
+        mod.Replayer(cache, GeomTensor, ctypes.cast(launch, ctypes.c_void_p).value, [])
+
+
 def test_launch_errors_come_back_negated(rig):
     mod, be, rp, cache, calls, verdict, t, _ = rig
     x, o = t((8, 8)), t((8, 8))

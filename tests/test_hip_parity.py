@@ -1129,3 +1129,45 @@ def test_split_column_reductions_with_strips_dealt_to_xcds_in_runs(hip, shape, d
         assert np.array_equal(am.get().ravel(), x.argmax(axis=0))
         m = x64.max(axis=0)
         assert_close(lse.get().ravel(), np.log(np.exp(x64 - m).sum(axis=0)) + m, rtol=RTOL32, atol=1e-5, what="log-sum-exp")
+
+
+@pytest.mark.parametrize("shape,dtype", [((32000, 256), np.float32), ((16000, 250), np.float32), ((30000, 264), np.float16),
+                                         ((8192, 1024), np.float32), ((40000, 96), np.float32), ((6000, 509), np.float16)])
+def test_split_column_reductions_finished_by_the_last_workgroups_of_a_strip(hip, shape, dtype):
+    """the split column family where the strip's last workgroups wait for the
+    others' tagged partials (a tag bit inside each 8-byte record, flipped every
+    launch): sum / max / argmax / min with NaNs / log-sum-exp against numpy on
+    fresh data, four launches in a row of every kernel so that both tag values
+    are met, widths with a ragged last strip and a ragged last vector included."""
+    tagged = 0
+    for rep in range(4):
+        rs = np.random.RandomState(rep + 77)
+        x = rs.standard_normal(shape).astype(dtype)
+        x[rs.randint(0, shape[0], 50), rs.randint(0, shape[1], 50)] = 3.5         # ties for argmax
+        xn = x.copy()
+        xn[rs.randint(0, shape[0], 3), rs.randint(0, shape[1], 3)] = np.nan
+        tx, tn = hip.array(x, dtype=dtype), hip.array(xn, dtype=dtype)
+        sm, mx, mn, lse = (hip.empty((1, shape[1])) for _ in range(4))
+        am = hip.empty((1, shape[1]), dtype=np.int32)
+        if rep == 0:
+            for issue in (lambda: sm.__setitem__(slice(None), hip.sum(tx, axis=0)),
+                          lambda: am.__setitem__(slice(None), hip.argmax(tx, axis=0))):
+                with hip.capture() as groups:
+                    issue()
+                spec = hip.time_group(groups[0], reps=1)[1].spec
+                assert spec.family == "colsplit"
+                tagged += bool(spec.params["lookback"])
+        sm[:] = hip.sum(tx, axis=0)
+        mx[:] = hip.max(tx, axis=0)
+        am[:] = hip.argmax(tx, axis=0)
+        mn[:] = hip.min(tn, axis=0)
+        lse[:] = hip.log(hip.sum(hip.exp(tx - hip.max(tx, axis=0)), axis=0)) + hip.max(tx, axis=0)
+        x64 = x.astype(np.float64)
+        assert_close(sm.get(), x64.sum(axis=0, keepdims=True), rtol=RTOL32, atol=2e-3 * np.sqrt(shape[0]), what="sum")
+        assert np.array_equal(mx.get(), x.astype(np.float32).max(axis=0, keepdims=True))
+        assert np.array_equal(am.get().ravel(), x.argmax(axis=0))
+        assert np.array_equal(mn.get(), xn.astype(np.float32).min(axis=0, keepdims=True), equal_nan=True)
+        m = x64.max(axis=0)
+        assert_close(lse.get().ravel(), np.log(np.exp(x64 - m).sum(axis=0)) + m, rtol=RTOL32, atol=1e-5, what="log-sum-exp")
+    if shape == (32000, 256):
+        assert tagged == 2, "the benchmark shape should take the tagged form"

@@ -89,7 +89,7 @@ def test_the_hand_offs_built_with_release_and_acquire_fences(hip, monkeypatch):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("family", ["colcoop", "rowcoop"])
+@pytest.mark.parametrize("family", ["colcoop", "rowcoop", "colsplit"])
 def test_a_cooperative_kernel_that_gave_up_is_reported_and_replaced(pair, family, monkeypatch):
     """Nothing is made to hang: the word an aborting workgroup would leave is
     written into the plan's workspace from the host.  The next synchronisation
@@ -103,6 +103,14 @@ def test_a_cooperative_kernel_that_gave_up_is_reported_and_replaced(pair, family
         def run(be):
             X, out = be.array(x), be.empty(x.shape)
             out[:] = be.exp(X - be.max(X, axis=0)) / be.sum(be.exp(X - be.max(X, axis=0)), axis=0)
+            return out
+    elif family == "colsplit":
+        # (the split family's tagged form: only the last workgroups of a strip wait)
+        x = (rs.standard_normal((32000, 256)) * 2).astype(np.float32)
+
+        def run(be):
+            X, out = be.array(x), be.empty((1, x.shape[1]))
+            out[:] = be.sum(be.exp(X - be.max(X, axis=0)), axis=0)
             return out
     else:
         x = (rs.standard_normal((6, 50000)) * 2).astype(np.float32)
@@ -131,3 +139,36 @@ def test_a_cooperative_kernel_that_gave_up_is_reported_and_replaced(pair, family
     assert all(p.status_ptr is None for k, p in hip.plans.items() if k not in before), \
         "the replacement must not wait between workgroups"
     del out
+
+
+@pytest.mark.gpu
+def test_a_replayed_cooperative_statement_is_still_checked(hip):
+    """the same statement over the same tensors is served from its recording
+    (by the C replayer where it is built): the plan must be looked at by the
+    next synchronisation all the same"""
+    rs = np.random.RandomState(4)
+    x = rs.standard_normal((31000, 256)).astype(np.float32)
+    X, out = hip.array(x), hip.empty((1, 256))
+    with hip.capture() as groups:
+        out[:] = hip.max(X, axis=0)
+    plan = hip.time_group(groups[0], reps=1)[1]
+    assert plan.spec.family == "colsplit" and plan.spec.params["lookback"] and plan.status_ptr is not None
+    for _ in range(3):
+        out[:] = hip.max(X, axis=0)
+    hip.synchronize()
+    assert np.array_equal(out.get(), x.max(axis=0, keepdims=True))
+    replayed = hip.plan_stats["replayed"]
+    assert not hip._coop_pending
+    out[:] = hip.max(X, axis=0)
+    assert hip.plan_stats["replayed"] == replayed + 1 and hip._coop_pending.get(plan.key) is plan
+    hip.synchronize()
+    assert not hip._coop_pending
+    hip.rt.memset(plan.status_ptr, 0xDEAD, 1, 4)
+    out[:] = hip.max(X, axis=0)
+    with pytest.raises(hiprt.HipError) as err:
+        hip.synchronize()
+    assert err.value.code == hiprt.NH_ECOOP and plan.key not in hip.plans
+    out[:] = hip.max(X, axis=0)                      # planned again, in the form that never waits
+    assert np.array_equal(out.get(), x.max(axis=0, keepdims=True))
+    again = hip.plans[plan.key]
+    assert again is not plan and again.status_ptr is None and not again.spec.params["lookback"]

@@ -305,11 +305,20 @@ def test_shape_class_selection(pb):
     assert ch.spec.family == "colcoop" and ch.grid[0] * ch.grid[1] <= 256 and ch.workspace is not None
     assert ch.spec.source.count("nh_part_store") == 1 and "NH_SPIN_LIMIT" in ch.spec.source
     assert "nh_op_lse" in ch.spec.source and ch.status_offset is not None
-    # cross-entropy with the one-hot made in the kernel: one pass, no waiting at all
+    # cross-entropy with the one-hot made in the kernel: one pass; only the strip's last workgroups wait,
+    # for tagged partials, and a program whose wait once expired gets the form that never waits
     i5 = pb.empty((1, 256), np.int32)
-    ch = plan_of(pb, lambda: pb.empty((1, 256)).__setitem__(slice(None), -pb.sum(
-        pb.onehot(i5, axis=0) * pb.log(pb.fprop_softmax(x5, 0)), axis=0)))
-    assert ch.spec.family == "colsplit" and "NH_SPIN_LIMIT" not in ch.spec.source and "nh_op_lse" in ch.spec.source
+    xent = lambda: pb.empty((1, 256)).__setitem__(slice(None), -pb.sum(
+        pb.onehot(i5, axis=0) * pb.log(pb.fprop_softmax(x5, 0)), axis=0))
+    ch = plan_of(pb, xent)
+    assert ch.spec.family == "colsplit" and "nh_op_lse" in ch.spec.source
+    assert ch.spec.params["lookback"] and ch.status_offset is not None and "nh_ticket_take" not in ch.spec.source
+    assert ch.spec.source.count("NH_SPIN_LIMIT") == 1 and "nh_tag_put" in ch.spec.source
+    pb.coop = False
+    ch = plan_of(pb, xent)
+    pb.coop = True
+    assert ch.spec.family == "colsplit" and not ch.spec.params["lookback"] and ch.status_offset is None
+    assert "NH_SPIN_LIMIT" not in ch.spec.source and "nh_ticket_take" in ch.spec.source
     huge = pb.empty((4000000, 256))
     with pytest.raises(planner.NeedsSplit):        # too many rows to keep on chip: evaluated stage by stage
         pb.empty((4000000, 256)).__setitem__(slice(None), pb.fprop_softmax(huge, 0))
