@@ -534,15 +534,34 @@ COLCOOP_MAX_BYTES_512 = max(COLCOOP_MAX_BYTES, int(os.environ.get("NEON_HIP_COLC
 # over a small matrix.  Softmax, cooperative / staged: (8192,1024) fp16, 16 MB: 26 / 20 us; (4096,1000)
 # fp32, 16 MB: 18.3 / 16.6; (3000,2000) fp32, 24 MB: 20.5 / 22.0; (16384,512) fp32, 32 MB: 24.3 / 26.4.
 COLCOOP_MIN_BYTES = int(os.environ.get("NEON_HIP_COLCOOP_MIN_MB", "20")) << 20
+COL_TINY_ONE_WORD = os.environ.get("NEON_HIP_COL_TINY_ONE_WORD", "1") != "0"
 ONLINE_LSE_IN_ONE_WORKGROUP = os.environ.get("NEON_HIP_ONLINE_LSE_COL", "0") != "0"
 
 
-def _plan_col(prog, cu_count, coop=True):
+def _plan_col(prog, cu_count, coop=True, one_word_lanes=None):
     R, C = prog.domain
     V = _vector_width(prog, tail_ok=True)
+    isz = max([t.dtype.itemsize for t in prog.tensors if t.shape[1] > 1] + [1])
+    if (one_word_lanes is None and COL_TINY_ONE_WORD and V > 4 // isz and isz in (2, 4)
+            and R * C * isz <= (4 << 20)):
+        # Tiny inputs whose rows stay in registers: one 32-bit word per lane and the strip's width made of
+        # adjacent lanes, instead of one 16-byte vector per lane -- a quarter of the registers, and the wave
+        # fold has one value (two 16-bit ones) to pass round instead of four (eight).  Softmax down the
+        # columns, 16 bytes / 4 bytes per lane: (1000,128) fp32 4.5 -> 4.0 us, (2000,128) 6.3 -> 5.3, (512,512)
+        # 4.2 -> 4.0, (300,1024) 4.1 -> 3.6, (100,4096) 3.9 -> 3.6, (64,2048) 3.4 -> 3.2, (1000,256) 4.8 -> 4.8;
+        # fp16 (1000,128) 4.9 -> 4.5, (2000,256) 7.1 -> 5.9.  Mean / variance normalisation (1000,128) fp32
+        # 4.7 -> 3.9, fp16 5.2 -> 3.9; argmax fp32 3.6 -> 3.2, fp16 4.1 -> 3.2; sum 2.6 -> 2.5.  From 8 MB on
+        # there is nothing in it ((2000,2048) fp32 softmax 11.8 / 12.0 us, (1000,4096) 9.1 / 9.2).
+        try:
+            ch = _plan_col(prog, cu_count, coop, one_word_lanes=True)
+            if ch.spec.family == "col":
+                return ch
+        except NeedsSplit:
+            pass
+    if one_word_lanes:
+        V = 4 // isz
     tail = (C % V) != 0
     nvec = _ceil_div(C, V)
-    isz = max([t.dtype.itemsize for t in prog.tensors if t.shape[1] > 1] + [1])
     words = _words_per_tile(prog, V, 0)
     line_only = all(st.out.shape[0] == 1 and R > 1 for st in prog.statements)
 

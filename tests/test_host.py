@@ -291,6 +291,14 @@ def test_shape_class_selection(pb):
     xs = pb.empty((1000, 128))
     ch = plan_of(pb, lambda: pb.empty((1000, 128)).__setitem__(slice(None), pb.fprop_softmax(xs, 0)))
     assert ch.spec.family == "col" and ch.spec.params["NR"] * ch.spec.params["LY"] >= 1000
+    # tiny inputs: one 32-bit word per lane, the 16-byte strip made of adjacent lanes
+    assert (ch.spec.params["V"], ch.spec.params["LX"]) == (1, 4)
+    xh = pb.empty((1000, 128), np.float16)
+    ch = plan_of(pb, lambda: pb.empty((1000, 128), np.float16).__setitem__(slice(None), pb.fprop_softmax(xh, 0)))
+    assert ch.spec.family == "col" and ch.spec.params["V"] == 2
+    xm = pb.empty((2000, 2048))
+    ch = plan_of(pb, lambda: pb.empty((2000, 2048)).__setitem__(slice(None), pb.fprop_softmax(xm, 0)))
+    assert ch.spec.family == "col" and ch.spec.params["V"] == 4
     x4, o4 = pb.empty((256, 100352), f16), pb.empty((256, 100352), f16)
     ch = plan_of(pb, lambda: o4.__setitem__(slice(None), (x4 - pb.mean(x4, axis=1)) / pb.sqrt(pb.var(x4, axis=1) + 1e-5)))
     assert ch.spec.family == "row" and ch.spec.params["V"] == 8 and ch.spec.params["NCH"] == 13
