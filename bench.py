@@ -19,7 +19,9 @@ Each row also carries ``kernel_us_rocprof`` -- the median rocprofv3 kernel
 duration of the same kernel from the committed summaries under ``profiles/``
 -- and ``traffic``, the HBM bytes per launch from hardware counters; both are
 looked up by kernel name and are null when the summaries were made from
-other kernels.  ``cpu_baseline`` times the numpy oracle on the same Adam step
+other kernels (the prebuilt kernels behind direct C-ABI entry points are found
+by a part of the compiler's name for them, which a change of their source does
+not alter: their rows are remade whenever ``kernels.hip`` changes).  ``cpu_baseline`` times the numpy oracle on the same Adam step
 on this machine's host cores.
 
 Other modes (each the program behind one of the summaries in ``profiles/``):
@@ -63,6 +65,13 @@ def rocprof_us(kernel_name, mode="hot"):
     ``kernel_name`` from the committed kernel-trace summary, or None"""
     from neon_amd.profile_summary import lookup
     rec = lookup(DURATION_SUMMARY[mode], kernel_name)
+    return rec["median_us"] if rec else None
+
+
+def rocprof_us_part(part, mode="hot"):
+    """as ``rocprof_us`` for a prebuilt kernel, found by a part of the compiler's name for it"""
+    from neon_amd.profile_summary import lookup_part
+    rec = lookup_part(DURATION_SUMMARY[mode], part)
     return rec["median_us"] if rec else None
 
 
@@ -388,7 +397,7 @@ def gpu_leg(steps, warmup, detail=True, no_cold=False, hot_cold_only=False):
     lib = rt.lib
     e0, e1 = rt.event(), rt.event()
 
-    def measure_abi(label, call, nbytes, elements, reps=30):
+    def measure_abi(label, part, call, nbytes, elements, reps=30):
         for _ in range(3):
             call()
         rt.synchronize()
@@ -399,20 +408,24 @@ def gpu_leg(steps, warmup, detail=True, no_cold=False, hot_cold_only=False):
         rt.event_sync(e1)
         assert rc == 0, lib.nh_last_error()
         ms_k = rt.event_elapsed_ms(e0, e1) / reps
+        us = rocprof_us_part(part, "hot")
         rows.append({"config": label, "bytes": nbytes, "kernels": 1, "ms": ms_k, "api_ms": ms_k,
-                     "timing": "HIP events around back-to-back C-ABI calls", "plan": "prebuilt (kernels.hip)",
+                     "timing": "HIP events around back-to-back C-ABI calls through ctypes: for a kernel of a few "
+                               "microseconds this is the rate of the calls, not the kernel (see kernel_us_rocprof)",
+                     "plan": "prebuilt (kernels.hip)",
                      "gbs": nbytes / (ms_k * 1e-3) / 1e9, "frac_of_hbm_peak": nbytes / (ms_k * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "elements_per_s": elements / (ms_k * 1e-3)})
+                     "elements_per_s": elements / (ms_k * 1e-3), "kernel_us_rocprof": us,
+                     "frac_rocprof": (nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS) if us else None})
 
-    measure_abi("C3 prebuilt nh_adam_step_f32 (5000,5000) f32",
+    measure_abi("C3 prebuilt nh_adam_step_f32 (5000,5000) f32", PREBUILT_PARTS["adam"],
                 lambda: lib.nh_adam_step_f32(p.ptr, m.ptr, v.ptr, g.ptr, 1e-3, 0.9, 0.1, 0.999, 0.001, 1e-8, n3, None),
                 configs.bytes_c3(fused=True), n3)
-    measure_abi("C4 prebuilt nh_rownorm_f16 (256,100352) f16",
+    measure_abi("C4 prebuilt nh_rownorm_f16 (256,100352) f16", PREBUILT_PARTS["rownorm"],
                 lambda: lib.nh_rownorm_f16(o4.ptr, x4.ptr, g4.ptr, b4.ptr, 1e-5, configs.C4_SHAPE[0],
                                            configs.C4_SHAPE[1], configs.C4_SHAPE[1], None),
                 configs.bytes_c4(), configs.C4_SHAPE[0] * configs.C4_SHAPE[1])
     ws = rt.malloc(lib.nh_colreduce_workspace_bytes(configs.C5_SHAPE[0], configs.C5_SHAPE[1]))
-    measure_abi("C5a+b prebuilt nh_colmax_argmax_f32 (32000,256) f32",
+    measure_abi("C5a+b prebuilt nh_colmax_argmax_f32 (32000,256) f32", PREBUILT_PARTS["colmax"],
                 lambda: lib.nh_colmax_argmax_f32(mx.ptr, am.ptr, x5.ptr, configs.C5_SHAPE[0], configs.C5_SHAPE[1],
                                                  configs.C5_SHAPE[1], ws, None),
                 configs.bytes_c5_reduce() + 4 * configs.C5_SHAPE[1], n5)
@@ -673,6 +686,8 @@ def counter_pass():
 
 
 TRACE_WARMUP, TRACE_LAUNCHES = 12, 60
+# a part of the compiler's name for each prebuilt kernel behind a direct C-ABI entry point
+PREBUILT_PARTS = {"adam": "AdamF", "rownorm": "rownorm_f16_kernel", "colmax": "colmax_kernel"}
 
 
 def trace_pass(mode):
@@ -714,7 +729,8 @@ def trace_pass(mode):
 def _trace_support_rows(be, table):
     """hot-pass rows beyond the benchmark configurations: the batch-norm pair on both of its
     shapes (one workgroup per row, and several cooperating workgroups per row), softmax down
-    cooperating column strips, and the two prebuilt kernels that stage data in LDS"""
+    cooperating column strips, the two prebuilt kernels that stage data in LDS, and the
+    hand-written kernels behind the direct C-ABI entry points of C3, C4 and C5"""
     from neon_amd import configs
     rs = np.random.RandomState(3)
     f16 = np.float16
@@ -760,6 +776,27 @@ def _trace_support_rows(be, table):
     t_in, t_out = _fresh(be, sq, rs=rs), be.empty(sq)
     prebuilt("copy_transpose (8192,8192) f32", "transpose_tile", 2 * sq[0] * sq[1] * 4,
              lambda: be.copy_transpose(t_in, t_out))
+    del t_in, t_out
+    # the hand-written kernels behind the direct C-ABI entry points of three configurations
+    lib = be.rt.lib
+    n3 = configs.C3_SHAPE[0] * configs.C3_SHAPE[1]
+    p, m, v, g = (_fresh(be, configs.C3_SHAPE, rs=rs, scale=1e-2) for _ in range(4))
+    prebuilt("C3 prebuilt nh_adam_step_f32 (5000,5000) f32", PREBUILT_PARTS["adam"], configs.bytes_c3(fused=True),
+             lambda: lib.nh_adam_step_f32(p.ptr, m.ptr, v.ptr, g.ptr, 1e-3, 0.9, 0.1, 0.999, 0.001, 1e-8, n3, None))
+    del p, m, v, g
+    K, N = configs.C4_SHAPE
+    x4 = _fresh(be, (K, N), dtype=f16, rs=rs, scale=2.0, shift=0.5)
+    o4, g4, b4 = be.empty((K, N), dtype=f16), _fresh(be, (K, 1), fill=1.0), _fresh(be, (K, 1), fill=0.0)
+    prebuilt("C4 prebuilt nh_rownorm_f16 (256,100352) f16", PREBUILT_PARTS["rownorm"], configs.bytes_c4(),
+             lambda: lib.nh_rownorm_f16(o4.ptr, x4.ptr, g4.ptr, b4.ptr, 1e-5, K, N, N, None))
+    del x4, o4
+    R5, C5 = configs.C5_SHAPE
+    x5, mx, am = _fresh(be, (R5, C5), rs=rs), be.empty((1, C5)), be.empty((1, C5), dtype=np.int32)
+    ws = be.rt.malloc(lib.nh_colreduce_workspace_bytes(R5, C5))
+    prebuilt("C5a+b prebuilt nh_colmax_argmax_f32 (32000,256) f32", PREBUILT_PARTS["colmax"],
+             configs.bytes_c5_reduce() + 4 * C5,
+             lambda: lib.nh_colmax_argmax_f32(mx.ptr, am.ptr, x5.ptr, R5, C5, C5, ws, None))
+    be.rt.free(ws)
 
 
 def shape_sweep(dtype_name):
@@ -881,6 +918,9 @@ def main():
                 d["kernel_us_rocprof"] = r.get("kernel_us_rocprof")
                 d["frac_rocprof"] = round(r["frac_rocprof"], 4) if r.get("frac_rocprof") else None
                 d["traffic"] = r.get("traffic")
+            elif r.get("kernel_us_rocprof"):           # a prebuilt kernel, found by a part of its name
+                d["kernel_us_rocprof"] = r["kernel_us_rocprof"]
+                d["frac_rocprof"] = round(r["frac_rocprof"], 4)
             return d
         line["per_config"] = [short(r) for r in per_config]
     print(json.dumps(line))

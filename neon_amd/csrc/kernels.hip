@@ -140,8 +140,8 @@ template <class F> int launch_ew(const F& f, size_t n, bool vec_ok, void* stream
 // Row normalisation, fp16 storage / fp32 statistics.  One workgroup of 1024
 // threads owns one row and keeps it in registers as raw fp16 vectors (NCH
 // chunks of 8 halves per thread), so the row is read from HBM exactly once:
-// sweep 1 sums, sweep 2 sums squared deviations, sweep 3 normalises and
-// stores.  Cross-lane sums use DPP; LDS only joins the 16 waves.
+// sweep 1 takes sum and second moment per lane while the tiles arrive, sweep 2
+// normalises and stores.  Cross-lane sums use DPP; LDS only joins the 16 waves.
 // ---------------------------------------------------------------------------
 constexpr int RN_T = 1024;
 constexpr int RN_V = 8;
@@ -174,31 +174,39 @@ __global__ __launch_bounds__(RN_T) void rownorm_f16_kernel(nh_f16* out, const nh
     const float g = gamma[row];
     const float b = beta[row];
 
+    // One pass over the tiles as they arrive takes the lane's sum and its squared deviations from a
+    // shift (the lane's first element: deviations stay small, nothing cancels); once the row's mean is
+    // known each lane's share of the row's squared deviations follows in closed form
+    //   sum (x - mean)^2 = M2_lane + n_lane * (mean_lane - mean)^2,
+    // so the second block-wide sum needs no second sweep over the registers.
     const float one = nh_opaque_one();
-    float s = 0.0f;
-#pragma unroll
-    for (int k = 0; k < NCH; ++k)
-#pragma unroll
-        for (int j = 0; j < RN_V / 2; ++j) s = nh_sum2_f16(raw[k][j], s);  // padding chunks hold zeros
-    const float mean = nh_block_allreduce<nh_op_sum, RN_T / 64>(s, slots) * inv_n;
-
-#pragma unroll
-    for (int k = 0; k < NCH; ++k) nh_keep_packed(raw[k]);
-    float q = 0.0f;
+    float s = 0.0f, sq = 0.0f, cnt = 0.0f;
+    const float shift = nh_f16_lo(raw[0][0]);           // (a lane without elements holds zeros and counts none)
 #pragma unroll
     for (int k = 0; k < NCH; ++k) {
         const uint32_t c = (uint32_t)(k * RN_T + tid) * RN_V;
         if (c < cols) {
+            cnt += (float)RN_V;
 #pragma unroll
             for (int j = 0; j < RN_V / 2; ++j) {
                 // widening and subtraction in one v_fma_mix_f32 each; the squares are
                 // accumulated with one rounding per term
-                const float d0 = __builtin_fmaf(nh_f16_lo(raw[k][j]), one, -mean);
-                const float d1 = __builtin_fmaf(nh_f16_hi(raw[k][j]), one, -mean);
-                q = __builtin_fmaf(d0, d0, q);
-                q = __builtin_fmaf(d1, d1, q);
+                const float d0 = __builtin_fmaf(nh_f16_lo(raw[k][j]), one, -shift);
+                const float d1 = __builtin_fmaf(nh_f16_hi(raw[k][j]), one, -shift);
+                sq = __builtin_fmaf(d0, d0, sq);
+                sq = __builtin_fmaf(d1, d1, sq);
+                s = nh_sum2_f16(raw[k][j], s);
             }
         }
+    }
+    const float mean = nh_block_allreduce<nh_op_sum, RN_T / 64>(s, slots) * inv_n;
+    float q = 0.0f;
+    if (cnt > 0.0f) {
+        const float sa = __builtin_fmaf(-cnt, shift, s);         // sum of (x - shift)
+        const float mu = sa / cnt;                               // lane mean - shift
+        const float m2 = nh_max(sq - sa * mu, 0.0f);             // squared deviations from the lane mean
+        const float e = (shift + mu) - mean;
+        q = __builtin_fmaf(cnt * e, e, m2);
     }
     const float var = nh_block_allreduce<nh_op_sum, RN_T / 64>(q, slots) * inv_n;
     // gamma * (x - mean) / sqrt(var + eps) + beta as (x - mean) * A + beta with A once

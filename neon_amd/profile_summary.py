@@ -47,6 +47,20 @@ def lookup(summary_path, kernel_name):
         return None
 
 
+def lookup_part(summary_path, part):
+    """as ``lookup`` for a prebuilt kernel, whose name is the compiler's: the first record
+    whose kernel name contains ``part``, or None"""
+    try:
+        with open(summary_path) as f:
+            lines = [l for l in f if l.startswith("json: ")]
+        for name, rec in json.loads(lines[-1][6:]).items():
+            if part in name:
+                return rec
+    except (IOError, OSError, IndexError, ValueError):
+        pass
+    return None
+
+
 def _dispatches(csv_path):
     """kernel name -> list of durations in ns, in dispatch order"""
     rows = []
