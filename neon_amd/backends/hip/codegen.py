@@ -2476,8 +2476,10 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
         # tag has the value.  The strip's LAST %d chunks each finish one tile of V columns: a wave per
         # column polls the records of all chunks, a wave-wide fold, and the lane that owns the tile
         # evaluates the statements.  Everybody else is done after its stores.  The finishing workgroups
-        # have the highest block numbers, so none of them starts before every other workgroup of the
-        # grid has been handed to a compute unit: they cannot keep a producer from running.
+        # have the highest block numbers.  Block numbers are dealt to the XCDs in turn and every XCD
+        # starts its share in order, so on each XCD the finishers start after all its other workgroups
+        # have: a workgroup that is still to start only ever queues behind workgroups that store and
+        # leave, never behind one that waits -- the finishers cannot keep a producer from running.
         G = S // V
         L("const int grp = (int)chunk - (nchunks - %d);" % G)
         L("if (grp < 0) return;")
