@@ -2311,7 +2311,7 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
         lds += S * (8 if g.is_pair(n) else 4)
     L("__shared__ int s_last;")
     g.declare_one()
-    lookback = bool(lookback and multi and not runs and V * 64 <= T)
+    lookback = int(lookback) if (lookback and multi and not runs and V * 64 <= T) else 0
     if lookback:
         L("__shared__ unsigned int s_tag;")
         L("__shared__ int s_abort;")
@@ -2485,29 +2485,45 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
         L("if (grp < 0) return;")
         L("const int pw = threadIdx.x >> 6, pq = threadIdx.x & 63;")
         L("const long long pc = c0 + grp * %d + pw;" % V)
-        L("const bool polls = (pw < %d) && (pq < nchunks) && (pc < C);" % V)
+        # (lane q takes the records of chunks q, q + 64, ...: PK of them)
+        PK = max(1, int(lookback))
+        L("const bool owns = (pw < %d) && (pc < C);" % V)
         for n in reds:
-            L("nh_pair rec%d = nh_pair{0.0f, 0};" % n.nid)
-        L.open("if (polls)")
+            L("nh_pair rec%d[%d];" % (n.nid, PK))
+            L("#pragma unroll")
+            L("for (int k = 0; k < %d; ++k) rec%d[k] = nh_pair{0.0f, 0};" % (PK, n.nid))
+        L.open("if (owns && pq < nchunks)")
         L("unsigned int spins = 0;")
         L.open("for (;;)")
+        L("bool seen = true;")
+        L("#pragma unroll")
+        L.open("for (int k = 0; k < %d; ++k)" % PK)
+        L.open("if (pq + 64 * k < nchunks)")
         for n in reds:
-            L("rec%d = nh_part_load(&part%d[(long long)pq * C + pc]);" % (n.nid, n.nid))
-        L("if (%s) break;" % " && ".join("nh_tag_is(rec%d, tag)" % n.nid for n in reds))
+            L("rec%d[k] = nh_part_load(&part%d[(long long)(pq + 64 * k) * C + pc]);" % (n.nid, n.nid))
+            L("seen = seen && nh_tag_is(rec%d[k], tag);" % n.nid)
+        L.close()
+        L.close()
+        L("if (seen) break;")
         L("__builtin_amdgcn_s_sleep(1);")
         L("if (++spins > NH_SPIN_LIMIT) { s_abort = 1; break; }")
         L.close()
         L.close()
         for n in reds:
             op = fold_op[n.nid]
+            ty_ = "nh_pair" if g.is_pair(n) else "float"
+            L("one%d = %s::init();" % (n.nid, op))
+            L("#pragma unroll")
+            L.open("for (int k = 0; k < %d; ++k)" % PK)
+            L.open("if (owns && pq + 64 * k < nchunks)")
             if n.is_index:
-                L("rec%d.i = (int)((nh_u32)rec%d.i | 0x80000000u);" % (n.nid, n.nid))
+                L("rec%d[k].i = (int)((nh_u32)rec%d[k].i | 0x80000000u);" % (n.nid, n.nid))
             elif g.is_pair(n):
-                L("rec%d.i = (int)((nh_u32)rec%d.i & 0x7fffffffu);" % (n.nid, n.nid))
-            if g.is_pair(n):
-                L("one%d = nh_wave_allreduce<%s, 64, nh_pair>(polls ? rec%d : %s::init());" % (n.nid, op, n.nid, op))
-            else:
-                L("one%d = nh_wave_allreduce<%s, 64, float>(polls ? rec%d.v : %s::init());" % (n.nid, op, n.nid, op))
+                L("rec%d[k].i = (int)((nh_u32)rec%d[k].i & 0x7fffffffu);" % (n.nid, n.nid))
+            L("one%d = %s::f(one%d, rec%d[k]%s);" % (n.nid, op, n.nid, n.nid, "" if g.is_pair(n) else ".v"))
+            L.close()
+            L.close()
+            L("one%d = nh_wave_allreduce<%s, 64, %s>(one%d);" % (n.nid, op, ty_, n.nid))
         L.open("if (pq == 0 && pw < %d)" % V)
         for n in reds:
             L("s_r%d[grp * %d + pw] = one%d;" % (n.nid, V, n.nid))
@@ -2612,4 +2628,4 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
     L.close()
     return _finish("colsplit", g, head, fmt, T, lds,
                    dict(V=V, LX=LX, LY=LY, NR=NR, NB=NB, NRED=len(reds), multi=bool(multi),
-                        stream=bool(stream), tail=bool(tail), runs=int(runs), lookback=bool(lookback and multi)))
+                        stream=bool(stream), tail=bool(tail), runs=int(runs), lookback=int(lookback)))

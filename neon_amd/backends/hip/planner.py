@@ -761,14 +761,18 @@ def _plan_col(prog, cu_count, coop=True, one_word_lanes=None):
                 runs = 128 // (LX * V * isz)
             elif (C * isz) % 128 != 0 and strips >= 16:
                 runs = 1
-        # The strip's last LX workgroups each finish one tile of V columns, a lane per chunk polling the
-        # others' tagged partials: needs a lane per chunk (<= 64), a wave per column of the tile, as many
-        # chunks as tiles, and block numbers that grow with the chunk (so that whoever waits was handed
-        # out after everybody it waits for).  (32000,256) fp32 on one box, ticket / tagged: max 5.6 -> 5.1
-        # us, argmax 6.9 -> 6.2 us, cross-entropy 8.3 -> 7.8 us.  Like the other waiting families it
-        # is dropped for a program whose wait once expired (coop=False).
-        lookback = (coop and COLSPLIT_LOOKBACK and not runs and 2 * LX <= chunks <= 64
+        # The strip's last LX workgroups each finish one tile of V columns, the lanes of a wave polling the
+        # chunks' tagged partials (up to four each): needs a wave per column of the tile, at least twice as
+        # many chunks as tiles, and block numbers that grow with the chunk (so that on every XCD whoever
+        # waits starts after everybody else).  (32000,256) fp32 on one box, ticket / tagged: max 5.6 -> 5.1
+        # us, argmax 6.9 -> 6.2 us, cross-entropy 8.3 -> 7.8 us; the more chunks the last ticket holder had
+        # to fold alone the more it brings: (131072,64) fp16, 128 chunks, sum 9.8 -> 6.0 us, argmax 13.0 ->
+        # 8.5; (802816,32) fp32, 224 chunks, 19.7 -> 16.3 / 21.5 -> 17.6; (400000,16) fp32 7.9 -> 5.9 /
+        # 9.5 -> 7.1.  Like the other waiting families it is dropped for a program whose wait once expired
+        # (coop=False).
+        lookback = (coop and COLSPLIT_LOOKBACK and not runs and 2 * LX <= chunks <= 256
                     and strips * chunks <= 2 * cu_count and V * 64 <= threads)
+        lookback = _ceil_div(chunks, 64) if lookback else 0      # records a polling lane takes
         spec = codegen.gen_colsplit(prog, V, LX, LY, _streams(prog), tail=tail, fold_batch=fold_batch, NR=NR,
                                     NB=codegen.COLSPLIT_SUBBATCH_ROWS, multi=chunks > 1, runs=runs, lookback=lookback)
         part_bytes = spec.params["NRED"] * chunks * C * 8
