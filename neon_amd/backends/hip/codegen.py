@@ -2311,7 +2311,7 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
         lds += S * (8 if g.is_pair(n) else 4)
     L("__shared__ int s_last;")
     g.declare_one()
-    lookback = int(lookback) if (lookback and multi and not runs and V * 64 <= T) else 0
+    lookback = int(lookback) if (lookback and multi and V * 64 <= T) else 0
     if lookback:
         L("__shared__ unsigned int s_tag;")
         L("__shared__ int s_abort;")
@@ -2334,6 +2334,7 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
         L("if (blockIdx.x % NH_XCDS >= nx || strip >= nstrips || chunk >= (unsigned int)nchunks) return;")
     else:
         L("const int nchunks = gridDim.y;")
+        L("const unsigned int nstrips = gridDim.x;")
         L("const unsigned int strip = blockIdx.x, chunk = blockIdx.y;")
     L("const int tx = threadIdx.x %% %d, ty = threadIdx.x / %d;" % (LX, LX))
     L("const long long c0 = (long long)strip * %d;" % S)
@@ -2476,10 +2477,11 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
         # tag has the value.  The strip's LAST %d chunks each finish one tile of V columns: a wave per
         # column polls the records of all chunks, a wave-wide fold, and the lane that owns the tile
         # evaluates the statements.  Everybody else is done after its stores.  The finishing workgroups
-        # have the highest block numbers.  Block numbers are dealt to the XCDs in turn and every XCD
-        # starts its share in order, so on each XCD the finishers start after all its other workgroups
-        # have: a workgroup that is still to start only ever queues behind workgroups that store and
-        # leave, never behind one that waits -- the finishers cannot keep a producer from running.
+        # are the last of their XCD to start: block numbers are dealt to the XCDs in turn, every XCD
+        # starts its share in order, and in all three block-to-(strip, chunk) mappings above the chunk
+        # grows with the block number within an XCD.  So a workgroup that is still to start only ever
+        # queues behind workgroups that store and leave, never behind one that waits -- the finishers
+        # cannot keep a producer from running.
         G = S // V
         L("const int grp = (int)chunk - (nchunks - %d);" % G)
         L("if (grp < 0) return;")
@@ -2579,7 +2581,7 @@ def gen_colsplit(prog, V, LX, LY, stream=False, tail=False, fold_batch=1, NR=4, 
         # a record never came (its workgroup was not running within the wait's bound): no result for
         # this tile, and the host is told through the plan's status word
         L.open("if (s_abort)")
-        L("unsigned int* status = reinterpret_cast<unsigned int*>(ws + ticket_offset) + %d * gridDim.x;" % TICKET_STRIDE_WORDS)
+        L("unsigned int* status = reinterpret_cast<unsigned int*>(ws + ticket_offset) + %d * nstrips;" % TICKET_STRIDE_WORDS)
         L("if (threadIdx.x == 0) __hip_atomic_store(status, NH_COOP_ABORTED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);")
         L("return;")
         L.close()

@@ -768,9 +768,11 @@ def _plan_col(prog, cu_count, coop=True, one_word_lanes=None):
         # us, argmax 6.9 -> 6.2 us, cross-entropy 8.3 -> 7.8 us; the more chunks the last ticket holder had
         # to fold alone the more it brings: (131072,64) fp16, 128 chunks, sum 9.8 -> 6.0 us, argmax 13.0 ->
         # 8.5; (802816,32) fp32, 224 chunks, 19.7 -> 16.3 / 21.5 -> 17.6; (400000,16) fp32 7.9 -> 5.9 /
-        # 9.5 -> 7.1.  Like the other waiting families it is dropped for a program whose wait once expired
-        # (coop=False).
-        lookback = (coop and COLSPLIT_LOOKBACK and not runs and 2 * LX <= chunks <= 256
+        # 9.5 -> 7.1; on the grids dealt to the XCDs in runs (rows that are no whole cache lines) (50000,250)
+        # fp16 11.4 -> 9.7 / 13.9 -> 12.0, (64000,300) fp32 23.5 -> 21.7 / 25.1 -> 23.0, (131072,1000) fp16
+        # 46.3 -> 44.4 / 56.5 -> 54.0.  Like the other waiting families it is dropped for a program whose
+        # wait once expired (coop=False).
+        lookback = (coop and COLSPLIT_LOOKBACK and 2 * LX <= chunks <= 256
                     and strips * chunks <= 2 * cu_count and V * 64 <= threads)
         lookback = _ceil_div(chunks, 64) if lookback else 0      # records a polling lane takes
         spec = codegen.gen_colsplit(prog, V, LX, LY, _streams(prog), tail=tail, fold_batch=fold_batch, NR=NR,

@@ -1133,7 +1133,8 @@ def test_split_column_reductions_with_strips_dealt_to_xcds_in_runs(hip, shape, d
 
 @pytest.mark.parametrize("shape,dtype", [((32000, 256), np.float32), ((16000, 250), np.float32), ((30000, 264), np.float16),
                                          ((8192, 1024), np.float32), ((40000, 96), np.float32), ((6000, 509), np.float16),
-                                         ((131072, 64), np.float32), ((100000, 64), np.float16), ((400000, 16), np.float32)])
+                                         ((131072, 64), np.float32), ((100000, 64), np.float16), ((400000, 16), np.float32),
+                                         ((50000, 250), np.float16), ((64000, 300), np.float32)])
 def test_split_column_reductions_finished_by_the_last_workgroups_of_a_strip(hip, shape, dtype):
     """the split column family where the strip's last workgroups wait for the
     others' tagged partials (a tag bit inside each 8-byte record, flipped every
@@ -1170,5 +1171,7 @@ def test_split_column_reductions_finished_by_the_last_workgroups_of_a_strip(hip,
         assert np.array_equal(mn.get(), xn.astype(np.float32).min(axis=0, keepdims=True), equal_nan=True)
         m = x64.max(axis=0)
         assert_close(lse.get().ravel(), np.log(np.exp(x64 - m).sum(axis=0)) + m, rtol=RTOL32, atol=1e-5, what="log-sum-exp")
-    if shape in ((32000, 256), (131072, 64), (100000, 64), (400000, 16)):   # (the last three: several records per polling lane)
+    # ((131072,64), (100000,64), (400000,16): several records per polling lane; (50000,250), (64000,300): grids
+    # that deal chunks to the XCDs in runs)
+    if shape in ((32000, 256), (131072, 64), (100000, 64), (400000, 16), (50000, 250), (64000, 300)):
         assert tagged == 2, "this shape should take the tagged form"

@@ -136,8 +136,14 @@ def test_a_cooperative_kernel_that_gave_up_is_reported_and_replaced(pair, family
     again = run(hip)
     got = again.get()
     assert_close(got, want, rtol=1e-5, atol=1e-6, what=family + " after the fallback")
-    assert all(p.status_ptr is None for k, p in hip.plans.items() if k not in before), \
-        "the replacement must not wait between workgroups"
+    # (a split column reduction among the replacement's stages may finish through tagged records: only the
+    # strip's last workgroups wait there, for workgroups that started before them, so it does not need the
+    # whole grid resident; the program that gave up itself is planned without any wait)
+    fresh = dict((k, p) for k, p in hip.plans.items() if k not in before)
+    assert all(p.spec.family not in ("colcoop", "rowcoop") for p in fresh.values()), \
+        "the replacement must not need all its workgroups resident at once"
+    if plan.key in fresh:
+        assert fresh[plan.key].status_ptr is None
     del out
 
 
