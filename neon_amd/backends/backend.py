@@ -47,18 +47,21 @@ _NO_OPERAND, _SCALAR_SHAPE = (0, 0), (1, 1)
 # builder of elementwise nodes in C (neon_amd/csrc/fastpath.c), installed by
 # ``use_c_node_builder``; None: nodes are built by ``OpTreeNode.build`` alone
 _c_ew_node = None
+_c_red_node = None
 
 
 def use_c_node_builder(module):
     """Let ``OpTreeNode.build`` hand elementwise nodes without keyword
-    arguments to ``module.ew_node`` (same nodes, a third of the time);
-    ``None`` switches back to Python."""
-    global _c_ew_node
+    arguments to ``module.ew_node``, and the reduction builders theirs
+    (one axis, no ``out=``) to ``module.red_node`` (same nodes, a third of
+    the time); ``None`` switches back to Python."""
+    global _c_ew_node, _c_red_node
     if module is None:
-        _c_ew_node = None
+        _c_ew_node = _c_red_node = None
         return
-    module.configure_builder(OpTreeNode, Tensor, sorted(_EW_NOT_ASSIGN))
+    module.configure_builder(OpTreeNode, Tensor, sorted(_EW_NOT_ASSIGN), sorted(OpCollection.reduction_ops))
     _c_ew_node = module.ew_node
+    _c_red_node = getattr(module, "red_node", None)
 
 
 def _shape_of_operand(x):
@@ -695,6 +698,10 @@ class Backend(metaclass=_BackendRegistry):
 
     # -- reductions and derived statistics (reference backend.py:1313-1502) ---
     def _reduce(self, op, a, axis, out):
+        if out is None and _c_red_node is not None:
+            node = _c_red_node(op, a, axis)          # (None: not an axis-0/1 reduction of a tensor or node)
+            if node is not None:
+                return node
         if axis is None:
             # whole-tensor reduction = axis 0 then axis 1
             inner = OpTreeNode.build(op, a, None, axis=0)
@@ -711,9 +718,17 @@ class Backend(metaclass=_BackendRegistry):
         return self._reduce("min", a, axis, out)
 
     def argmax(self, a, axis=1, out=None, keepdims=True):
+        if out is None and _c_red_node is not None:
+            node = _c_red_node("argmax", a, axis)
+            if node is not None:
+                return node
         return OpTreeNode.build("argmax", a, None, axis=axis, out=out)
 
     def argmin(self, a, axis=1, out=None, keepdims=True):
+        if out is None and _c_red_node is not None:
+            node = _c_red_node("argmin", a, axis)
+            if node is not None:
+                return node
         return OpTreeNode.build("argmin", a, None, axis=axis, out=out)
 
     def mean(self, a, axis=None, partial=None, out=None, keepdims=True):
@@ -907,3 +922,73 @@ class Backend(metaclass=_BackendRegistry):
             out = self.empty_like(ary) if hasattr(ary, "shape") else self.empty((1, 1))
         out[:] = self.multiply(ary, ap2)
         return out
+
+
+# -- the operators and builders above, entered through the C node builder ----------------------
+# Every arithmetic operator and elementwise builder is a Python call into ``OpTreeNode.build``,
+# which (for the common case) is a call into ``ew_node``: the wrappers below go to ``ew_node``
+# first and to the definition above whenever it says "not mine" (or is not installed), which
+# saves a Python frame and a keyword dictionary per node -- a quarter of a microsecond each.
+def _operator_via_c(op, slow, swap):
+    if swap:
+        def method(self, other):
+            f = _c_ew_node
+            if f is not None:
+                node = f(op, other, self)
+                if node is not None:
+                    return node
+            return slow(self, other)
+    else:
+        def method(self, other):
+            f = _c_ew_node
+            if f is not None:
+                node = f(op, self, other)
+                if node is not None:
+                    return node
+            return slow(self, other)
+    method.__name__, method.__qualname__, method.__doc__ = slow.__name__, slow.__qualname__, slow.__doc__
+    return method
+
+
+def _builder_via_c(op, slow, operands):
+    if operands == 1:
+        def method(self, a, out=None):
+            if out is None:
+                f = _c_ew_node
+                if f is not None:
+                    node = f(op, a, None)
+                    if node is not None:
+                        return node
+            return slow(self, a, out)
+    else:
+        def method(self, a, b, out=None):
+            if out is None:
+                f = _c_ew_node
+                if f is not None:
+                    node = f(op, a, b)
+                    if node is not None:
+                        return node
+            return slow(self, a, b, out)
+    method.__name__, method.__qualname__, method.__doc__ = slow.__name__, slow.__qualname__, slow.__doc__
+    return method
+
+
+for _name, _op, _swap in (("__add__", "add", False), ("__radd__", "add", True), ("__sub__", "sub", False),
+                          ("__rsub__", "sub", True), ("__mul__", "mul", False), ("__rmul__", "mul", True),
+                          ("__truediv__", "div", False), ("__rtruediv__", "div", True), ("__pow__", "pow", False),
+                          ("__rpow__", "pow", True), ("__eq__", "eq", False), ("__ne__", "ne", False),
+                          ("__lt__", "lt", False), ("__le__", "le", False), ("__gt__", "gt", False),
+                          ("__ge__", "ge", False)):
+    setattr(_LazyOperators, _name, _operator_via_c(_op, getattr(_LazyOperators, _name), _swap))
+_LazyOperators.__div__, _LazyOperators.__rdiv__ = _LazyOperators.__truediv__, _LazyOperators.__rtruediv__
+for _name, _op, _n in (("add", "add", 2), ("subtract", "sub", 2), ("multiply", "mul", 2), ("divide", "div", 2),
+                       ("power", "pow", 2), ("negative", "neg", 1), ("sgn", "sgn", 1), ("absolute", "abs", 1),
+                       ("sqrt", "sqrt", 1), ("square", "sqr", 1), ("exp", "exp", 1), ("exp2", "exp2", 1),
+                       ("safelog", "safelog", 1), ("log", "log", 1), ("log2", "log2", 1), ("sig", "sig", 1),
+                       ("sig2", "sig2", 1), ("tanh", "tanh", 1), ("tanh2", "tanh2", 1), ("finite", "finite", 1),
+                       ("rint", "rint", 1), ("equal", "eq", 2), ("not_equal", "ne", 2), ("less", "lt", 2),
+                       ("less_equal", "le", 2), ("greater", "gt", 2), ("greater_equal", "ge", 2),
+                       ("maximum", "maximum", 2), ("minimum", "minimum", 2)):
+    setattr(Backend, _name, _builder_via_c(_op, getattr(Backend, _name), _n))
+Backend.true_divide, Backend.fabs = Backend.divide, Backend.absolute
+del _name, _op, _swap, _n

@@ -444,11 +444,12 @@ static PyTypeObject ReplayerType = {
  * shapes; numbers are 1x1, a missing operand 0x0, 1-d shapes padded to 2-d).  Anything it
  * is not sure about -- an op outside the set, an operand of an unknown type, a shape that is
  * not one or two integers -- is answered with None and Python takes over. */
-static PyObject *b_node_cls, *b_tensor_cls, *b_ew_ops, *s_shape, *t_scalar, *t_none;
+static PyObject *b_node_cls, *b_tensor_cls, *b_ew_ops, *b_red_ops, *s_shape, *t_scalar, *t_none;
 
 static PyObject* builder_configure(PyObject* self, PyObject* args) {
-    PyObject *node_cls, *tensor_cls, *ops;
-    if (!PyArg_ParseTuple(args, "O!O!O:configure_builder", &PyType_Type, &node_cls, &PyType_Type, &tensor_cls, &ops))
+    PyObject *node_cls, *tensor_cls, *ops, *red_ops = NULL;
+    if (!PyArg_ParseTuple(args, "O!O!O|O:configure_builder", &PyType_Type, &node_cls, &PyType_Type, &tensor_cls, &ops,
+                          &red_ops))
         return NULL;
     if (!PyType_IsSubtype((PyTypeObject*)node_cls, &PyTuple_Type)) {
         PyErr_SetString(PyExc_TypeError, "the node class must derive from tuple");
@@ -456,9 +457,12 @@ static PyObject* builder_configure(PyObject* self, PyObject* args) {
     }
     PyObject* frozen = PyFrozenSet_New(ops);
     if (!frozen) return NULL;
+    PyObject* frozen_red = PyFrozenSet_New(red_ops);      /* (NULL: the empty set) */
+    if (!frozen_red) { Py_DECREF(frozen); return NULL; }
     Py_INCREF(node_cls); Py_XSETREF(b_node_cls, node_cls);
     Py_INCREF(tensor_cls); Py_XSETREF(b_tensor_cls, tensor_cls);
     Py_XSETREF(b_ew_ops, frozen);
+    Py_XSETREF(b_red_ops, frozen_red);
     Py_RETURN_NONE;
 }
 
@@ -529,9 +533,45 @@ static PyObject* builder_ew_node(PyObject* self, PyObject* const* args, Py_ssize
     return node;
 }
 
+/* OpTreeNode.build(op, a, None, axis=axis) for a reduction along axis 0 or 1 of a two-dimensional operand:
+ * {"op", "shape", "axis"} with the operand's shape, that axis set to 1.  None: Python builds it. */
+static PyObject* builder_red_node(PyObject* self, PyObject* const* args, Py_ssize_t nargs) {
+    if (nargs != 3) { PyErr_SetString(PyExc_TypeError, "red_node(op, a, axis)"); return NULL; }
+    if (!b_node_cls || !b_red_ops || !PyLong_CheckExact(args[2])) Py_RETURN_NONE;
+    int known = PySet_Contains(b_red_ops, args[0]);
+    if (known < 0) return NULL;
+    if (!known) Py_RETURN_NONE;
+    const long axis = PyLong_AsLong(args[2]);
+    if (axis == -1 && PyErr_Occurred()) { PyErr_Clear(); Py_RETURN_NONE; }
+    if (axis != 0 && axis != 1) Py_RETURN_NONE;
+    Py_ssize_t ra, ca;
+    PyObject* ka;
+    if (args[1] == Py_None || PyFloat_Check(args[1]) || PyLong_Check(args[1])) Py_RETURN_NONE;
+    int ok = operand_shape(args[1], &ra, &ca, &ka);
+    if (ok < 0) return NULL;
+    if (!ok) Py_RETURN_NONE;
+    PyObject* shape = axis == 0 ? Py_BuildValue("(in)", 1, ca) : Py_BuildValue("(ni)", ra, 1);
+    if (!shape) return NULL;
+    PyObject* d = PyDict_New();
+    if (!d || PyDict_SetItem(d, s_op, args[0]) < 0 || PyDict_SetItem(d, s_shape, shape) < 0 ||
+        PyDict_SetItem(d, s_axis, args[2]) < 0) {
+        Py_XDECREF(d); Py_DECREF(shape); return NULL;
+    }
+    Py_DECREF(shape);
+    PyTypeObject* cls = (PyTypeObject*)b_node_cls;
+    PyObject* node = cls->tp_alloc(cls, 3);
+    if (!node) { Py_DECREF(d); return NULL; }
+    PyTuple_SET_ITEM(node, 0, d);
+    Py_INCREF(args[1]); PyTuple_SET_ITEM(node, 1, args[1]);
+    Py_INCREF(Py_None); PyTuple_SET_ITEM(node, 2, Py_None);
+    return node;
+}
+
 static PyMethodDef module_methods[] = {
     {"configure_builder", builder_configure, METH_VARARGS,
-     "configure_builder(node class, tensor class, elementwise op names)"},
+     "configure_builder(node class, tensor class, elementwise op names[, reduction op names])"},
+    {"red_node", (PyCFunction)(void (*)(void))builder_red_node, METH_FASTCALL,
+     "red_node(op, a, axis) -> node, or None when Python has to build it"},
     {"ew_node", (PyCFunction)(void (*)(void))builder_ew_node, METH_FASTCALL,
      "ew_node(op, a, b) -> node, or None when Python has to build it"},
     {NULL, NULL, 0, NULL}};

@@ -411,6 +411,79 @@ def test_c_node_builder_builds_the_nodes_python_builds():
     assert checked > 2000
 
 
+def test_c_node_builder_builds_the_reductions_python_builds():
+    """every reduction over every kind of operand and axis through the
+    backend's builders, with the C builder and without: same node class, same
+    op dict (same key order), same operand -- or the same refusal; and the
+    operators and elementwise builders that go to the C builder first give
+    what ``OpTreeNode.build`` gives"""
+    import neon_amd.backends  # noqa: F401
+    from neon_amd.backends import backend as api
+    from neon_amd.backends.backend import OpCollection, OpTreeNode
+    assert api._c_red_node is not None
+    be = PlanBackend(compile_kernels=False)
+    full, col, row, one = be.empty((5, 7)), be.empty((5, 1)), be.empty((1, 7)), be.empty((1, 1))
+    vec = ShapeTensor(be, (9,))
+    vec.shape = (9,)
+    cube = be.empty((5, 1))
+    cube.shape = (2, 3, 4)
+    node = full * col
+    operands = [full, col, row, one, vec, cube, node, be.sum(full, axis=0), 2.5, 3, None, "text"]
+    axes = [0, 1, None, -1, 2, True, 1.0, "0"]
+    c_ew, c_red = api._c_ew_node, api._c_red_node
+
+    def both(make):
+        results = []
+        for use_c in (True, False):
+            api._c_ew_node, api._c_red_node = (c_ew, c_red) if use_c else (None, None)
+            try:
+                results.append(make())
+            except Exception as e:                       # noqa: BLE001  (compared, not handled)
+                results.append(type(e))
+        api._c_ew_node, api._c_red_node = c_ew, c_red
+        return results
+
+    def same(got, want, what):
+        if isinstance(want, tuple):
+            assert type(got) is type(want) is OpTreeNode, what
+            assert got[0] == want[0] and list(got[0]) == list(want[0]), (what, got[0], want[0])
+            assert type(got[0]["shape"]) is tuple
+            for g, w in zip(got[1:], want[1:]):
+                if isinstance(w, tuple):
+                    same(g, w, what)                     # (sum over everything: a reduction of a reduction)
+                else:
+                    assert g is w, what
+        else:
+            assert got is want, (what, got, want)
+
+    built = 0
+    for name in sorted(OpCollection.reduction_ops):
+        for a in operands:
+            for axis in axes:
+                got, want = both(lambda: getattr(be, name)(a, axis=axis))
+                same(got, want, (name, a, axis))
+                built += isinstance(want, tuple)
+                direct = c_red(name, a, axis)
+                assert direct is None or (axis in (0, 1) and type(axis) is int and isinstance(want, tuple))
+    assert built > 150
+    assert c_red("add", full, 0) is None and c_red("bogus", full, 0) is None
+    with pytest.raises(TypeError):
+        c_red("sum", full)
+    # operators and elementwise builders
+    pairs = [(full, col), (col, full), (full, 2.5), (3, row), (node, one), (full, "text"), (None, full)]
+    for a, b in pairs:
+        for make in (lambda: a + b, lambda: a - b, lambda: a * b, lambda: a / b, lambda: a ** b, lambda: a == b,
+                     lambda: a != b, lambda: a < b, lambda: a <= b, lambda: a > b, lambda: a >= b,
+                     lambda: be.add(a, b), lambda: be.subtract(a, b), lambda: be.multiply(a, b), lambda: be.divide(a, b),
+                     lambda: be.maximum(a, b), lambda: be.minimum(a, b), lambda: be.power(a, b), lambda: be.less(a, b),
+                     lambda: be.exp(a), lambda: be.log(b), lambda: be.sqrt(a), lambda: be.sig(a), lambda: be.tanh(b),
+                     lambda: be.square(a), lambda: be.absolute(a), lambda: be.negative(b), lambda: be.rint(a)):
+            got, want = both(make)
+            same(got, want, (a, b))
+    assert be.true_divide.__func__ is be.divide.__func__ and be.fabs.__func__ is be.absolute.__func__
+    assert type(full).__div__ is type(full).__truediv__
+
+
 def test_the_extension_is_clean_under_address_and_undefined_behaviour_sanitizers(tmp_path):
     """fastpath.c built with -fsanitize=address,undefined and this file's CPU
     tests (key walks, node builder, records, error paths) run against that
